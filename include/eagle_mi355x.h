@@ -1,0 +1,199 @@
+/*
+ * eagle_mi355x.h - C ABI of the MI355X (gfx950) EAGLE-2 tree-verification kernels.
+ *
+ * Plain pointers and sizes only.  Every pointer argument named `*_dev` or typed
+ * as tensor data is a DEVICE pointer; `stream` is a hipStream_t passed as void*.
+ * All entry points are asynchronous and stream ordered, never synchronise,
+ * never allocate and never retain pointers.  Half-precision tensors are IEEE
+ * binary16.  Return value: 0 on success, an eagle_status code otherwise;
+ * argument errors are detected on the host before any device work is issued.
+ *
+ * Each declaration cites the reference interface it replaces
+ * (file:line in 0seba/mlx-eagle-spec-decoding-tree).
+ */
+#ifndef EAGLE_MI355X_H
+#define EAGLE_MI355X_H
+
+#include <stddef.h>
+#include <stdint.h>
+
+#ifdef __cplusplus
+extern "C" {
+#endif
+
+typedef void* eagle_stream_t; /* hipStream_t */
+
+enum eagle_status {
+  EAGLE_OK = 0,
+  EAGLE_ERR_NULL = 1,        /* required pointer is NULL */
+  EAGLE_ERR_SHAPE = 2,       /* a dimension is out of the supported range */
+  EAGLE_ERR_ALIGN = 3,       /* pointer not 16-byte aligned */
+  EAGLE_ERR_UNSUPPORTED = 4, /* group_size != 64 or bits != 4 */
+  EAGLE_ERR_WORKSPACE = 5,   /* workspace missing or too small */
+  EAGLE_ERR_HIP = 6,         /* the HIP runtime reported a launch error */
+  EAGLE_ERR_ARCH = 7         /* current device is not gfx950 */
+};
+
+#define EAGLE_MAX_TREE 32    /* tree tokens per verify step (root + 31 nodes) */
+#define EAGLE_MAX_M 32       /* rows of x accepted by the quantised matmul */
+
+const char* eagle_status_string(int status);
+int eagle_abi_version(void);
+/* 0 if the current HIP device is gfx950, EAGLE_ERR_ARCH / EAGLE_ERR_HIP otherwise. */
+int eagle_check_device(void);
+
+/* ---------------------------------------------------------------------------
+ * 4-bit affine quantised matmul, group size 64 (MLX layout).
+ *   out[m,n] = fp16( sum_k x[m,k] * (scales[n,k/64]*q[n,k] + biases[n,k/64]) ) (+ bias[n])
+ *   q[n,k] = (wq[n,k/8] >> 4*(k%8)) & 15
+ *   x [M,K] fp16 row-major, wq [N,K/8] uint32, scales/biases [N,K/64] fp16,
+ *   bias [N] fp16 or NULL (added in fp16 after rounding), out [M,N] fp16.
+ * Constraints: 1 <= M <= 32, K % 64 == 0, N % 8 == 0, group_size == 64, bits == 4.
+ * Replaces qmm_kernel.matmul (qmm_kernel.py:84-164) with the body
+ * kernels/progression/simd_no_swizzle_cast.metal, the mx.quantized_matmul
+ * fallback of the patched layer (mlx_model_fwd_bench.py:65-73) and its bias add
+ * (:70-71).
+ * `workspace` holds split-K partial sums and arrival counters; its first
+ * EAGLE_QMM_COUNTER_BYTES bytes must be zero before the first call (they are
+ * left zero by every call).  Calls sharing a workspace must be stream ordered.
+ * ------------------------------------------------------------------------- */
+#define EAGLE_QMM_COUNTER_BYTES 16384
+size_t eagle_qmm_workspace_bytes(int M, int N, int K);
+int eagle_qmm_w4g64_f16(const void* x, const uint32_t* wq, const void* scales,
+                        const void* biases, const void* bias, void* out,
+                        int M, int N, int K, int group_size, int bits,
+                        void* workspace, size_t workspace_bytes, eagle_stream_t stream);
+/* Same, with the launch configuration forced (tuning sweeps and tests):
+ * variant indexes the compiled tile shapes, splits is the split-K factor.
+ * eagle_qmm_num_variants() variants exist; variant < 0 selects the heuristic. */
+int eagle_qmm_num_variants(void);
+size_t eagle_qmm_workspace_bytes_cfg(int M, int N, int K, int variant, int splits);
+const char* eagle_qmm_variant_name(int variant);
+int eagle_qmm_w4g64_f16_cfg(const void* x, const uint32_t* wq, const void* scales,
+                            const void* biases, const void* bias, void* out,
+                            int M, int N, int K, int variant, int splits,
+                            void* workspace, size_t workspace_bytes, eagle_stream_t stream);
+
+/* Quantised embedding gather: out[t,:] = fp16(scales*q + biases) of row ids[t].
+ * ids [T] int32, out [T,D] fp16, D % 64 == 0.  Replaces the quantised
+ * nn.Embedding lookup of mlx_llama.py:273. */
+int eagle_embed_w4g64_f16(const int32_t* ids, const uint32_t* wq, const void* scales,
+                          const void* biases, void* out, int T, int D, int V,
+                          eagle_stream_t stream);
+
+/* ---------------------------------------------------------------------------
+ * RoPE with one position per (batch, token), half-split pairing, fp32 math.
+ *   x, out [B,H,L,hd] fp16 contiguous; positions [B,L] int32; inv_freqs [hd/2] fp32.
+ * Replaces rope_positions (mlx_arrayed_rope_kernel.py:46-152).
+ * ------------------------------------------------------------------------- */
+int eagle_rope_arrayed_f16(const void* x, const int32_t* positions, const float* inv_freqs,
+                           float scaling_factor, void* out, int B, int H, int L, int hd,
+                           eagle_stream_t stream);
+
+/* Fused form used inside the decoder layer: takes the token-major projections
+ * q_lin [T,H*hd], k_lin [T,G*hd], v_lin [T,G*hd], rotates q and k at
+ * positions[t] and writes q_out [H,T,hd] plus rows *cache_len_dev + t of the
+ * K/V caches ([G,capacity,hd]).  Covers mlx_llama.py:134-161 and the cache
+ * append of :178. */
+int eagle_rope_kv_append_f16(const void* q_lin, const void* k_lin, const void* v_lin,
+                             const int32_t* positions, const float* inv_freqs,
+                             float scaling_factor, void* q_out, void* k_cache, void* v_cache,
+                             const int32_t* cache_len_dev, int T, int H, int G, int hd,
+                             long capacity, eagle_stream_t stream);
+
+/* ---------------------------------------------------------------------------
+ * Tree-masked grouped-query attention of T <= 32 tree tokens against the cache.
+ *   q [H,T,hd] fp16 (rotated), k_cache/v_cache [G,capacity,hd] fp16 holding
+ *   P = *cache_len_dev prefix rows followed by the T tree rows,
+ *   tree_mask_bits [T] uint32: bit j of word i set iff tree token j is visible
+ *   to tree token i; prefix rows are visible to every token.
+ *   out [T,H*hd] fp16 = softmax(scale*q.k + mask) v, laid out for o_proj.
+ * hd must be 64 or 128.  Replaces scaled_dot_product_attention with the additive
+ * tree mask (mlx_llama.py:185-195, mask from mlx_eagle.py:337-338).
+ * ------------------------------------------------------------------------- */
+/* max_len bounds prefix + tree rows (P + T) for every launch that uses the workspace. */
+size_t eagle_tree_attention_workspace_bytes(int H, int hd, int max_len);
+int eagle_tree_attention_f16(const void* q, const void* k_cache, const void* v_cache,
+                             const uint32_t* tree_mask_bits, const int32_t* cache_len_dev,
+                             void* out, int T, int H, int G, int hd, long capacity,
+                             int max_len, float scale, void* workspace,
+                             size_t workspace_bytes, eagle_stream_t stream);
+
+/* RMSNorm (mlx_llama.py:225-228,240,247,286): out = w * x * rsqrt(mean(x^2)+eps),
+ * fp32 math; x, out [T,D] fp16, w [D] fp16.  With `residual` non-NULL the kernel
+ * first forms h = fp16(x + residual), stores it to h_out and normalises h
+ * (the residual adds of mlx_llama.py:246,248 fused with the following norm). */
+int eagle_rmsnorm_f16(const void* x, const void* residual, const void* w, float eps,
+                      void* h_out, void* out, int T, int D, eagle_stream_t stream);
+
+/* out = fp16( fp16(silu(g)) * u ); g, u are the two halves of gate_up [T,2*I]
+ * when `up` is NULL (g = gate_up[:, :I], u = gate_up[:, I:]) or separate [T,I]
+ * tensors.  mlx_llama.py:215. */
+int eagle_silu_mul_f16(const void* gate, const void* up, void* out, int T, int I,
+                       eagle_stream_t stream);
+
+/* out = fp16(a + b), n elements (residual add, mlx_llama.py:246,248). */
+int eagle_add_f16(const void* a, const void* b, void* out, long n, eagle_stream_t stream);
+
+/* Row argmax of fp16 logits [R,V], lowest index among equal maxima
+ * (mx.argmax at mlx_eagle.py:316,534,596).  out [R] int32. */
+size_t eagle_argmax_workspace_bytes(int R, long V);
+int eagle_argmax_rows_f16(const void* logits, int32_t* out, int R, long V,
+                          void* workspace, size_t workspace_bytes, eagle_stream_t stream);
+
+/* ---------------------------------------------------------------------------
+ * Tree construction and acceptance (integer work, single workgroup kernels).
+ * ------------------------------------------------------------------------- */
+
+/* process_draft_tree (mlx_eagle.py:217-250): from C = k + k*k*depth candidate
+ * scores (fp16, flat), their token ids and the parent table, pick the `total`
+ * best (descending score, ties to the lowest flat index), order them by flat
+ * index and emit
+ *   tree_position_ids [T] int32, mask_index [total] int32, draft_tokens [T] int32,
+ *   tree_mask_bits [T] uint32 (ancestor-or-self rows), T = total + 1 <= 32.
+ * parents_list [C/k] uint32: 0 for the root's children, else parent flat id + 1.
+ * sampled_token_dev: the root token. */
+int eagle_process_draft_tree(const void* scores, const int32_t* tokens,
+                             const uint32_t* parents_list, const int32_t* sampled_token_dev,
+                             int C, int k, int total, int32_t* tree_position_ids,
+                             int32_t* mask_index, int32_t* draft_tokens,
+                             uint32_t* tree_mask_bits, eagle_stream_t stream);
+
+/* post_process_draft_tree (mlx_eagle.py:254-295) without the host round trip:
+ * retrieve_indices [32,32] int32 (row r = path of the r-th leaf, -1 padded),
+ * shape_out [2] int32 = {leaf_num, max_depth + 1}. */
+int eagle_post_process_draft_tree(const int32_t* tree_position_ids, const int32_t* mask_index,
+                                  int total, int32_t* retrieve_indices, int32_t* shape_out,
+                                  eagle_stream_t stream);
+
+/* Greedy acceptance (evaluate_posterior_greedy, mlx_eagle.py:311-326, with the
+ * gathers of :582-589).  node_argmax [T] is the argmax token of each tree node's
+ * logits.  retrieve_indices [32,32] / shape as produced above; a -1 entry
+ * selects node T-1, as the reference's negative gather index does.
+ * result [4 + 32] int32 = {best, accept_length, bonus_node, next_token,
+ * accept_indices[0..accept_length)}; accepted_tokens [32] int32. */
+int eagle_greedy_accept(const int32_t* node_argmax, const int32_t* draft_tokens,
+                        const int32_t* retrieve_indices, const int32_t* shape, int T,
+                        int32_t* result, int32_t* accepted_tokens, eagle_stream_t stream);
+
+/* accept_candidate (mlx_eagle.py:349-376) for n_caches K or V buffers at once:
+ * rows P + accept_indices[j] move to P + 1 + j for j < accept_length (gather
+ * first, then scatter), then *cache_len_dev = P + accept_length + 1.
+ * caches: device array of n_caches pointers to [G,capacity,hd] fp16 buffers.
+ * accept [4 + 32] int32 in the layout of eagle_greedy_accept's result. */
+int eagle_kv_compact_f16(void* const* caches_dev, int n_caches, const int32_t* accept,
+                         int32_t* cache_len_dev, int G, int hd, long capacity,
+                         eagle_stream_t stream);
+
+/* Small device-side helpers for graph-replayed steps. */
+int eagle_fill_i32(int32_t* dst, int32_t value, long n, eagle_stream_t stream);
+/* positions[t] = *cache_len_dev + tree_position_ids[t] (mlx_eagle.py:343). */
+int eagle_tree_positions(const int32_t* tree_position_ids, const int32_t* cache_len_dev,
+                         int32_t* positions, int T, eagle_stream_t stream);
+/* *cache_len_dev += delta (KVCache.offset bookkeeping after an append). */
+int eagle_advance_len(int32_t* cache_len_dev, int delta, eagle_stream_t stream);
+
+#ifdef __cplusplus
+}
+#endif
+#endif /* EAGLE_MI355X_H */

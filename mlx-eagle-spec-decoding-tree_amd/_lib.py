@@ -1,0 +1,81 @@
+"""ctypes binding of libeagle_mi355x.so (declared in include/eagle_mi355x.h).
+
+The library is never built or replaced at import time: a missing library is a
+hard error (there is no CPU or eager fallback).  Build it with
+`python -m mlx_eagle_spec_decoding_tree_amd.build`.
+"""
+import ctypes
+import os
+from ctypes import c_char_p, c_float, c_int, c_int32, c_long, c_size_t, c_void_p
+
+HERE = os.path.dirname(os.path.abspath(__file__))
+LIB_PATH = os.path.join(HERE, "libeagle_mi355x.so")
+
+_lib = None
+
+# name -> (restype, argtypes); must list every symbol the header declares
+SIGNATURES = {
+    "eagle_status_string": (c_char_p, [c_int]),
+    "eagle_abi_version": (c_int, []),
+    "eagle_check_device": (c_int, []),
+    "eagle_qmm_workspace_bytes": (c_size_t, [c_int, c_int, c_int]),
+    "eagle_qmm_w4g64_f16": (c_int, [c_void_p] * 6 + [c_int] * 5 + [c_void_p, c_size_t, c_void_p]),
+    "eagle_qmm_num_variants": (c_int, []),
+    "eagle_qmm_workspace_bytes_cfg": (c_size_t, [c_int] * 5),
+    "eagle_qmm_variant_name": (c_char_p, [c_int]),
+    "eagle_qmm_w4g64_f16_cfg": (c_int, [c_void_p] * 6 + [c_int] * 5 + [c_void_p, c_size_t, c_void_p]),
+    "eagle_embed_w4g64_f16": (c_int, [c_void_p] * 5 + [c_int] * 3 + [c_void_p]),
+    "eagle_rope_arrayed_f16": (c_int, [c_void_p] * 3 + [c_float, c_void_p] + [c_int] * 4 + [c_void_p]),
+    "eagle_rope_kv_append_f16": (c_int, [c_void_p] * 5 + [c_float] + [c_void_p] * 4 + [c_int] * 4
+                                 + [c_long, c_void_p]),
+    "eagle_tree_attention_workspace_bytes": (c_size_t, [c_int, c_int, c_int]),
+    "eagle_tree_attention_f16": (c_int, [c_void_p] * 6 + [c_int] * 4 + [c_long, c_int, c_float,
+                                                                       c_void_p, c_size_t, c_void_p]),
+    "eagle_rmsnorm_f16": (c_int, [c_void_p] * 3 + [c_float] + [c_void_p] * 2 + [c_int] * 2 + [c_void_p]),
+    "eagle_silu_mul_f16": (c_int, [c_void_p] * 3 + [c_int] * 2 + [c_void_p]),
+    "eagle_add_f16": (c_int, [c_void_p] * 3 + [c_long, c_void_p]),
+    "eagle_argmax_workspace_bytes": (c_size_t, [c_int, c_long]),
+    "eagle_argmax_rows_f16": (c_int, [c_void_p] * 2 + [c_int, c_long, c_void_p, c_size_t, c_void_p]),
+    "eagle_process_draft_tree": (c_int, [c_void_p] * 4 + [c_int] * 3 + [c_void_p] * 5),
+    "eagle_post_process_draft_tree": (c_int, [c_void_p] * 2 + [c_int] + [c_void_p] * 3),
+    "eagle_greedy_accept": (c_int, [c_void_p] * 4 + [c_int] + [c_void_p] * 3),
+    "eagle_kv_compact_f16": (c_int, [c_void_p, c_int, c_void_p, c_void_p, c_int, c_int, c_long, c_void_p]),
+    "eagle_fill_i32": (c_int, [c_void_p, c_int32, c_long, c_void_p]),
+    "eagle_tree_positions": (c_int, [c_void_p] * 3 + [c_int, c_void_p]),
+    "eagle_advance_len": (c_int, [c_void_p, c_int, c_void_p]),
+}
+
+
+class EagleLibraryMissing(RuntimeError):
+    pass
+
+
+def lib():
+    """The loaded C-ABI library; raises if it has not been built."""
+    global _lib
+    if _lib is None:
+        if not os.path.exists(LIB_PATH):
+            raise EagleLibraryMissing(
+                f"{LIB_PATH} not found: build the HIP extension first "
+                "(python -m mlx_eagle_spec_decoding_tree_amd.build); there is no fallback path")
+        handle = ctypes.CDLL(LIB_PATH)
+        for name, (res, args) in SIGNATURES.items():
+            fn = getattr(handle, name)
+            fn.restype = res
+            fn.argtypes = args
+        _lib = handle
+    return _lib
+
+
+def status_string(rc):
+    return lib().eagle_status_string(rc).decode()
+
+
+def check(rc, what):
+    """Raise the Python error that corresponds to a non-zero status."""
+    if rc == 0:
+        return
+    msg = f"{what}: {status_string(rc)} (status {rc})"
+    if rc in (1, 2, 3, 4, 5):
+        raise ValueError(msg)
+    raise RuntimeError(msg)

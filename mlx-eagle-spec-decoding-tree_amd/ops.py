@@ -1,0 +1,273 @@
+"""Operator front end: reference call signatures on torch tensors, executed by the
+HIP kernels of libeagle_mi355x.so through its C ABI.
+
+torch only supplies device memory and the current stream.  There is no eager
+or CPU fallback: every function raises if the library is missing or the tensor
+is not on a GPU.
+"""
+import math
+from functools import reduce
+
+import torch
+
+from . import _lib
+
+_WS = {}  # (device index, tag) -> workspace tensor
+
+
+def _stream():
+    return torch.cuda.current_stream().cuda_stream
+
+
+def _ptr(t):
+    return None if t is None else t.data_ptr()
+
+
+def _need_cuda(*ts):
+    for t in ts:
+        if t is not None and not t.is_cuda:
+            raise RuntimeError("eagle ops need GPU tensors (there is no CPU path)")
+
+
+def _f16(t, name):
+    if t.dtype != torch.float16:
+        raise TypeError(f"{name} must be float16, got {t.dtype}")
+    return t.contiguous()
+
+
+def workspace(tag, nbytes, device):
+    """A zero-initialised device buffer that persists between calls (and across
+    HIP-graph replays).  It only grows; growing is not graph-capture safe, so
+    capture callers size it first."""
+    key = (device.index, tag)
+    buf = _WS.get(key)
+    if buf is None or buf.numel() < nbytes:
+        buf = torch.zeros(max(int(nbytes), 1 << 16), dtype=torch.uint8, device=device)
+        _WS[key] = buf
+    return buf
+
+
+def as_packed_u32(w_q):
+    """MLX packs into uint32; torch has weak uint32 support, so int32 storage of
+    the same bits is accepted too."""
+    if w_q.dtype not in (torch.uint32, torch.int32):
+        raise TypeError(f"packed weights must be uint32/int32, got {w_q.dtype}")
+    return w_q.contiguous()
+
+
+def quantized_matmul(x, w_q, scales, biases, transpose=True, group_size=64, bits=4, bias=None,
+                     out=None, variant=-1, splits=0):
+    """`mx.quantized_matmul(x, w, scales, biases, transpose=True, group_size=64, bits=4)`
+    for 1..32 rows of x (any leading dims, flattened as qmm_kernel.py:99-100,136).
+    `bias` ([N] fp16) is added after rounding, as the patched linear layer does
+    (mlx_model_fwd_bench.py:70-71)."""
+    if not transpose:
+        raise ValueError("only transpose=True (x @ dequant(w).T) is implemented")
+    _need_cuda(x, w_q, scales, biases, bias)
+    x = _f16(x, "x")
+    w_q = as_packed_u32(w_q)
+    scales, biases = _f16(scales, "scales"), _f16(biases, "biases")
+    *lead, K = x.shape
+    M = reduce(lambda a, b: a * b, lead, 1)
+    N = w_q.shape[0]
+    if w_q.shape[1] * 8 != K or tuple(scales.shape) != (N, K // 64) or tuple(biases.shape) != (N, K // 64):
+        raise ValueError(f"shape mismatch: x {tuple(x.shape)}, w {tuple(w_q.shape)}, "
+                         f"scales {tuple(scales.shape)}, biases {tuple(biases.shape)}")
+    if bias is not None:
+        bias = _f16(bias, "bias")
+        if tuple(bias.shape) != (N,):
+            raise ValueError("bias must have shape [N]")
+    if out is None:
+        out = torch.empty((*lead, N), dtype=torch.float16, device=x.device)
+    L = _lib.lib()
+    need = L.eagle_qmm_workspace_bytes_cfg(M, N, K, variant, splits)
+    ws = workspace("qmm", need, x.device)
+    if variant < 0:
+        rc = L.eagle_qmm_w4g64_f16(_ptr(x), _ptr(w_q), _ptr(scales), _ptr(biases), _ptr(bias),
+                                   _ptr(out), M, N, K, group_size, bits, _ptr(ws), ws.numel(),
+                                   _stream())
+    else:
+        if group_size != 64 or bits != 4:
+            raise ValueError("only group_size=64, bits=4 is supported")
+        rc = L.eagle_qmm_w4g64_f16_cfg(_ptr(x), _ptr(w_q), _ptr(scales), _ptr(biases), _ptr(bias),
+                                       _ptr(out), M, N, K, variant, splits, _ptr(ws), ws.numel(),
+                                       _stream())
+    _lib.check(rc, "quantized_matmul")
+    return out
+
+
+def matmul(x, w, s, b, group_size, **_ignored):
+    """Same contract as the reference's `qmm_kernel.matmul` (qmm_kernel.py:84-164):
+    returns a one-element list.  The Metal tuning keywords are accepted and ignored."""
+    return [quantized_matmul(x, w, s, b, group_size=group_size, bits=4)]
+
+
+def default_inv_freqs(head_dim, base=10000.0, device=None):
+    """inv_freq[i] = 2 ** (-log2(base) * 2i / head_dim) in fp32 (mlx_llama.py:109-113)."""
+    expo = -torch.log2(torch.tensor(float(base), dtype=torch.float32)) * \
+        torch.arange(0, head_dim, 2, dtype=torch.float32) / float(head_dim)
+    return torch.exp2(expo).to(device)
+
+
+def arrayed_rope(x, positions, inv_freqs=None, scaling_factor=1.0, base=10000.0):
+    """RoPE with a position per (batch, token).  x [B,H,L,hd] fp16, positions [B,L]
+    (or [L] for B=1) integer.  Same semantics as `rope_positions`
+    (mlx_arrayed_rope_kernel.py:46-152)."""
+    _need_cuda(x, positions)
+    x = _f16(x, "x")
+    if x.dim() != 4:
+        raise ValueError("x must be [B, H, L, head_dim]")
+    B, H, L, hd = x.shape
+    pos = positions.to(torch.int32).contiguous()
+    if pos.numel() != B * L:
+        raise ValueError(f"positions must hold B*L = {B * L} entries")
+    if inv_freqs is None:
+        inv_freqs = default_inv_freqs(hd, base, x.device)
+    inv = inv_freqs.to(device=x.device, dtype=torch.float32).contiguous()
+    if inv.numel() != hd // 2:
+        raise ValueError("inv_freqs must have head_dim/2 entries")
+    out = torch.empty_like(x)
+    rc = _lib.lib().eagle_rope_arrayed_f16(_ptr(x), _ptr(pos), _ptr(inv), float(scaling_factor),
+                                           _ptr(out), B, H, L, hd, _stream())
+    _lib.check(rc, "arrayed_rope")
+    return out
+
+
+def rope_positions(inp, offsets, inv_freqs, scaling_factor, verbose=False):
+    """Reference name and argument order (mlx_arrayed_rope_kernel.py:47-53)."""
+    return arrayed_rope(inp, offsets, inv_freqs, scaling_factor)
+
+
+def rope_kv_append(q_lin, k_lin, v_lin, positions, inv_freqs, scaling_factor, q_out, k_cache,
+                   v_cache, cache_len_dev, H, G, hd):
+    T = q_lin.shape[0]
+    rc = _lib.lib().eagle_rope_kv_append_f16(
+        _ptr(q_lin), _ptr(k_lin), _ptr(v_lin), _ptr(positions), _ptr(inv_freqs),
+        float(scaling_factor), _ptr(q_out), _ptr(k_cache), _ptr(v_cache), _ptr(cache_len_dev),
+        T, H, G, hd, k_cache.shape[1], _stream())
+    _lib.check(rc, "rope_kv_append")
+
+
+def mask_to_bits(tree_mask):
+    """[T,T] additive ({0,-inf}) or boolean visibility matrix -> [T] int32 row bitmasks."""
+    m = tree_mask
+    vis = m if m.dtype == torch.bool else (m == 0)
+    T = vis.shape[-1]
+    if vis.shape[-2] != T or T > 32:
+        raise ValueError("tree mask must be [T,T] with T <= 32")
+    weights = (torch.ones(T, dtype=torch.int64, device=vis.device) << torch.arange(T, device=vis.device))
+    bits = (vis.reshape(T, T).to(torch.int64) * weights[None, :]).sum(1)
+    bits = torch.where(bits >= 2 ** 31, bits - 2 ** 32, bits)   # bit 31 -> sign bit of int32
+    return bits.to(torch.int32)
+
+
+def tree_attention(q, k_cache, v_cache, tree_mask_bits, cache_len_dev, scale, max_len=None,
+                   out=None):
+    """q [H,T,hd]; k_cache, v_cache [G,capacity,hd] holding *cache_len_dev prefix rows
+    followed by the T tree rows; tree_mask_bits [T] int32.  Returns [T, H*hd]."""
+    _need_cuda(q, k_cache, v_cache, tree_mask_bits, cache_len_dev)
+    H, T, hd = q.shape
+    G, cap, _ = k_cache.shape
+    if max_len is None:
+        max_len = cap
+    if out is None:
+        out = torch.empty((T, H * hd), dtype=torch.float16, device=q.device)
+    L = _lib.lib()
+    need = L.eagle_tree_attention_workspace_bytes(H, hd, max_len)
+    ws = workspace("attn", need, q.device)
+    rc = L.eagle_tree_attention_f16(_ptr(q), _ptr(k_cache), _ptr(v_cache), _ptr(tree_mask_bits),
+                                    _ptr(cache_len_dev), _ptr(out), T, H, G, hd, cap, max_len,
+                                    float(scale), _ptr(ws), ws.numel(), _stream())
+    _lib.check(rc, "tree_attention")
+    return out
+
+
+def scaled_dot_product_attention(queries, keys, values, cache=None, scale=None, mask=None):
+    """Drop-in for the call at mlx_llama.py:185-192 on the tree path:
+    queries [1,H,T,hd], keys/values [1,G,S,hd] (prefix then the T tree rows),
+    mask [1,1,T,S] additive whose prefix part is zero.  Returns [1,H,T,hd]."""
+    _need_cuda(queries, keys, values, mask)
+    B, H, T, hd = queries.shape
+    if B != 1:
+        raise ValueError("batch size 1 only")
+    G, S = keys.shape[1], keys.shape[2]
+    if scale is None:
+        scale = hd ** -0.5
+    P = S - T
+    if mask is None:
+        raise ValueError("the tree path always passes a mask")
+    m = mask.reshape(T, S)
+    bits = mask_to_bits(m[:, P:])
+    len_dev = torch.tensor([P], dtype=torch.int32, device=queries.device)
+    out = tree_attention(_f16(queries[0], "q"), _f16(keys[0], "k"), _f16(values[0], "v"), bits,
+                         len_dev, scale, max_len=S)
+    return out.reshape(T, H, hd).permute(1, 0, 2).unsqueeze(0).contiguous()
+
+
+def rms_norm(x, weight, eps, residual=None):
+    """`mx.fast.rms_norm(x, weight, eps)`; with `residual` returns (h, norm(h)),
+    h = fp16(x + residual)."""
+    _need_cuda(x, weight, residual)
+    x = _f16(x, "x")
+    D = x.shape[-1]
+    T = x.numel() // D
+    out = torch.empty_like(x)
+    h = torch.empty_like(x) if residual is not None else None
+    rc = _lib.lib().eagle_rmsnorm_f16(_ptr(x), _ptr(residual), _ptr(_f16(weight, "weight")),
+                                      float(eps), _ptr(h), _ptr(out), T, D, _stream())
+    _lib.check(rc, "rms_norm")
+    return out if residual is None else (h, out)
+
+
+def silu_mul(gate, up=None):
+    """fp16(fp16(silu(gate)) * up); with up=None, `gate` is the fused [T, 2*I] tensor."""
+    _need_cuda(gate, up)
+    gate = _f16(gate, "gate")
+    if up is None:
+        I = gate.shape[-1] // 2
+    else:
+        up = _f16(up, "up")
+        I = gate.shape[-1]
+    T = gate.numel() // gate.shape[-1]
+    out = torch.empty((*gate.shape[:-1], I), dtype=torch.float16, device=gate.device)
+    rc = _lib.lib().eagle_silu_mul_f16(_ptr(gate), _ptr(up), _ptr(out), T, I, _stream())
+    _lib.check(rc, "silu_mul")
+    return out
+
+
+def add(a, b):
+    _need_cuda(a, b)
+    a, b = _f16(a, "a"), _f16(b, "b")
+    out = torch.empty_like(a)
+    rc = _lib.lib().eagle_add_f16(_ptr(a), _ptr(b), _ptr(out), a.numel(), _stream())
+    _lib.check(rc, "add")
+    return out
+
+
+def embed(ids, w_q, scales, biases):
+    """Quantised embedding lookup: ids [...] int -> [..., D] fp16."""
+    _need_cuda(ids, w_q, scales, biases)
+    w_q = as_packed_u32(w_q)
+    V, D = w_q.shape[0], w_q.shape[1] * 8
+    ids32 = ids.to(torch.int32).contiguous()
+    out = torch.empty((*ids.shape, D), dtype=torch.float16, device=ids.device)
+    rc = _lib.lib().eagle_embed_w4g64_f16(_ptr(ids32), _ptr(w_q), _ptr(_f16(scales, "scales")),
+                                          _ptr(_f16(biases, "biases")), _ptr(out), ids32.numel(),
+                                          D, V, _stream())
+    _lib.check(rc, "embed")
+    return out
+
+
+def argmax_rows(logits, out=None):
+    """argmax over the last axis, lowest index among equal maxima; int32."""
+    _need_cuda(logits)
+    logits = _f16(logits, "logits")
+    V = logits.shape[-1]
+    R = logits.numel() // V
+    if out is None:
+        out = torch.empty(logits.shape[:-1], dtype=torch.int32, device=logits.device)
+    L = _lib.lib()
+    ws = workspace("argmax", L.eagle_argmax_workspace_bytes(R, V), logits.device)
+    rc = L.eagle_argmax_rows_f16(_ptr(logits), _ptr(out), R, V, _ptr(ws), ws.numel(), _stream())
+    _lib.check(rc, "argmax_rows")
+    return out

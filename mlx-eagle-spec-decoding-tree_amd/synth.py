@@ -1,0 +1,184 @@
+"""Seeded synthetic inputs for every benchmark configuration.
+
+numpy `default_rng(seed)` (PCG64) is platform-stable, so the generator code is
+what ships, not data: the same call yields the same arrays for the HIP path and
+for the CPU checker.  Value distributions follow the benchmark configuration
+text: packed uint4 uniform in 0..15, scales ~ U(0.005, 0.02) fp16,
+biases = fp16(-8*scale + N(0, 1e-3)), activations ~ N(0, 1) fp16.
+"""
+from dataclasses import dataclass, field
+from typing import Dict, Optional
+
+import numpy as np
+
+
+@dataclass
+class ModelArgs:
+    """Same fields as the reference's ModelArgs (mlx_llama.py:21-58)."""
+    model_type: str = "qwen2"
+    hidden_size: int = 3584
+    num_hidden_layers: int = 28
+    intermediate_size: int = 18944
+    num_attention_heads: int = 28
+    rms_norm_eps: float = 1e-6
+    vocab_size: int = 152064
+    head_dim: Optional[int] = None
+    max_position_embeddings: Optional[int] = None
+    num_key_value_heads: Optional[int] = None
+    attention_bias: bool = False
+    mlp_bias: bool = False
+    rope_theta: float = 10000.0
+    rope_traditional: bool = False
+    rope_scaling: Optional[Dict] = None
+    tie_word_embeddings: bool = True
+    group_size: int = 64
+    bits: int = 4
+
+    def __post_init__(self):
+        if self.num_key_value_heads is None:
+            self.num_key_value_heads = self.num_attention_heads
+        if self.head_dim is None:
+            self.head_dim = self.hidden_size // self.num_attention_heads
+        if self.rope_scaling:
+            if "factor" not in self.rope_scaling:
+                raise ValueError("rope_scaling must contain 'factor'")
+            rope_type = self.rope_scaling.get("type") or self.rope_scaling.get("rope_type")
+            if rope_type is None:
+                raise ValueError("rope_scaling must contain either 'type' or 'rope_type'")
+            if rope_type not in ("linear", "dynamic", "llama3"):
+                raise ValueError("rope_scaling 'type' supports 'linear', 'dynamic' or 'llama3'")
+
+
+def qwen25_7b():
+    return ModelArgs(model_type="qwen2", hidden_size=3584, num_hidden_layers=28,
+                     intermediate_size=18944, num_attention_heads=28, num_key_value_heads=4,
+                     head_dim=128, vocab_size=152064, rms_norm_eps=1e-6, rope_theta=1e6,
+                     attention_bias=True, tie_word_embeddings=False)
+
+
+def qwen25_05b():
+    return ModelArgs(model_type="qwen2", hidden_size=896, num_hidden_layers=24,
+                     intermediate_size=4864, num_attention_heads=14, num_key_value_heads=2,
+                     head_dim=64, vocab_size=152064, rms_norm_eps=1e-6, rope_theta=1e6,
+                     attention_bias=True, tie_word_embeddings=True)
+
+
+def llama3_8b():
+    return ModelArgs(model_type="llama", hidden_size=4096, num_hidden_layers=32,
+                     intermediate_size=14336, num_attention_heads=32, num_key_value_heads=8,
+                     head_dim=128, vocab_size=128256, rms_norm_eps=1e-5, rope_theta=5e5,
+                     attention_bias=False, tie_word_embeddings=False)
+
+
+def tiny(layers=2, hidden=256, inter=512, heads=4, kv_heads=2, head_dim=64, vocab=1024,
+         attention_bias=True, tie=False, theta=1e6):
+    return ModelArgs(model_type="qwen2", hidden_size=hidden, num_hidden_layers=layers,
+                     intermediate_size=inter, num_attention_heads=heads,
+                     num_key_value_heads=kv_heads, head_dim=head_dim, vocab_size=vocab,
+                     rms_norm_eps=1e-6, rope_theta=theta, attention_bias=attention_bias,
+                     tie_word_embeddings=tie)
+
+
+def make_qlinear(rng, N, K, bias=False):
+    """Random 4-bit group-64 linear layer in the packed layout
+    (weight uint32 [N, K/8], nibble i of a word = element 8*word + i)."""
+    assert K % 64 == 0
+    w = rng.integers(0, 1 << 32, size=(N, K // 8), dtype=np.uint32)
+    s = rng.uniform(0.005, 0.02, size=(N, K // 64)).astype(np.float16)
+    b = (-8.0 * s.astype(np.float32)
+         + rng.normal(0.0, 1e-3, size=s.shape).astype(np.float32)).astype(np.float16)
+    out = {"weight": w, "scales": s, "biases": b}
+    if bias:
+        out["bias"] = rng.normal(0.0, 0.02, size=(N,)).astype(np.float16)
+    return out
+
+
+def unpack_nibbles(w):
+    """uint32 [N, K/8] -> uint8 [N, K] (element 8*j+i = bits 4i..4i+3 of word j)."""
+    N, K8 = w.shape
+    sh = (np.arange(8, dtype=np.uint32) * 4)[None, None, :]
+    return ((w[:, :, None] >> sh) & np.uint32(15)).astype(np.uint8).reshape(N, K8 * 8)
+
+
+def pack_nibbles(q):
+    """uint8 [N, K] with values 0..15 -> uint32 [N, K/8]."""
+    N, K = q.shape
+    q = q.reshape(N, K // 8, 8).astype(np.uint32)
+    sh = (np.arange(8, dtype=np.uint32) * 4)[None, None, :]
+    return (q << sh).sum(axis=2, dtype=np.uint64).astype(np.uint32)
+
+
+def dequantize(layer, dtype=np.float64):
+    q = unpack_nibbles(layer["weight"]).astype(dtype)
+    s = np.repeat(layer["scales"].astype(dtype), 64, axis=1)
+    b = np.repeat(layer["biases"].astype(dtype), 64, axis=1)
+    return s * q + b
+
+
+def make_x(rng, *shape):
+    return rng.normal(0.0, 1.0, size=shape).astype(np.float16)
+
+
+def make_model_weights(args: ModelArgs, seed=42, layers=None):
+    """All tensors of a random-init quantised decoder as a flat dict of numpy
+    arrays keyed like an MLX-community checkpoint
+    (`model.layers.3.self_attn.q_proj.weight` / `.scales` / `.biases` / `.bias`)."""
+    rng = np.random.default_rng(seed)
+    D, I, V = args.hidden_size, args.intermediate_size, args.vocab_size
+    H, G, hd = args.num_attention_heads, args.num_key_value_heads, args.head_dim
+    out = {}
+
+    def put(prefix, layer):
+        for k, v in layer.items():
+            out[f"{prefix}.{k}"] = v
+
+    put("model.embed_tokens", make_qlinear(rng, V, D))
+    n_layers = args.num_hidden_layers if layers is None else layers
+    for i in range(n_layers):
+        p = f"model.layers.{i}"
+        put(f"{p}.self_attn.q_proj", make_qlinear(rng, H * hd, D, args.attention_bias))
+        put(f"{p}.self_attn.k_proj", make_qlinear(rng, G * hd, D, args.attention_bias))
+        put(f"{p}.self_attn.v_proj", make_qlinear(rng, G * hd, D, args.attention_bias))
+        put(f"{p}.self_attn.o_proj", make_qlinear(rng, D, H * hd))
+        put(f"{p}.mlp.gate_proj", make_qlinear(rng, I, D, args.mlp_bias))
+        put(f"{p}.mlp.up_proj", make_qlinear(rng, I, D, args.mlp_bias))
+        put(f"{p}.mlp.down_proj", make_qlinear(rng, D, I, args.mlp_bias))
+        out[f"{p}.input_layernorm.weight"] = (1.0 + rng.normal(0, 0.02, D)).astype(np.float16)
+        out[f"{p}.post_attention_layernorm.weight"] = (1.0 + rng.normal(0, 0.02, D)).astype(np.float16)
+    out["model.norm.weight"] = (1.0 + rng.normal(0, 0.02, D)).astype(np.float16)
+    if not args.tie_word_embeddings:
+        put("lm_head", make_qlinear(rng, V, D))
+    return out
+
+
+def inv_freqs(args: ModelArgs):
+    """fp32 inverse-frequency table and scaling factor for the default / linear
+    rope types: inv_freq[i] = 2 ** (-log2(theta) * 2i / head_dim)
+    (mlx_llama.py:105-113)."""
+    rope_type = "default"
+    if args.rope_scaling is not None:
+        rope_type = args.rope_scaling.get("type") or args.rope_scaling.get("rope_type", "default")
+    if rope_type not in ("default", "linear"):
+        raise NotImplementedError("only default/linear rope tables are generated here")
+    hd = args.head_dim
+    expo = (-np.log2(np.float32(args.rope_theta)) * np.arange(0, hd, 2, dtype=np.float32)
+            / np.float32(hd)).astype(np.float32)
+    inv = np.exp2(expo).astype(np.float32)
+    scale = 1.0 / args.rope_scaling["factor"] if rope_type == "linear" else 1.0
+    return inv, float(scale)
+
+
+def random_tree(rng, n_nodes=32, max_depth=4, max_children=4):
+    """Parents (node ids, for nodes 1..n-1) of a random tree with topologically
+    sorted ids, depth <= max_depth, at most max_children children per node."""
+    depth = [0]
+    children = [0]
+    parents = []
+    for node in range(1, n_nodes):
+        ok = [p for p in range(node) if depth[p] < max_depth and children[p] < max_children]
+        p = int(ok[rng.integers(len(ok))])
+        parents.append(p)
+        children[p] += 1
+        children.append(0)
+        depth.append(depth[p] + 1)
+    return np.array(parents, np.int32)

@@ -1,0 +1,98 @@
+"""HIP quantised matmul vs the CPU oracle, through the C ABI."""
+import numpy as np
+import pytest
+import torch
+
+from mlx_eagle_spec_decoding_tree_amd import _lib, ops, synth
+from oracle import oracle
+from util import TOL, layer_to_dev, rel_err, to_dev
+
+pytestmark = pytest.mark.gpu
+
+
+def run_case(dev, M, N, K, seed=0, bias=False, variant=-1, splits=0):
+    rng = np.random.default_rng(seed)
+    layer = synth.make_qlinear(rng, N, K, bias=bias)
+    x = synth.make_x(rng, M, K)
+    want = oracle.qmm(x, layer["weight"], layer["scales"], layer["biases"], layer.get("bias"))
+    d = layer_to_dev(layer, dev)
+    got = ops.quantized_matmul(to_dev(x, dev), d["weight"], d["scales"], d["biases"],
+                               bias=d.get("bias"), variant=variant, splits=splits)
+    torch.cuda.synchronize()
+    err = rel_err(got.cpu().numpy(), want)
+    assert err <= TOL, f"M={M} N={N} K={K} variant={variant} splits={splits}: rel err {err:.3e}"
+    return err
+
+
+@pytest.mark.parametrize("M", [1, 2, 7, 8, 16, 17, 24, 32])
+def test_cfg1_shape_all_m(dev, M):
+    print(f"qmm cfg1 M={M}", flush=True)
+    run_case(dev, M, 8192, 2048, seed=42)
+
+
+@pytest.mark.parametrize("variant", range(6))
+@pytest.mark.parametrize("splits", [1, 2, 5])
+@pytest.mark.parametrize("M", [8, 32])
+def test_every_variant_and_split(dev, variant, splits, M):
+    print(f"qmm variant={variant} splits={splits} M={M}", flush=True)
+    run_case(dev, M, 1536, 3584, seed=variant * 10 + splits, variant=variant, splits=splits)
+
+
+@pytest.mark.parametrize("N,K", [(8, 64), (8, 128), (24, 192), (40, 896), (136, 2944), (512, 3584)])
+def test_edge_shapes(dev, N, K):
+    for M in (1, 5, 32):
+        print(f"qmm edge N={N} K={K} M={M}", flush=True)
+        for variant in (-1, 0, 3):
+            run_case(dev, M, N, K, seed=N + K + M, variant=variant, splits=3)
+
+
+def test_bias_and_leading_dims(dev):
+    rng = np.random.default_rng(3)
+    layer = synth.make_qlinear(rng, 512, 896, bias=True)
+    x = synth.make_x(rng, 1, 8, 896)
+    want = oracle.qmm(x, layer["weight"], layer["scales"], layer["biases"], layer["bias"])
+    d = layer_to_dev(layer, dev)
+    got = ops.quantized_matmul(to_dev(x, dev), d["weight"], d["scales"], d["biases"], bias=d["bias"])
+    assert tuple(got.shape) == (1, 8, 512)
+    assert rel_err(got.cpu().numpy(), want) <= TOL
+    lst = ops.matmul(to_dev(x, dev), d["weight"], d["scales"], d["biases"], 64)
+    assert isinstance(lst, list) and len(lst) == 1
+
+
+def test_one_hot_rows_reproduce_dequantised_columns(dev):
+    """x = e_k picks column k of dequant(W): pins nibble order and group indexing exactly."""
+    rng = np.random.default_rng(5)
+    N, K = 64, 256
+    layer = synth.make_qlinear(rng, N, K)
+    wd = synth.dequantize(layer, np.float32)
+    d = layer_to_dev(layer, dev)
+    for k0 in range(0, K, 32):
+        x = np.zeros((32, K), np.float16)
+        for m in range(32):
+            x[m, k0 + m] = 1.0
+        got = ops.quantized_matmul(to_dev(x, dev), d["weight"], d["scales"], d["biases"]).cpu().numpy()
+        want = wd[:, k0:k0 + 32].T.astype(np.float16)
+        np.testing.assert_allclose(got.astype(np.float32), want.astype(np.float32), rtol=0, atol=2e-3)
+
+
+def test_deterministic_split_k(dev):
+    rng = np.random.default_rng(9)
+    layer = synth.make_qlinear(rng, 512, 3584)
+    x = to_dev(synth.make_x(rng, 32, 3584), dev)
+    d = layer_to_dev(layer, dev)
+    ref = ops.quantized_matmul(x, d["weight"], d["scales"], d["biases"], variant=3, splits=7)
+    for _ in range(5):
+        again = ops.quantized_matmul(x, d["weight"], d["scales"], d["biases"], variant=3, splits=7)
+        assert torch.equal(ref, again)
+
+
+def test_argument_errors(dev):
+    x = torch.zeros(33, 128, dtype=torch.float16, device=dev)
+    w = torch.zeros(8, 16, dtype=torch.int32, device=dev)
+    s = torch.zeros(8, 2, dtype=torch.float16, device=dev)
+    with pytest.raises(ValueError):
+        ops.quantized_matmul(x, w, s, s)              # M > 32
+    with pytest.raises(ValueError):
+        ops.quantized_matmul(x[:8], w, s, s, group_size=32)
+    with pytest.raises(ValueError):
+        ops.quantized_matmul(x[:8], w, s, s, bits=8)

@@ -1,0 +1,24 @@
+"""Shared helpers of the test-suite."""
+import numpy as np
+import torch
+
+TOL = 2e-2   # max |err| <= TOL * RMS(reference output): the bound stated for fp16 QMM / RoPE / attention
+
+
+def to_dev(a, dev):
+    """numpy -> torch on the device; uint32 travels as int32 bits."""
+    if isinstance(a, np.ndarray) and a.dtype == np.uint32:
+        return torch.from_numpy(a.view(np.int32)).to(dev)
+    return torch.from_numpy(np.ascontiguousarray(a)).to(dev)
+
+
+def rel_err(got, want):
+    """max |got - want| / RMS(want), computed in float64."""
+    g = np.asarray(got, dtype=np.float64)
+    w = np.asarray(want, dtype=np.float64)
+    rms = np.sqrt(np.mean(w * w))
+    return float(np.max(np.abs(g - w)) / max(rms, 1e-30))
+
+
+def layer_to_dev(layer, dev):
+    return {k: to_dev(v, dev) for k, v in layer.items()}
