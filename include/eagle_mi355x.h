@@ -48,7 +48,8 @@ int eagle_check_device(void);
  *   q[n,k] = (wq[n,k/8] >> 4*(k%8)) & 15
  *   x [M,K] fp16 row-major, wq [N,K/8] uint32, scales/biases [N,K/64] fp16,
  *   bias [N] fp16 or NULL (added in fp16 after rounding), out [M,N] fp16.
- * Constraints: 1 <= M <= 32, K % 64 == 0, N % 8 == 0, group_size == 64, bits == 4.
+ * Constraints: 1 <= M <= 32, K % 64 == 0, K <= 32768, N % 8 == 0, group_size == 64,
+ * bits == 4.
  * Replaces qmm_kernel.matmul (qmm_kernel.py:84-164) with the body
  * kernels/progression/simd_no_swizzle_cast.metal, the mx.quantized_matmul
  * fallback of the patched layer (mlx_model_fwd_bench.py:65-73) and its bias add
@@ -57,22 +58,24 @@ int eagle_check_device(void);
  * EAGLE_QMM_COUNTER_BYTES bytes must be zero before the first call (they are
  * left zero by every call).  Calls sharing a workspace must be stream ordered.
  * ------------------------------------------------------------------------- */
-#define EAGLE_QMM_COUNTER_BYTES 16384
+#define EAGLE_QMM_COUNTER_BYTES 65536
 size_t eagle_qmm_workspace_bytes(int M, int N, int K);
 int eagle_qmm_w4g64_f16(const void* x, const uint32_t* wq, const void* scales,
                         const void* biases, const void* bias, void* out,
                         int M, int N, int K, int group_size, int bits,
                         void* workspace, size_t workspace_bytes, eagle_stream_t stream);
-/* Same, with the launch configuration forced (tuning sweeps and tests):
- * variant indexes the compiled tile shapes, splits is the split-K factor.
- * eagle_qmm_num_variants() variants exist; variant < 0 selects the heuristic. */
-int eagle_qmm_num_variants(void);
-size_t eagle_qmm_workspace_bytes_cfg(int M, int N, int K, int variant, int splits);
-const char* eagle_qmm_variant_name(int variant);
-int eagle_qmm_w4g64_f16_cfg(const void* x, const uint32_t* wq, const void* scales,
-                            const void* biases, const void* bias, void* out,
-                            int M, int N, int K, int variant, int splits,
-                            void* workspace, size_t workspace_bytes, eagle_stream_t stream);
+/* The launch shape the library would pick: plan7 = {tiles per wave, tile slots per
+ * round, waves per tile, K slabs, columns per slab, row groups, rounds}. */
+int eagle_qmm_plan(int M, int N, int K, int* plan7);
+/* Same matmul with the launch shape forced (tuning sweeps and tests).  The shape
+ * must cover N and K and fit LDS, else EAGLE_ERR_SHAPE. */
+size_t eagle_qmm_workspace_bytes_tuned(int M, int rt, int wt, int wk, int splits,
+                                       int row_groups, int rounds);
+int eagle_qmm_w4g64_f16_tuned(const void* x, const uint32_t* wq, const void* scales,
+                              const void* biases, const void* bias, void* out,
+                              int M, int N, int K, int rt, int wt, int wk, int splits,
+                              int slab_k, int row_groups, int rounds,
+                              void* workspace, size_t workspace_bytes, eagle_stream_t stream);
 
 /* Quantised embedding gather: out[t,:] = fp16(scales*q + biases) of row ids[t].
  * ids [T] int32, out [T,D] fp16, D % 64 == 0.  Replaces the quantised

@@ -9,7 +9,8 @@ import os
 from ctypes import c_char_p, c_float, c_int, c_int32, c_long, c_size_t, c_void_p
 
 HERE = os.path.dirname(os.path.abspath(__file__))
-LIB_PATH = os.path.join(HERE, "libeagle_mi355x.so")
+# EAGLE_MI355X_LIB selects another build of the same library (kernel experiments)
+LIB_PATH = os.environ.get("EAGLE_MI355X_LIB") or os.path.join(HERE, "libeagle_mi355x.so")
 
 _lib = None
 
@@ -20,10 +21,9 @@ SIGNATURES = {
     "eagle_check_device": (c_int, []),
     "eagle_qmm_workspace_bytes": (c_size_t, [c_int, c_int, c_int]),
     "eagle_qmm_w4g64_f16": (c_int, [c_void_p] * 6 + [c_int] * 5 + [c_void_p, c_size_t, c_void_p]),
-    "eagle_qmm_num_variants": (c_int, []),
-    "eagle_qmm_workspace_bytes_cfg": (c_size_t, [c_int] * 5),
-    "eagle_qmm_variant_name": (c_char_p, [c_int]),
-    "eagle_qmm_w4g64_f16_cfg": (c_int, [c_void_p] * 6 + [c_int] * 5 + [c_void_p, c_size_t, c_void_p]),
+    "eagle_qmm_plan": (c_int, [c_int, c_int, c_int, c_void_p]),
+    "eagle_qmm_workspace_bytes_tuned": (c_size_t, [c_int] * 7),
+    "eagle_qmm_w4g64_f16_tuned": (c_int, [c_void_p] * 6 + [c_int] * 10 + [c_void_p, c_size_t, c_void_p]),
     "eagle_embed_w4g64_f16": (c_int, [c_void_p] * 5 + [c_int] * 3 + [c_void_p]),
     "eagle_rope_arrayed_f16": (c_int, [c_void_p] * 3 + [c_float, c_void_p] + [c_int] * 4 + [c_void_p]),
     "eagle_rope_kv_append_f16": (c_int, [c_void_p] * 5 + [c_float] + [c_void_p] * 4 + [c_int] * 4

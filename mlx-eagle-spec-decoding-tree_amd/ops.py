@@ -56,7 +56,7 @@ def as_packed_u32(w_q):
 
 
 def quantized_matmul(x, w_q, scales, biases, transpose=True, group_size=64, bits=4, bias=None,
-                     out=None, variant=-1, splits=0):
+                     out=None, tuned=None):
     """`mx.quantized_matmul(x, w, scales, biases, transpose=True, group_size=64, bits=4)`
     for 1..32 rows of x (any leading dims, flattened as qmm_kernel.py:99-100,136).
     `bias` ([N] fp16) is added after rounding, as the patched linear layer does
@@ -80,20 +80,32 @@ def quantized_matmul(x, w_q, scales, biases, transpose=True, group_size=64, bits
     if out is None:
         out = torch.empty((*lead, N), dtype=torch.float16, device=x.device)
     L = _lib.lib()
-    need = L.eagle_qmm_workspace_bytes_cfg(M, N, K, variant, splits)
-    ws = workspace("qmm", need, x.device)
-    if variant < 0:
+    if tuned is None:
+        ws = workspace("qmm", L.eagle_qmm_workspace_bytes(M, N, K), x.device)
         rc = L.eagle_qmm_w4g64_f16(_ptr(x), _ptr(w_q), _ptr(scales), _ptr(biases), _ptr(bias),
                                    _ptr(out), M, N, K, group_size, bits, _ptr(ws), ws.numel(),
                                    _stream())
     else:
+        # tuned = (rt, wt, wk, splits, slab_k, row_groups, rounds): forced launch shape
         if group_size != 64 or bits != 4:
             raise ValueError("only group_size=64, bits=4 is supported")
-        rc = L.eagle_qmm_w4g64_f16_cfg(_ptr(x), _ptr(w_q), _ptr(scales), _ptr(biases), _ptr(bias),
-                                       _ptr(out), M, N, K, variant, splits, _ptr(ws), ws.numel(),
-                                       _stream())
+        rt, wt, wk, splits, slab_k, row_groups, rounds = (int(v) for v in tuned)
+        need = L.eagle_qmm_workspace_bytes_tuned(M, rt, wt, wk, splits, row_groups, rounds)
+        ws = workspace("qmm", need, x.device)
+        rc = L.eagle_qmm_w4g64_f16_tuned(_ptr(x), _ptr(w_q), _ptr(scales), _ptr(biases),
+                                         _ptr(bias), _ptr(out), M, N, K, rt, wt, wk, splits,
+                                         slab_k, row_groups, rounds, _ptr(ws), ws.numel(),
+                                         _stream())
     _lib.check(rc, "quantized_matmul")
     return out
+
+
+def qmm_plan(M, N, K):
+    """The launch shape the library picks: (rt, wt, wk, splits, slab_k, row_groups, rounds)."""
+    import ctypes
+    plan = (ctypes.c_int * 7)()
+    _lib.check(_lib.lib().eagle_qmm_plan(M, N, K, plan), "qmm_plan")
+    return tuple(plan)
 
 
 def matmul(x, w, s, b, group_size, **_ignored):

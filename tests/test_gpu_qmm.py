@@ -10,17 +10,32 @@ from util import TOL, layer_to_dev, rel_err, to_dev
 pytestmark = pytest.mark.gpu
 
 
-def run_case(dev, M, N, K, seed=0, bias=False, variant=-1, splits=0):
+def shape_for(M, N, K, rt, wt, wk, splits, rounds):
+    """A forced launch shape (or None if it cannot hold the x slab in LDS)."""
+    mp = 16 if M <= 16 else 32
+    slab_k = -(-(-(-K // splits)) // 256) * 256
+    splits = -(-K // slab_k)
+    tiles = -(-N // 16)
+    row_groups = -(-tiles // (rounds * wt * rt))
+    units = -(-(slab_k // 256) // wk)
+    lds = (mp * (slab_k * 2 + 16) + ((wk - 1) * wt * rt * (mp // 16) * 1024 if wk > 1 else 0)
+           + wt * wk * rt * 2 * 16 * (units | 1) * 8)
+    if lds > 160 * 1024 - 512 or units > 16 or wt * wk > 12 or rt != 1:
+        return None
+    return (rt, wt, wk, splits, slab_k, row_groups, rounds)
+
+
+def run_case(dev, M, N, K, seed=0, bias=False, tuned=None):
     rng = np.random.default_rng(seed)
     layer = synth.make_qlinear(rng, N, K, bias=bias)
     x = synth.make_x(rng, M, K)
     want = oracle.qmm(x, layer["weight"], layer["scales"], layer["biases"], layer.get("bias"))
     d = layer_to_dev(layer, dev)
     got = ops.quantized_matmul(to_dev(x, dev), d["weight"], d["scales"], d["biases"],
-                               bias=d.get("bias"), variant=variant, splits=splits)
+                               bias=d.get("bias"), tuned=tuned)
     torch.cuda.synchronize()
     err = rel_err(got.cpu().numpy(), want)
-    assert err <= TOL, f"M={M} N={N} K={K} variant={variant} splits={splits}: rel err {err:.3e}"
+    assert err <= TOL, f"M={M} N={N} K={K} tuned={tuned}: rel err {err:.3e}"
     return err
 
 
@@ -30,20 +45,30 @@ def test_cfg1_shape_all_m(dev, M):
     run_case(dev, M, 8192, 2048, seed=42)
 
 
-@pytest.mark.parametrize("variant", range(6))
+@pytest.mark.parametrize("rt", [1])
+@pytest.mark.parametrize("wt,wk", [(4, 1), (2, 4), (1, 7), (12, 1), (2, 5), (3, 2)])
 @pytest.mark.parametrize("splits", [1, 2, 5])
+@pytest.mark.parametrize("rounds", [1, 3])
 @pytest.mark.parametrize("M", [8, 32])
-def test_every_variant_and_split(dev, variant, splits, M):
-    print(f"qmm variant={variant} splits={splits} M={M}", flush=True)
-    run_case(dev, M, 1536, 3584, seed=variant * 10 + splits, variant=variant, splits=splits)
+def test_forced_launch_shapes(dev, rt, wt, wk, splits, rounds, M):
+    N, K = 1536, 3584
+    tuned = shape_for(M, N, K, rt, wt, wk, splits, rounds)
+    if tuned is None:
+        pytest.skip("shape does not fit LDS / chunk count")
+    print(f"qmm tuned={tuned} M={M}", flush=True)
+    run_case(dev, M, N, K, seed=rt * 100 + wt * 10 + splits, tuned=tuned)
 
 
-@pytest.mark.parametrize("N,K", [(8, 64), (8, 128), (24, 192), (40, 896), (136, 2944), (512, 3584)])
+@pytest.mark.parametrize("N,K", [(8, 64), (8, 128), (24, 192), (40, 896), (136, 2944), (512, 3584),
+                                 (64, 18944)])
 def test_edge_shapes(dev, N, K):
     for M in (1, 5, 32):
         print(f"qmm edge N={N} K={K} M={M}", flush=True)
-        for variant in (-1, 0, 3):
-            run_case(dev, M, N, K, seed=N + K + M, variant=variant, splits=3)
+        run_case(dev, M, N, K, seed=N + K + M)
+        for cfg in ((1, 1, 1, 1, 1), (1, 2, 1, 3, 2), (1, 2, 2, 2, 1)):
+            tuned = shape_for(M, N, K, *cfg)
+            if tuned is not None:
+                run_case(dev, M, N, K, seed=N + K + M, tuned=tuned)
 
 
 def test_bias_and_leading_dims(dev):
@@ -80,10 +105,21 @@ def test_deterministic_split_k(dev):
     layer = synth.make_qlinear(rng, 512, 3584)
     x = to_dev(synth.make_x(rng, 32, 3584), dev)
     d = layer_to_dev(layer, dev)
-    ref = ops.quantized_matmul(x, d["weight"], d["scales"], d["biases"], variant=3, splits=7)
+    tuned = shape_for(32, 512, 3584, 1, 2, 2, 7, 2)
+    ref = ops.quantized_matmul(x, d["weight"], d["scales"], d["biases"], tuned=tuned)
     for _ in range(5):
-        again = ops.quantized_matmul(x, d["weight"], d["scales"], d["biases"], variant=3, splits=7)
+        again = ops.quantized_matmul(x, d["weight"], d["scales"], d["biases"], tuned=tuned)
         assert torch.equal(ref, again)
+
+
+def test_plan_covers_benchmark_shapes(dev):
+    for M in (1, 8, 16, 24, 32):
+        for N, K in ((3584, 3584), (512, 3584), (18944, 3584), (3584, 18944), (152064, 3584),
+                     (8192, 2048), (896, 896), (128, 896), (4864, 896), (896, 4864),
+                     (4096, 4096), (1024, 4096), (14336, 4096), (4096, 14336), (128256, 4096)):
+            rt, wt, wk, splits, slab_k, row_groups, rounds = ops.qmm_plan(M, N, K)
+            assert slab_k * splits >= K and row_groups * rounds * wt * rt * 16 >= N
+            assert wt * wk <= 16
 
 
 def test_argument_errors(dev):
