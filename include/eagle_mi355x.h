@@ -48,7 +48,7 @@ int eagle_check_device(void);
  *   q[n,k] = (wq[n,k/8] >> 4*(k%8)) & 15
  *   x [M,K] fp16 row-major, wq [N,K/8] uint32, scales/biases [N,K/64] fp16,
  *   bias [N] fp16 or NULL (added in fp16 after rounding), out [M,N] fp16.
- * Constraints: 1 <= M <= 32, K % 64 == 0, K <= 32768, N % 8 == 0, group_size == 64,
+ * Constraints: 1 <= M <= 32, K % 64 == 0, K <= 32768 (65536 for M <= 16), N % 8 == 0, group_size == 64,
  * bits == 4.
  * Replaces qmm_kernel.matmul (qmm_kernel.py:84-164) with the body
  * kernels/progression/simd_no_swizzle_cast.metal, the mx.quantized_matmul

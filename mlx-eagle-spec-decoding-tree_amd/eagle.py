@@ -1,0 +1,312 @@
+"""Tree speculative-decoding step: the reference's function names, argument order
+and return tuples (mlx_eagle.py:24-93, 217-376) on torch tensors, plus
+`TreeVerifier`, the same step as one HIP-graph replay with no host round trip.
+
+All index work runs in the single-workgroup kernels of csrc/tree.hip; the
+float work in the kernels of qmm / ops / attn.
+"""
+import math
+
+import torch
+
+from . import _lib, ops
+from .cache import KVCache
+
+MAXT = 32
+
+
+def _ptr(t):
+    return None if t is None else t.data_ptr()
+
+
+def _stream():
+    return torch.cuda.current_stream().cuda_stream
+
+
+def topk(x, k, axis=-1, stable=False):
+    """(indices, values) of the k largest entries, descending; equal values keep the
+    lowest index first.  The reference's non-stable branch (mlx_eagle.py:30-32) leaves
+    that order to argpartition; here both branches are stable."""
+    vals, idx = torch.sort(x.float(), dim=axis, descending=True, stable=True)
+    idx = idx.narrow(axis, 0, k)
+    return idx, torch.gather(x, axis, idx)
+
+
+def search_sorted(arr, target, left=True):
+    """Vectorised binary search with ceil(log2(n)) steps on uint32 bounds
+    (mlx_eagle.py:61-93).  int64 holds the uint32 values."""
+    n = arr.numel()
+    tgt = target.to(torch.int64) & 0xFFFFFFFF
+    low = torch.zeros_like(tgt)
+    high = torch.full_like(tgt, n)
+    a = arr.to(torch.int64) & 0xFFFFFFFF
+    for _ in range(int(math.ceil(math.log2(n))) if n > 1 else 0):
+        mid = (low + high) // 2
+        inside = mid < n
+        vals = a[torch.clamp(mid, max=n - 1)]
+        if left:
+            lt = (vals < tgt) & inside
+            ge = (vals >= tgt) & inside
+        else:
+            lt = (vals <= tgt) & inside
+            ge = (vals > tgt) & inside
+        low = torch.where(lt, mid + 1, low)
+        high = torch.where(ge, mid, high)
+    return low
+
+
+def bits_to_mask(bits, dtype=torch.bfloat16):
+    """[T] int32 row bitmasks -> [T,T] additive mask (0 where visible, -inf elsewhere)."""
+    T = bits.numel()
+    b = bits.to(torch.int64) & 0xFFFFFFFF
+    vis = ((b[:, None] >> torch.arange(T, device=bits.device)[None, :]) & 1).bool()
+    zero = torch.zeros((), dtype=dtype, device=bits.device)
+    return torch.where(vis, zero, torch.full((), -math.inf, dtype=dtype, device=bits.device))
+
+
+def process_draft_tree_device(scores, tokens, parents_list, sampled_token_id, k, total_tokens,
+                              out=None):
+    """Device-only form: flat fp16 scores [C], int32 tokens [C], parents [C/k] ->
+    (tree_position_ids [T], mask_index [V], draft_tokens [T], tree_mask_bits [T]), int32."""
+    dev = scores.device
+    T = total_tokens + 1
+    C = scores.numel()
+    if out is None:
+        out = (torch.empty(T, dtype=torch.int32, device=dev),
+               torch.empty(total_tokens, dtype=torch.int32, device=dev),
+               torch.empty(T, dtype=torch.int32, device=dev),
+               torch.empty(T, dtype=torch.int32, device=dev))
+    pos, midx, toks, bits = out
+    rc = _lib.lib().eagle_process_draft_tree(
+        _ptr(scores), _ptr(tokens), _ptr(parents_list), _ptr(sampled_token_id), C, k,
+        total_tokens, _ptr(pos), _ptr(midx), _ptr(toks), _ptr(bits), _stream())
+    _lib.check(rc, "process_draft_tree")
+    return out
+
+
+def process_draft_tree(scores_list, ss_token, parents_list, sampled_token_id, k, total_tokens):
+    """mlx_eagle.py:217-250.  Lists of per-level tensors in, and
+    (tree_position_ids [T], mask_index [V], draft_tokens [1,T], tree_mask [T,T] bf16) out."""
+    scores = torch.cat([s.reshape(s.shape[0], -1) for s in scores_list], dim=1).flatten()
+    tokens = torch.cat([t.reshape(t.shape[0], -1) for t in ss_token], dim=1).flatten()
+    parents = torch.cat([p.flatten() for p in parents_list], dim=0)
+    pos, midx, toks, bits = process_draft_tree_device(
+        scores.to(torch.float16).contiguous(), tokens.to(torch.int32).contiguous(),
+        parents.to(torch.int32).contiguous(),
+        sampled_token_id.to(torch.int32).reshape(-1)[:1].contiguous(), k, total_tokens)
+    return pos, midx, toks[None], bits_to_mask(bits)
+
+
+def post_process_draft_tree_device(tree_position_ids, total_tokens, mask_index, out=None):
+    """retrieve_indices [32,32] (-1 padded) and shape [2] = {leaf_num, max_depth+1}, on device."""
+    dev = tree_position_ids.device
+    if out is None:
+        out = (torch.empty((MAXT, MAXT), dtype=torch.int32, device=dev),
+               torch.empty(2, dtype=torch.int32, device=dev))
+    rc = _lib.lib().eagle_post_process_draft_tree(_ptr(tree_position_ids), _ptr(mask_index),
+                                                  total_tokens, _ptr(out[0]), _ptr(out[1]),
+                                                  _stream())
+    _lib.check(rc, "post_process_draft_tree")
+    return out
+
+
+def post_process_draft_tree(tree_position_ids, total_tokens, mask_index):
+    """mlx_eagle.py:254-295: retrieve_indices [leaf_num, max_depth+1]; like the reference
+    this form synchronises with the host (to learn the shape)."""
+    full, shape = post_process_draft_tree_device(tree_position_ids.to(torch.int32).contiguous(),
+                                                 total_tokens,
+                                                 mask_index.to(torch.int32).contiguous())
+    leaf_num, cols = (int(v) for v in shape.tolist())
+    return full[:leaf_num, :cols].contiguous()
+
+
+def evaluate_posterior_greedy(logits, candidates):
+    """mlx_eagle.py:311-326.  logits [n_leaves, cols, vocab], candidates [n_leaves, cols]."""
+    am = ops.argmax_rows(logits[:, :-1].contiguous())
+    posterior = (candidates[:, 1:].to(torch.int32) == am).to(torch.int32)
+    lens = torch.cumprod(posterior, dim=1).sum(dim=1)
+    accept_length = lens.max()
+    # first maximum (torch.argmax does not promise it): smallest index reaching the max
+    first = torch.nonzero(lens == accept_length)[0, 0]
+    best = torch.where(accept_length == 0, torch.zeros_like(first), first).to(torch.int32)
+    return best, accept_length, logits[best.long(), accept_length.long()]
+
+
+def tree_decoding(token_ids, tree_mask, tree_position_ids, base_model, cache):
+    """mlx_eagle.py:329-346."""
+    offset = cache[0].offset
+    T = tree_mask.shape[0]
+    mask = torch.zeros((1, 1, T, offset), dtype=tree_mask.dtype, device=tree_mask.device)
+    mask = torch.cat((mask, tree_mask[None, None]), dim=-1)
+    return base_model(token_ids, cache, position_ids=tree_position_ids[None] + offset, mask=mask)
+
+
+def accept_candidate(cache, accept_indices, accept_length, offset):
+    """mlx_eagle.py:349-376: for every layer move rows offset+accept_indices to
+    offset+1.., then set every cache length to offset + accept_length + 1."""
+    accept_length = int(accept_length)
+    if accept_length > 0:
+        dev = cache[0].keys.device
+        acc = torch.zeros(4 + MAXT, dtype=torch.int32, device=dev)
+        acc[1] = accept_length
+        acc[4:4 + accept_length] = accept_indices.to(torch.int32).reshape(-1)[:accept_length]
+        len_dev = torch.tensor([offset], dtype=torch.int32, device=dev)
+        ptrs = torch.tensor([c.keys.data_ptr() for c in cache] + [c.values.data_ptr() for c in cache],
+                            dtype=torch.int64, device=dev)
+        G, cap, hd = cache[0].keys.shape[1:]
+        rc = _lib.lib().eagle_kv_compact_f16(_ptr(ptrs), ptrs.numel(), _ptr(acc), _ptr(len_dev),
+                                             G, hd, cap, _stream())
+        _lib.check(rc, "accept_candidate")
+    for c in cache:
+        c.offset = offset + accept_length + 1
+
+
+class TreeVerifier:
+    """One target-model tree-verification step with static buffers, so that it can be
+    captured once in a HIP graph and replayed: embedding, all decoder layers, final norm,
+    output head, per-node argmax, greedy acceptance and KV compaction.  Inputs are written
+    into `tokens`, `tree_position_ids`, `mask_index` and `mask_bits`; results appear in
+    `logits`, `node_argmax`, `result` (best, accept_length, bonus_node, next_token,
+    accept_indices...) and `accepted_tokens`; the cache length advances on the device.
+    Same kernels and operator order as Model.__call__ + the host functions above."""
+
+    def __init__(self, model, cache, total_tokens=31, max_len=None, compact=True):
+        args = model.args
+        self.model, self.cache, self.args = model, cache, args
+        self.V = total_tokens
+        self.T = T = total_tokens + 1
+        dev = model.device
+        self.dev = dev
+        D, I = args.hidden_size, args.intermediate_size
+        H, G, hd = args.num_attention_heads, args.num_key_value_heads, args.head_dim
+        self.capacity = cache[0].capacity
+        self.max_len = max_len or self.capacity
+        self.compact = compact
+        i32 = dict(dtype=torch.int32, device=dev)
+        f16 = dict(dtype=torch.float16, device=dev)
+        self.tokens = torch.zeros(T, **i32)
+        self.tree_position_ids = torch.zeros(T, **i32)
+        self.mask_index = torch.zeros(total_tokens, **i32)
+        self.mask_bits = torch.zeros(T, **i32)
+        self.positions = torch.zeros(T, **i32)
+        self.retrieve = torch.zeros((MAXT, MAXT), **i32)
+        self.shape = torch.zeros(2, **i32)
+        self.node_argmax = torch.zeros(T, **i32)
+        self.result = torch.zeros(4 + MAXT, **i32)
+        self.accepted_tokens = torch.zeros(MAXT, **i32)
+        self.h = torch.empty((T, D), **f16)
+        self.hn = torch.empty((T, D), **f16)
+        self.q = torch.empty((T, H * hd), **f16)
+        self.k = torch.empty((T, G * hd), **f16)
+        self.v = torch.empty((T, G * hd), **f16)
+        self.q_rot = torch.empty((H, T, hd), **f16)
+        self.attn = torch.empty((T, H * hd), **f16)
+        self.o = torch.empty((T, D), **f16)
+        self.gate = torch.empty((T, I), **f16)
+        self.up = torch.empty((T, I), **f16)
+        self.act = torch.empty((T, I), **f16)
+        self.down = torch.empty((T, D), **f16)
+        self.logits = torch.empty((T, args.vocab_size), **f16)
+        self.len_dev = cache[0].len_dev
+        self.cache_ptrs = torch.tensor([c.keys.data_ptr() for c in cache]
+                                       + [c.values.data_ptr() for c in cache],
+                                       dtype=torch.int64, device=dev)
+        self.graph = None
+        # size every workspace before any capture
+        L = _lib.lib()
+        head = model.lm_head if not args.tie_word_embeddings else model.model.embed_tokens
+        need = max(L.eagle_qmm_workspace_bytes(T, n, k) for n, k in
+                   ((H * hd, D), (G * hd, D), (D, H * hd), (I, D), (D, I), (head.weight.shape[0], D)))
+        ops.workspace("qmm", need, dev)
+        ops.workspace("attn", L.eagle_tree_attention_workspace_bytes(H, hd, self.max_len), dev)
+        ops.workspace("argmax", L.eagle_argmax_workspace_bytes(T, args.vocab_size), dev)
+
+    def set_tree(self, tokens, tree_position_ids, mask_index, mask_bits):
+        self.tokens.copy_(tokens.reshape(-1))
+        self.tree_position_ids.copy_(tree_position_ids.reshape(-1))
+        self.mask_index.copy_(mask_index.reshape(-1))
+        self.mask_bits.copy_(mask_bits.reshape(-1))
+
+    def forward(self):
+        """Enqueue the whole step on the current stream (no synchronisation)."""
+        L = _lib.lib()
+        m = self.model
+        args = self.args
+        T = self.T
+        H, G, hd = args.num_attention_heads, args.num_key_value_heads, args.head_dim
+        st = _stream()
+        _lib.check(L.eagle_tree_positions(_ptr(self.tree_position_ids), _ptr(self.len_dev),
+                                          _ptr(self.positions), T, st), "tree_positions")
+        post_process_draft_tree_device(self.tree_position_ids, self.V, self.mask_index,
+                                       out=(self.retrieve, self.shape))
+        emb = m.model.embed_tokens
+        ops.embed(self.tokens, emb.weight, emb.scales, emb.biases, out=self.h)
+        layers = m.model.layers
+        ops.rms_norm(self.h, layers[0].input_layernorm.weight, args.rms_norm_eps, out=self.hn)
+        for i, layer in enumerate(layers):
+            at = layer.self_attn
+            for lin, out in ((at.q_proj, self.q), (at.k_proj, self.k), (at.v_proj, self.v)):
+                ops.quantized_matmul(self.hn, lin.weight, lin.scales, lin.biases, bias=lin.bias, out=out)
+            c = self.cache[i]
+            ops.rope_kv_append(self.q, self.k, self.v, self.positions, at._inv_freqs,
+                               at._scaling_factor, self.q_rot, c.keys[0], c.values[0],
+                               self.len_dev, H, G, hd)
+            ops.tree_attention(self.q_rot, c.keys[0], c.values[0], self.mask_bits, self.len_dev,
+                               at.scale, max_len=self.max_len, out=self.attn)
+            ops.quantized_matmul(self.attn, at.o_proj.weight, at.o_proj.scales, at.o_proj.biases,
+                                 bias=at.o_proj.bias, out=self.o)
+            ops.rms_norm(self.o, layer.post_attention_layernorm.weight, args.rms_norm_eps,
+                         residual=self.h, out=self.hn, h_out=self.h)
+            mlp = layer.mlp
+            ops.quantized_matmul(self.hn, mlp.gate_proj.weight, mlp.gate_proj.scales,
+                                 mlp.gate_proj.biases, bias=mlp.gate_proj.bias, out=self.gate)
+            ops.quantized_matmul(self.hn, mlp.up_proj.weight, mlp.up_proj.scales,
+                                 mlp.up_proj.biases, bias=mlp.up_proj.bias, out=self.up)
+            ops.silu_mul(self.gate, self.up, out=self.act)
+            ops.quantized_matmul(self.act, mlp.down_proj.weight, mlp.down_proj.scales,
+                                 mlp.down_proj.biases, bias=mlp.down_proj.bias, out=self.down)
+            nxt = layers[i + 1].input_layernorm.weight if i + 1 < len(layers) else m.model.norm.weight
+            ops.rms_norm(self.down, nxt, args.rms_norm_eps, residual=self.h, out=self.hn, h_out=self.h)
+        head = m.model.embed_tokens if args.tie_word_embeddings else m.lm_head
+        ops.quantized_matmul(self.hn, head.weight, head.scales, head.biases, out=self.logits)
+        ops.argmax_rows(self.logits, out=self.node_argmax)
+        _lib.check(L.eagle_greedy_accept(_ptr(self.node_argmax), _ptr(self.tokens),
+                                         _ptr(self.retrieve), _ptr(self.shape), T,
+                                         _ptr(self.result), _ptr(self.accepted_tokens), st),
+                   "greedy_accept")
+        if self.compact:
+            c0 = self.cache[0]
+            _lib.check(L.eagle_kv_compact_f16(_ptr(self.cache_ptrs), self.cache_ptrs.numel(),
+                                              _ptr(self.result), _ptr(self.len_dev), G, hd,
+                                              c0.capacity, st), "kv_compact")
+
+    def capture(self):
+        """Record forward() into a HIP graph (after one eager warm-up on a side stream)."""
+        saved_len = self.len_dev.clone()
+        side = torch.cuda.Stream()
+        side.wait_stream(torch.cuda.current_stream())
+        with torch.cuda.stream(side):
+            self.forward()
+        torch.cuda.current_stream().wait_stream(side)
+        torch.cuda.synchronize()
+        self.len_dev.copy_(saved_len)
+        self.graph = torch.cuda.CUDAGraph()
+        with torch.cuda.graph(self.graph):
+            self.forward()
+        self.len_dev.copy_(saved_len)
+        torch.cuda.synchronize()
+        return self
+
+    def step(self):
+        """Run one verification step (graph replay when captured)."""
+        if self.graph is not None:
+            self.graph.replay()
+        else:
+            self.forward()
+
+    def sync_host_offsets(self):
+        """Bring the host-side cache offsets in line with the device length (one D2H copy)."""
+        n = int(self.len_dev.item())
+        for c in self.cache:
+            c.offset = n
+        return n

@@ -211,27 +211,33 @@ def scaled_dot_product_attention(queries, keys, values, cache=None, scale=None, 
     m = mask.reshape(T, S)
     bits = mask_to_bits(m[:, P:])
     len_dev = torch.tensor([P], dtype=torch.int32, device=queries.device)
-    out = tree_attention(_f16(queries[0], "q"), _f16(keys[0], "k"), _f16(values[0], "v"), bits,
-                         len_dev, scale, max_len=S)
+    if cache is not None and keys.data_ptr() == cache.keys.data_ptr():
+        k_buf, v_buf = cache.keys[0], cache.values[0]        # the fetched views alias the cache
+    else:
+        k_buf, v_buf = _f16(keys[0], "k"), _f16(values[0], "v")
+    out = tree_attention(_f16(queries[0], "q"), k_buf, v_buf, bits, len_dev, scale, max_len=S)
     return out.reshape(T, H, hd).permute(1, 0, 2).unsqueeze(0).contiguous()
 
 
-def rms_norm(x, weight, eps, residual=None):
+def rms_norm(x, weight, eps, residual=None, out=None, h_out=None):
     """`mx.fast.rms_norm(x, weight, eps)`; with `residual` returns (h, norm(h)),
-    h = fp16(x + residual)."""
+    h = fp16(x + residual) (h_out may alias residual for an in-place update)."""
     _need_cuda(x, weight, residual)
     x = _f16(x, "x")
     D = x.shape[-1]
     T = x.numel() // D
-    out = torch.empty_like(x)
-    h = torch.empty_like(x) if residual is not None else None
+    if out is None:
+        out = torch.empty_like(x)
+    h = None
+    if residual is not None:
+        h = h_out if h_out is not None else torch.empty_like(x)
     rc = _lib.lib().eagle_rmsnorm_f16(_ptr(x), _ptr(residual), _ptr(_f16(weight, "weight")),
                                       float(eps), _ptr(h), _ptr(out), T, D, _stream())
     _lib.check(rc, "rms_norm")
     return out if residual is None else (h, out)
 
 
-def silu_mul(gate, up=None):
+def silu_mul(gate, up=None, out=None):
     """fp16(fp16(silu(gate)) * up); with up=None, `gate` is the fused [T, 2*I] tensor."""
     _need_cuda(gate, up)
     gate = _f16(gate, "gate")
@@ -241,7 +247,8 @@ def silu_mul(gate, up=None):
         up = _f16(up, "up")
         I = gate.shape[-1]
     T = gate.numel() // gate.shape[-1]
-    out = torch.empty((*gate.shape[:-1], I), dtype=torch.float16, device=gate.device)
+    if out is None:
+        out = torch.empty((*gate.shape[:-1], I), dtype=torch.float16, device=gate.device)
     rc = _lib.lib().eagle_silu_mul_f16(_ptr(gate), _ptr(up), _ptr(out), T, I, _stream())
     _lib.check(rc, "silu_mul")
     return out
@@ -256,13 +263,14 @@ def add(a, b):
     return out
 
 
-def embed(ids, w_q, scales, biases):
+def embed(ids, w_q, scales, biases, out=None):
     """Quantised embedding lookup: ids [...] int -> [..., D] fp16."""
     _need_cuda(ids, w_q, scales, biases)
     w_q = as_packed_u32(w_q)
     V, D = w_q.shape[0], w_q.shape[1] * 8
     ids32 = ids.to(torch.int32).contiguous()
-    out = torch.empty((*ids.shape, D), dtype=torch.float16, device=ids.device)
+    if out is None:
+        out = torch.empty((*ids.shape, D), dtype=torch.float16, device=ids.device)
     rc = _lib.lib().eagle_embed_w4g64_f16(_ptr(ids32), _ptr(w_q), _ptr(_f16(scales, "scales")),
                                           _ptr(_f16(biases, "biases")), _ptr(out), ids32.numel(),
                                           D, V, _stream())

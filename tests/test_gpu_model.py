@@ -1,0 +1,199 @@
+"""Whole tree-verification step on small random-init decoders: HIP path vs the CPU oracle."""
+import numpy as np
+import pytest
+import torch
+
+from mlx_eagle_spec_decoding_tree_amd import eagle, llama, ops, synth
+from mlx_eagle_spec_decoding_tree_amd.cache import make_prompt_cache
+from oracle import model_oracle, oracle, tree_oracle
+from util import TOL, rel_err, to_dev
+
+pytestmark = pytest.mark.gpu
+
+CONFIGS = {
+    "qwen_like": dict(layers=2, hidden=256, inter=512, heads=4, kv_heads=2, head_dim=64, vocab=1024,
+                      attention_bias=True, tie=False),
+    "llama_like_tied": dict(layers=2, hidden=512, inter=768, heads=4, kv_heads=4, head_dim=128, vocab=640,
+                            attention_bias=False, tie=True, theta=5e5),
+}
+
+
+def build(dev, name, P, T, seed=0, cap=None):
+    args = synth.tiny(**CONFIGS[name])
+    weights = synth.make_model_weights(args, seed=seed)
+    model = llama.Model.from_numpy(args, weights, dev)
+    cap = cap or (P + T + 16)
+    rng = np.random.default_rng(seed + 1)
+    G, hd = args.num_key_value_heads, args.head_dim
+    prefix = [(rng.normal(size=(G, P, hd)).astype(np.float16), rng.normal(size=(G, P, hd)).astype(np.float16))
+              for _ in range(args.num_hidden_layers)]
+    cache = make_prompt_cache(model, capacity=cap)
+    ocache = model_oracle.new_cache(args, cap)
+    for c, (k, v), (ok, ov) in zip(cache, prefix, ocache):
+        c.keys[0, :, :P].copy_(to_dev(k, dev)); c.values[0, :, :P].copy_(to_dev(v, dev))
+        c.offset = P
+        ok[:, :P] = k; ov[:, :P] = v
+    cache[0].sync_len()
+    parents = synth.random_tree(rng, T)
+    depth, anc = tree_oracle.tree_from_parents(parents)
+    tokens = rng.integers(0, args.vocab_size, T).astype(np.int32)
+    inv, sc = synth.inv_freqs(args)
+    return dict(args=args, weights=weights, model=model, cache=cache, ocache=ocache, parents=parents,
+                depth=depth, anc=anc, tokens=tokens, inv=inv, sc=sc, P=P, T=T)
+
+
+def margins(logits):
+    srt = np.sort(logits.astype(np.float32), axis=-1)
+    return srt[:, -1] - srt[:, -2]
+
+
+@pytest.mark.parametrize("name", list(CONFIGS))
+@pytest.mark.parametrize("P,T", [(40, 8), (300, 32)])
+def test_tree_decoding_matches_oracle(dev, name, P, T):
+    print(f"model {name} P={P} T={T}", flush=True)
+    s = build(dev, name, P, T)
+    mask_np = np.concatenate([np.zeros((T, P), np.float16), tree_oracle.additive_mask(s["anc"])], axis=1)
+    want = model_oracle.tree_forward(s["args"], s["weights"], s["inv"], s["sc"], s["tokens"],
+                                     s["depth"] + P, mask_np, s["ocache"], P)
+    tree_mask = to_dev(tree_oracle.additive_mask(s["anc"]), dev).to(torch.bfloat16)
+    logits = eagle.tree_decoding(to_dev(s["tokens"][None], dev), tree_mask, to_dev(s["depth"], dev),
+                                 s["model"], s["cache"])
+    assert tuple(logits.shape) == (1, T, s["args"].vocab_size)
+    got = logits[0].cpu().numpy()
+    assert rel_err(got, want) <= TOL
+    assert s["cache"][0].offset == P + T
+    # argmax tokens agree wherever the oracle's top-2 margin exceeds the observed error
+    err = np.abs(got.astype(np.float32) - want.astype(np.float32)).max()
+    am_g, am_w = np.argmax(got.astype(np.float32), -1), oracle.argmax_rows(want)
+    clear = margins(want) > 2 * err
+    assert clear.sum() >= T // 2 and np.array_equal(am_g[clear], am_w[clear])
+    # the appended KV rows match the oracle's
+    for c, (ok, ov) in zip(s["cache"], s["ocache"]):
+        assert rel_err(c.keys[0, :, P:P + T].cpu().numpy(), ok[:, P:P + T]) <= TOL
+        assert rel_err(c.values[0, :, P:P + T].cpu().numpy(), ov[:, P:P + T]) <= TOL
+
+
+def run_verifier(s, dev, graph):
+    T = s["T"]
+    ver = eagle.TreeVerifier(s["model"], s["cache"], total_tokens=T - 1, max_len=s["cache"][0].capacity)
+    ver.set_tree(to_dev(s["tokens"], dev), to_dev(s["depth"], dev), to_dev(s["parents"], dev),
+                 to_dev(tree_oracle.mask_bits(s["anc"]).view(np.int32), dev))
+    if graph:
+        ver.capture()
+    return ver
+
+
+@pytest.mark.parametrize("name", list(CONFIGS))
+def test_fused_step_equals_module_path_and_oracle(dev, name):
+    P, T = 200, 32
+    s = build(dev, name, P, T, seed=3)
+    # module path (reference-shaped) on a copy of the cache
+    s2 = build(dev, name, P, T, seed=3)
+    tree_mask = to_dev(tree_oracle.additive_mask(s2["anc"]), dev).to(torch.bfloat16)
+    ref_logits = eagle.tree_decoding(to_dev(s2["tokens"][None], dev), tree_mask, to_dev(s2["depth"], dev),
+                                     s2["model"], s2["cache"])[0]
+    ver = run_verifier(s, dev, graph=False)
+    ver.step()
+    torch.cuda.synchronize()
+    assert torch.equal(ver.logits, ref_logits), "fused step and module path must be bit-identical"
+    want = model_oracle.verify_step(s["args"], s["weights"], s["inv"], s["sc"], s["tokens"], s["depth"],
+                                    s["parents"], s["anc"], s["ocache"], P)
+    assert rel_err(ver.logits.cpu().numpy(), want["logits"]) <= TOL
+    # integer stages are bit-exact given the device's own argmax
+    am = ver.node_argmax.cpu().numpy()
+    assert np.array_equal(am, oracle.argmax_rows(ver.logits.cpu().numpy()))
+    ri = tree_oracle.post_process_draft_tree(s["depth"], T - 1, s["parents"])
+    best, al, bonus = tree_oracle.greedy_accept(am, s["tokens"], ri)
+    r = ver.result.cpu().numpy()
+    assert (r[0], r[1], r[2], r[3]) == (best, al, bonus, am[bonus])
+    assert ver.sync_host_offsets() == P + al + 1
+    # and equal to the oracle's decision whenever its argmax margins are clear
+    err = np.abs(ver.logits.cpu().numpy().astype(np.float32) - want["logits"].astype(np.float32)).max()
+    if (margins(want["logits"]) > 2 * err).all():
+        assert (best, al, am[bonus]) == (want["best"], want["accept_length"], want["next_token"])
+
+
+@pytest.mark.parametrize("name", list(CONFIGS))
+def test_graph_replays_match_eager(dev, name):
+    """Replay the captured step several times with eager work and synchronisation in
+    between; every replay must reproduce the eager result."""
+    P, T = 120, 32
+    s = build(dev, name, P, T, seed=5)
+    eager = run_verifier(s, dev, graph=False)
+    eager.step()
+    torch.cuda.synchronize()
+    want_logits, want_result = eager.logits.clone(), eager.result.clone()
+    want_k = [c.keys.clone() for c in s["cache"]]
+    s2 = build(dev, name, P, T, seed=5)
+    ver = run_verifier(s2, dev, graph=True)
+    for rep in range(4):
+        s2["cache"][0].offset = P
+        s2["cache"][0].sync_len()
+        _ = ops.add(ver.h, ver.h)                       # unrelated eager work between replays
+        torch.cuda.synchronize()
+        ver.step()
+        torch.cuda.synchronize()
+        assert torch.equal(ver.logits, want_logits), f"replay {rep}"
+        assert torch.equal(ver.result, want_result), f"replay {rep}"
+        for c, k in zip(s2["cache"], want_k):
+            assert torch.equal(c.keys, k)
+        assert int(ver.len_dev.item()) == P + int(want_result[1]) + 1
+
+
+def test_accepted_path_cache_equals_sequential_decode(dev):
+    """mlx_eagle_tests.py:135-170: after acceptance the speculative cache equals the cache of a
+    plain sequential decode of the accepted tokens.  The tree is built so that one path is
+    accepted in full: each node's token is the target's own greedy continuation."""
+    name, P = "qwen_like", 64
+    s = build(dev, name, P, 2, seed=9)
+    args, model = s["args"], s["model"]
+    # sequential greedy decode of 5 tokens from a random root, one token at a time
+    rng = np.random.default_rng(1)
+    root = int(rng.integers(0, args.vocab_size))
+    seq_cache = s["cache"]
+    toks = [root]
+    one = to_dev(tree_oracle.additive_mask(np.ones((1, 1), bool)), dev).to(torch.bfloat16)
+    for step in range(5):
+        lg = eagle.tree_decoding(torch.tensor([[toks[-1]]], dtype=torch.int32, device=dev), one,
+                                 torch.zeros(1, dtype=torch.int32, device=dev), model, seq_cache)
+        toks.append(int(ops.argmax_rows(lg[0])[0]))
+    # speculative: a chain root -> t1 -> t2 -> t3 -> t4 plus a wrong sibling at every level
+    s2 = build(dev, name, P, 2, seed=9)
+    parents = np.array([0, 0, 1, 1, 3, 3, 5, 5], np.int32)            # nodes 1,3,5,7 form the chain
+    T = len(parents) + 1
+    depth, anc = tree_oracle.tree_from_parents(parents)
+    tokens = np.zeros(T, np.int32)
+    tokens[0] = root
+    for lvl, node in enumerate([1, 3, 5, 7]):
+        tokens[node] = toks[lvl + 1]
+        tokens[node + 1] = (toks[lvl + 1] + 1) % args.vocab_size
+    s2.update(parents=parents, depth=depth, anc=anc, tokens=tokens, T=T)
+    ver = run_verifier(s2, dev, graph=False)
+    ver.step()
+    torch.cuda.synchronize()
+    r = ver.result.cpu().numpy()
+    assert r[1] == 4 and list(r[4:8]) == [1, 3, 5, 7] and r[3] == toks[5]
+    n = ver.sync_host_offsets()
+    assert n == P + 5 == seq_cache[0].offset
+    for a, b in zip(s2["cache"], seq_cache):
+        assert rel_err(a.keys[0, :, :n].cpu().numpy(), b.keys[0, :, :n].cpu().numpy()) <= 5e-3
+        assert rel_err(a.values[0, :, :n].cpu().numpy(), b.values[0, :, :n].cpu().numpy()) <= 5e-3
+
+
+def test_patch_model_uses_the_supplied_kernel(dev):
+    s = build(dev, "qwen_like", 30, 8, seed=11)
+    calls = []
+
+    def kernel(x, w, sc, b, group_size):
+        calls.append(tuple(x.shape))
+        return ops.matmul(x, w, sc, b, group_size)[0]
+
+    base = build(dev, "qwen_like", 30, 8, seed=11)
+    tree_mask = to_dev(tree_oracle.additive_mask(s["anc"]), dev).to(torch.bfloat16)
+    want = eagle.tree_decoding(to_dev(base["tokens"][None], dev), tree_mask, to_dev(base["depth"], dev),
+                               base["model"], base["cache"])
+    llama.patch_model(s["model"], kernel)
+    got = eagle.tree_decoding(to_dev(s["tokens"][None], dev), tree_mask, to_dev(s["depth"], dev),
+                              s["model"], s["cache"])
+    assert len(calls) == 2 * 7 + 1 and all(c == (1, 8, c[2]) for c in calls)
+    assert torch.equal(got, want)

@@ -1,0 +1,112 @@
+"""CPU-only checks of the C-ABI library: it loads, exports every symbol the header
+declares, and rejects bad arguments on the host before any device work."""
+import ctypes
+import os
+import re
+
+import pytest
+import torch
+
+from mlx_eagle_spec_decoding_tree_amd import _lib, ops
+
+ROOT = os.path.dirname(os.path.dirname(os.path.abspath(__file__)))
+HEADER = os.path.join(ROOT, "include", "eagle_mi355x.h")
+
+
+def declared_symbols():
+    text = open(HEADER).read()
+    text = re.sub(r"/\*.*?\*/", "", text, flags=re.S)
+    return sorted(set(re.findall(r"\b(eagle_[a-z0-9_]+)\s*\(", text)))
+
+
+def test_library_exports_every_declared_symbol():
+    lib = ctypes.CDLL(_lib.LIB_PATH)
+    names = declared_symbols()
+    assert len(names) >= 25
+    for n in names:
+        assert hasattr(lib, n), f"{n} declared in the header but not exported"
+    # and the Python binding knows each of them
+    assert set(names) == set(_lib.SIGNATURES), set(names) ^ set(_lib.SIGNATURES)
+
+
+def test_status_strings_and_version():
+    L = _lib.lib()
+    assert L.eagle_abi_version() == 1
+    assert L.eagle_status_string(0) == b"ok"
+    for rc in range(1, 8):
+        assert len(L.eagle_status_string(rc)) > 3
+
+
+def test_qmm_argument_errors_are_detected_on_the_host():
+    L = _lib.lib()
+    buf = (ctypes.c_char * 4096)()
+    p = ctypes.addressof(buf)
+    p = (p + 15) & ~15
+    call = lambda **kw: L.eagle_qmm_w4g64_f16(kw.get("x", p), kw.get("w", p), kw.get("s", p), kw.get("b", p),
+                                              None, kw.get("out", p), kw.get("M", 8), kw.get("N", 64),
+                                              kw.get("K", 128), kw.get("gs", 64), kw.get("bits", 4),
+                                              None, 0, None)
+    assert call(x=None) == 1                       # EAGLE_ERR_NULL
+    assert call(out=None) == 1
+    assert call(M=0) == 2 and call(M=33) == 2      # EAGLE_ERR_SHAPE
+    assert call(K=100) == 2 and call(N=12) == 2 and call(K=128 * 1024) == 2
+    assert call(x=p + 2) == 3                      # EAGLE_ERR_ALIGN
+    assert call(gs=32) == 4 and call(bits=8) == 4  # EAGLE_ERR_UNSUPPORTED
+    # a K-split launch needs a workspace
+    assert L.eagle_qmm_w4g64_f16(p, p, p, p, None, p, 32, 3584, 3584, 64, 4, None, 0, None) == 5
+    assert L.eagle_qmm_workspace_bytes(32, 3584, 3584) > 65536
+    assert L.eagle_qmm_workspace_bytes(8, 152064, 3584) == 65536
+
+
+def test_other_entry_points_reject_bad_arguments():
+    L = _lib.lib()
+    buf = (ctypes.c_char * 4096)()
+    p = (ctypes.addressof(buf) + 15) & ~15
+    assert L.eagle_rope_arrayed_f16(None, p, p, 1.0, p, 1, 1, 1, 64, None) == 1
+    assert L.eagle_rope_arrayed_f16(p, p, p, 1.0, p, 1, 1, 1, 63, None) == 2
+    assert L.eagle_rope_kv_append_f16(p, p, p, p, p, 1.0, p, p, p, p, 33, 4, 2, 64, 100, None) == 2
+    assert L.eagle_tree_attention_f16(p, p, p, p, p, p, 32, 28, 4, 96, 4096, 2080, 0.1, p, 1 << 30, None) == 2
+    assert L.eagle_tree_attention_f16(p, p, p, p, p, p, 32, 28, 4, 128, 4096, 2080, 0.1, None, 0, None) == 5
+    assert L.eagle_rmsnorm_f16(p, None, p, 1e-6, None, p, 4, 100, None) == 2
+    assert L.eagle_rmsnorm_f16(p, p, p, 1e-6, None, p, 4, 128, None) == 1      # residual needs h_out
+    assert L.eagle_silu_mul_f16(p, None, p, 4, 12, None) == 2
+    assert L.eagle_add_f16(p, p, p + 2, 16, None) == 3
+    assert L.eagle_embed_w4g64_f16(p, p, p, p, p, 4, 100, 10, None) == 2
+    assert L.eagle_argmax_rows_f16(p, p, 4, 1000, None, 0, None) == 5
+    assert L.eagle_process_draft_tree(p, p, p, p, 200, 8, 32, p, p, p, p, None) == 2    # total must be < 32
+    assert L.eagle_process_draft_tree(p, p, p, p, 2000, 8, 31, p, p, p, p, None) == 2   # too many candidates
+    assert L.eagle_post_process_draft_tree(p, p, 0, p, p, None) == 2
+    assert L.eagle_greedy_accept(p, p, p, p, 40, p, p, None) == 2
+    assert L.eagle_kv_compact_f16(None, 4, p, p, 4, 128, 100, None) == 1
+    assert L.eagle_tree_positions(p, p, p, 0, None) == 2
+
+
+def test_plan_is_consistent_for_benchmark_shapes():
+    for M in (1, 8, 16, 24, 32):
+        for N, K in ((3584, 3584), (512, 3584), (18944, 3584), (3584, 18944), (152064, 3584),
+                     (8192, 2048), (896, 896), (128, 896), (4864, 896), (896, 4864), (151936, 896),
+                     (4096, 4096), (1024, 4096), (14336, 4096), (4096, 14336), (128256, 4096)):
+            rt, wt, wk, splits, slab_k, row_groups, rounds = ops.qmm_plan(M, N, K)
+            assert slab_k % 256 == 0 and slab_k * splits >= K > slab_k * (splits - 1)
+            assert row_groups * rounds * wt * rt * 16 >= N
+            assert 1 <= wt * wk <= 12 and slab_k <= (4096 if M <= 16 else 2048)
+
+
+def test_ops_refuse_cpu_tensors():
+    x = torch.zeros(8, 128, dtype=torch.float16)
+    w = torch.zeros(8, 16, dtype=torch.int32)
+    s = torch.zeros(8, 2, dtype=torch.float16)
+    with pytest.raises(RuntimeError):
+        ops.quantized_matmul(x, w, s, s)
+    with pytest.raises(RuntimeError):
+        ops.arrayed_rope(torch.zeros(1, 1, 2, 64, dtype=torch.float16), torch.zeros(1, 2, dtype=torch.int32))
+
+
+def test_mask_bit_helpers_round_trip():
+    from mlx_eagle_spec_decoding_tree_amd import eagle
+    vis = torch.tril(torch.ones(32, 32, dtype=torch.bool))
+    bits = ops.mask_to_bits(vis)
+    assert bits.dtype == torch.int32 and bits[0].item() == 1 and bits[31].item() == -1
+    back = eagle.bits_to_mask(bits, torch.float32)
+    assert torch.equal(back == 0, vis)
+    assert torch.equal(ops.mask_to_bits(back), bits)

@@ -1,0 +1,188 @@
+"""Pins the integer oracle (oracle/tree_oracle.py) against the reference's golden tree,
+brute force with explicit parent pointers, and the documented quirks.  CPU only."""
+import json
+import os
+
+import numpy as np
+import pytest
+
+from mlx_eagle_spec_decoding_tree_amd import synth
+from oracle import tree_oracle as to
+
+HERE = os.path.dirname(os.path.abspath(__file__))
+
+
+@pytest.fixture(scope="module")
+def fixture():
+    with open(os.path.join(HERE, "golden", "tree_fixture.json")) as f:
+        return json.load(f)
+
+
+def test_reference_fixture_mask_depth_paths(fixture):
+    parents = np.array(fixture["mask_index"], np.int32)
+    depth, anc = to.tree_from_parents(parents)
+    assert anc.astype(int).tolist() == fixture["tree_mask"]
+    assert depth.tolist() == fixture["tree_position_ids"]
+    ri = to.post_process_draft_tree(depth, fixture["total_tokens"], parents)
+    assert ri.tolist() == fixture["retrieve_indices"]
+
+
+def test_reference_fixture_greedy_accept(fixture):
+    ri = np.array(fixture["retrieve_indices"])
+    T = 8
+    tokens = np.arange(100, 100 + T)                 # node j carries token 100 + j
+    path = ri[fixture["correct_draft_index"]]
+    node_argmax = np.full(T, -1)
+    for a, b in zip(path[:-1], path[1:]):            # the target agrees along path 1
+        node_argmax[a] = tokens[b]
+    node_argmax[path[-1]] = 33894                    # bonus token id of mlx_eagle_tests.py:124
+    best, al, bonus = to.greedy_accept(node_argmax, tokens, ri)
+    assert (best, al) == (fixture["expected_best_candidate"], fixture["expected_accept_length"])
+    assert node_argmax[bonus] == 33894
+    # array form on synthetic logits gives the same answer
+    V = 40000
+    logits = np.full((T, V), -1.0, np.float16)
+    for j in range(T):
+        logits[j, node_argmax[j] if node_argmax[j] >= 0 else 7] = 1.0
+    cand = tokens[ri]                                # -1 wraps to the last node, as in the reference
+    b2, al2, row = to.evaluate_posterior_greedy(logits[ri], cand)
+    assert (b2, al2) == (best, al) and int(np.argmax(row)) == 33894
+
+
+def simulate_draft(rng, depth, k=8, tie_levels=None):
+    """Ground-truth simulation of the draft expansion that feeds process_draft_tree:
+    returns flat scores, tokens, parents_list and, separately tracked, the true parent
+    candidate id of every candidate (-1 = root)."""
+    scores, tokens, true_parent = [], [], []
+    parents_list = [0]
+    # level 0: the root's k children
+    lvl_scores = -np.sort(rng.uniform(0.1, 3.0, k))                     # descending log-probs
+    if tie_levels:
+        lvl_scores = np.round(lvl_scores * tie_levels) / tie_levels
+    scores += list(lvl_scores); tokens += list(rng.integers(0, 1000, k)); true_parent += [-1] * k
+    frontier_ids = list(range(k))                                       # flat ids of the selected nodes
+    frontier_scores = lvl_scores
+    for i in range(depth):
+        base = k + k * k * i
+        child = frontier_scores[:, None] - np.sort(rng.uniform(0.1, 3.0, (k, k)), axis=1)
+        if tie_levels:
+            child = np.round(child * tie_levels) / tie_levels
+        for r in range(k):
+            parents_list.append(frontier_ids[r] + 1)                    # parent flat id + 1
+            for c in range(k):
+                scores.append(child[r, c]); tokens.append(int(rng.integers(0, 1000)))
+                true_parent.append(frontier_ids[r])
+        flat = child.reshape(-1)
+        top = np.argsort(-flat, kind="stable")[:k]
+        frontier_ids = [base + int(t) for t in top]
+        frontier_scores = flat[top]
+    return (np.array(scores, np.float16), np.array(tokens, np.int32),
+            np.array(parents_list, np.uint32), np.array(true_parent))
+
+
+@pytest.mark.parametrize("depth", [0, 1, 2, 3, 5])
+@pytest.mark.parametrize("V", [7, 15, 23, 31])
+def test_process_draft_tree_against_parent_pointers(depth, V):
+    rng = np.random.default_rng(depth * 100 + V)
+    for trial in range(25):
+        scores, tokens, parents_list, true_parent = simulate_draft(rng, depth, tie_levels=(8 if trial % 2 else None))
+        if V > scores.size:
+            pytest.skip("fewer candidates than requested nodes")
+        pos, midx, dtoks, anc = to.process_draft_tree(scores, tokens, parents_list, np.array([[5]]), 8, V)
+        order = np.argsort(-scores.astype(np.float64), kind="stable")[:V]
+        sel = np.sort(order)
+        assert dtoks[0, 0] == 5 and np.array_equal(dtoks[0, 1:], tokens[sel])
+        # brute force: parent node = 1 + rank of the true parent candidate among the selected
+        rank = {int(c): i for i, c in enumerate(sel)}
+        for j, c in enumerate(sel):
+            tp = int(true_parent[c])
+            want = 0 if tp < 0 else 1 + rank[tp]          # the parent of a selected node is selected
+            assert midx[j] == want and want <= j
+        d2, anc2 = to.tree_from_parents(midx)
+        assert np.array_equal(anc, anc2) and np.array_equal(pos, d2)
+        assert pos.max() <= depth + 1
+        # paths
+        ri = to.post_process_draft_tree(pos, V, midx)
+        inner = set(int(m) for m in midx)
+        leaves = [n for n in range(V + 1) if n not in inner]
+        assert ri.shape == (len(leaves), pos.max() + 1)
+        for row, leaf in zip(ri, leaves):
+            path = [leaf]
+            while path[-1] != 0:
+                path.append(int(midx[path[-1] - 1]))
+            path = path[::-1]
+            assert list(row[:len(path)]) == path and all(v == -1 for v in row[len(path):])
+
+
+def test_topk_ties_keep_lowest_index():
+    x = np.array([1.0, 3.0, 3.0, 2.0, 3.0], np.float16)
+    idx, vals = to.topk(x, 3)
+    assert idx.tolist() == [1, 2, 4] and vals.tolist() == [3.0, 3.0, 3.0]
+
+
+def test_search_sorted_matches_numpy_on_found_targets():
+    """ceil(log2(n)) steps resolve n+1 possible answers for the node counts the reference
+    uses (7, 15, 23, 31); the step count is part of the restated behaviour."""
+    rng = np.random.default_rng(0)
+    for n in (7, 15, 23, 31):
+        arr = np.sort(rng.choice(200, n, replace=False)).astype(np.uint32)
+        tgt = rng.choice(arr, 12)
+        assert np.array_equal(to.search_sorted(arr, tgt), np.searchsorted(arr, tgt, side="left"))
+    # n = 2 gets a single step, one too few: the fixed step count of mlx_eagle.py:76 is kept
+    assert to.search_sorted(np.array([102, 126], np.uint32), np.array([126])).tolist() == [0]
+
+
+def brute_greedy(node_argmax, tokens, ri):
+    T = len(tokens)
+    best, best_len = 0, 0
+    for r, row in enumerate(ri):
+        n = 0
+        for a, b in zip(row[:-1], row[1:]):
+            if tokens[b % T] == node_argmax[a % T]:
+                n += 1
+            else:
+                break
+        if n > best_len:
+            best, best_len = r, n
+    return best, best_len
+
+
+def test_greedy_accept_brute_force_and_padding_quirk():
+    rng = np.random.default_rng(3)
+    for trial in range(200):
+        T = int(rng.integers(2, 33))
+        parents = synth.random_tree(rng, T)
+        depth, anc = to.tree_from_parents(parents)
+        ri = to.post_process_draft_tree(depth, T - 1, parents)
+        tokens = rng.integers(0, 6, T)
+        node_argmax = rng.integers(0, 6, T)
+        best, al, bonus = to.greedy_accept(node_argmax, tokens, ri)
+        assert (best, al) == brute_greedy(node_argmax, tokens, ri)
+        assert bonus == ri[best, al] % T
+        lg = np.zeros((T, 6), np.float16)
+        lg[np.arange(T), node_argmax] = 1
+        b2, al2, _ = to.evaluate_posterior_greedy(lg[ri], tokens[ri])
+        assert (b2, al2) == (best, al)
+    # a -1 pad selects the last node (mlx_eagle.py:582,584): the short path of the fixture is
+    # extended when the target's argmax at its leaf equals the last node's token
+    ri = np.array([[0, 1, 2, 4, 6, -1], [0, 1, 2, 3, 5, 7]])
+    tokens = np.array([0, 1, 2, 3, 4, 5, 6, 7])
+    node_argmax = np.array([1, 2, 4, 9, 6, 9, 7, 9])      # path 0 all right, then leaf 6 -> token 7
+    best, al, bonus = to.greedy_accept(node_argmax, tokens, ri)
+    assert (best, al, bonus) == (0, 5, 7)
+
+
+def test_accept_candidate_gather_then_scatter():
+    rng = np.random.default_rng(4)
+    G, cap, hd, P = 2, 64, 8, 20
+    k0 = rng.normal(size=(G, cap, hd)).astype(np.float16)
+    v0 = rng.normal(size=(G, cap, hd)).astype(np.float16)
+    for idx in ([1, 2, 3], [2, 5, 9], [3], [1, 4], [-1, 5]):
+        k, v = k0.copy(), v0.copy()
+        new = to.accept_candidate(k, v, np.array(idx), len(idx), P)
+        assert new == P + len(idx) + 1
+        for j, i in enumerate(idx):
+            assert np.array_equal(k[:, P + 1 + j], k0[:, P + i]) and np.array_equal(v[:, P + 1 + j], v0[:, P + i])
+        assert np.array_equal(k[:, :P + 1], k0[:, :P + 1])
+    k, v = k0.copy(), v0.copy()
+    assert to.accept_candidate(k, v, np.array([], int), 0, P) == P + 1 and np.array_equal(k, k0)
