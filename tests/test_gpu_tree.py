@@ -91,7 +91,8 @@ def test_greedy_accept_kernel_bit_exact(dev):
         full, shape = eagle.post_process_draft_tree_device(to_dev(depth, dev), T - 1, to_dev(parents, dev))
         result = torch.zeros(36, dtype=torch.int32, device=dev)
         acc_t = torch.zeros(32, dtype=torch.int32, device=dev)
-        rc = L.eagle_greedy_accept(to_dev(am, dev).data_ptr(), to_dev(tokens, dev).data_ptr(), full.data_ptr(),
+        am_d, tok_d = to_dev(am, dev), to_dev(tokens, dev)
+        rc = L.eagle_greedy_accept(am_d.data_ptr(), tok_d.data_ptr(), full.data_ptr(),
                                    shape.data_ptr(), T, result.data_ptr(), acc_t.data_ptr(), None)
         assert rc == 0
         torch.cuda.synchronize()
@@ -111,7 +112,8 @@ def test_padding_quirk_on_device(dev):
     result = torch.zeros(36, dtype=torch.int32, device=dev)
     acc_t = torch.zeros(32, dtype=torch.int32, device=dev)
     shape = torch.tensor([2, 6], dtype=torch.int32, device=dev)
-    rc = L.eagle_greedy_accept(to_dev(am, dev).data_ptr(), to_dev(tokens, dev).data_ptr(), to_dev(ri, dev).data_ptr(),
+    am_d, tok_d, ri_d = to_dev(am, dev), to_dev(tokens, dev), to_dev(ri, dev)
+    rc = L.eagle_greedy_accept(am_d.data_ptr(), tok_d.data_ptr(), ri_d.data_ptr(),
                                shape.data_ptr(), 8, result.data_ptr(), acc_t.data_ptr(), None)
     assert rc == 0
     r = result.cpu().numpy()
