@@ -1,0 +1,264 @@
+#!/usr/bin/env python3
+"""Tree-verification step benchmark on one MI355X.
+
+A step is one full verification forward of a random-init Qwen2.5-7B-shaped 4-bit (group 64)
+target over 32 tree tokens (root + 31 nodes of a seeded random tree) against a 2048-token
+fp16 KV prefix: embedding, 28 decoder layers, output head, per-node argmax, greedy
+longest-accepted-path selection and KV compaction, replayed as one HIP graph with every
+input resident in HBM.  Prints ONE JSON line.
+
+  python bench.py [--gpus 1] [--steps K] [--warmup W] [--no-cpu] [--sweep]
+
+--sweep additionally prints (to stderr) the per-shape QMM table for M in {1,8,16,24,32}.
+"""
+import argparse
+import json
+import os
+import sys
+import time
+
+import numpy as np
+
+ROOT = os.path.dirname(os.path.abspath(__file__))
+sys.path.insert(0, ROOT)
+
+HBM_PEAK_GBS = 8000.0
+# HBM bytes per QMM launch of this workload (FETCH_SIZE + WRITE_SIZE from two rocprofv3 --pmc
+# runs of this script, scaled by a copy kernel of known size); None until measured.
+QMM_TRAFFIC_BYTES_PER_LAUNCH = None
+PREFIX = 2048
+NODES = 32
+
+
+def qmm_bytes(M, N, K):
+    """Algorithmic bytes of one 4-bit group-64 QMM: packed weights + fp16 scale and bias per
+    64 weights (0.5625 B per weight) + fp16 activations in and out."""
+    return 0.5625 * N * K + 2.0 * M * (K + N)
+
+
+def qmm_shapes(args):
+    D, I, V = args.hidden_size, args.intermediate_size, args.vocab_size
+    H, G, hd = args.num_attention_heads, args.num_key_value_heads, args.head_dim
+    per_layer = [("q", H * hd, D), ("k", G * hd, D), ("v", G * hd, D), ("o", D, H * hd),
+                 ("gate", I, D), ("up", I, D), ("down", D, I)]
+    return per_layer, ("lm_head", V, D)
+
+
+def graph_time_ms(torch, fn, reps, warm=2):
+    """Capture fn() once in a HIP graph and time `reps` replays with events on the
+    replay stream; returns the list of per-replay milliseconds."""
+    side = torch.cuda.Stream()
+    side.wait_stream(torch.cuda.current_stream())
+    with torch.cuda.stream(side):
+        fn()
+    torch.cuda.current_stream().wait_stream(side)
+    torch.cuda.synchronize()
+    g = torch.cuda.CUDAGraph()
+    with torch.cuda.graph(g):
+        fn()
+    for _ in range(warm):
+        g.replay()
+    torch.cuda.synchronize()
+    out = []
+    for _ in range(reps):
+        e0 = torch.cuda.Event(enable_timing=True)
+        e1 = torch.cuda.Event(enable_timing=True)
+        e0.record()
+        g.replay()
+        e1.record()
+        torch.cuda.synchronize()
+        out.append(e0.elapsed_time(e1))
+    return out, g
+
+
+def main():
+    ap = argparse.ArgumentParser()
+    ap.add_argument("--gpus", type=int, default=1)
+    ap.add_argument("--steps", type=int, default=50)
+    ap.add_argument("--warmup", type=int, default=5)
+    ap.add_argument("--seed", type=int, default=1234)
+    ap.add_argument("--no-cpu", action="store_true", help="skip the CPU baseline / full-size parity leg")
+    ap.add_argument("--sweep", action="store_true", help="also print the per-shape QMM table to stderr")
+    opt = ap.parse_args()
+    if opt.gpus != 1:
+        print("bench.py: this build runs on one GPU only; run with --gpus 1", file=sys.stderr)
+        sys.exit(2)
+
+    import torch
+    from mlx_eagle_spec_decoding_tree_amd import _lib, eagle, llama, ops, synth
+    from mlx_eagle_spec_decoding_tree_amd.cache import make_prompt_cache
+
+    if not torch.cuda.is_available():
+        print("bench.py: no GPU visible", file=sys.stderr)
+        sys.exit(2)
+    dev = torch.device("cuda:0")
+    _lib.check(_lib.lib().eagle_check_device(), "device check")
+
+    args = synth.qwen25_7b()
+    t0 = time.time()
+    weights = synth.make_model_weights(args, seed=opt.seed)
+    print(f"[bench] synthetic weights: {sum(v.nbytes for v in weights.values()) / 1e9:.2f} GB "
+          f"in {time.time() - t0:.1f} s", file=sys.stderr, flush=True)
+    model = llama.Model.from_numpy(args, weights, dev)
+    rng = np.random.default_rng(opt.seed + 1)
+    G, hd, L = args.num_key_value_heads, args.head_dim, args.num_hidden_layers
+    cap = 4096
+    cache = make_prompt_cache(model, capacity=cap)
+    prefix = []
+    for c in cache:
+        k = rng.standard_normal((G, PREFIX, hd), dtype=np.float32).astype(np.float16)
+        v = rng.standard_normal((G, PREFIX, hd), dtype=np.float32).astype(np.float16)
+        c.keys[0, :, :PREFIX].copy_(torch.from_numpy(k).to(dev))
+        c.values[0, :, :PREFIX].copy_(torch.from_numpy(v).to(dev))
+        c.offset = PREFIX
+        prefix.append((k, v))
+    cache[0].sync_len()
+
+    parents = synth.random_tree(rng, NODES)
+    depth, anc, bits = synth.tree_arrays(parents)
+    tokens = rng.integers(0, args.vocab_size, NODES).astype(np.int32)
+
+    ver = eagle.TreeVerifier(model, cache, total_tokens=NODES - 1, max_len=cap)
+    ver.set_tree(torch.from_numpy(tokens).to(dev), torch.from_numpy(depth.astype(np.int32)).to(dev),
+                 torch.from_numpy(parents).to(dev),
+                 torch.from_numpy(bits.view(np.int32)).to(dev))
+    len0 = torch.tensor([PREFIX], dtype=torch.int32, device=dev)
+
+    def one_step():
+        ver.len_dev.copy_(len0)               # rewind: every step sees the same 2048-token prefix
+        ver.forward()
+
+    # ---- timed region: W warm-up replays, then exactly K replays ----
+    _, graph = graph_time_ms(torch, one_step, reps=1, warm=0)
+    for _ in range(opt.warmup):
+        graph.replay()
+    torch.cuda.synchronize()
+    t_start = time.perf_counter()
+    e0 = torch.cuda.Event(enable_timing=True)
+    e1 = torch.cuda.Event(enable_timing=True)
+    e0.record()
+    for _ in range(opt.steps):
+        graph.replay()
+    e1.record()
+    torch.cuda.synchronize()
+    wall_ms = (time.perf_counter() - t_start) * 1e3 / opt.steps
+    ms_per_step = e0.elapsed_time(e1) / opt.steps
+    result = ver.result.cpu().numpy().copy()
+    gpu_logits = ver.logits.cpu().numpy().copy()
+
+    # ---- dominant kernel: the QMM launches of one step, replayed alone ----
+    per_layer, head = qmm_shapes(args)
+    launches = []
+    for i, layer in enumerate(model.layers):
+        at, mlp = layer.self_attn, layer.mlp
+        for lin, x, out in ((at.q_proj, ver.hn, ver.q), (at.k_proj, ver.hn, ver.k), (at.v_proj, ver.hn, ver.v),
+                            (at.o_proj, ver.attn, ver.o), (mlp.gate_proj, ver.hn, ver.gate),
+                            (mlp.up_proj, ver.hn, ver.up), (mlp.down_proj, ver.act, ver.down)):
+            launches.append((lin, x, out))
+    launches.append((model.lm_head, ver.hn, ver.logits))
+    ver.hn.normal_()
+    ver.attn.normal_()
+    ver.act.normal_()
+
+    def qmm_only():
+        for lin, x, out in launches:
+            ops.quantized_matmul(x, lin.weight, lin.scales, lin.biases, bias=lin.bias, out=out)
+
+    qt, _ = graph_time_ms(torch, qmm_only, reps=10)
+    qmm_ms = float(np.median(qt))
+    n_launch = len(launches)
+    alg = sum(qmm_bytes(NODES, n, k) for _, n, k in per_layer) * L + qmm_bytes(NODES, head[1], head[2])
+    kv_bytes = 2 * L * G * (PREFIX + NODES) * hd * 2
+    achieved = alg / (qmm_ms * 1e-3) / 1e9
+    traffic = QMM_TRAFFIC_BYTES_PER_LAUNCH
+    roofline = {"bound": "hbm", "kernel": "qmm_w4g64_kernel", "achieved": round(achieved, 1),
+                "peak": HBM_PEAK_GBS, "unit": "GB/s", "frac": round(achieved / HBM_PEAK_GBS, 4),
+                "traffic": traffic, "launches_per_step": n_launch,
+                "avg_launch_us": round(qmm_ms * 1e3 / n_launch, 3),
+                "algorithmic_bytes_per_launch": round(alg / n_launch),
+                "step_frac": round((alg + kv_bytes) / (ms_per_step * 1e-3) / 1e9 / HBM_PEAK_GBS, 4)}
+
+    if opt.sweep:
+        sweep(torch, ops, dev, args)
+
+    # ---- CPU baseline: the CPU restatement of the same step on the host cores, same inputs ----
+    cpu = None
+    parity = None
+    if not opt.no_cpu:
+        from oracle import model_oracle, oracle
+        oracle.build()
+        cores = int(os.environ.get("OMP_NUM_THREADS", 0)) or min(16, os.cpu_count() or 1)
+        inv, sc = synth.inv_freqs(args)
+        ocache = model_oracle.new_cache(args, PREFIX + NODES)
+        for (ok, ov), (k, v) in zip(ocache, prefix):
+            ok[:, :PREFIX] = k
+            ov[:, :PREFIX] = v
+        print("[bench] CPU baseline: one full step on the host ...", file=sys.stderr, flush=True)
+        t0 = time.perf_counter()
+        want = model_oracle.verify_step(args, weights, inv, sc, tokens, depth, parents, anc, ocache, PREFIX)
+        cpu_ms = (time.perf_counter() - t0) * 1e3
+        cpu = {"value": round(cpu_ms, 1), "unit": "ms", "cores": cores, "kind": "port",
+               "sample": "1 full step (28 layers + head, 32 nodes, 2048-token prefix), same weights and inputs, "
+                         "OpenMP C restatement, single timing after page-in"}
+        wl = want["logits"].astype(np.float32)
+        gl = gpu_logits.astype(np.float32)
+        abs_err = float(np.abs(gl - wl).max())
+        err = abs_err / float(np.sqrt(np.mean(wl * wl)))
+        srt = np.sort(wl, axis=-1)
+        clear = (srt[:, -1] - srt[:, -2]) > 2 * abs_err       # nodes whose top-2 margin exceeds the error
+        am_gpu = np.argmax(gl, -1)
+        parity = {"finite": bool(np.isfinite(gl).all() and np.isfinite(wl).all()),
+                  "logits_max_abs_err_over_rms": round(err, 5), "tolerance": 2e-2,
+                  "node_argmax_equal": int((am_gpu == want["node_argmax"]).sum()),
+                  "nodes_with_clear_margin": int(clear.sum()),
+                  "clear_margin_argmax_equal": int((am_gpu[clear] == want["node_argmax"][clear]).sum()),
+                  "nodes": NODES,
+                  "accept_equal": bool(result[0] == want["best"] and result[1] == want["accept_length"]
+                                       and result[3] == want["next_token"])}
+
+    line = {"metric": "tree_verify_step_ms", "value": round(ms_per_step, 4), "unit": "ms", "n_gpus": 1,
+            "steps": opt.steps, "warmup": opt.warmup, "ms_per_step": round(ms_per_step, 4),
+            "higher_is_better": False, "scaling": "weak", "vs_baseline": None, "dtype": "f16",
+            "data": "synthetic",
+            "config": {"workload": "qwen2.5-7b-shape 4-bit g64 target, 28 layers, 32 tree nodes, "
+                                   "2048-token fp16 KV prefix, greedy accept + KV compaction, HIP-graph replay",
+                       "nodes": NODES, "prefix": PREFIX, "wall_ms_per_step": round(wall_ms, 4),
+                       "accept_length": int(result[1]),
+                       "tokens_per_target_forward": int(result[1]) + 1},
+            "roofline": roofline, "cpu_baseline": cpu}
+    if parity is not None:
+        line["parity"] = parity
+    print(json.dumps(line), flush=True)
+
+
+def sweep(torch, ops, dev, args):
+    """QMM microbenchmark over the projection shapes, weights rotated over > 1 GB of
+    distinct copies so that no replay is served from cache."""
+    per_layer, head = qmm_shapes(args)
+    shapes = [("cfg1", 8192, 2048)] + [s for s in per_layer if s[0] in ("q", "k", "gate", "down")] + [head]
+    print(f"{'shape':>8} {'N':>7} {'K':>6} {'M':>3} {'us':>9} {'GB/s':>8} {'frac':>6}", file=sys.stderr)
+    for name, N, K in shapes:
+        wbytes = 0.5625 * N * K
+        ncopy = 4 if wbytes > 3e8 else min(40, max(2, int(1.2e9 // wbytes)))
+        ws = [torch.randint(-2 ** 31, 2 ** 31 - 1, (N, K // 8), dtype=torch.int32, device=dev) for _ in range(ncopy)]
+        ss = [(torch.rand(N, K // 64, device=dev) * 0.015 + 0.005).half() for _ in range(ncopy)]
+        bs = [(-8 * s.float()).half() for s in ss]
+        for M in (1, 8, 16, 24, 32):
+            x = torch.randn(M, K, device=dev).half()
+            o = torch.empty(M, N, device=dev, dtype=torch.float16)
+            iters = 40
+
+            def fn():
+                for i in range(iters):
+                    ops.quantized_matmul(x, ws[i % ncopy], ss[i % ncopy], bs[i % ncopy], out=o)
+
+            ts, _ = graph_time_ms(torch, fn, reps=5)
+            us = float(np.median(ts)) * 1e3 / iters
+            gbs = qmm_bytes(M, N, K) / us / 1e3
+            print(f"{name:>8} {N:>7} {K:>6} {M:>3} {us:>9.2f} {gbs:>8.0f} {gbs / HBM_PEAK_GBS:>6.3f}",
+                  file=sys.stderr, flush=True)
+        del ws, ss, bs
+
+
+if __name__ == "__main__":
+    main()

@@ -79,14 +79,27 @@ def tiny(layers=2, hidden=256, inter=512, heads=4, kv_heads=2, head_dim=64, voca
                      tie_word_embeddings=tie)
 
 
-def make_qlinear(rng, N, K, bias=False):
+def make_qlinear(rng, N, K, bias=False, gain=None):
     """Random 4-bit group-64 linear layer in the packed layout
-    (weight uint32 [N, K/8], nibble i of a word = element 8*word + i)."""
+    (weight uint32 [N, K/8], nibble i of a word = element 8*word + i).
+
+    gain=None: the single-matmul benchmark distribution (scales ~ U(0.005, 0.02),
+    biases = -8*scale + N(0, 1e-3)); the dequantised weights then have mean -0.5*scale
+    and rms 0.061, which is what a lone matmul is measured with.
+    gain=g: the same shapes of distribution rescaled for whole-model use: zero-mean
+    weights (biases = -7.5*scale + small noise) of rms g / sqrt(K), so that activations
+    stay O(1) through dozens of layers instead of overflowing fp16 in the first MLP."""
     assert K % 64 == 0
     w = rng.integers(0, 1 << 32, size=(N, K // 8), dtype=np.uint32)
-    s = rng.uniform(0.005, 0.02, size=(N, K // 64)).astype(np.float16)
-    b = (-8.0 * s.astype(np.float32)
-         + rng.normal(0.0, 1e-3, size=s.shape).astype(np.float32)).astype(np.float16)
+    s32 = rng.uniform(0.005, 0.02, size=(N, K // 64))
+    noise = rng.normal(0.0, 1e-3, size=s32.shape)
+    if gain is None:
+        s = s32.astype(np.float16)
+        b = (-8.0 * s.astype(np.float32) + noise.astype(np.float32)).astype(np.float16)
+    else:
+        f = gain / (0.0610 * np.sqrt(K))
+        s = (s32 * f).astype(np.float16)
+        b = (-7.5 * s.astype(np.float32) + (noise * f).astype(np.float32)).astype(np.float16)
     out = {"weight": w, "scales": s, "biases": b}
     if bias:
         out["bias"] = rng.normal(0.0, 0.02, size=(N,)).astype(np.float16)
@@ -119,7 +132,7 @@ def make_x(rng, *shape):
     return rng.normal(0.0, 1.0, size=shape).astype(np.float16)
 
 
-def make_model_weights(args: ModelArgs, seed=42, layers=None):
+def make_model_weights(args: ModelArgs, seed=42, layers=None, gain=1.0):
     """All tensors of a random-init quantised decoder as a flat dict of numpy
     arrays keyed like an MLX-community checkpoint
     (`model.layers.3.self_attn.q_proj.weight` / `.scales` / `.biases` / `.bias`)."""
@@ -132,22 +145,22 @@ def make_model_weights(args: ModelArgs, seed=42, layers=None):
         for k, v in layer.items():
             out[f"{prefix}.{k}"] = v
 
-    put("model.embed_tokens", make_qlinear(rng, V, D))
+    put("model.embed_tokens", make_qlinear(rng, V, D, gain=gain))
     n_layers = args.num_hidden_layers if layers is None else layers
     for i in range(n_layers):
         p = f"model.layers.{i}"
-        put(f"{p}.self_attn.q_proj", make_qlinear(rng, H * hd, D, args.attention_bias))
-        put(f"{p}.self_attn.k_proj", make_qlinear(rng, G * hd, D, args.attention_bias))
-        put(f"{p}.self_attn.v_proj", make_qlinear(rng, G * hd, D, args.attention_bias))
-        put(f"{p}.self_attn.o_proj", make_qlinear(rng, D, H * hd))
-        put(f"{p}.mlp.gate_proj", make_qlinear(rng, I, D, args.mlp_bias))
-        put(f"{p}.mlp.up_proj", make_qlinear(rng, I, D, args.mlp_bias))
-        put(f"{p}.mlp.down_proj", make_qlinear(rng, D, I, args.mlp_bias))
+        put(f"{p}.self_attn.q_proj", make_qlinear(rng, H * hd, D, args.attention_bias, gain=gain))
+        put(f"{p}.self_attn.k_proj", make_qlinear(rng, G * hd, D, args.attention_bias, gain=gain))
+        put(f"{p}.self_attn.v_proj", make_qlinear(rng, G * hd, D, args.attention_bias, gain=gain))
+        put(f"{p}.self_attn.o_proj", make_qlinear(rng, D, H * hd, gain=gain))
+        put(f"{p}.mlp.gate_proj", make_qlinear(rng, I, D, args.mlp_bias, gain=gain))
+        put(f"{p}.mlp.up_proj", make_qlinear(rng, I, D, args.mlp_bias, gain=gain))
+        put(f"{p}.mlp.down_proj", make_qlinear(rng, D, I, args.mlp_bias, gain=gain))
         out[f"{p}.input_layernorm.weight"] = (1.0 + rng.normal(0, 0.02, D)).astype(np.float16)
         out[f"{p}.post_attention_layernorm.weight"] = (1.0 + rng.normal(0, 0.02, D)).astype(np.float16)
     out["model.norm.weight"] = (1.0 + rng.normal(0, 0.02, D)).astype(np.float16)
     if not args.tie_word_embeddings:
-        put("lm_head", make_qlinear(rng, V, D))
+        put("lm_head", make_qlinear(rng, V, D, gain=gain))
     return out
 
 
@@ -182,3 +195,17 @@ def random_tree(rng, n_nodes=32, max_depth=4, max_children=4):
         children.append(0)
         depth.append(depth[p] + 1)
     return np.array(parents, np.int32)
+
+
+def tree_arrays(parents):
+    """(depth [T] int32, ancestor-or-self visibility [T,T] bool, row bitmasks [T] uint32)
+    of the tree given by `parents` (as returned by random_tree)."""
+    T = len(parents) + 1
+    depth = np.zeros(T, np.int32)
+    vis = np.eye(T, dtype=bool)
+    for node in range(1, T):
+        p = int(parents[node - 1])
+        depth[node] = depth[p] + 1
+        vis[node] |= vis[p]
+    bits = (vis.astype(np.uint64) << np.arange(T, dtype=np.uint64)[None, :]).sum(1).astype(np.uint32)
+    return depth, vis, bits
