@@ -79,6 +79,9 @@ def main():
     ap.add_argument("--seed", type=int, default=1234)
     ap.add_argument("--no-cpu", action="store_true", help="skip the CPU baseline / full-size parity leg")
     ap.add_argument("--sweep", action="store_true", help="also print the per-shape QMM table to stderr")
+    ap.add_argument("--calibrate-copy", action="store_true",
+                    help="before anything else run one 1 GiB device copy (a kernel of known traffic: "
+                         "1 GiB read + 1 GiB written) so that profiler byte counters can be scaled")
     opt = ap.parse_args()
     if opt.gpus != 1:
         print("bench.py: this build runs on one GPU only; run with --gpus 1", file=sys.stderr)
@@ -93,6 +96,13 @@ def main():
         sys.exit(2)
     dev = torch.device("cuda:0")
     _lib.check(_lib.lib().eagle_check_device(), "device check")
+
+    if opt.calibrate_copy:
+        src = torch.empty(1 << 30, dtype=torch.uint8, device=dev).random_(0, 255)
+        dst = torch.empty_like(src)
+        dst.copy_(src)
+        torch.cuda.synchronize()
+        del src, dst
 
     args = synth.qwen25_7b()
     t0 = time.time()
