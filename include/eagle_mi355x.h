@@ -48,7 +48,7 @@ int eagle_check_device(void);
  *   q[n,k] = (wq[n,k/8] >> 4*(k%8)) & 15
  *   x [M,K] fp16 row-major, wq [N,K/8] uint32, scales/biases [N,K/64] fp16,
  *   bias [N] fp16 or NULL (added in fp16 after rounding), out [M,N] fp16.
- * Constraints: 1 <= M <= 32, K % 64 == 0, K <= 32768 (65536 for M <= 16), N % 8 == 0, group_size == 64,
+ * Constraints: 1 <= M <= 32, K % 64 == 0, N % 8 == 0, N * K / 2 < 2^32, group_size == 64,
  * bits == 4.
  * Replaces qmm_kernel.matmul (qmm_kernel.py:84-164) with the body
  * kernels/progression/simd_no_swizzle_cast.metal, the mx.quantized_matmul
@@ -64,17 +64,17 @@ int eagle_qmm_w4g64_f16(const void* x, const uint32_t* wq, const void* scales,
                         const void* biases, const void* bias, void* out,
                         int M, int N, int K, int group_size, int bits,
                         void* workspace, size_t workspace_bytes, eagle_stream_t stream);
-/* The launch shape the library would pick: plan7 = {tiles per wave, tile slots per
- * round, waves per tile, K slabs, columns per slab, row groups, rounds}. */
-int eagle_qmm_plan(int M, int N, int K, int* plan7);
-/* Same matmul with the launch shape forced (tuning sweeps and tests).  The shape
- * must cover N and K and fit LDS, else EAGLE_ERR_SHAPE. */
-size_t eagle_qmm_workspace_bytes_tuned(int M, int rt, int wt, int wk, int splits,
-                                       int row_groups, int rounds);
+/* The launch shape the library would pick: plan3 = {streaming waves per workgroup
+ * (= column units per K slab; a unit is 256 columns for M <= 16, 128 above), K slabs,
+ * tile ranges (workgroups per slab)}. */
+int eagle_qmm_plan(int M, int N, int K, int* plan3);
+/* Same matmul with the launch shape forced (tuning sweeps and tests).  nw <= 14,
+ * nw * splits must cover K with no empty slab, 1 <= ranges <= ceil(N / 16), else
+ * EAGLE_ERR_SHAPE. */
+size_t eagle_qmm_workspace_bytes_tuned(int M, int N, int splits);
 int eagle_qmm_w4g64_f16_tuned(const void* x, const uint32_t* wq, const void* scales,
                               const void* biases, const void* bias, void* out,
-                              int M, int N, int K, int rt, int wt, int wk, int splits,
-                              int slab_k, int row_groups, int rounds,
+                              int M, int N, int K, int nw, int splits, int ranges,
                               void* workspace, size_t workspace_bytes, eagle_stream_t stream);
 
 /* Quantised embedding gather: out[t,:] = fp16(scales*q + biases) of row ids[t].

@@ -6,39 +6,61 @@
 // 8*word + i; scales/biases [N, K/64] fp16.  (Reference contract:
 // qmm_kernel.py:84-164, kernels/progression/simd_no_swizzle_cast.metal.)
 //
-// Structure: a weight streamer with x resident in LDS.
+// Structure: a weight streamer with x resident in registers.
 //
-//  * A workgroup owns one K slab (at most 4096 columns for M <= 16, 2048 for M <= 32)
-//    and a contiguous range of 16-row weight tiles.  It first copies its slab of x
-//    into LDS (element order 0,4,1,5,2,6,3,7 inside every group of eight, matching
-//    the nibble pairs below), once; after that the only memory traffic of the main
-//    loop is the weight stream, and there is no barrier per K step.
-//  * Tiles are processed in rounds of WT tiles; WK waves share a tile and split its
-//    K chunks (256 columns each).  Per chunk a lane issues two 128-bit loads: the
-//    four lanes that share a row read 64 contiguous bytes per instruction, one full
-//    128-byte line per chunk.  PF chunks are kept in flight in a register ring that
-//    runs across tile rounds.
-//  * Nibbles are expanded in registers with the fp16 magic-number trick
-//    ((w & 0x000f000f) | 0x6400 = 1024 + q, (w & 0x00f000f0) | 0x5400 = 64 + q), giving
-//    the pairs (q0,q4) (q1,q5) (q2,q6) (q3,q7), scaled with packed fp16 FMAs and fed to
-//    v_mfma_f32_16x16x32_f16 as the A operand (rows = output features); the B operand
-//    (columns = rows of x) is read from the LDS slab; accumulation is fp32.
-//  * The WK partial tiles of a round are added through LDS.  K slabs (blockIdx.y) are
-//    added through fp32 partials in a workspace: the last workgroup to arrive sums
-//    them in slab order, so results are deterministic.  The partials travel as
-//    device-scope relaxed atomics (write-through stores, L2-bypassing loads): no
-//    L2 write-back / invalidate fence, which costs microseconds on a multi-XCD part.
+//  * A workgroup owns one K slab and a contiguous range of 16-row weight tiles.  Each of
+//    its `nw` streaming waves owns one column unit of the slab (256 columns for M <= 16,
+//    128 for M <= 32) for the whole launch: it loads that unit of x ONCE, straight into
+//    MFMA operand registers, and then walks down the rows.  Per tile a lane issues one or
+//    two 128-bit loads; the four lanes that share a row read 64 contiguous bytes per
+//    instruction and the waves of the workgroup together read whole rows.  Four tiles are
+//    in flight per wave in a register ring.
+//  * Nibbles are expanded with the fp16 magic-number trick only:
+//    (w & 0x000f000f) | 0x6400 = 1024 + q and (w & 0x00f000f0) | 0x5400 = 64 + q give the
+//    pairs (q0,q4) (q1,q5) (q2,q6) (q3,q7) as MFMA operands without subtracting the offsets
+//    or applying scale and bias per weight.  v_mfma_f32_16x16x32_f16 accumulates one
+//    quantisation group at a time, t[m,n] = sum_k x[m,k] (off_k + q[n,k]); the group result
+//    is folded in with one fp32 FMA per accumulator, acc += s[n,g] * t.  What that leaves,
+//        sum_g b[n,g] * xs[m,g]  -  sum_g s[n,g] * (1024 * xsE[m,g] + 64 * xsO[m,g])
+//    (xs = per-group sums of x, over even / odd columns), is one more MFMA per tile whose
+//    x-side operand is computed once per launch (split into fp16 high and low parts, so
+//    that it carries 22 bits) and whose weight-side operand is the tile's scales and biases.
+//    v_permlane32_swap regroups the loaded words so that all four lanes of a row feed one
+//    quantisation group per MFMA.
+//  * Scales and biases of a batch of tiles are staged through LDS by the streaming waves
+//    (whole row segments, coalesced) one batch ahead.
+//  * Each streaming wave leaves its 16 x M partial tile in LDS; two further waves of the
+//    workgroup only add the partials in wave order and store the results, one batch
+//    behind the streamers (double-buffered, one barrier per batch).  Streaming waves
+//    therefore never have stores in flight and their prefetch ring is waited on exactly.
+//  * K slabs (blockIdx.y), needed when K exceeds what 14 waves cover, are added through
+//    fp32 partials in a workspace: the last workgroup of a tile range to arrive sums the
+//    slabs in slab order, so results are deterministic.  The partials travel as
+//    device-scope relaxed atomics (write-through stores, L2-bypassing loads): no L2
+//    write-back / invalidate fence, which costs microseconds on a multi-XCD part.
 #include "common.h"
+
+#ifdef EAGLE_DBG_TIMES
+__device__ unsigned long long eagle_dbg_times[1024 * 16];
+#define TSTAMP(k) do { if (lane == 0 && (wave == 0 || wave == nw)) eagle_dbg_times[blockIdx.x * 16 + (k)] = wall_clock64(); } while (0)
+EAGLE_EXPORT int eagle_dbg_read_times(unsigned long long* host) {
+  return hipMemcpyFromSymbol(host, HIP_SYMBOL(eagle_dbg_times), sizeof(eagle_dbg_times)) == hipSuccess ? 0 : 6;
+}
+#else
+#define TSTAMP(k) do { } while (0)
+#endif
 
 namespace {
 
-constexpr int CHUNK_K = 256;          // K columns per wave step (4 quantisation groups)
-constexpr int MAX_ROW_BLOCKS = EAGLE_QMM_COUNTER_BYTES / 4;
-constexpr int MAX_SPLITS = 16;
-constexpr int MAX_WAVES = 12;          // per workgroup: 768 threads, up to 170 VGPRs each
-constexpr int LDS_BUDGET = 160 * 1024 - 512;
+constexpr int MAX_STREAM_WAVES = 14;   // + 2 reducing waves = 1024 threads
+constexpr int NWR = 2;                 // reducing waves per workgroup
+constexpr int MAX_SPLITS = 64;
+constexpr int MAX_RANGES = EAGLE_QMM_COUNTER_BYTES / 4;
+constexpr int LDS_MAX = 160 * 1024;
+constexpr int NUM_CU = 256;
 
 __device__ inline half2_t as_h2(uint32_t u) { return __builtin_bit_cast(half2_t, u); }
+__device__ inline uint32_t as_u32(half2_t h) { return __builtin_bit_cast(uint32_t, h); }
 
 // (v & mask) | bits in one VALU op.  The compiler splits the two-literal form into
 // v_and + v_or; holding `bits` in a VGPR and `mask` in an SGPR makes it encodable.
@@ -48,525 +70,478 @@ __device__ inline uint32_t and_or(uint32_t v, uint32_t mask, uint32_t bits) {
   return r;
 }
 
-struct DequantConsts {
-  uint32_t magic_lo, magic_hi;   // VGPR copies of 0x64006400 / 0x54005400
-};
-
-// 8 nibbles of one packed word -> 8 fp16 weights in the order q0,q4,q1,q5,q2,q6,q3,q7.
-__device__ inline half8_t dequant8(uint32_t v, half2_t ss, half2_t bb, const DequantConsts& c) {
-  const half2_t k1024 = {(half_t)1024.0f, (half_t)1024.0f};
-  const half2_t k64 = {(half_t)64.0f, (half_t)64.0f};
+// 8 nibbles of one packed word -> fp16 (1024+q0, 1024+q4, 64+q1, 64+q5, 1024+q2, 1024+q6,
+// 64+q3, 64+q7): five VALU operations.
+__device__ inline half8_t expand8(uint32_t v, uint32_t magic_lo, uint32_t magic_hi) {
   const uint32_t v2 = v >> 8;
-  half2_t a0 = as_h2(and_or(v, 0x000f000fu, c.magic_lo)) - k1024;    // 1024 + q  -> q
-  half2_t a1 = as_h2(and_or(v, 0x00f000f0u, c.magic_hi)) - k64;      //   64 + q  -> q
-  half2_t a2 = as_h2(and_or(v2, 0x000f000fu, c.magic_lo)) - k1024;
-  half2_t a3 = as_h2(and_or(v2, 0x00f000f0u, c.magic_hi)) - k64;
-  a0 = a0 * ss + bb;
-  a1 = a1 * ss + bb;
-  a2 = a2 * ss + bb;
-  a3 = a3 * ss + bb;
-  half8_t r;
-  r[0] = a0[0]; r[1] = a0[1]; r[2] = a1[0]; r[3] = a1[1];
-  r[4] = a2[0]; r[5] = a2[1]; r[6] = a3[0]; r[7] = a3[1];
-  return r;
+  uint4_t u;
+  u[0] = and_or(v, 0x000f000fu, magic_lo);
+  u[1] = and_or(v, 0x00f000f0u, magic_hi);
+  u[2] = and_or(v2, 0x000f000fu, magic_lo);
+  u[3] = and_or(v2, 0x00f000f0u, magic_hi);
+  return __builtin_bit_cast(half8_t, u);
 }
 
-// One chunk of one 16-row tile as held by a lane, exactly as loaded (nothing may be
-// computed from these registers before the chunk is consumed, or the wait for it would
-// drain the whole prefetch ring): 2 x 32 nibbles of its row.
-struct WRegs {
-  uint4_t lo, hi;
+// Exchange the upper 32 lanes of `a` with the lower 32 lanes of `b`.
+__device__ inline void swap32(uint32_t& a, uint32_t& b) {
+  const uint2_t r = __builtin_amdgcn_permlane32_swap(a, b, false, false);
+  a = r[0];
+  b = r[1];
+}
+
+// Workgroup barrier that orders LDS traffic only.  __syncthreads() also waits for every
+// outstanding global load (vmcnt(0)), which would drain the prefetch ring at each batch.
+__device__ inline void lds_barrier() {
+  asm volatile("s_waitcnt lgkmcnt(0)\n\ts_barrier" ::: "memory");
+}
+
+#ifndef EAGLE_RING
+#define EAGLE_RING 4
+#endif
+
+template <int NT, int GW>
+struct Cfg {
+  static constexpr int RING = EAGLE_RING;       // tiles in flight per streaming wave
+  static constexpr int B = 4 / NT;              // tiles per batch (one barrier per batch)
+  static constexpr int CW = GW * 64;            // columns owned by a streaming wave
+  static constexpr int NL = GW / 2;             // 128-bit weight loads per lane per tile
+  static constexpr int NMF = GW * 2;            // MFMAs per 16 rows of x per tile
+  static constexpr int UNIT = GW * 2;           // bytes of scales (or biases) per row per wave
+  static constexpr int SB_ARRAY = 16 * B * 16 * UNIT;   // LDS bytes: one array, one buffer
+  static constexpr int SB_BUF = 2 * SB_ARRAY;
+  static constexpr int NSU = B / 2;             // staging units per streaming thread per batch
 };
+
+__host__ __device__ inline int pbuf_bytes(int nw) { return 2 * nw * 4096; }
 
 struct Launch {
-  int rt;          // 16-row tiles per wave (1 or 2)
-  int wt;          // tile slots per round (waves along N)
-  int wk;          // waves sharing a tile (each takes a contiguous run of the slab's chunks)
-  int splits;      // K slabs (gridDim.y)
-  int slab_k;      // columns per slab, multiple of 256
-  int row_groups;  // gridDim.x
-  int rounds;      // tile rounds per workgroup
-  int pf;          // ring depth (4, 5 or 7): the divisor of the run length that wastes least
+  int nw;       // streaming waves per workgroup = column units per K slab
+  int splits;   // K slabs (gridDim.y)
+  int ranges;   // tile ranges (gridDim.x)
 };
 
-constexpr int SB_ITERS = 4;   // 64 lanes x 4 cover the 16 rows x (<= 16 chunks) of a wave's run
-
-// LDS stride (in 8-byte units) of one row of a wave's scale / bias block: odd, so that the
-// 16 rows read by one quarter wave fall into 16 different bank pairs.
-__host__ __device__ inline int sb_row_units(int units) { return units | 1; }
-
-// PF = weight chunks in flight per wave (depth of the register ring).
-template <int NT, int RT, int PF, bool SLOW_SB>
-__global__ __launch_bounds__(768) void qmm_w4g64_kernel(
+// NT: 16-row blocks of x (1 or 2).  GW: quantisation groups per streaming wave.
+// SLOWSB: scales / biases are fetched element by element (odd group counts, rows shorter
+// than a unit, unaligned arrays).
+template <int NT, int GW, bool SLOWSB>
+__global__ __launch_bounds__(1024) void qmm_w4g64_kernel(
     const half_t* __restrict__ x, const uint32_t* __restrict__ w,
     const half_t* __restrict__ s, const half_t* __restrict__ b,
     const half_t* __restrict__ bias, half_t* __restrict__ out,
     float* __restrict__ partial, unsigned* __restrict__ counters,
-    int M, int N, int K, int WT, int WK, int slab_k, int rounds) {
-  constexpr int MP = 16 * NT;                     // padded rows of x
+    int M, int N, int K, int nw) {
+  using C = Cfg<NT, GW>;
+  constexpr int B = C::B;
   extern __shared__ __attribute__((aligned(16))) unsigned char lds[];
-  __shared__ int s_last;
+  float4_t* pbuf4 = reinterpret_cast<float4_t*>(lds);                 // [2][nw][256] float4
+  unsigned char* sbuf = lds + pbuf_bytes(nw);                         // [2][2][16B][16] units
 
   const int tid = threadIdx.x;
-  const int nthr = blockDim.x;
   const int lane = tid & 63;
   const int wave = tid >> 6;
-  const int wt = wave % WT;
-  const int wk = wave / WT;
-  const int r = lane & 15;   // row inside a 16-row tile (A operand) / column m (B operand)
-  const int h = lane >> 4;   // which 32-nibble quarter of a 128-nibble half chunk
+  const int r = lane & 15;   // x row (A operand) / weight row of the tile (B operand)
+  const int h = lane >> 4;   // K block of the MFMA this lane feeds
   const int G = K >> 6;
   const int K8 = K >> 3;
   const int nsplit = gridDim.y;
+  const int slab = blockIdx.y;
+  const int tiles_total = (N + 15) >> 4;
+  const int t_lo = (int)(((long)blockIdx.x * tiles_total) / gridDim.x);
+  const int t_hi = (int)(((long)(blockIdx.x + 1) * tiles_total) / gridDim.x);
+  const int nss = (t_hi - t_lo + C::RING - 1) / C::RING;   // super-steps of RING tiles
+  const bool to_out = nsplit == 1;
 
-  const int k0 = blockIdx.y * slab_k;
-  const int klen = min(slab_k, K - k0);
-  const int nchunks = (klen + CHUNK_K - 1) / CHUNK_K;      // chunks of this slab
-  const int cbase = k0 / CHUNK_K;                          // first chunk of the slab in K
-  // this wave's contiguous run of chunks inside the slab
-  const int U = (slab_k / CHUNK_K + WK - 1) / WK;
-  const int c_lo = wk * U;
-  const int cpw = max(min(nchunks, c_lo + U) - c_lo, 0);
-  const int UP = sb_row_units(U);
+  TSTAMP(0);
+  if (wave < nw) {
+    // ------------------------------------------------------------------ streaming wave
+    const int unit = slab * nw + wave;
+    const int col0 = unit * C::CW;
+    const uint32_t magic_lo = 0x64006400u, magic_hi = 0x54005400u;
+    const uint32_t row_bytes = (uint32_t)K8 * 4u;
 
-  // LDS: [x slab][WK reduction buffer][per-wave scale/bias blocks]
-  const int xrow = slab_k * 2 + 16;               // bytes per x row (+16: conflict-free b128)
-  unsigned char* red = lds + MP * xrow;
-  const int red_bytes = WK > 1 ? (WK - 1) * WT * RT * NT * 1024 : 0;
-  const int sb_tile_bytes = 2 * 16 * UP * 8;      // scales then biases of one 16-row tile run
-  unsigned char* sbw = red + red_bytes + wave * (RT * sb_tile_bytes);
-
-  const int tiles_per_round = WT * RT;
-  const int tile_base = (blockIdx.x * rounds) * tiles_per_round + wt * RT;
-
-  // ---- scales / biases of a round: global -> staging registers -> this wave's LDS block ----
-  // Unit (row, u) = the four scales (or biases) of chunk c_lo + u of tile row `row`, 8 bytes.
-  // Rows of a tile are adjacent in memory, so a full-K run is one contiguous block.
-  uint2_t st_s[RT][SB_ITERS], st_b[RT][SB_ITERS];
-  auto load_sb = [&](int round) {
+    // byte offset of this lane's words inside a weight row, clamped into the row
+    uint32_t woff[C::NL];
 #pragma unroll
-    for (int rt = 0; rt < RT; ++rt)
+    for (int ld = 0; ld < C::NL; ++ld) {
+      int word = unit * (C::CW / 8) + ld * 16 + h * 4;
+      if (word > K8 - 4) word = K8 - 4;
+      woff[ld] = (uint32_t)word * 4u;
+    }
+    auto load_w = [&](int tile, uint4_t (&dst)[C::NL]) {
+      int t = tile < t_hi ? tile : t_hi - 1;
+      int row = t * 16 + r;
+      if (row > N - 1) row = N - 1;
+      const unsigned char* p = reinterpret_cast<const unsigned char*>(w) + (uint32_t)row * row_bytes;
 #pragma unroll
-      for (int it = 0; it < SB_ITERS; ++it) {
-        const int idx = lane + 64 * it;
-        const int row = idx / U;
-        const int u = idx - row * U;
-        const bool ok = round < rounds && idx < 16 * U && u < cpw;
-        const int n = min((tile_base + min(round, rounds - 1) * tiles_per_round + rt) * 16 + min(row, 15), N - 1);
-        const int c4 = (cbase + c_lo + min(u, max(cpw - 1, 0))) * 4;
-        if (SLOW_SB) {
-          // fewer than four groups per row, or an odd group count: element-wise
-          uint32_t sv[4], bv[4];
+      for (int ld = 0; ld < C::NL; ++ld)
+#ifdef EAGLE_DBG_NT
+        dst[ld] = __builtin_nontemporal_load(reinterpret_cast<const uint4_t*>(p + woff[ld]));
+#else
+        dst[ld] = *reinterpret_cast<const uint4_t*>(p + woff[ld]);
+#endif
+    };
+
+    // ---- scale / bias staging: this thread's units of a batch
+    const int nthr_s = nw * 64;
+    int su_row[C::NSU], su_g[C::NSU], su_lds[C::NSU];
+    const half_t* su_arr[C::NSU];
 #pragma unroll
-          for (int i = 0; i < 4; ++i) {
-            const bool oki = ok && (c4 + i) < G;
-            const size_t off = (size_t)n * G + min(c4 + i, G - 1);
-            sv[i] = oki ? (uint32_t) * reinterpret_cast<const uint16_t*>(s + off) : 0u;
-            bv[i] = oki ? (uint32_t) * reinterpret_cast<const uint16_t*>(b + off) : 0u;
+    for (int k = 0; k < C::NSU; ++k) {
+      const int u = tid + k * nthr_s;
+      const int per_arr = 16 * B * nw;
+      const int a = u / per_arr;
+      const int rem = u - a * per_arr;
+      const int row = rem / nw;
+      const int c = rem - row * nw;
+      su_row[k] = row;
+      int g = (slab * nw + c) * GW;
+      if (!SLOWSB && g > G - GW) g = G - GW;
+      su_g[k] = g;
+      su_arr[k] = a ? b : s;
+      su_lds[k] = ((a * 16 * B + row) * 16 + (c ^ (row & 15))) * C::UNIT;
+    }
+    uint2_t su_val[C::NSU];
+    auto stage_load = [&](int tile0) {
+#pragma unroll
+      for (int k = 0; k < C::NSU; ++k) {
+        int row = tile0 * 16 + su_row[k];
+        if (row > N - 1) row = N - 1;
+        const half_t* p = su_arr[k] + (size_t)row * G;
+        if (SLOWSB) {
+          half_t v[4];
+#pragma unroll
+          for (int e = 0; e < GW; ++e) {
+            int g = su_g[k] + e;
+            if (g > G - 1) g = G - 1;
+            v[e] = p[g];
           }
-          st_s[rt][it] = uint2_t{sv[0] | (sv[1] << 16), sv[2] | (sv[3] << 16)};
-          st_b[rt][it] = uint2_t{bv[0] | (bv[1] << 16), bv[2] | (bv[3] << 16)};
+          half2_t lo = {v[0], v[1]};
+          su_val[k][0] = as_u32(lo);
+          if (GW == 4) {
+            half2_t hi = {v[2], v[3]};
+            su_val[k][1] = as_u32(hi);
+          }
+        } else if (GW == 4) {
+          su_val[k] = *reinterpret_cast<const uint2_t*>(p + su_g[k]);
         } else {
-          // A last chunk with fewer than four groups reads the row's last four groups
-          // instead (in range); compute() shifts them into place.
-          const size_t off = (size_t)n * G + min(c4, G - 4);
-#ifdef EAGLE_DBG_NOSB
-          st_s[rt][it] = uint2_t{(uint32_t)off, 0u}; st_b[rt][it] = uint2_t{0u, (uint32_t)n};
-#else
-          st_s[rt][it] = *reinterpret_cast<const uint2_t*>(s + off);   // unconditional, see load_w
-          st_b[rt][it] = *reinterpret_cast<const uint2_t*>(b + off);
-#endif
-          (void)ok;
+          su_val[k][0] = *reinterpret_cast<const uint32_t*>(p + su_g[k]);
         }
       }
-  };
-  auto commit_sb = [&]() {
+    };
+    auto stage_store = [&](int buf) {
 #pragma unroll
-    for (int rt = 0; rt < RT; ++rt)
+      for (int k = 0; k < C::NSU; ++k) {
+        unsigned char* q = sbuf + buf * C::SB_BUF + su_lds[k];
+        if (GW == 4) *reinterpret_cast<uint2_t*>(q) = su_val[k];
+        else *reinterpret_cast<uint32_t*>(q) = su_val[k][0];
+      }
+    };
+
+    // ---- prologue: scales/biases of batch 0, this wave's unit of x, first four tiles
+    stage_load(t_lo);
+
+    half8_t xop[NT][C::NMF];
+    float sE[NT][GW], sO[NT][GW];
 #pragma unroll
-      for (int it = 0; it < SB_ITERS; ++it) {
-        const int idx = lane + 64 * it;
-        const int row = idx / U;
-        const int u = idx - row * U;
-        if (idx < 16 * U) {
-          unsigned char* dst = sbw + rt * sb_tile_bytes + (row * UP + u) * 8;
-          *reinterpret_cast<uint2_t*>(dst) = st_s[rt][it];
-          *reinterpret_cast<uint2_t*>(dst + 16 * UP * 8) = st_b[rt][it];
+    for (int t = 0; t < NT; ++t)
+#pragma unroll
+      for (int g = 0; g < GW; ++g) sE[t][g] = sO[t][g] = 0.f;
+    const int hperm = ((h & 1) << 2) | (h & 2);          // 0, 4, 2, 6
+#pragma unroll
+    for (int t = 0; t < NT; ++t) {
+#pragma unroll
+      for (int j = 0; j < C::NMF; ++j) {
+        const int wi = 16 * (j >> 2) + 8 * ((j >> 1) & 1) + (j & 1) + hperm;
+        const int col = col0 + 8 * wi;
+        const int m = 16 * t + r;
+        uint4_t u = uint4_t{0u, 0u, 0u, 0u};
+        if (m < M && col < K) u = *reinterpret_cast<const uint4_t*>(x + (size_t)m * K + col);
+        uint4_t o;
+        o[0] = __builtin_amdgcn_perm(u[2], u[0], 0x05040100u);   // (x0, x4)
+        o[1] = __builtin_amdgcn_perm(u[2], u[0], 0x07060302u);   // (x1, x5)
+        o[2] = __builtin_amdgcn_perm(u[3], u[1], 0x05040100u);   // (x2, x6)
+        o[3] = __builtin_amdgcn_perm(u[3], u[1], 0x07060302u);   // (x3, x7)
+        xop[t][j] = __builtin_bit_cast(half8_t, o);
+        const half2_t e0 = as_h2(o[0]), o0 = as_h2(o[1]), e1 = as_h2(o[2]), o1 = as_h2(o[3]);
+        sE[t][j >> 1] += ((float)e0[0] + (float)e0[1]) + ((float)e1[0] + (float)e1[1]);
+        sO[t][j >> 1] += ((float)o0[0] + (float)o0[1]) + ((float)o1[0] + (float)o1[1]);
+      }
+    }
+    uint4_t ring[C::RING][C::NL];
+#pragma unroll
+    for (int p = 0; p < C::RING; ++p) load_w(t_lo + p, ring[p]);
+    TSTAMP(1);
+
+    // x-side operand of the bias / offset MFMA: K block 0 carries the group sums of x
+    // (high and low fp16 parts), K block 1 carries -(16 * even sum + odd sum); the other
+    // two blocks are zero.
+    half8_t xaux[NT];
+#pragma unroll
+    for (int t = 0; t < NT; ++t) {
+      half8_t a;
+#pragma unroll
+      for (int e = 0; e < 8; ++e) a[e] = (half_t)0.f;
+#pragma unroll
+      for (int g = 0; g < GW; ++g) {
+        float se = sE[t][g], so = sO[t][g];
+        se += __shfl_xor(se, 16, 64);
+        se += __shfl_xor(se, 32, 64);
+        so += __shfl_xor(so, 16, 64);
+        so += __shfl_xor(so, 32, 64);
+        const float v = h == 0 ? se + so : -(16.f * se + so);
+        const half_t hi = (half_t)v;
+        const half_t lo = (half_t)(v - (float)hi);
+        a[g] = h < 2 ? hi : (half_t)0.f;
+        a[4 + g] = h < 2 ? lo : (half_t)0.f;
+      }
+      xaux[t] = a;
+    }
+    const half2_t kmul = h == 0 ? half2_t{(half_t)1.f, (half_t)1.f} : half2_t{(half_t)64.f, (half_t)64.f};
+
+    TSTAMP(2);
+    stage_store(0);
+    __syncthreads();
+    TSTAMP(3);
+
+    // ---- main loop: super-steps of RING tiles, ring slots are compile-time indices
+    for (int ss = 0; ss < nss; ++ss) {
+      const int tb = t_lo + C::RING * ss;
+#pragma unroll
+      for (int p = 0; p < C::RING; ++p) {
+        const int j = p % B;                       // tile inside its batch
+        const int bi = ss * (C::RING / B) + p / B; // batch index
+        const int buf = bi & 1;
+#ifndef EAGLE_DBG_PURE
+        if (j == 0) stage_load(tb + p + B);        // next batch's scales and biases
+#endif
+        const int tile = tb + p;
+        if (tile < t_hi) {
+          // this tile's scales and biases: row j*16 + r, column (wave ^ r)
+          const unsigned char* sp = sbuf + buf * C::SB_BUF + (((j * 16 + r) * 16) + (wave ^ r)) * C::UNIT;
+          uint2_t sv, bv;
+          if (GW == 4) {
+            sv = *reinterpret_cast<const uint2_t*>(sp);
+            bv = *reinterpret_cast<const uint2_t*>(sp + C::SB_ARRAY);
+          } else {
+            sv[0] = *reinterpret_cast<const uint32_t*>(sp);
+            bv[0] = *reinterpret_cast<const uint32_t*>(sp + C::SB_ARRAY);
+            sv[1] = sv[0];
+            bv[1] = bv[0];
+          }
+          // weight-side operand of the bias / offset MFMA: biases in K block 0, 64 * scales
+          // in K block 1 (blocks 2 and 3 meet zeros)
+          uint4_t aux;
+          {
+            const half2_t s0 = as_h2(sv[0]) * kmul, s1 = as_h2(sv[1]) * kmul;
+            const uint32_t q0 = h == 0 ? bv[0] : as_u32(s0);
+            const uint32_t q1 = h == 0 ? bv[1] : as_u32(s1);
+            aux[0] = q0; aux[1] = q1; aux[2] = q0; aux[3] = q1;
+          }
+          float4_t acc[NT];
+#pragma unroll
+          for (int t = 0; t < NT; ++t)
+            acc[t] = __builtin_amdgcn_mfma_f32_16x16x32_f16(
+                xaux[t], __builtin_bit_cast(half8_t, aux), float4_t{0.f, 0.f, 0.f, 0.f}, 0, 0, 0);
+#ifndef EAGLE_DBG_NOCOMP
+#pragma unroll
+          for (int ld = 0; ld < C::NL; ++ld) {
+            uint32_t q[4] = {ring[p][ld][0], ring[p][ld][1], ring[p][ld][2], ring[p][ld][3]};
+            swap32(q[0], q[2]);
+            swap32(q[1], q[3]);
+#pragma unroll
+            for (int gl = 0; gl < 2; ++gl) {
+              const int g = 2 * ld + gl;
+              float4_t tt[NT];
+#pragma unroll
+              for (int t = 0; t < NT; ++t) tt[t] = float4_t{0.f, 0.f, 0.f, 0.f};
+#pragma unroll
+              for (int pp = 0; pp < 2; ++pp) {
+                const half8_t wop = expand8(q[2 * gl + pp], magic_lo, magic_hi);
+#pragma unroll
+                for (int t = 0; t < NT; ++t)
+                  tt[t] = __builtin_amdgcn_mfma_f32_16x16x32_f16(xop[t][4 * ld + 2 * gl + pp], wop,
+                                                                 tt[t], 0, 0, 0);
+              }
+              const half_t sg = as_h2(sv[g >> 1])[g & 1];
+#pragma unroll
+              for (int t = 0; t < NT; ++t)
+#pragma unroll
+                for (int i = 0; i < 4; ++i) acc[t][i] = __builtin_fmaf((float)sg, tt[t][i], acc[t][i]);
+            }
+          }
+#else
+#pragma unroll
+          for (int ld = 0; ld < C::NL; ++ld) acc[0][0] += __builtin_bit_cast(float, ring[p][ld][0] ^ ring[p][ld][3]);
+#endif
+#pragma unroll
+          for (int t = 0; t < NT; ++t)
+            pbuf4[(buf * nw + wave) * 256 + (j * NT + t) * 64 + lane] = acc[t];
+          if (ss == 0 && p == 0) TSTAMP(4);
+        }
+#ifndef EAGLE_DBG_NOW
+        load_w(tb + p + C::RING, ring[p]);
+#endif
+        if (j == B - 1) {
+#ifndef EAGLE_DBG_PURE
+          stage_store(buf ^ 1);
+          lds_barrier();
+#endif
         }
       }
-  };
-
-  const uint32_t gsel = (h & 2) ? 0x03020302u : 0x01000100u;   // byte selector of group h/2
-  DequantConsts dq;
-  asm volatile("v_mov_b32 %0, 0x64006400" : "=v"(dq.magic_lo));
-  asm volatile("v_mov_b32 %0, 0x54005400" : "=v"(dq.magic_hi));
-
-  // item (round, j): chunk c_lo + j of the slab, for the RT tiles of this wave.  The lane
-  // reads nibbles 32h..32h+31 (group 4c + h/2) and 128+32h.. (group 4c + 2 + h/2) of it.
-  // Loads are unconditional: a conditional load makes the compiler fall back to waiting
-  // for every outstanding load.  Out-of-range rounds, rows, chunks and groups are clamped to
-  // an in-range address instead; what they fetch is multiplied by the zeros that pad x in
-  // LDS (columns >= K) or never consumed (dummy items, rows >= N).
-  auto load_w = [&](int round, int j, WRegs (&dst)[RT]) {
-    const int c = cbase + c_lo + j;
-    const int col = c * 32 + h * 4;                       // in 32-bit words, 4 per load
-#pragma unroll
-    for (int rt = 0; rt < RT; ++rt) {
-      const int rr = min(round, rounds - 1);
-      const int n = min((tile_base + rr * tiles_per_round + rt) * 16 + r, N - 1);
-      const uint32_t* row = w + (size_t)n * K8;
-#ifdef EAGLE_DBG_NOW
-      dst[rt].lo = uint4_t{(uint32_t)n, 0, 0, 0}; dst[rt].hi = uint4_t{0, 0, 0, (uint32_t)col}; (void)row;
-#else
-      dst[rt].lo = __builtin_nontemporal_load(reinterpret_cast<const uint4_t*>(row + min(col, K8 - 4)));
-      dst[rt].hi = __builtin_nontemporal_load(reinterpret_cast<const uint4_t*>(row + min(col + 16, K8 - 4)));
+    }
+    TSTAMP(5);
+  } else {
+    // ------------------------------------------------------------------ reducing wave
+    const int wl = tid - nw * 64;     // 0 .. 127
+    __syncthreads();
+    const int nb = nss * (C::RING / B);
+    for (int bi = 0; bi < nb; ++bi) {
+#ifndef EAGLE_DBG_PURE
+      lds_barrier();
 #endif
-    }
-  };
-
-  float4_t acc[RT][NT];
+      const int buf = bi & 1;
+      const int tile0 = t_lo + bi * B;
 #pragma unroll
-  for (int i = 0; i < RT; ++i)
-#pragma unroll
-    for (int j = 0; j < NT; ++j) acc[i][j] = float4_t{0.f, 0.f, 0.f, 0.f};
-
-  auto compute = [&](const WRegs (&cur)[RT], int j) {
-    // B operand of step t: 8 halves of x row m = 16 nt + r at slab column
-    // 256 (c_lo + j) + 32h + 8t (t < 4) or + 128 + 32h + 8(t-4)
-    const unsigned char* xb = lds + r * xrow + (c_lo + j) * (CHUNK_K * 2) + h * 64;
-    // the lane's groups are h/2 (first half chunk) and 2 + h/2: broadcast that half of
-    // the {g0,g1} / {g2,g3} pairs into both halves of a register
-    half2_t ss[RT][2], bb[RT][2];
-    const int c4 = (cbase + c_lo + j) * 4;
-    const int shift = SLOW_SB ? 0 : 16 * (c4 - min(c4, G - 4));   // tail chunk: see load_sb
-#pragma unroll
-    for (int rt = 0; rt < RT; ++rt) {
-      const unsigned char* sp = sbw + rt * sb_tile_bytes + (r * UP + j) * 8;
-      const uint2_t s4 = *reinterpret_cast<const uint2_t*>(sp);
-      const uint2_t b4 = *reinterpret_cast<const uint2_t*>(sp + 16 * UP * 8);
-      uint32_t s01 = s4[0], s23 = s4[1], b01 = b4[0], b23 = b4[1];
-      if (shift) {
-        const uint64_t sv = (((uint64_t)s23 << 32) | s01) >> shift;
-        const uint64_t bv = (((uint64_t)b23 << 32) | b01) >> shift;
-        s01 = (uint32_t)sv; s23 = (uint32_t)(sv >> 32);
-        b01 = (uint32_t)bv; b23 = (uint32_t)(bv >> 32);
-      }
-      ss[rt][0] = as_h2(__builtin_amdgcn_perm(s01, s01, gsel));
-      bb[rt][0] = as_h2(__builtin_amdgcn_perm(b01, b01, gsel));
-      ss[rt][1] = as_h2(__builtin_amdgcn_perm(s23, s23, gsel));
-      bb[rt][1] = as_h2(__builtin_amdgcn_perm(b23, b23, gsel));
-    }
-#pragma unroll
-    for (int t = 0; t < 8; ++t) {
-      half8_t bx[NT];
-#pragma unroll
-      for (int nt = 0; nt < NT; ++nt)
-        bx[nt] = *reinterpret_cast<const half8_t*>(xb + nt * 16 * xrow + (t >> 2) * 256 + (t & 3) * 16);
-#pragma unroll
-      for (int rt = 0; rt < RT; ++rt) {
-        const uint32_t word = (t < 4) ? cur[rt].lo[t & 3] : cur[rt].hi[t & 3];
-        const half8_t a = dequant8(word, ss[rt][t >> 2], bb[rt][t >> 2], dq);
-#pragma unroll
-        for (int nt = 0; nt < NT; ++nt)
-          acc[rt][nt] = __builtin_amdgcn_mfma_f32_16x16x32_f16(a, bx[nt], acc[rt][nt], 0, 0, 0);
-      }
-    }
-  };
-
-  // End of a round: add the WK partial tiles, combine K slabs, store.
-  auto finish_round = [&](int round) {
-    if (WK > 1) {
-      float4_t* rb = reinterpret_cast<float4_t*>(red);
-      __syncthreads();                 // previous round's readers are done with `red`
-      if (wk > 0) {
-#pragma unroll
-        for (int rt = 0; rt < RT; ++rt)
-#pragma unroll
-          for (int nt = 0; nt < NT; ++nt)
-            rb[((((wk - 1) * WT + wt) * RT + rt) * NT + nt) * 64 + lane] = acc[rt][nt];
-      }
-      __syncthreads();
-      if (wk == 0) {
-        for (int k2 = 1; k2 < WK; ++k2)
-#pragma unroll
-          for (int rt = 0; rt < RT; ++rt)
-#pragma unroll
-            for (int nt = 0; nt < NT; ++nt)
-              acc[rt][nt] += rb[((((k2 - 1) * WT + wt) * RT + rt) * NT + nt) * 64 + lane];
-      }
-    }
-    const bool owner = wk == 0;
-    bool write_out = owner;
-    if (nsplit > 1) {
-      const int rblock = blockIdx.x * rounds + round;       // row block of this round
-      const int per_blk = WT * RT * NT * 64;                // float4 per (row block, slab)
-      float* pbase = partial + ((size_t)rblock * nsplit) * per_blk * 4;
-      if (owner) {
-        float* mine = pbase + (size_t)blockIdx.y * per_blk * 4;
-#pragma unroll
-        for (int rt = 0; rt < RT; ++rt)
-#pragma unroll
-          for (int nt = 0; nt < NT; ++nt)
+      for (int it = 0; it < 2; ++it) {
+        const int l4 = wl + it * 128;            // 0 .. 255
+        const int jt = l4 >> 6;
+        const int j = jt / NT, t = jt % NT;
+        const int tile = tile0 + j;
+        if (tile >= t_hi) continue;
+        float4_t sum = pbuf4[(buf * nw) * 256 + l4];
+#ifndef EAGLE_DBG_NORED
+        for (int wv = 1; wv < nw; ++wv) sum += pbuf4[(buf * nw + wv) * 256 + l4];
+#endif
+        const int ln = l4 & 63;
+        const int n = tile * 16 + (ln & 15);
+        const int m0 = 16 * t + 4 * (ln >> 4);
+        if (to_out) {
+          if (n < N) {
+            half_t bn = (half_t)0.f;
+            if (bias) bn = bias[n];
 #pragma unroll
             for (int i = 0; i < 4; ++i)
-              __hip_atomic_store(mine + ((((wt * RT + rt) * NT + nt) * 64 + lane) << 2) + i,
-                                 acc[rt][nt][i], __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
-      }
-      __builtin_amdgcn_s_waitcnt(0x0F70);   // vmcnt(0): this wave's partial stores are done
-      __syncthreads();
-      if (tid == 0) {
-        const unsigned old = __hip_atomic_fetch_add(&counters[rblock], 1u, __ATOMIC_RELAXED,
-                                                    __HIP_MEMORY_SCOPE_AGENT);
-        s_last = (old == (unsigned)(nsplit - 1));
-      }
-      __syncthreads();
-      const bool last = s_last != 0;
-      write_out = owner && last;
-      if (write_out) {
-#pragma unroll
-        for (int rt = 0; rt < RT; ++rt)
-#pragma unroll
-          for (int nt = 0; nt < NT; ++nt) {
-            float4_t sum = float4_t{0.f, 0.f, 0.f, 0.f};
-            for (int sp = 0; sp < nsplit; ++sp) {
-              const float* src = pbase + (size_t)sp * per_blk * 4 +
-                                 ((((wt * RT + rt) * NT + nt) * 64 + lane) << 2);
-#pragma unroll
-              for (int i = 0; i < 4; ++i)
-                sum[i] += __hip_atomic_load(src + i, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
-            }
-            acc[rt][nt] = sum;
+              if (m0 + i < M) {
+                half_t o = (half_t)sum[i];
+                if (bias) o = o + bn;
+                out[(size_t)(m0 + i) * N + n] = o;
+              }
           }
-      }
-      if (last && tid == 0)
-        __hip_atomic_store(&counters[rblock], 0u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
-    }
-    // lane holds out[m = 16 nt + r][n = tile*16 + 4 h + i], i = 0..3
-    if (write_out) {
+        } else {
+          // partial[slab][tile][t][i][64]
+          float* dst = partial + ((((size_t)slab * tiles_total + tile) * NT + t) * 4) * 64 + ln;
 #pragma unroll
-      for (int rt = 0; rt < RT; ++rt) {
-        const int n0 = (tile_base + round * tiles_per_round + rt) * 16 + 4 * h;
-        if (n0 >= N) continue;   // N % 8 == 0, so a group of four is all in or all out
-#pragma unroll
-        for (int nt = 0; nt < NT; ++nt) {
-          const int m = nt * 16 + r;
-          if (m >= M) continue;
-          half4_t o;
-#pragma unroll
-          for (int i = 0; i < 4; ++i) {
-            half_t v = (half_t)acc[rt][nt][i];
-            if (bias) v = (half_t)((float)v + (float)bias[n0 + i]);
-            o[i] = v;
-          }
-          *reinterpret_cast<half4_t*>(out + (size_t)m * N + n0) = o;
+          for (int i = 0; i < 4; ++i)
+            __hip_atomic_store(dst + i * 64, sum[i], __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
         }
       }
     }
-#pragma unroll
-    for (int rt = 0; rt < RT; ++rt)
-#pragma unroll
-      for (int nt = 0; nt < NT; ++nt) acc[rt][nt] = float4_t{0.f, 0.f, 0.f, 0.f};
-    // Stores and loads retire out of order with respect to each other, so a counted wait
-    // on the weight ring is only exact while no store is pending: drain here, once per
-    // round, instead of at every chunk.  (0x0F70 = vmcnt(0), other counters untouched.)
-    __builtin_amdgcn_s_waitcnt(0x0F70);
-  };
-
-  // ---- prologue: first loads in flight, then the x slab ---------------------------------
-  // Every wave walks UPAD = U rounded up to a multiple of PF items per round, so that the
-  // ring slot of an item is a compile-time constant; items past its real run are dummies
-  // (no load, no compute).
-  const int UPAD = (U + PF - 1) / PF * PF;
-  // Order matters: the x loads go out first and in one batch where possible (they sit on
-  // the critical path to the first barrier), the weight ring next; waiting for x then
-  // leaves the younger ring loads in flight.
-  load_sb(0);
-  {
-    constexpr int XB = 12;
-    const int vec_row = slab_k >> 3;
-    const int total = MP * vec_row;
-    for (int v0 = tid; v0 < total; v0 += nthr * XB) {
-      half8_t a[XB];
-#pragma unroll
-      for (int i = 0; i < XB; ++i) {
-        // always load from an in-range address and zero afterwards: no branch, so the
-        // XB loads are in flight together
-        const int v = v0 + i * nthr;
-        const int row = v / vec_row;
-        const int c8 = v - row * vec_row;
-        const int k = k0 + c8 * 8;
-        const bool ok = v < total && row < M && k < K;
-        const half8_t ld = *reinterpret_cast<const half8_t*>(
-            x + (size_t)min(row, M - 1) * K + min(k, K - 8));
-        a[i] = ok ? ld : half8_t{0, 0, 0, 0, 0, 0, 0, 0};
-      }
-#pragma unroll
-      for (int i = 0; i < XB; ++i) {
-        const int v = v0 + i * nthr;
-        const int row = v / vec_row;
-        const int c8 = v - row * vec_row;
-        half8_t p;   // element order matching dequant8: 0,4,1,5,2,6,3,7
-        p[0] = a[i][0]; p[1] = a[i][4]; p[2] = a[i][1]; p[3] = a[i][5];
-        p[4] = a[i][2]; p[5] = a[i][6]; p[6] = a[i][3]; p[7] = a[i][7];
-        if (v < total) *reinterpret_cast<half8_t*>(lds + row * xrow + c8 * 16) = p;
-      }
-    }
   }
-  WRegs ring[PF][RT];
-#pragma unroll
-  for (int p = 0; p < PF; ++p) load_w(0, p, ring[p]);
-  commit_sb();
-  load_sb(1);
-  __syncthreads();                      // the x slab is in LDS
 
-  // ---- main loop -------------------------------------------------------------------------
-  // The chunk loop is free of stores and of round bookkeeping, so the counted waits on the
-  // ring stay exact; the ring runs across rounds (the last PF items of a round already
-  // load the first PF of the next).
-  for (int round = 0; round < rounds; ++round) {
-    for (int jb = 0; jb < UPAD; jb += PF) {
-#pragma unroll
-      for (int p = 0; p < PF; ++p) {
-        const int j = jb + p;
-        if (j < cpw) {
-#ifdef EAGLE_DBG_NOCOMP
-          acc[0][0][0] += __builtin_bit_cast(float, ring[p][0].lo[0] ^ ring[p][0].hi[3]);
-#else
-          compute(ring[p], j);
-#endif
+  TSTAMP(wave == 0 ? 6 : 9);
+  if (nsplit > 1) {
+    // ---- the last workgroup of this tile range to arrive adds the slabs, in slab order
+    int* flag = reinterpret_cast<int*>(lds);
+    __builtin_amdgcn_s_waitcnt(0x0F70);   // vmcnt(0): this wave's partial stores are done
+    __syncthreads();
+    if (tid == 0) {
+      const unsigned old = __hip_atomic_fetch_add(&counters[blockIdx.x], 1u, __ATOMIC_RELAXED,
+                                                  __HIP_MEMORY_SCOPE_AGENT);
+      *flag = old == (unsigned)(nsplit - 1);
+      if (old == (unsigned)(nsplit - 1))
+        __hip_atomic_store(&counters[blockIdx.x], 0u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+    }
+    __syncthreads();
+    TSTAMP(wave == 0 ? 7 : 10);
+    if (*flag) {
+      const int per_tile = NT * 256;                       // floats
+      const int total = (t_hi - t_lo) * per_tile;
+      const size_t slab_stride = (size_t)tiles_total * per_tile;
+      for (int idx = tid; idx < total; idx += blockDim.x) {
+        const int tile = t_lo + idx / per_tile;
+        const int rem = idx % per_tile;                    // (t*4 + i)*64 + ln
+        const int ln = rem & 63;
+        const int ti = rem >> 6;
+        const int t = ti >> 2, i = ti & 3;
+        const float* src = partial + (size_t)tile * per_tile + rem;
+        float v = 0.f;
+        for (int sp = 0; sp < nsplit; ++sp)
+          v += __hip_atomic_load(src + sp * slab_stride, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+        const int n = tile * 16 + (ln & 15);
+        const int m = 16 * t + 4 * (ln >> 4) + i;
+        if (n < N && m < M) {
+          half_t o = (half_t)v;
+          if (bias) o = o + bias[n];
+          out[(size_t)m * N + n] = o;
         }
-        int nj = j + PF, nr = round;
-        if (nj >= UPAD) { nj -= UPAD; ++nr; }
-        load_w(nr, nj, ring[p]);
       }
     }
-#ifndef EAGLE_DBG_NOSTORE
-    finish_round(round);
-#endif
-    commit_sb();               // staged while the round that just ended was running
-    load_sb(round + 2);
   }
+  TSTAMP(wave == 0 ? 8 : 11);
 }
 
 // ------------------------------------------------------------------------------------------
 // host side
 // ------------------------------------------------------------------------------------------
-// Ring depth for a run of `units` chunks: the depth whose multiple overshoots the run least
-// (the overshoot only costs empty loop iterations); deeper wins ties.
-int pick_pf(int units) {
-  int best = 7, best_waste = 1 << 30;
-  const int cands[3] = {7, 5, 4};
-  for (int pf : cands) {
-    const int waste = (units + pf - 1) / pf * pf - units;
-    if (waste < best_waste) { best = pf; best_waste = waste; }
-  }
-  return best;
-}
+inline int nt_of(int M) { return M <= 16 ? 1 : 2; }
+inline int cw_of(int M) { return M <= 16 ? 256 : 128; }
 
-int lds_bytes(int mp, const Launch& L) {
-  const int nt = mp / 16;
-  const int xs = mp * (L.slab_k * 2 + 16);
-  const int red = L.wk > 1 ? (L.wk - 1) * L.wt * L.rt * nt * 1024 : 0;
-  const int units = (L.slab_k / CHUNK_K + L.wk - 1) / L.wk;
-  const int sb = L.wt * L.wk * L.rt * 2 * 16 * sb_row_units(units) * 8;
-  return xs + red + sb;
+int lds_bytes(int M, const Launch& L) {
+  const int sb = M <= 16 ? 2 * Cfg<1, 4>::SB_BUF : 2 * Cfg<2, 2>::SB_BUF;
+  return pbuf_bytes(L.nw) + sb;
 }
 
 int validate_launch(int M, int N, int K, const Launch& L) {
-  const int mp = M <= 16 ? 16 : 32;
-  if (L.rt != 1 || L.wt < 1 || L.wk < 1 || L.wt * L.wk > MAX_WAVES) return EAGLE_ERR_SHAPE;
-  if (L.pf != 4 && L.pf != 5 && L.pf != 7) return EAGLE_ERR_SHAPE;
-  if (L.splits < 1 || L.splits > MAX_SPLITS || L.slab_k < CHUNK_K || (L.slab_k % CHUNK_K) != 0)
+  if (L.nw < 1 || L.nw > MAX_STREAM_WAVES || L.splits < 1 || L.splits > MAX_SPLITS)
     return EAGLE_ERR_SHAPE;
-  if ((long)L.slab_k * L.splits < K || (long)L.slab_k * (L.splits - 1) >= K) return EAGLE_ERR_SHAPE;
-  const int units = (L.slab_k / CHUNK_K + L.wk - 1) / L.wk;
-  if (units > 16) return EAGLE_ERR_SHAPE;            // a wave's run must fit its staging registers
-  if (L.row_groups < 1 || L.rounds < 1) return EAGLE_ERR_SHAPE;
-  const long tiles = (N + 15) / 16;
-  if ((long)L.row_groups * L.rounds * L.wt * L.rt < tiles) return EAGLE_ERR_SHAPE;
-  if (lds_bytes(mp, L) > LDS_BUDGET) return EAGLE_ERR_SHAPE;
-  if (L.splits > 1 && (long)L.row_groups * L.rounds > MAX_ROW_BLOCKS) return EAGLE_ERR_SHAPE;
+  const int units = (K + cw_of(M) - 1) / cw_of(M);
+  if ((long)L.nw * L.splits < units || (long)L.nw * (L.splits - 1) >= units) return EAGLE_ERR_SHAPE;
+  const int tiles = (N + 15) / 16;
+  if (L.ranges < 1 || L.ranges > tiles || L.ranges > MAX_RANGES) return EAGLE_ERR_SHAPE;
+  if (lds_bytes(M, L) > LDS_MAX) return EAGLE_ERR_SHAPE;
   return EAGLE_OK;
 }
 
-size_t partial_bytes(int M, const Launch& L) {
+size_t partial_bytes(int M, int N, const Launch& L) {
   if (L.splits <= 1) return 0;
-  const size_t mp = M <= 16 ? 16 : 32;
-  return (size_t)L.row_groups * L.rounds * L.splits * L.wt * L.rt * 16 * mp * sizeof(float);
+  const size_t tiles = (N + 15) / 16;
+  return (size_t)L.splits * tiles * nt_of(M) * 256 * sizeof(float);
 }
 
-// Launch shape.  K slabs only as far as LDS capacity forces them (every extra slab costs
-// a partial-sum round trip): the x slab plus the per-wave scale/bias blocks must leave room
-// for at least 12 waves.  One workgroup per compute unit when the slab is large, up to four
-// when it is small.  As many waves along N as the tile count can feed; the rest of the
-// parallelism comes from splitting a tile's chunk run over waves.
+// Launch shape: as few K slabs as 14 streaming waves allow, the units spread evenly over the
+// slabs, and about one workgroup per compute unit (two when a workgroup is at most 8 waves).
 void choose(int M, int N, int K, Launch* out) {
-  const int mp = M <= 16 ? 16 : 32;
+  const int units = (K + cw_of(M) - 1) / cw_of(M);
   const int tiles = (N + 15) / 16;
   Launch L;
-  L.rt = 1;
-  int waves = 4, wg_per_cu = 1;
-  bool found = false;
-  for (L.splits = 1; L.splits <= MAX_SPLITS && !found; ++L.splits) {
-    L.slab_k = ((K + L.splits - 1) / L.splits + CHUNK_K - 1) / CHUNK_K * CHUNK_K;
-    const int chunks = L.slab_k / CHUNK_K;
-    if (chunks > 16) continue;                               // staging registers hold 16 chunks
-    const int x_lds = mp * (L.slab_k * 2 + 16);
-    const int sb_wave = 2 * 16 * sb_row_units(chunks) * 8;
-    const bool last_try = L.splits == MAX_SPLITS || L.slab_k == CHUNK_K;
-    for (int wg = 4; wg >= 1 && !found; --wg) {
-      int w = (LDS_BUDGET / wg - 1024 - x_lds) / sb_wave;
-      if (w > 16 / wg) w = 16 / wg;
-      if (w > MAX_WAVES) w = MAX_WAVES;
-      w = w / 4 * 4;
-      if (w >= 4 && (wg * w >= 12 || (last_try && wg == 1))) {
-        waves = w;
-        wg_per_cu = wg;
-        found = true;
-      }
-    }
-    if (found) break;
-  }
-  L.splits = (K + L.slab_k - 1) / L.slab_k;
-  const int chunks = L.slab_k / CHUNK_K;
-  const int nchunks_last = (K - L.slab_k * (L.splits - 1) + CHUNK_K - 1) / CHUNK_K;
-  int groups = (256 * wg_per_cu) / L.splits;
-  if (groups < 1) groups = 1;
-  if (groups > tiles) groups = tiles;
-  const int tiles_per_group = (tiles + groups - 1) / groups;
-  if (tiles_per_group >= waves) {
-    L.wk = 1;
-    L.rounds = (tiles_per_group + waves - 1) / waves;
-    L.wt = (tiles_per_group + L.rounds - 1) / L.rounds;      // even out the rounds
-  } else {
-    L.wt = tiles_per_group;
-    L.wk = waves / L.wt;
-    if (L.wk > chunks) L.wk = chunks;
-    // every wave should own at least one chunk of the (shorter) last slab
-    while (L.wk > 1 && ((chunks + L.wk - 1) / L.wk) * (L.wk - 1) >= nchunks_last) --L.wk;
-    L.rounds = 1;
-  }
-  L.row_groups = (tiles + L.rounds * L.wt - 1) / (L.rounds * L.wt);
-  L.pf = pick_pf((chunks + L.wk - 1) / L.wk);
+  L.splits = (units + MAX_STREAM_WAVES - 1) / MAX_STREAM_WAVES;
+  L.nw = (units + L.splits - 1) / L.splits;
+  L.splits = (units + L.nw - 1) / L.nw;
+  const int wg_per_cu = (L.nw + NWR) <= 8 && 2 * lds_bytes(M, L) <= LDS_MAX ? 2 : 1;
+  int ranges = (NUM_CU * wg_per_cu) / L.splits;
+  if (ranges < 1) ranges = 1;
+  if (ranges > tiles) ranges = tiles;
+  if (ranges > MAX_RANGES) ranges = MAX_RANGES;
+  L.ranges = ranges;
   *out = L;
 }
 
-template <int NT, int PF, bool SLOW_SB>
+template <int NT, int GW, bool SLOWSB>
 int launch(const void* x, const uint32_t* wq, const void* s, const void* b, const void* bias,
            void* out, float* partial, unsigned* counters, int M, int N, int K, const Launch& L,
            hipStream_t stream) {
-  const int lds = lds_bytes(16 * NT, L);
+  const int lds = lds_bytes(M, L);
   static bool attr_set = false;   // more than 64 KB of LDS needs an explicit opt-in, once
   if (lds > 65536 && !attr_set) {
-    if (hipFuncSetAttribute(reinterpret_cast<const void*>(&qmm_w4g64_kernel<NT, 1, PF, SLOW_SB>),
-                            hipFuncAttributeMaxDynamicSharedMemorySize, LDS_BUDGET) != hipSuccess)
+    if (hipFuncSetAttribute(reinterpret_cast<const void*>(&qmm_w4g64_kernel<NT, GW, SLOWSB>),
+                            hipFuncAttributeMaxDynamicSharedMemorySize, LDS_MAX) != hipSuccess)
       return EAGLE_ERR_HIP;
     attr_set = true;
   }
-  hipLaunchKernelGGL((qmm_w4g64_kernel<NT, 1, PF, SLOW_SB>), dim3(L.row_groups, L.splits),
-                     dim3(64 * L.wt * L.wk), lds, stream, (const half_t*)x, wq,
+  hipLaunchKernelGGL((qmm_w4g64_kernel<NT, GW, SLOWSB>), dim3(L.ranges, L.splits),
+                     dim3(64 * (L.nw + NWR)), lds, stream, (const half_t*)x, wq,
                      (const half_t*)s, (const half_t*)b, (const half_t*)bias, (half_t*)out,
-                     partial, counters, M, N, K, L.wt, L.wk, L.slab_k, L.rounds);
+                     partial, counters, M, N, K, L.nw);
   return eagle_launch_status();
 }
 
@@ -575,8 +550,8 @@ int validate(const void* x, const uint32_t* wq, const void* s, const void* b, co
   if (!x || !wq || !s || !b || !out) return EAGLE_ERR_NULL;
   if (M < 1 || M > EAGLE_MAX_M || N < 8 || (N % 8) != 0 || K < 64 || (K % 64) != 0)
     return EAGLE_ERR_SHAPE;
-  const int slab_max = M <= 16 ? 4096 : 2048;
-  if (K > slab_max * MAX_SPLITS) return EAGLE_ERR_SHAPE;
+  if ((long)K > (long)cw_of(M) * MAX_STREAM_WAVES * MAX_SPLITS) return EAGLE_ERR_SHAPE;
+  if ((long)N * (K / 2) >= (1L << 32)) return EAGLE_ERR_SHAPE;   // 32-bit byte offsets
   if (!eagle_aligned16(x) || !eagle_aligned16(wq) || !eagle_aligned16(out) ||
       (reinterpret_cast<uintptr_t>(s) & 1u) || (reinterpret_cast<uintptr_t>(b) & 1u) ||
       (bias && (reinterpret_cast<uintptr_t>(bias) & 1u)))
@@ -591,30 +566,23 @@ int run(const void* x, const uint32_t* wq, const void* scales, const void* biase
   unsigned* counters = nullptr;
   if (L.splits > 1) {
     if (!workspace || !eagle_aligned16(workspace) ||
-        workspace_bytes < (size_t)EAGLE_QMM_COUNTER_BYTES + partial_bytes(M, L))
+        workspace_bytes < (size_t)EAGLE_QMM_COUNTER_BYTES + partial_bytes(M, N, L))
       return EAGLE_ERR_WORKSPACE;
     counters = reinterpret_cast<unsigned*>(workspace);
     partial = reinterpret_cast<float*>(static_cast<unsigned char*>(workspace) +
                                        EAGLE_QMM_COUNTER_BYTES);
   }
-  // rows with fewer than four groups, or an odd group count (unaligned 8-byte reads),
-  // fetch scales and biases one by one
+  // vector fetches of scales / biases need whole, aligned units in every row
   const int G = K / 64;
-  const bool slow = G < 4 || (G & 1);
-#define EAGLE_QMM_GO(NT_, PF_)                                                               \
-  return slow ? launch<NT_, PF_, true>(x, wq, scales, biases, bias, out, partial, counters, \
-                                       M, N, K, L, st)                                      \
-              : launch<NT_, PF_, false>(x, wq, scales, biases, bias, out, partial, counters, \
-                                        M, N, K, L, st)
-  if (M <= 16) {
-    if (L.pf == 7) EAGLE_QMM_GO(1, 7);
-    if (L.pf == 5) EAGLE_QMM_GO(1, 5);
-    EAGLE_QMM_GO(1, 4);
-  }
-  if (L.pf == 7) EAGLE_QMM_GO(2, 7);
-  if (L.pf == 5) EAGLE_QMM_GO(2, 5);
-  EAGLE_QMM_GO(2, 4);
-#undef EAGLE_QMM_GO
+  const int gw = M <= 16 ? 4 : 2;
+  const uintptr_t amask = gw == 4 ? 7u : 3u;
+  const bool slow = (G % gw) != 0 || (reinterpret_cast<uintptr_t>(scales) & amask) ||
+                    (reinterpret_cast<uintptr_t>(biases) & amask);
+  if (M <= 16)
+    return slow ? launch<1, 4, true>(x, wq, scales, biases, bias, out, partial, counters, M, N, K, L, st)
+                : launch<1, 4, false>(x, wq, scales, biases, bias, out, partial, counters, M, N, K, L, st);
+  return slow ? launch<2, 2, true>(x, wq, scales, biases, bias, out, partial, counters, M, N, K, L, st)
+              : launch<2, 2, false>(x, wq, scales, biases, bias, out, partial, counters, M, N, K, L, st);
 }
 
 }  // namespace
@@ -623,35 +591,32 @@ EAGLE_EXPORT size_t eagle_qmm_workspace_bytes(int M, int N, int K) {
   if (M < 1 || M > EAGLE_MAX_M || N < 1 || K < 64) return 0;
   Launch L;
   choose(M, N, K, &L);
-  return (size_t)EAGLE_QMM_COUNTER_BYTES + partial_bytes(M, L);
+  return (size_t)EAGLE_QMM_COUNTER_BYTES + partial_bytes(M, N, L);
 }
 
-EAGLE_EXPORT size_t eagle_qmm_workspace_bytes_tuned(int M, int rt, int wt, int wk, int splits,
-                                                    int row_groups, int rounds) {
-  if (M < 1 || rt < 1 || wt < 1 || wk < 1 || splits < 1 || row_groups < 1 || rounds < 1) return 0;
-  Launch L{rt, wt, wk, splits, 0, row_groups, rounds, 4};
-  return (size_t)EAGLE_QMM_COUNTER_BYTES + partial_bytes(M, L);
+EAGLE_EXPORT size_t eagle_qmm_workspace_bytes_tuned(int M, int N, int splits) {
+  if (M < 1 || M > EAGLE_MAX_M || N < 1 || splits < 1) return 0;
+  Launch L{1, splits, 1};
+  return (size_t)EAGLE_QMM_COUNTER_BYTES + partial_bytes(M, N, L);
 }
 
-EAGLE_EXPORT int eagle_qmm_plan(int M, int N, int K, int* plan7) {
-  if (!plan7) return EAGLE_ERR_NULL;
+EAGLE_EXPORT int eagle_qmm_plan(int M, int N, int K, int* plan3) {
+  if (!plan3) return EAGLE_ERR_NULL;
   if (M < 1 || M > EAGLE_MAX_M || N < 8 || K < 64 || (K % 64) != 0) return EAGLE_ERR_SHAPE;
   Launch L;
   choose(M, N, K, &L);
-  plan7[0] = L.rt; plan7[1] = L.wt; plan7[2] = L.wk; plan7[3] = L.splits;
-  plan7[4] = L.slab_k; plan7[5] = L.row_groups; plan7[6] = L.rounds;
+  plan3[0] = L.nw; plan3[1] = L.splits; plan3[2] = L.ranges;
   return EAGLE_OK;
 }
 
 EAGLE_EXPORT int eagle_qmm_w4g64_f16_tuned(const void* x, const uint32_t* wq, const void* scales,
                                            const void* biases, const void* bias, void* out, int M,
-                                           int N, int K, int rt, int wt, int wk, int splits,
-                                           int slab_k, int row_groups, int rounds, void* workspace,
-                                           size_t workspace_bytes, eagle_stream_t stream) {
+                                           int N, int K, int nw, int splits, int ranges,
+                                           void* workspace, size_t workspace_bytes,
+                                           eagle_stream_t stream) {
   int rc = validate(x, wq, scales, biases, bias, out, M, N, K);
   if (rc != EAGLE_OK) return rc;
-  Launch L{rt, wt, wk, splits, slab_k, row_groups, rounds, 0};
-  L.pf = pick_pf((slab_k / CHUNK_K + (wk > 0 ? wk : 1) - 1) / (wk > 0 ? wk : 1));
+  Launch L{nw, splits, ranges};
   rc = validate_launch(M, N, K, L);
   if (rc != EAGLE_OK) return rc;
   return run(x, wq, scales, biases, bias, out, M, N, K, L, workspace, workspace_bytes,

@@ -10,19 +10,16 @@ from util import TOL, layer_to_dev, rel_err, to_dev
 pytestmark = pytest.mark.gpu
 
 
-def shape_for(M, N, K, rt, wt, wk, splits, rounds):
-    """A forced launch shape (or None if it cannot hold the x slab in LDS)."""
-    mp = 16 if M <= 16 else 32
-    slab_k = -(-(-(-K // splits)) // 256) * 256
-    splits = -(-K // slab_k)
+def shape_for(M, N, K, nw, ranges):
+    """A forced launch shape: `nw` streaming waves per workgroup (the K slabs follow from it)
+    and `ranges` workgroups per slab; None if it cannot be launched."""
+    cw = 256 if M <= 16 else 128
+    units = -(-K // cw)
+    splits = -(-units // nw)
     tiles = -(-N // 16)
-    row_groups = -(-tiles // (rounds * wt * rt))
-    units = -(-(slab_k // 256) // wk)
-    lds = (mp * (slab_k * 2 + 16) + ((wk - 1) * wt * rt * (mp // 16) * 1024 if wk > 1 else 0)
-           + wt * wk * rt * 2 * 16 * (units | 1) * 8)
-    if lds > 160 * 1024 - 512 or units > 16 or wt * wk > 12 or rt != 1:
+    if nw > 14 or nw * (splits - 1) >= units or ranges > tiles or splits > 64:
         return None
-    return (rt, wt, wk, splits, slab_k, row_groups, rounds)
+    return (nw, splits, ranges)
 
 
 def run_case(dev, M, N, K, seed=0, bias=False, tuned=None):
@@ -45,18 +42,16 @@ def test_cfg1_shape_all_m(dev, M):
     run_case(dev, M, 8192, 2048, seed=42)
 
 
-@pytest.mark.parametrize("rt", [1])
-@pytest.mark.parametrize("wt,wk", [(4, 1), (2, 4), (1, 7), (12, 1), (2, 5), (3, 2)])
-@pytest.mark.parametrize("splits", [1, 2, 5])
-@pytest.mark.parametrize("rounds", [1, 3])
+@pytest.mark.parametrize("nw", [1, 2, 3, 5, 7, 13, 14])
+@pytest.mark.parametrize("ranges", [1, 7, 96])
 @pytest.mark.parametrize("M", [8, 32])
-def test_forced_launch_shapes(dev, rt, wt, wk, splits, rounds, M):
+def test_forced_launch_shapes(dev, nw, ranges, M):
     N, K = 1536, 3584
-    tuned = shape_for(M, N, K, rt, wt, wk, splits, rounds)
+    tuned = shape_for(M, N, K, nw, ranges)
     if tuned is None:
-        pytest.skip("shape does not fit LDS / chunk count")
+        pytest.skip("shape cannot be launched")
     print(f"qmm tuned={tuned} M={M}", flush=True)
-    run_case(dev, M, N, K, seed=rt * 100 + wt * 10 + splits, tuned=tuned)
+    run_case(dev, M, N, K, seed=nw * 100 + ranges, tuned=tuned)
 
 
 @pytest.mark.parametrize("N,K", [(8, 64), (8, 128), (24, 192), (40, 896), (136, 2944), (512, 3584),
@@ -65,7 +60,7 @@ def test_edge_shapes(dev, N, K):
     for M in (1, 5, 32):
         print(f"qmm edge N={N} K={K} M={M}", flush=True)
         run_case(dev, M, N, K, seed=N + K + M)
-        for cfg in ((1, 1, 1, 1, 1), (1, 2, 1, 3, 2), (1, 2, 2, 2, 1)):
+        for cfg in ((1, 1), (3, 2), (14, 3)):
             tuned = shape_for(M, N, K, *cfg)
             if tuned is not None:
                 run_case(dev, M, N, K, seed=N + K + M, tuned=tuned)
@@ -105,7 +100,8 @@ def test_deterministic_split_k(dev):
     layer = synth.make_qlinear(rng, 512, 3584)
     x = to_dev(synth.make_x(rng, 32, 3584), dev)
     d = layer_to_dev(layer, dev)
-    tuned = shape_for(32, 512, 3584, 1, 2, 2, 7, 2)
+    tuned = shape_for(32, 512, 3584, 4, 5)
+    assert tuned[1] == 7
     ref = ops.quantized_matmul(x, d["weight"], d["scales"], d["biases"], tuned=tuned)
     for _ in range(5):
         again = ops.quantized_matmul(x, d["weight"], d["scales"], d["biases"], tuned=tuned)
@@ -117,9 +113,10 @@ def test_plan_covers_benchmark_shapes(dev):
         for N, K in ((3584, 3584), (512, 3584), (18944, 3584), (3584, 18944), (152064, 3584),
                      (8192, 2048), (896, 896), (128, 896), (4864, 896), (896, 4864),
                      (4096, 4096), (1024, 4096), (14336, 4096), (4096, 14336), (128256, 4096)):
-            rt, wt, wk, splits, slab_k, row_groups, rounds = ops.qmm_plan(M, N, K)
-            assert slab_k * splits >= K and row_groups * rounds * wt * rt * 16 >= N
-            assert wt * wk <= 16
+            nw, splits, ranges = ops.qmm_plan(M, N, K)
+            cw = 256 if M <= 16 else 128
+            assert nw * splits * cw >= K > nw * (splits - 1) * cw
+            assert 1 <= nw <= 14 and 1 <= ranges <= -(-N // 16)
 
 
 def test_argument_errors(dev):

@@ -49,7 +49,7 @@ def test_qmm_argument_errors_are_detected_on_the_host():
     assert call(x=None) == 1                       # EAGLE_ERR_NULL
     assert call(out=None) == 1
     assert call(M=0) == 2 and call(M=33) == 2      # EAGLE_ERR_SHAPE
-    assert call(K=100) == 2 and call(N=12) == 2 and call(K=128 * 1024) == 2
+    assert call(K=100) == 2 and call(N=12) == 2 and call(K=256 * 1024) == 2
     assert call(x=p + 2) == 3                      # EAGLE_ERR_ALIGN
     assert call(gs=32) == 4 and call(bits=8) == 4  # EAGLE_ERR_UNSUPPORTED
     # a K-split launch needs a workspace
@@ -86,10 +86,11 @@ def test_plan_is_consistent_for_benchmark_shapes():
         for N, K in ((3584, 3584), (512, 3584), (18944, 3584), (3584, 18944), (152064, 3584),
                      (8192, 2048), (896, 896), (128, 896), (4864, 896), (896, 4864), (151936, 896),
                      (4096, 4096), (1024, 4096), (14336, 4096), (4096, 14336), (128256, 4096)):
-            rt, wt, wk, splits, slab_k, row_groups, rounds = ops.qmm_plan(M, N, K)
-            assert slab_k % 256 == 0 and slab_k * splits >= K > slab_k * (splits - 1)
-            assert row_groups * rounds * wt * rt * 16 >= N
-            assert 1 <= wt * wk <= 12 and slab_k <= (4096 if M <= 16 else 2048)
+            nw, splits, ranges = ops.qmm_plan(M, N, K)
+            cw = 256 if M <= 16 else 128
+            assert nw * splits * cw >= K > nw * (splits - 1) * cw
+            assert 1 <= nw <= 14 and 1 <= ranges <= -(-N // 16)
+            assert ranges * splits <= 512
 
 
 def test_ops_refuse_cpu_tensors():
