@@ -64,17 +64,17 @@ int eagle_qmm_w4g64_f16(const void* x, const uint32_t* wq, const void* scales,
                         const void* biases, const void* bias, void* out,
                         int M, int N, int K, int group_size, int bits,
                         void* workspace, size_t workspace_bytes, eagle_stream_t stream);
-/* The launch shape the library would pick: plan3 = {streaming waves per workgroup
- * (= column units per K slab; a unit is 256 columns for M <= 16, 128 above), K slabs,
- * tile ranges (workgroups per slab)}. */
-int eagle_qmm_plan(int M, int N, int K, int* plan3);
+/* The launch shape the library would pick: plan4 = {streaming waves per workgroup,
+ * phases (column units each streaming wave owns, one after the other; a unit is 256
+ * columns for M <= 16, 128 above), K slabs, tile ranges (workgroups per slab)}. */
+int eagle_qmm_plan(int M, int N, int K, int* plan4);
 /* Same matmul with the launch shape forced (tuning sweeps and tests).  nw <= 14,
- * nw * splits must cover K with no empty slab, 1 <= ranges <= ceil(N / 16), else
- * EAGLE_ERR_SHAPE. */
+ * phases <= 8, nw * phases * splits must cover K with no empty slab,
+ * 1 <= ranges <= ceil(N / 16), and the shape must fit LDS, else EAGLE_ERR_SHAPE. */
 size_t eagle_qmm_workspace_bytes_tuned(int M, int N, int splits);
 int eagle_qmm_w4g64_f16_tuned(const void* x, const uint32_t* wq, const void* scales,
                               const void* biases, const void* bias, void* out,
-                              int M, int N, int K, int nw, int splits, int ranges,
+                              int M, int N, int K, int nw, int phases, int splits, int ranges,
                               void* workspace, size_t workspace_bytes, eagle_stream_t stream);
 
 /* Quantised embedding gather: out[t,:] = fp16(scales*q + biases) of row ids[t].

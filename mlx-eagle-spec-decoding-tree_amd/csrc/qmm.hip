@@ -95,14 +95,11 @@ __device__ inline void lds_barrier() {
   asm volatile("s_waitcnt lgkmcnt(0)\n\ts_barrier" ::: "memory");
 }
 
-#ifndef EAGLE_RING
-#define EAGLE_RING 4
-#endif
-
 template <int NT, int GW>
 struct Cfg {
-  static constexpr int RING = EAGLE_RING;       // tiles in flight per streaming wave
+  static constexpr int RING = 4;                // tiles in flight per streaming wave
   static constexpr int B = 4 / NT;              // tiles per batch (one barrier per batch)
+  static constexpr int BPS = RING / B;          // batches per super-step of RING tiles
   static constexpr int CW = GW * 64;            // columns owned by a streaming wave
   static constexpr int NL = GW / 2;             // 128-bit weight loads per lane per tile
   static constexpr int NMF = GW * 2;            // MFMAs per 16 rows of x per tile
@@ -115,12 +112,19 @@ struct Cfg {
 __host__ __device__ inline int pbuf_bytes(int nw) { return 2 * nw * 4096; }
 
 struct Launch {
-  int nw;       // streaming waves per workgroup = column units per K slab
-  int splits;   // K slabs (gridDim.y)
+  int nw;       // streaming waves per workgroup
+  int phases;   // column units a streaming wave owns, one after the other
+  int splits;   // K slabs (gridDim.y); a slab is nw * phases units
   int ranges;   // tile ranges (gridDim.x)
 };
 
-// NT: 16-row blocks of x (1 or 2).  GW: quantisation groups per streaming wave.
+template <int V>
+struct Mode { static constexpr int value = V; };
+constexpr int STEP_MID = 0;    // more tiles of this phase follow: reload the ring from it
+constexpr int STEP_NEXT = 1;   // last super-step of a phase, another phase follows
+constexpr int STEP_LAST = 2;   // last super-step of the last phase: nothing to prefetch
+
+// NT: 16-row blocks of x (1 or 2).  GW: quantisation groups per streaming wave and phase.
 // SLOWSB: scales / biases are fetched element by element (odd group counts, rows shorter
 // than a unit, unaligned arrays).
 template <int NT, int GW, bool SLOWSB>
@@ -129,12 +133,13 @@ __global__ __launch_bounds__(1024) void qmm_w4g64_kernel(
     const half_t* __restrict__ s, const half_t* __restrict__ b,
     const half_t* __restrict__ bias, half_t* __restrict__ out,
     float* __restrict__ partial, unsigned* __restrict__ counters,
-    int M, int N, int K, int nw) {
+    int M, int N, int K, int nw, int phases, int t_q, int t_r) {
   using C = Cfg<NT, GW>;
   constexpr int B = C::B;
   extern __shared__ __attribute__((aligned(16))) unsigned char lds[];
   float4_t* pbuf4 = reinterpret_cast<float4_t*>(lds);                 // [2][nw][256] float4
   unsigned char* sbuf = lds + pbuf_bytes(nw);                         // [2][2][16B][16] units
+  float4_t* accl4 = reinterpret_cast<float4_t*>(sbuf + 2 * C::SB_BUF); // [batches][256] float4
 
   const int tid = threadIdx.x;
   const int lane = tid & 63;
@@ -146,72 +151,76 @@ __global__ __launch_bounds__(1024) void qmm_w4g64_kernel(
   const int nsplit = gridDim.y;
   const int slab = blockIdx.y;
   const int tiles_total = (N + 15) >> 4;
-  const int t_lo = (int)(((long)blockIdx.x * tiles_total) / gridDim.x);
-  const int t_hi = (int)(((long)(blockIdx.x + 1) * tiles_total) / gridDim.x);
-  const int nss = (t_hi - t_lo + C::RING - 1) / C::RING;   // super-steps of RING tiles
+  const int bx = blockIdx.x;
+  const int t_lo = bx * t_q + (bx < t_r ? bx : t_r);
+  const int t_hi = t_lo + t_q + (bx < t_r ? 1 : 0);
+  const int nss = (t_hi - t_lo + C::RING - 1) / C::RING;   // super-steps per phase
+  const int nbp = nss * C::BPS;                             // batches per phase
   const bool to_out = nsplit == 1;
 
   TSTAMP(0);
   if (wave < nw) {
     // ------------------------------------------------------------------ streaming wave
-    const int unit = slab * nw + wave;
-    const int col0 = unit * C::CW;
     const uint32_t magic_lo = 0x64006400u, magic_hi = 0x54005400u;
     const uint32_t row_bytes = (uint32_t)K8 * 4u;
+    const int unit0 = slab * phases * nw + wave;            // this wave's unit in phase 0
 
     // byte offset of this lane's words inside a weight row, clamped into the row
-    uint32_t woff[C::NL];
+    auto unit_woff = [&](int unit, uint32_t (&o)[C::NL]) {
 #pragma unroll
-    for (int ld = 0; ld < C::NL; ++ld) {
-      int word = unit * (C::CW / 8) + ld * 16 + h * 4;
-      if (word > K8 - 4) word = K8 - 4;
-      woff[ld] = (uint32_t)word * 4u;
-    }
-    auto load_w = [&](int tile, uint4_t (&dst)[C::NL]) {
+      for (int ld = 0; ld < C::NL; ++ld) {
+        int word = unit * (C::CW / 8) + ld * 16 + h * 4;
+        if (word > K8 - 4) word = K8 - 4;
+        o[ld] = (uint32_t)word * 4u;
+      }
+    };
+    auto load_w = [&](int tile, const uint32_t (&o)[C::NL], uint4_t (&dst)[C::NL]) {
       int t = tile < t_hi ? tile : t_hi - 1;
       int row = t * 16 + r;
       if (row > N - 1) row = N - 1;
       const unsigned char* p = reinterpret_cast<const unsigned char*>(w) + (uint32_t)row * row_bytes;
 #pragma unroll
-      for (int ld = 0; ld < C::NL; ++ld)
-#ifdef EAGLE_DBG_NT
-        dst[ld] = __builtin_nontemporal_load(reinterpret_cast<const uint4_t*>(p + woff[ld]));
-#else
-        dst[ld] = *reinterpret_cast<const uint4_t*>(p + woff[ld]);
-#endif
+      for (int ld = 0; ld < C::NL; ++ld) dst[ld] = *reinterpret_cast<const uint4_t*>(p + o[ld]);
     };
 
-    // ---- scale / bias staging: this thread's units of a batch
+    // ---- scale / bias staging: this thread's units of a batch (16*B rows x nw units x 2 arrays)
     const int nthr_s = nw * 64;
-    int su_row[C::NSU], su_g[C::NSU], su_lds[C::NSU];
+    int su_row[C::NSU], su_c[C::NSU], su_lds[C::NSU];
     const half_t* su_arr[C::NSU];
+    const float inv_nw = 1.0f / (float)nw;
 #pragma unroll
     for (int k = 0; k < C::NSU; ++k) {
-      const int u = tid + k * nthr_s;
-      const int per_arr = 16 * B * nw;
-      const int a = u / per_arr;
-      const int rem = u - a * per_arr;
-      const int row = rem / nw;
+      // NT == 1: two units per thread, unit k of array k.  NT == 2: one unit, array = upper half.
+      const int a = NT == 1 ? k : (tid >= 32 * nw ? 1 : 0);
+      const int rem = NT == 1 ? tid : tid - a * 32 * nw;
+      int row = (int)(((float)rem + 0.5f) * inv_nw);
+      if (row * nw > rem) --row;
+      if ((row + 1) * nw <= rem) ++row;
       const int c = rem - row * nw;
       su_row[k] = row;
-      int g = (slab * nw + c) * GW;
-      if (!SLOWSB && g > G - GW) g = G - GW;
-      su_g[k] = g;
+      su_c[k] = c;
       su_arr[k] = a ? b : s;
       su_lds[k] = ((a * 16 * B + row) * 16 + (c ^ (row & 15))) * C::UNIT;
     }
-    uint2_t su_val[C::NSU];
-    auto stage_load = [&](int tile0) {
+    // Staged values travel in registers from the load to the LDS store.  The vmcnt counter
+    // retires loads in order, so waiting for a staged value also waits for every weight load
+    // issued before it: the staging load must be at least as old as the ring slot consumed
+    // at the time of the store.  With two batches per super-step (NT == 2) that takes a
+    // lookahead of two batches and two register sets.
+    constexpr int NSET = NT == 2 ? 2 : 1;
+    uint2_t su_vals[NSET][C::NSU];
+    auto stage_load = [&](int tile0, int ph, uint2_t (&su_val)[C::NSU]) {
 #pragma unroll
       for (int k = 0; k < C::NSU; ++k) {
         int row = tile0 * 16 + su_row[k];
         if (row > N - 1) row = N - 1;
         const half_t* p = su_arr[k] + (size_t)row * G;
+        int g0 = ((slab * phases + ph) * nw + su_c[k]) * GW;
         if (SLOWSB) {
           half_t v[4];
 #pragma unroll
           for (int e = 0; e < GW; ++e) {
-            int g = su_g[k] + e;
+            int g = g0 + e;
             if (g > G - 1) g = G - 1;
             v[e] = p[g];
           }
@@ -221,14 +230,14 @@ __global__ __launch_bounds__(1024) void qmm_w4g64_kernel(
             half2_t hi = {v[2], v[3]};
             su_val[k][1] = as_u32(hi);
           }
-        } else if (GW == 4) {
-          su_val[k] = *reinterpret_cast<const uint2_t*>(p + su_g[k]);
         } else {
-          su_val[k][0] = *reinterpret_cast<const uint32_t*>(p + su_g[k]);
+          if (g0 > G - GW) g0 = G - GW;
+          if (GW == 4) su_val[k] = *reinterpret_cast<const uint2_t*>(p + g0);
+          else su_val[k][0] = *reinterpret_cast<const uint32_t*>(p + g0);
         }
       }
     };
-    auto stage_store = [&](int buf) {
+    auto stage_store = [&](int buf, const uint2_t (&su_val)[C::NSU]) {
 #pragma unroll
       for (int k = 0; k < C::NSU; ++k) {
         unsigned char* q = sbuf + buf * C::SB_BUF + su_lds[k];
@@ -237,202 +246,234 @@ __global__ __launch_bounds__(1024) void qmm_w4g64_kernel(
       }
     };
 
-    // ---- prologue: scales/biases of batch 0, this wave's unit of x, first four tiles
-    stage_load(t_lo);
-
+    // ---- x side: this wave's unit of x as MFMA operands, and the operand of the bias /
+    // offset MFMA: K block 0 carries the group sums of x (high and low fp16 parts), K block 1
+    // carries -(16 * even sum + odd sum); the other two blocks are zero.
     half8_t xop[NT][C::NMF];
-    float sE[NT][GW], sO[NT][GW];
-#pragma unroll
-    for (int t = 0; t < NT; ++t)
-#pragma unroll
-      for (int g = 0; g < GW; ++g) sE[t][g] = sO[t][g] = 0.f;
-    const int hperm = ((h & 1) << 2) | (h & 2);          // 0, 4, 2, 6
-#pragma unroll
-    for (int t = 0; t < NT; ++t) {
-#pragma unroll
-      for (int j = 0; j < C::NMF; ++j) {
-        const int wi = 16 * (j >> 2) + 8 * ((j >> 1) & 1) + (j & 1) + hperm;
-        const int col = col0 + 8 * wi;
-        const int m = 16 * t + r;
-        uint4_t u = uint4_t{0u, 0u, 0u, 0u};
-        if (m < M && col < K) u = *reinterpret_cast<const uint4_t*>(x + (size_t)m * K + col);
-        uint4_t o;
-        o[0] = __builtin_amdgcn_perm(u[2], u[0], 0x05040100u);   // (x0, x4)
-        o[1] = __builtin_amdgcn_perm(u[2], u[0], 0x07060302u);   // (x1, x5)
-        o[2] = __builtin_amdgcn_perm(u[3], u[1], 0x05040100u);   // (x2, x6)
-        o[3] = __builtin_amdgcn_perm(u[3], u[1], 0x07060302u);   // (x3, x7)
-        xop[t][j] = __builtin_bit_cast(half8_t, o);
-        const half2_t e0 = as_h2(o[0]), o0 = as_h2(o[1]), e1 = as_h2(o[2]), o1 = as_h2(o[3]);
-        sE[t][j >> 1] += ((float)e0[0] + (float)e0[1]) + ((float)e1[0] + (float)e1[1]);
-        sO[t][j >> 1] += ((float)o0[0] + (float)o0[1]) + ((float)o1[0] + (float)o1[1]);
-      }
-    }
-    uint4_t ring[C::RING][C::NL];
-#pragma unroll
-    for (int p = 0; p < C::RING; ++p) load_w(t_lo + p, ring[p]);
-    TSTAMP(1);
-
-    // x-side operand of the bias / offset MFMA: K block 0 carries the group sums of x
-    // (high and low fp16 parts), K block 1 carries -(16 * even sum + odd sum); the other
-    // two blocks are zero.
     half8_t xaux[NT];
+    const int hperm = ((h & 1) << 2) | (h & 2);          // 0, 4, 2, 6
+    auto load_x = [&](int unit) {
+      const int col0 = unit * C::CW;
+      float sE[NT][GW], sO[NT][GW];
 #pragma unroll
-    for (int t = 0; t < NT; ++t) {
-      half8_t a;
+      for (int t = 0; t < NT; ++t)
 #pragma unroll
-      for (int e = 0; e < 8; ++e) a[e] = (half_t)0.f;
+        for (int g = 0; g < GW; ++g) sE[t][g] = sO[t][g] = 0.f;
 #pragma unroll
-      for (int g = 0; g < GW; ++g) {
-        float se = sE[t][g], so = sO[t][g];
-        se += __shfl_xor(se, 16, 64);
-        se += __shfl_xor(se, 32, 64);
-        so += __shfl_xor(so, 16, 64);
-        so += __shfl_xor(so, 32, 64);
-        const float v = h == 0 ? se + so : -(16.f * se + so);
-        const half_t hi = (half_t)v;
-        const half_t lo = (half_t)(v - (float)hi);
-        a[g] = h < 2 ? hi : (half_t)0.f;
-        a[4 + g] = h < 2 ? lo : (half_t)0.f;
+      for (int t = 0; t < NT; ++t) {
+#pragma unroll
+        for (int j = 0; j < C::NMF; ++j) {
+          const int wi = 16 * (j >> 2) + 8 * ((j >> 1) & 1) + (j & 1) + hperm;
+          const int col = col0 + 8 * wi;
+          const int m = 16 * t + r;
+          uint4_t u = uint4_t{0u, 0u, 0u, 0u};
+          if (m < M && col < K) u = *reinterpret_cast<const uint4_t*>(x + (size_t)m * K + col);
+          uint4_t o;
+          o[0] = __builtin_amdgcn_perm(u[2], u[0], 0x05040100u);   // (x0, x4)
+          o[1] = __builtin_amdgcn_perm(u[2], u[0], 0x07060302u);   // (x1, x5)
+          o[2] = __builtin_amdgcn_perm(u[3], u[1], 0x05040100u);   // (x2, x6)
+          o[3] = __builtin_amdgcn_perm(u[3], u[1], 0x07060302u);   // (x3, x7)
+          xop[t][j] = __builtin_bit_cast(half8_t, o);
+          const half2_t e0 = as_h2(o[0]), o0 = as_h2(o[1]), e1 = as_h2(o[2]), o1 = as_h2(o[3]);
+          sE[t][j >> 1] += ((float)e0[0] + (float)e0[1]) + ((float)e1[0] + (float)e1[1]);
+          sO[t][j >> 1] += ((float)o0[0] + (float)o0[1]) + ((float)o1[0] + (float)o1[1]);
+        }
       }
-      xaux[t] = a;
-    }
+#pragma unroll
+      for (int t = 0; t < NT; ++t) {
+        half8_t a;
+#pragma unroll
+        for (int e = 0; e < 8; ++e) a[e] = (half_t)0.f;
+#pragma unroll
+        for (int g = 0; g < GW; ++g) {
+          float se = sE[t][g], so = sO[t][g];
+          se += __shfl_xor(se, 16, 64);
+          se += __shfl_xor(se, 32, 64);
+          so += __shfl_xor(so, 16, 64);
+          so += __shfl_xor(so, 32, 64);
+          const float v = h == 0 ? se + so : -(16.f * se + so);
+          const half_t hi = (half_t)v;
+          const half_t lo = (half_t)(v - (float)hi);
+          a[g] = h < 2 ? hi : (half_t)0.f;
+          a[4 + g] = h < 2 ? lo : (half_t)0.f;
+        }
+        xaux[t] = a;
+      }
+    };
     const half2_t kmul = h == 0 ? half2_t{(half_t)1.f, (half_t)1.f} : half2_t{(half_t)64.f, (half_t)64.f};
 
+    // ---- prologue: first tiles of the weight stream, batch 0 of scales / biases, x
+    uint32_t woff[C::NL];
+    unit_woff(unit0, woff);
+    stage_load(t_lo, 0, su_vals[0]);
+    if (NT == 2) stage_load(t_lo + B < t_hi ? t_lo + B : t_lo, 0, su_vals[NSET - 1]);
+    uint4_t ring[C::RING][C::NL];
+#pragma unroll
+    for (int p = 0; p < C::RING; ++p) load_w(t_lo + p, woff, ring[p]);
+    TSTAMP(1);
+    load_x(unit0);
     TSTAMP(2);
-    stage_store(0);
-    __syncthreads();
+    stage_store(0, su_vals[0]);
+    lds_barrier();
     TSTAMP(3);
 
-    // ---- main loop: super-steps of RING tiles, ring slots are compile-time indices
-    for (int ss = 0; ss < nss; ++ss) {
+    // One tile: bias / offset MFMA, then per quantisation group two MFMAs and the scale FMAs.
+    auto tile_compute = [&](const uint4_t (&wq)[C::NL], int sbuf_idx, int pbuf_idx, int j) {
+      const unsigned char* sp = sbuf + sbuf_idx * C::SB_BUF + (((j * 16 + r) * 16) + (wave ^ r)) * C::UNIT;
+      uint2_t sv, bv;
+      if (GW == 4) {
+        sv = *reinterpret_cast<const uint2_t*>(sp);
+        bv = *reinterpret_cast<const uint2_t*>(sp + C::SB_ARRAY);
+      } else {
+        sv[0] = *reinterpret_cast<const uint32_t*>(sp);
+        bv[0] = *reinterpret_cast<const uint32_t*>(sp + C::SB_ARRAY);
+        sv[1] = sv[0];
+        bv[1] = bv[0];
+      }
+      // weight-side operand of the bias / offset MFMA: biases in K block 0, 64 * scales in
+      // K block 1 (blocks 2 and 3 meet zeros)
+      uint4_t aux;
+      {
+        const half2_t s0 = as_h2(sv[0]) * kmul, s1 = as_h2(sv[1]) * kmul;
+        const uint32_t q0 = h == 0 ? bv[0] : as_u32(s0);
+        const uint32_t q1 = h == 0 ? bv[1] : as_u32(s1);
+        aux[0] = q0; aux[1] = q1; aux[2] = q0; aux[3] = q1;
+      }
+      float4_t acc[NT];
+#pragma unroll
+      for (int t = 0; t < NT; ++t)
+        acc[t] = __builtin_amdgcn_mfma_f32_16x16x32_f16(
+            xaux[t], __builtin_bit_cast(half8_t, aux), float4_t{0.f, 0.f, 0.f, 0.f}, 0, 0, 0);
+#pragma unroll
+      for (int ld = 0; ld < C::NL; ++ld) {
+        uint32_t q[4] = {wq[ld][0], wq[ld][1], wq[ld][2], wq[ld][3]};
+        swap32(q[0], q[2]);
+        swap32(q[1], q[3]);
+#pragma unroll
+        for (int gl = 0; gl < 2; ++gl) {
+          const int g = 2 * ld + gl;
+          float4_t tt[NT];
+#pragma unroll
+          for (int t = 0; t < NT; ++t) tt[t] = float4_t{0.f, 0.f, 0.f, 0.f};
+#pragma unroll
+          for (int pp = 0; pp < 2; ++pp) {
+            const half8_t wop = expand8(q[2 * gl + pp], magic_lo, magic_hi);
+#pragma unroll
+            for (int t = 0; t < NT; ++t)
+              tt[t] = __builtin_amdgcn_mfma_f32_16x16x32_f16(xop[t][4 * ld + 2 * gl + pp], wop,
+                                                             tt[t], 0, 0, 0);
+          }
+          const half_t sg = as_h2(sv[g >> 1])[g & 1];
+#pragma unroll
+          for (int t = 0; t < NT; ++t)
+#pragma unroll
+            for (int i = 0; i < 4; ++i) acc[t][i] = __builtin_fmaf((float)sg, tt[t][i], acc[t][i]);
+        }
+      }
+#pragma unroll
+      for (int t = 0; t < NT; ++t)
+        pbuf4[(pbuf_idx * nw + wave) * 256 + (j * NT + t) * 64 + lane] = acc[t];
+    };
+
+    // ---- main loop over super-steps of RING tiles (ring slots are compile-time indices) and
+    // phases.  Every load of the loop is unconditional: targets beyond the work are
+    // redirected to addresses that are already cached.
+    const int nvs = phases * nss;
+    int ph = 0, ss = 0;
+    for (int vs = 0; vs < nvs; ++vs) {
+      const bool last_ss = ss == nss - 1;
+      const bool more_phases = ph + 1 < phases;
+      if (ss == 0 && ph > 0) load_x(unit0 + ph * nw);
+      if (last_ss && more_phases) unit_woff(unit0 + (ph + 1) * nw, woff);   // reloads now target the next phase
       const int tb = t_lo + C::RING * ss;
+      const int nbase = last_ss ? (more_phases ? t_lo : t_hi) : tb + C::RING;
 #pragma unroll
       for (int p = 0; p < C::RING; ++p) {
         const int j = p % B;                       // tile inside its batch
-        const int bi = ss * (C::RING / B) + p / B; // batch index
-        const int buf = bi & 1;
-#ifndef EAGLE_DBG_PURE
-        if (j == 0) stage_load(tb + p + B);        // next batch's scales and biases
-#endif
-        const int tile = tb + p;
-        if (tile < t_hi) {
-          // this tile's scales and biases: row j*16 + r, column (wave ^ r)
-          const unsigned char* sp = sbuf + buf * C::SB_BUF + (((j * 16 + r) * 16) + (wave ^ r)) * C::UNIT;
-          uint2_t sv, bv;
-          if (GW == 4) {
-            sv = *reinterpret_cast<const uint2_t*>(sp);
-            bv = *reinterpret_cast<const uint2_t*>(sp + C::SB_ARRAY);
-          } else {
-            sv[0] = *reinterpret_cast<const uint32_t*>(sp);
-            bv[0] = *reinterpret_cast<const uint32_t*>(sp + C::SB_ARRAY);
-            sv[1] = sv[0];
-            bv[1] = bv[0];
+        const int bq = p / B;
+        const int buf = (vs * C::BPS + bq) & 1;    // batch parity over all phases
+        if (j == 0) {
+          // scales and biases of a later batch: the next one (NT == 1) or the same batch of
+          // the next super-step (NT == 2)
+          int n_tile0 = NT == 1 ? tb + p + B : tb + C::RING + p, n_ph = ph;
+          if ((NT == 2 || bq == C::BPS - 1) && last_ss) {
+            n_tile0 = NT == 1 ? t_lo : t_lo + p;
+            n_ph = ph + 1;
           }
-          // weight-side operand of the bias / offset MFMA: biases in K block 0, 64 * scales
-          // in K block 1 (blocks 2 and 3 meet zeros)
-          uint4_t aux;
-          {
-            const half2_t s0 = as_h2(sv[0]) * kmul, s1 = as_h2(sv[1]) * kmul;
-            const uint32_t q0 = h == 0 ? bv[0] : as_u32(s0);
-            const uint32_t q1 = h == 0 ? bv[1] : as_u32(s1);
-            aux[0] = q0; aux[1] = q1; aux[2] = q0; aux[3] = q1;
+          if (n_ph >= phases || n_tile0 >= t_hi) {   // no such batch: fetch the current one again
+            n_tile0 = tb + p;
+            n_ph = ph;
           }
-          float4_t acc[NT];
-#pragma unroll
-          for (int t = 0; t < NT; ++t)
-            acc[t] = __builtin_amdgcn_mfma_f32_16x16x32_f16(
-                xaux[t], __builtin_bit_cast(half8_t, aux), float4_t{0.f, 0.f, 0.f, 0.f}, 0, 0, 0);
-#ifndef EAGLE_DBG_NOCOMP
-#pragma unroll
-          for (int ld = 0; ld < C::NL; ++ld) {
-            uint32_t q[4] = {ring[p][ld][0], ring[p][ld][1], ring[p][ld][2], ring[p][ld][3]};
-            swap32(q[0], q[2]);
-            swap32(q[1], q[3]);
-#pragma unroll
-            for (int gl = 0; gl < 2; ++gl) {
-              const int g = 2 * ld + gl;
-              float4_t tt[NT];
-#pragma unroll
-              for (int t = 0; t < NT; ++t) tt[t] = float4_t{0.f, 0.f, 0.f, 0.f};
-#pragma unroll
-              for (int pp = 0; pp < 2; ++pp) {
-                const half8_t wop = expand8(q[2 * gl + pp], magic_lo, magic_hi);
-#pragma unroll
-                for (int t = 0; t < NT; ++t)
-                  tt[t] = __builtin_amdgcn_mfma_f32_16x16x32_f16(xop[t][4 * ld + 2 * gl + pp], wop,
-                                                                 tt[t], 0, 0, 0);
-              }
-              const half_t sg = as_h2(sv[g >> 1])[g & 1];
-#pragma unroll
-              for (int t = 0; t < NT; ++t)
-#pragma unroll
-                for (int i = 0; i < 4; ++i) acc[t][i] = __builtin_fmaf((float)sg, tt[t][i], acc[t][i]);
-            }
-          }
-#else
-#pragma unroll
-          for (int ld = 0; ld < C::NL; ++ld) acc[0][0] += __builtin_bit_cast(float, ring[p][ld][0] ^ ring[p][ld][3]);
-#endif
-#pragma unroll
-          for (int t = 0; t < NT; ++t)
-            pbuf4[(buf * nw + wave) * 256 + (j * NT + t) * 64 + lane] = acc[t];
-          if (ss == 0 && p == 0) TSTAMP(4);
+          stage_load(n_tile0, n_ph, su_vals[NT == 2 ? bq : 0]);
         }
-#ifndef EAGLE_DBG_NOW
-        load_w(tb + p + C::RING, ring[p]);
-#endif
+        if (tb + p < t_hi) tile_compute(ring[p], buf, buf, j);
+        if (vs == 0 && p == 0) TSTAMP(4);
+        load_w(nbase + p, woff, ring[p]);
         if (j == B - 1) {
-#ifndef EAGLE_DBG_PURE
-          stage_store(buf ^ 1);
+          stage_store(buf ^ 1, su_vals[NT == 2 ? (bq ^ 1) : 0]);
           lds_barrier();
-#endif
         }
+      }
+      if (++ss == nss) {
+        ss = 0;
+        ++ph;
       }
     }
     TSTAMP(5);
   } else {
     // ------------------------------------------------------------------ reducing wave
     const int wl = tid - nw * 64;     // 0 .. 127
-    __syncthreads();
-    const int nb = nss * (C::RING / B);
-    for (int bi = 0; bi < nb; ++bi) {
-#ifndef EAGLE_DBG_PURE
-      lds_barrier();
-#endif
-      const int buf = bi & 1;
-      const int tile0 = t_lo + bi * B;
+    lds_barrier();
+    for (int ph = 0; ph < phases; ++ph) {
+      for (int bi = 0; bi < nbp; ++bi) {
+        lds_barrier();
+        const int buf = (ph * nbp + bi) & 1;
+        const int tile0 = t_lo + bi * B;
 #pragma unroll
-      for (int it = 0; it < 2; ++it) {
-        const int l4 = wl + it * 128;            // 0 .. 255
-        const int jt = l4 >> 6;
-        const int j = jt / NT, t = jt % NT;
-        const int tile = tile0 + j;
-        if (tile >= t_hi) continue;
-        float4_t sum = pbuf4[(buf * nw) * 256 + l4];
-#ifndef EAGLE_DBG_NORED
-        for (int wv = 1; wv < nw; ++wv) sum += pbuf4[(buf * nw + wv) * 256 + l4];
-#endif
-        const int ln = l4 & 63;
-        const int n = tile * 16 + (ln & 15);
-        const int m0 = 16 * t + 4 * (ln >> 4);
-        if (to_out) {
-          if (n < N) {
-            half_t bn = (half_t)0.f;
-            if (bias) bn = bias[n];
+        for (int it = 0; it < 2; ++it) {
+          const int l4 = wl + it * 128;            // 0 .. 255
+          const int jt = l4 >> 6;
+          const int j = jt / NT, t = jt % NT;
+          const int tile = tile0 + j;
+          if (tile >= t_hi) continue;
+          // all partials are fetched before the first add; waves beyond nw re-read the last one
+          float4_t v[MAX_STREAM_WAVES];
+#pragma unroll
+          for (int wv = 0; wv < MAX_STREAM_WAVES; ++wv)
+            v[wv] = pbuf4[(buf * nw + (wv < nw ? wv : nw - 1)) * 256 + l4];
+          float4_t sum = v[0];
+#pragma unroll
+          for (int wv = 1; wv < MAX_STREAM_WAVES; ++wv)
+            if (wv < nw) sum += v[wv];
+          if (phases > 1) {
+            if (ph > 0) sum += accl4[bi * 256 + l4];
+            if (ph + 1 < phases) {
+              accl4[bi * 256 + l4] = sum;
+              continue;
+            }
+          }
+          const int ln = l4 & 63;
+          const int n = tile * 16 + (ln & 15);
+          const int m0 = 16 * t + 4 * (ln >> 4);
+          if (to_out) {
+            if (n < N) {
+              half_t bn = (half_t)0.f;
+              if (bias) bn = bias[n];
+#pragma unroll
+              for (int i = 0; i < 4; ++i)
+                if (m0 + i < M) {
+                  half_t o = (half_t)sum[i];
+                  if (bias) o = o + bn;
+                  out[(size_t)(m0 + i) * N + n] = o;
+                }
+            }
+          } else {
+            // partial[slab][tile][t][i][64]
+            float* dst = partial + ((((size_t)slab * tiles_total + tile) * NT + t) * 4) * 64 + ln;
 #pragma unroll
             for (int i = 0; i < 4; ++i)
-              if (m0 + i < M) {
-                half_t o = (half_t)sum[i];
-                if (bias) o = o + bn;
-                out[(size_t)(m0 + i) * N + n] = o;
-              }
+              __hip_atomic_store(dst + i * 64, sum[i], __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
           }
-        } else {
-          // partial[slab][tile][t][i][64]
-          float* dst = partial + ((((size_t)slab * tiles_total + tile) * NT + t) * 4) * 64 + ln;
-#pragma unroll
-          for (int i = 0; i < 4; ++i)
-            __hip_atomic_store(dst + i * 64, sum[i], __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
         }
       }
     }
@@ -465,8 +506,17 @@ __global__ __launch_bounds__(1024) void qmm_w4g64_kernel(
         const int t = ti >> 2, i = ti & 3;
         const float* src = partial + (size_t)tile * per_tile + rem;
         float v = 0.f;
-        for (int sp = 0; sp < nsplit; ++sp)
-          v += __hip_atomic_load(src + sp * slab_stride, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+        for (int sp0 = 0; sp0 < nsplit; sp0 += 8) {       // eight loads in flight, added in slab order
+          float pv[8];
+#pragma unroll
+          for (int k = 0; k < 8; ++k) {
+            const int sp = sp0 + k < nsplit ? sp0 + k : nsplit - 1;
+            pv[k] = __hip_atomic_load(src + sp * slab_stride, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+          }
+#pragma unroll
+          for (int k = 0; k < 8; ++k)
+            if (sp0 + k < nsplit) v += pv[k];
+        }
         const int n = tile * 16 + (ln & 15);
         const int m = 16 * t + 4 * (ln >> 4) + i;
         if (n < N && m < M) {
@@ -485,44 +535,66 @@ __global__ __launch_bounds__(1024) void qmm_w4g64_kernel(
 // ------------------------------------------------------------------------------------------
 inline int nt_of(int M) { return M <= 16 ? 1 : 2; }
 inline int cw_of(int M) { return M <= 16 ? 256 : 128; }
+constexpr int MAX_PHASES = 8;
 
-int lds_bytes(int M, const Launch& L) {
+int lds_bytes(int M, int N, const Launch& L) {
   const int sb = M <= 16 ? 2 * Cfg<1, 4>::SB_BUF : 2 * Cfg<2, 2>::SB_BUF;
-  return pbuf_bytes(L.nw) + sb;
+  int acc = 0;
+  if (L.phases > 1) {
+    const int tiles = (N + 15) / 16;
+    const int per_range = (tiles + L.ranges - 1) / L.ranges;
+    acc = (per_range + 3) / 4 * 4 * nt_of(M) * 1024;        // fp32 16 x M per tile, whole super-steps
+  }
+  return pbuf_bytes(L.nw) + sb + acc;
 }
 
 int validate_launch(int M, int N, int K, const Launch& L) {
-  if (L.nw < 1 || L.nw > MAX_STREAM_WAVES || L.splits < 1 || L.splits > MAX_SPLITS)
+  if (L.nw < 1 || L.nw > MAX_STREAM_WAVES || L.splits < 1 || L.splits > MAX_SPLITS ||
+      L.phases < 1 || L.phases > MAX_PHASES)
     return EAGLE_ERR_SHAPE;
   const int units = (K + cw_of(M) - 1) / cw_of(M);
-  if ((long)L.nw * L.splits < units || (long)L.nw * (L.splits - 1) >= units) return EAGLE_ERR_SHAPE;
+  const long per_slab = (long)L.nw * L.phases;
+  if (per_slab * L.splits < units || per_slab * (L.splits - 1) >= units) return EAGLE_ERR_SHAPE;
   const int tiles = (N + 15) / 16;
   if (L.ranges < 1 || L.ranges > tiles || L.ranges > MAX_RANGES) return EAGLE_ERR_SHAPE;
-  if (lds_bytes(M, L) > LDS_MAX) return EAGLE_ERR_SHAPE;
+  if (lds_bytes(M, N, L) > LDS_MAX) return EAGLE_ERR_SHAPE;
   return EAGLE_OK;
 }
 
-size_t partial_bytes(int M, int N, const Launch& L) {
-  if (L.splits <= 1) return 0;
+size_t partial_bytes(int M, int N, int splits) {
+  if (splits <= 1) return 0;
   const size_t tiles = (N + 15) / 16;
-  return (size_t)L.splits * tiles * nt_of(M) * 256 * sizeof(float);
+  return (size_t)splits * tiles * nt_of(M) * 256 * sizeof(float);
 }
 
-// Launch shape: as few K slabs as 14 streaming waves allow, the units spread evenly over the
-// slabs, and about one workgroup per compute unit (two when a workgroup is at most 8 waves).
+// Launch shape.  A workgroup covers nw * phases column units; K slabs beyond that cost a
+// round trip of fp32 partials, so there are only as many as 14 waves x 2 phases force, or as
+// it takes to give every compute unit a workgroup when there are few row tiles.  Tile ranges:
+// about one workgroup per compute unit, more when the per-range accumulators of a
+// multi-phase launch would not fit LDS.
 void choose(int M, int N, int K, Launch* out) {
   const int units = (K + cw_of(M) - 1) / cw_of(M);
   const int tiles = (N + 15) / 16;
   Launch L;
-  L.splits = (units + MAX_STREAM_WAVES - 1) / MAX_STREAM_WAVES;
-  L.nw = (units + L.splits - 1) / L.splits;
-  L.splits = (units + L.nw - 1) / L.nw;
-  const int wg_per_cu = (L.nw + NWR) <= 8 && 2 * lds_bytes(M, L) <= LDS_MAX ? 2 : 1;
-  int ranges = (NUM_CU * wg_per_cu) / L.splits;
+  int splits = (units + 2 * MAX_STREAM_WAVES - 1) / (2 * MAX_STREAM_WAVES);
+  int fill = tiles >= 160 ? 1 : (NUM_CU + tiles - 1) / tiles;
+  if (fill > 4) fill = 4;
+  if (splits < fill) splits = fill;
+  if (splits > units) splits = units;
+  int per_slab = (units + splits - 1) / splits;
+  L.phases = (per_slab + MAX_STREAM_WAVES - 1) / MAX_STREAM_WAVES;
+  L.nw = (per_slab + L.phases - 1) / L.phases;
+  per_slab = L.nw * L.phases;
+  L.splits = (units + per_slab - 1) / per_slab;
+  int ranges = NUM_CU / L.splits;
   if (ranges < 1) ranges = 1;
   if (ranges > tiles) ranges = tiles;
   if (ranges > MAX_RANGES) ranges = MAX_RANGES;
   L.ranges = ranges;
+  while (lds_bytes(M, N, L) > LDS_MAX && L.ranges < tiles && L.ranges < MAX_RANGES) {
+    L.ranges += NUM_CU / L.splits > 0 ? NUM_CU / L.splits : 1;
+    if (L.ranges > tiles) L.ranges = tiles;
+  }
   *out = L;
 }
 
@@ -530,7 +602,7 @@ template <int NT, int GW, bool SLOWSB>
 int launch(const void* x, const uint32_t* wq, const void* s, const void* b, const void* bias,
            void* out, float* partial, unsigned* counters, int M, int N, int K, const Launch& L,
            hipStream_t stream) {
-  const int lds = lds_bytes(M, L);
+  const int lds = lds_bytes(M, N, L);
   static bool attr_set = false;   // more than 64 KB of LDS needs an explicit opt-in, once
   if (lds > 65536 && !attr_set) {
     if (hipFuncSetAttribute(reinterpret_cast<const void*>(&qmm_w4g64_kernel<NT, GW, SLOWSB>),
@@ -538,10 +610,11 @@ int launch(const void* x, const uint32_t* wq, const void* s, const void* b, cons
       return EAGLE_ERR_HIP;
     attr_set = true;
   }
+  const int tiles = (N + 15) / 16;
   hipLaunchKernelGGL((qmm_w4g64_kernel<NT, GW, SLOWSB>), dim3(L.ranges, L.splits),
                      dim3(64 * (L.nw + NWR)), lds, stream, (const half_t*)x, wq,
                      (const half_t*)s, (const half_t*)b, (const half_t*)bias, (half_t*)out,
-                     partial, counters, M, N, K, L.nw);
+                     partial, counters, M, N, K, L.nw, L.phases, tiles / L.ranges, tiles % L.ranges);
   return eagle_launch_status();
 }
 
@@ -550,7 +623,7 @@ int validate(const void* x, const uint32_t* wq, const void* s, const void* b, co
   if (!x || !wq || !s || !b || !out) return EAGLE_ERR_NULL;
   if (M < 1 || M > EAGLE_MAX_M || N < 8 || (N % 8) != 0 || K < 64 || (K % 64) != 0)
     return EAGLE_ERR_SHAPE;
-  if ((long)K > (long)cw_of(M) * MAX_STREAM_WAVES * MAX_SPLITS) return EAGLE_ERR_SHAPE;
+  if ((long)K > (long)cw_of(M) * MAX_STREAM_WAVES * 2 * MAX_SPLITS) return EAGLE_ERR_SHAPE;
   if ((long)N * (K / 2) >= (1L << 32)) return EAGLE_ERR_SHAPE;   // 32-bit byte offsets
   if (!eagle_aligned16(x) || !eagle_aligned16(wq) || !eagle_aligned16(out) ||
       (reinterpret_cast<uintptr_t>(s) & 1u) || (reinterpret_cast<uintptr_t>(b) & 1u) ||
@@ -566,7 +639,7 @@ int run(const void* x, const uint32_t* wq, const void* scales, const void* biase
   unsigned* counters = nullptr;
   if (L.splits > 1) {
     if (!workspace || !eagle_aligned16(workspace) ||
-        workspace_bytes < (size_t)EAGLE_QMM_COUNTER_BYTES + partial_bytes(M, N, L))
+        workspace_bytes < (size_t)EAGLE_QMM_COUNTER_BYTES + partial_bytes(M, N, L.splits))
       return EAGLE_ERR_WORKSPACE;
     counters = reinterpret_cast<unsigned*>(workspace);
     partial = reinterpret_cast<float*>(static_cast<unsigned char*>(workspace) +
@@ -591,32 +664,31 @@ EAGLE_EXPORT size_t eagle_qmm_workspace_bytes(int M, int N, int K) {
   if (M < 1 || M > EAGLE_MAX_M || N < 1 || K < 64) return 0;
   Launch L;
   choose(M, N, K, &L);
-  return (size_t)EAGLE_QMM_COUNTER_BYTES + partial_bytes(M, N, L);
+  return (size_t)EAGLE_QMM_COUNTER_BYTES + partial_bytes(M, N, L.splits);
 }
 
 EAGLE_EXPORT size_t eagle_qmm_workspace_bytes_tuned(int M, int N, int splits) {
   if (M < 1 || M > EAGLE_MAX_M || N < 1 || splits < 1) return 0;
-  Launch L{1, splits, 1};
-  return (size_t)EAGLE_QMM_COUNTER_BYTES + partial_bytes(M, N, L);
+  return (size_t)EAGLE_QMM_COUNTER_BYTES + partial_bytes(M, N, splits);
 }
 
-EAGLE_EXPORT int eagle_qmm_plan(int M, int N, int K, int* plan3) {
-  if (!plan3) return EAGLE_ERR_NULL;
+EAGLE_EXPORT int eagle_qmm_plan(int M, int N, int K, int* plan4) {
+  if (!plan4) return EAGLE_ERR_NULL;
   if (M < 1 || M > EAGLE_MAX_M || N < 8 || K < 64 || (K % 64) != 0) return EAGLE_ERR_SHAPE;
   Launch L;
   choose(M, N, K, &L);
-  plan3[0] = L.nw; plan3[1] = L.splits; plan3[2] = L.ranges;
+  plan4[0] = L.nw; plan4[1] = L.phases; plan4[2] = L.splits; plan4[3] = L.ranges;
   return EAGLE_OK;
 }
 
 EAGLE_EXPORT int eagle_qmm_w4g64_f16_tuned(const void* x, const uint32_t* wq, const void* scales,
                                            const void* biases, const void* bias, void* out, int M,
-                                           int N, int K, int nw, int splits, int ranges,
+                                           int N, int K, int nw, int phases, int splits, int ranges,
                                            void* workspace, size_t workspace_bytes,
                                            eagle_stream_t stream) {
   int rc = validate(x, wq, scales, biases, bias, out, M, N, K);
   if (rc != EAGLE_OK) return rc;
-  Launch L{nw, splits, ranges};
+  Launch L{nw, phases, splits, ranges};
   rc = validate_launch(M, N, K, L);
   if (rc != EAGLE_OK) return rc;
   return run(x, wq, scales, biases, bias, out, M, N, K, L, workspace, workspace_bytes,

@@ -10,16 +10,24 @@ from util import TOL, layer_to_dev, rel_err, to_dev
 pytestmark = pytest.mark.gpu
 
 
-def shape_for(M, N, K, nw, ranges):
-    """A forced launch shape: `nw` streaming waves per workgroup (the K slabs follow from it)
-    and `ranges` workgroups per slab; None if it cannot be launched."""
+def shape_for(M, N, K, nw, phases, ranges):
+    """A forced launch shape: `nw` streaming waves per workgroup, each owning `phases` column
+    units in turn (the K slabs follow from both), `ranges` workgroups per slab; None if it
+    cannot be launched."""
     cw = 256 if M <= 16 else 128
+    nt = 1 if M <= 16 else 2
     units = -(-K // cw)
-    splits = -(-units // nw)
+    per_slab = nw * phases
+    splits = -(-units // per_slab)
     tiles = -(-N // 16)
-    if nw > 14 or nw * (splits - 1) >= units or ranges > tiles or splits > 64:
+    if nw > 14 or phases > 8 or per_slab * (splits - 1) >= units or ranges > tiles or splits > 64:
         return None
-    return (nw, splits, ranges)
+    lds = 2 * nw * 4096 + (32768 if nt == 1 else 8192)
+    if phases > 1:
+        lds += -(-(-(-tiles // ranges)) // 4) * 4 * nt * 1024
+    if lds > 160 * 1024:
+        return None
+    return (nw, phases, splits, ranges)
 
 
 def run_case(dev, M, N, K, seed=0, bias=False, tuned=None):
@@ -42,16 +50,17 @@ def test_cfg1_shape_all_m(dev, M):
     run_case(dev, M, 8192, 2048, seed=42)
 
 
-@pytest.mark.parametrize("nw", [1, 2, 3, 5, 7, 13, 14])
+@pytest.mark.parametrize("nw,phases", [(1, 1), (2, 1), (3, 2), (5, 3), (7, 1), (7, 2), (13, 1), (14, 1), (14, 2),
+                                       (2, 7), (4, 8)])
 @pytest.mark.parametrize("ranges", [1, 7, 96])
 @pytest.mark.parametrize("M", [8, 32])
-def test_forced_launch_shapes(dev, nw, ranges, M):
+def test_forced_launch_shapes(dev, nw, phases, ranges, M):
     N, K = 1536, 3584
-    tuned = shape_for(M, N, K, nw, ranges)
+    tuned = shape_for(M, N, K, nw, phases, ranges)
     if tuned is None:
         pytest.skip("shape cannot be launched")
     print(f"qmm tuned={tuned} M={M}", flush=True)
-    run_case(dev, M, N, K, seed=nw * 100 + ranges, tuned=tuned)
+    run_case(dev, M, N, K, seed=nw * 100 + ranges + phases, tuned=tuned)
 
 
 @pytest.mark.parametrize("N,K", [(8, 64), (8, 128), (24, 192), (40, 896), (136, 2944), (512, 3584),
@@ -60,7 +69,7 @@ def test_edge_shapes(dev, N, K):
     for M in (1, 5, 32):
         print(f"qmm edge N={N} K={K} M={M}", flush=True)
         run_case(dev, M, N, K, seed=N + K + M)
-        for cfg in ((1, 1), (3, 2), (14, 3)):
+        for cfg in ((1, 1, 1), (3, 2, 2), (14, 1, 3), (2, 3, 1)):
             tuned = shape_for(M, N, K, *cfg)
             if tuned is not None:
                 run_case(dev, M, N, K, seed=N + K + M, tuned=tuned)
@@ -100,8 +109,8 @@ def test_deterministic_split_k(dev):
     layer = synth.make_qlinear(rng, 512, 3584)
     x = to_dev(synth.make_x(rng, 32, 3584), dev)
     d = layer_to_dev(layer, dev)
-    tuned = shape_for(32, 512, 3584, 4, 5)
-    assert tuned[1] == 7
+    tuned = shape_for(32, 512, 3584, 2, 2, 5)
+    assert tuned[2] == 7
     ref = ops.quantized_matmul(x, d["weight"], d["scales"], d["biases"], tuned=tuned)
     for _ in range(5):
         again = ops.quantized_matmul(x, d["weight"], d["scales"], d["biases"], tuned=tuned)
@@ -113,9 +122,9 @@ def test_plan_covers_benchmark_shapes(dev):
         for N, K in ((3584, 3584), (512, 3584), (18944, 3584), (3584, 18944), (152064, 3584),
                      (8192, 2048), (896, 896), (128, 896), (4864, 896), (896, 4864),
                      (4096, 4096), (1024, 4096), (14336, 4096), (4096, 14336), (128256, 4096)):
-            nw, splits, ranges = ops.qmm_plan(M, N, K)
+            nw, phases, splits, ranges = ops.qmm_plan(M, N, K)
             cw = 256 if M <= 16 else 128
-            assert nw * splits * cw >= K > nw * (splits - 1) * cw
+            assert nw * phases * splits * cw >= K > nw * phases * (splits - 1) * cw
             assert 1 <= nw <= 14 and 1 <= ranges <= -(-N // 16)
 
 

@@ -49,12 +49,12 @@ def test_qmm_argument_errors_are_detected_on_the_host():
     assert call(x=None) == 1                       # EAGLE_ERR_NULL
     assert call(out=None) == 1
     assert call(M=0) == 2 and call(M=33) == 2      # EAGLE_ERR_SHAPE
-    assert call(K=100) == 2 and call(N=12) == 2 and call(K=256 * 1024) == 2
+    assert call(K=100) == 2 and call(N=12) == 2 and call(K=1024 * 1024) == 2
     assert call(x=p + 2) == 3                      # EAGLE_ERR_ALIGN
     assert call(gs=32) == 4 and call(bits=8) == 4  # EAGLE_ERR_UNSUPPORTED
     # a K-split launch needs a workspace
-    assert L.eagle_qmm_w4g64_f16(p, p, p, p, None, p, 32, 3584, 3584, 64, 4, None, 0, None) == 5
-    assert L.eagle_qmm_workspace_bytes(32, 3584, 3584) > 65536
+    assert L.eagle_qmm_w4g64_f16(p, p, p, p, None, p, 32, 512, 3584, 64, 4, None, 0, None) == 5
+    assert L.eagle_qmm_workspace_bytes(32, 512, 3584) > 65536
     assert L.eagle_qmm_workspace_bytes(8, 152064, 3584) == 65536
 
 
@@ -86,11 +86,11 @@ def test_plan_is_consistent_for_benchmark_shapes():
         for N, K in ((3584, 3584), (512, 3584), (18944, 3584), (3584, 18944), (152064, 3584),
                      (8192, 2048), (896, 896), (128, 896), (4864, 896), (896, 4864), (151936, 896),
                      (4096, 4096), (1024, 4096), (14336, 4096), (4096, 14336), (128256, 4096)):
-            nw, splits, ranges = ops.qmm_plan(M, N, K)
+            nw, phases, splits, ranges = ops.qmm_plan(M, N, K)
             cw = 256 if M <= 16 else 128
-            assert nw * splits * cw >= K > nw * (splits - 1) * cw
-            assert 1 <= nw <= 14 and 1 <= ranges <= -(-N // 16)
-            assert ranges * splits <= 512
+            assert nw * phases * splits * cw >= K > nw * phases * (splits - 1) * cw
+            assert 1 <= nw <= 14 and 1 <= phases <= 2 and 1 <= ranges <= -(-N // 16)
+            assert ranges * splits <= 1024
 
 
 def test_ops_refuse_cpu_tensors():
