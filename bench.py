@@ -157,27 +157,19 @@ def main():
     gpu_logits = ver.logits.cpu().numpy().copy()
 
     # ---- dominant kernel: the QMM launches of one step, replayed alone ----
-    per_layer, head = qmm_shapes(args)
-    launches = []
-    for i, layer in enumerate(model.layers):
-        at, mlp = layer.self_attn, layer.mlp
-        for lin, x, out in ((at.q_proj, ver.hn, ver.q), (at.k_proj, ver.hn, ver.k), (at.v_proj, ver.hn, ver.v),
-                            (at.o_proj, ver.attn, ver.o), (mlp.gate_proj, ver.hn, ver.gate),
-                            (mlp.up_proj, ver.hn, ver.up), (mlp.down_proj, ver.act, ver.down)):
-            launches.append((lin, x, out))
-    launches.append((model.lm_head, ver.hn, ver.logits))
+    launches = ver.qmm_launches()
     ver.hn.normal_()
     ver.attn.normal_()
     ver.act.normal_()
 
     def qmm_only():
-        for lin, x, out in launches:
-            ops.quantized_matmul(x, lin.weight, lin.scales, lin.biases, bias=lin.bias, out=out)
+        for wq, sc, bi, bias, x, out in launches:
+            ops.quantized_matmul(x, wq, sc, bi, bias=bias, out=out)
 
     qt, _ = graph_time_ms(torch, qmm_only, reps=10)
     qmm_ms = float(np.median(qt))
     n_launch = len(launches)
-    alg = sum(qmm_bytes(NODES, n, k) for _, n, k in per_layer) * L + qmm_bytes(NODES, head[1], head[2])
+    alg = sum(qmm_bytes(NODES, wq.shape[0], wq.shape[1] * 8) for wq, *_ in launches)
     kv_bytes = 2 * L * G * (PREFIX + NODES) * hd * 2
     achieved = alg / (qmm_ms * 1e-3) / 1e9
     traffic = QMM_TRAFFIC_BYTES_PER_LAUNCH

@@ -96,13 +96,15 @@ int eagle_rope_arrayed_f16(const void* x, const int32_t* positions, const float*
 /* Fused form used inside the decoder layer: takes the token-major projections
  * q_lin [T,H*hd], k_lin [T,G*hd], v_lin [T,G*hd], rotates q and k at
  * positions[t] and writes q_out [H,T,hd] plus rows *cache_len_dev + t of the
- * K/V caches ([G,capacity,hd]).  Covers mlx_llama.py:134-161 and the cache
- * append of :178. */
+ * K/V caches ([G,capacity,hd]).  row_stride = 0: the three inputs are packed as
+ * above; row_stride > 0: all three are column blocks of one [T,row_stride] matrix
+ * (a fused q|k|v projection) and consecutive tokens are row_stride elements apart.
+ * Covers mlx_llama.py:134-161 and the cache append of :178. */
 int eagle_rope_kv_append_f16(const void* q_lin, const void* k_lin, const void* v_lin,
                              const int32_t* positions, const float* inv_freqs,
                              float scaling_factor, void* q_out, void* k_cache, void* v_cache,
                              const int32_t* cache_len_dev, int T, int H, int G, int hd,
-                             long capacity, eagle_stream_t stream);
+                             long capacity, long row_stride, eagle_stream_t stream);
 
 /* ---------------------------------------------------------------------------
  * Tree-masked grouped-query attention of T <= 32 tree tokens against the cache.

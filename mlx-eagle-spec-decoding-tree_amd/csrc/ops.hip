@@ -83,7 +83,7 @@ __global__ void rope_kv_append_kernel(const half_t* __restrict__ q_lin,
                                       half_t* __restrict__ q_out, half_t* __restrict__ k_cache,
                                       half_t* __restrict__ v_cache,
                                       const int32_t* __restrict__ len_dev, int T, int H, int G,
-                                      int hd, long cap) {
+                                      int hd, long cap, long ld_q, long ld_kv) {
   const int half = hd >> 1;
   const int per_row = half >> 3;
   const int heads = H + 2 * G;
@@ -98,7 +98,7 @@ __global__ void rope_kv_append_kernel(const half_t* __restrict__ q_lin,
   if (hh < H + G) {
     const bool is_q = hh < H;
     const int head = is_q ? hh : hh - H;
-    const half_t* src = is_q ? q_lin + ((long)t * H + head) * hd : k_lin + ((long)t * G + head) * hd;
+    const half_t* src = is_q ? q_lin + t * ld_q + (long)head * hd : k_lin + t * ld_kv + (long)head * hd;
     half_t* dst = is_q ? q_out + ((long)head * T + t) * hd : k_cache + ((long)head * cap + P + t) * hd;
     const half8_t lo = *reinterpret_cast<const half8_t*>(src + c * 8);
     const half8_t hi = *reinterpret_cast<const half8_t*>(src + half + c * 8);
@@ -108,7 +108,7 @@ __global__ void rope_kv_append_kernel(const half_t* __restrict__ q_lin,
     *reinterpret_cast<half8_t*>(dst + half + c * 8) = ohi;
   } else {
     const int head = hh - H - G;
-    const half_t* src = v_lin + ((long)t * G + head) * hd;
+    const half_t* src = v_lin + t * ld_kv + (long)head * hd;
     half_t* dst = v_cache + ((long)head * cap + P + t) * hd;
     *reinterpret_cast<half8_t*>(dst + c * 8) = *reinterpret_cast<const half8_t*>(src + c * 8);
     *reinterpret_cast<half8_t*>(dst + half + c * 8) =
@@ -316,13 +316,14 @@ EAGLE_EXPORT int eagle_rope_kv_append_f16(const void* q_lin, const void* k_lin, 
                                           const int32_t* positions, const float* inv_freqs,
                                           float scaling_factor, void* q_out, void* k_cache,
                                           void* v_cache, const int32_t* cache_len_dev, int T,
-                                          int H, int G, int hd, long capacity,
+                                          int H, int G, int hd, long capacity, long row_stride,
                                           eagle_stream_t stream) {
   if (!q_lin || !k_lin || !v_lin || !positions || !inv_freqs || !q_out || !k_cache || !v_cache ||
       !cache_len_dev)
     return EAGLE_ERR_NULL;
   if (T < 1 || T > EAGLE_MAX_TREE || H < 1 || G < 1 || (H % G) != 0 || hd < 16 || (hd % 16) != 0 ||
-      capacity < T)
+      capacity < T || row_stride < 0 || (row_stride % 8) != 0 ||
+      (row_stride > 0 && row_stride < (long)H * hd))
     return EAGLE_ERR_SHAPE;
   if (!eagle_aligned16(q_lin) || !eagle_aligned16(k_lin) || !eagle_aligned16(v_lin) ||
       !eagle_aligned16(q_out) || !eagle_aligned16(k_cache) || !eagle_aligned16(v_cache))
@@ -331,7 +332,8 @@ EAGLE_EXPORT int eagle_rope_kv_append_f16(const void* q_lin, const void* k_lin, 
   hipLaunchKernelGGL(rope_kv_append_kernel, dim3(blocks_for(total, 256)), dim3(256), 0,
                      static_cast<hipStream_t>(stream), (const half_t*)q_lin, (const half_t*)k_lin,
                      (const half_t*)v_lin, positions, inv_freqs, scaling_factor, (half_t*)q_out,
-                     (half_t*)k_cache, (half_t*)v_cache, cache_len_dev, T, H, G, hd, capacity);
+                     (half_t*)k_cache, (half_t*)v_cache, cache_len_dev, T, H, G, hd, capacity,
+                     row_stride ? row_stride : (long)H * hd, row_stride ? row_stride : (long)G * hd);
   return eagle_launch_status();
 }
 

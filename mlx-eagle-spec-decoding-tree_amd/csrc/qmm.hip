@@ -40,16 +40,6 @@
 //    write-back / invalidate fence, which costs microseconds on a multi-XCD part.
 #include "common.h"
 
-#ifdef EAGLE_DBG_TIMES
-__device__ unsigned long long eagle_dbg_times[1024 * 16];
-#define TSTAMP(k) do { if (lane == 0 && (wave == 0 || wave == nw)) eagle_dbg_times[blockIdx.x * 16 + (k)] = wall_clock64(); } while (0)
-EAGLE_EXPORT int eagle_dbg_read_times(unsigned long long* host) {
-  return hipMemcpyFromSymbol(host, HIP_SYMBOL(eagle_dbg_times), sizeof(eagle_dbg_times)) == hipSuccess ? 0 : 6;
-}
-#else
-#define TSTAMP(k) do { } while (0)
-#endif
-
 namespace {
 
 constexpr int MAX_STREAM_WAVES = 14;   // + 2 reducing waves = 1024 threads
@@ -158,7 +148,6 @@ __global__ __launch_bounds__(1024) void qmm_w4g64_kernel(
   const int nbp = nss * C::BPS;                             // batches per phase
   const bool to_out = nsplit == 1;
 
-  TSTAMP(0);
   if (wave < nw) {
     // ------------------------------------------------------------------ streaming wave
     const uint32_t magic_lo = 0x64006400u, magic_hi = 0x54005400u;
@@ -207,7 +196,7 @@ __global__ __launch_bounds__(1024) void qmm_w4g64_kernel(
     // issued before it: the staging load must be at least as old as the ring slot consumed
     // at the time of the store.  With two batches per super-step (NT == 2) that takes a
     // lookahead of two batches and two register sets.
-    constexpr int NSET = NT == 2 ? 2 : 1;
+    constexpr int NSET = NT == 2 ? C::BPS : 1;
     uint2_t su_vals[NSET][C::NSU];
     auto stage_load = [&](int tile0, int ph, uint2_t (&su_val)[C::NSU]) {
 #pragma unroll
@@ -306,16 +295,16 @@ __global__ __launch_bounds__(1024) void qmm_w4g64_kernel(
     uint32_t woff[C::NL];
     unit_woff(unit0, woff);
     stage_load(t_lo, 0, su_vals[0]);
-    if (NT == 2) stage_load(t_lo + B < t_hi ? t_lo + B : t_lo, 0, su_vals[NSET - 1]);
+    if (NT == 2) {
+#pragma unroll
+      for (int q = 1; q < NSET; ++q) stage_load(t_lo + q * B < t_hi ? t_lo + q * B : t_lo, 0, su_vals[q]);
+    }
     uint4_t ring[C::RING][C::NL];
 #pragma unroll
     for (int p = 0; p < C::RING; ++p) load_w(t_lo + p, woff, ring[p]);
-    TSTAMP(1);
     load_x(unit0);
-    TSTAMP(2);
     stage_store(0, su_vals[0]);
     lds_barrier();
-    TSTAMP(3);
 
     // One tile: bias / offset MFMA, then per quantisation group two MFMAs and the scale FMAs.
     auto tile_compute = [&](const uint4_t (&wq)[C::NL], int sbuf_idx, int pbuf_idx, int j) {
@@ -407,10 +396,9 @@ __global__ __launch_bounds__(1024) void qmm_w4g64_kernel(
           stage_load(n_tile0, n_ph, su_vals[NT == 2 ? bq : 0]);
         }
         if (tb + p < t_hi) tile_compute(ring[p], buf, buf, j);
-        if (vs == 0 && p == 0) TSTAMP(4);
         load_w(nbase + p, woff, ring[p]);
         if (j == B - 1) {
-          stage_store(buf ^ 1, su_vals[NT == 2 ? (bq ^ 1) : 0]);
+          stage_store(buf ^ 1, su_vals[NT == 2 ? (bq + 1) % C::BPS : 0]);
           lds_barrier();
         }
       }
@@ -419,7 +407,6 @@ __global__ __launch_bounds__(1024) void qmm_w4g64_kernel(
         ++ph;
       }
     }
-    TSTAMP(5);
   } else {
     // ------------------------------------------------------------------ reducing wave
     const int wl = tid - nw * 64;     // 0 .. 127
@@ -479,7 +466,6 @@ __global__ __launch_bounds__(1024) void qmm_w4g64_kernel(
     }
   }
 
-  TSTAMP(wave == 0 ? 6 : 9);
   if (nsplit > 1) {
     // ---- the last workgroup of this tile range to arrive adds the slabs, in slab order
     int* flag = reinterpret_cast<int*>(lds);
@@ -493,7 +479,6 @@ __global__ __launch_bounds__(1024) void qmm_w4g64_kernel(
         __hip_atomic_store(&counters[blockIdx.x], 0u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
     }
     __syncthreads();
-    TSTAMP(wave == 0 ? 7 : 10);
     if (*flag) {
       const int per_tile = NT * 256;                       // floats
       const int total = (t_hi - t_lo) * per_tile;
@@ -527,7 +512,6 @@ __global__ __launch_bounds__(1024) void qmm_w4g64_kernel(
       }
     }
   }
-  TSTAMP(wave == 0 ? 8 : 11);
 }
 
 // ------------------------------------------------------------------------------------------

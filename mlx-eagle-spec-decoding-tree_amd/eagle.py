@@ -170,7 +170,7 @@ class TreeVerifier:
     accept_indices...) and `accepted_tokens`; the cache length advances on the device.
     Same kernels and operator order as Model.__call__ + the host functions above."""
 
-    def __init__(self, model, cache, total_tokens=31, max_len=None, compact=True):
+    def __init__(self, model, cache, total_tokens=31, max_len=None, compact=True, fuse=True):
         args = model.args
         self.model, self.cache, self.args = model, cache, args
         self.V = total_tokens
@@ -182,6 +182,9 @@ class TreeVerifier:
         self.capacity = cache[0].capacity
         self.max_len = max_len or self.capacity
         self.compact = compact
+        self.fuse = fuse
+        if fuse:
+            self._fuse_projections()
         i32 = dict(dtype=torch.int32, device=dev)
         f16 = dict(dtype=torch.float16, device=dev)
         self.tokens = torch.zeros(T, **i32)
@@ -196,12 +199,15 @@ class TreeVerifier:
         self.accepted_tokens = torch.zeros(MAXT, **i32)
         self.h = torch.empty((T, D), **f16)
         self.hn = torch.empty((T, D), **f16)
+        # q | k | v of a token side by side: one fused projection writes all three
+        self.qkv = torch.empty((T, (H + 2 * G) * hd), **f16)
         self.q = torch.empty((T, H * hd), **f16)
         self.k = torch.empty((T, G * hd), **f16)
         self.v = torch.empty((T, G * hd), **f16)
         self.q_rot = torch.empty((H, T, hd), **f16)
         self.attn = torch.empty((T, H * hd), **f16)
         self.o = torch.empty((T, D), **f16)
+        self.gate_up = torch.empty((T, 2 * I), **f16)        # gate | up of a token side by side
         self.gate = torch.empty((T, I), **f16)
         self.up = torch.empty((T, I), **f16)
         self.act = torch.empty((T, I), **f16)
@@ -216,10 +222,62 @@ class TreeVerifier:
         L = _lib.lib()
         head = model.lm_head if not args.tie_word_embeddings else model.model.embed_tokens
         need = max(L.eagle_qmm_workspace_bytes(T, n, k) for n, k in
-                   ((H * hd, D), (G * hd, D), (D, H * hd), (I, D), (D, I), (head.weight.shape[0], D)))
+                   ((H * hd, D), (G * hd, D), ((H + 2 * G) * hd, D), (D, H * hd), (I, D), (2 * I, D),
+                    (D, I), (head.weight.shape[0], D)))
         ops.workspace("qmm", need, dev)
         ops.workspace("attn", L.eagle_tree_attention_workspace_bytes(H, hd, self.max_len), dev)
         ops.workspace("argmax", L.eagle_argmax_workspace_bytes(T, args.vocab_size), dev)
+
+    def _fuse_projections(self):
+        """Lay q/k/v and gate/up of every layer out as one matrix each (rows concatenated) and
+        re-point the layers' tensors at row blocks of it, so that one matmul launch serves
+        the three (two) projections; memory use is unchanged."""
+        self.qkv_w, self.gu_w = [], []
+
+        def fuse(lins):
+            parts = [[l.weight, l.scales, l.biases] for l in lins]
+            fused = [torch.cat([p[k] for p in parts], dim=0).contiguous() for k in range(3)]
+            bias = None
+            if any(l.bias is not None for l in lins):
+                bias = torch.cat([l.bias if l.bias is not None
+                                  else torch.zeros(l.weight.shape[0], dtype=torch.float16,
+                                                   device=l.weight.device) for l in lins]).contiguous()
+            row = 0
+            for l in lins:
+                n = l.weight.shape[0]
+                l.weight, l.scales, l.biases = (f[row:row + n] for f in fused)
+                if l.bias is not None:
+                    l.bias = bias[row:row + n]
+                row += n
+            return (*fused, bias)
+
+        for layer in self.model.model.layers:
+            at, mlp = layer.self_attn, layer.mlp
+            self.qkv_w.append(fuse([at.q_proj, at.k_proj, at.v_proj]))
+            self.gu_w.append(fuse([mlp.gate_proj, mlp.up_proj]))
+
+    def qmm_launches(self):
+        """(weight, scales, biases, bias, x, out) of every quantised matmul of one step, in order."""
+        m = self.model
+        out = []
+        for i, layer in enumerate(m.model.layers):
+            at, mlp = layer.self_attn, layer.mlp
+            if self.fuse:
+                out.append((*self.qkv_w[i], self.hn, self.qkv))
+            else:
+                for lin, o in ((at.q_proj, self.q), (at.k_proj, self.k), (at.v_proj, self.v)):
+                    out.append((lin.weight, lin.scales, lin.biases, lin.bias, self.hn, o))
+            out.append((at.o_proj.weight, at.o_proj.scales, at.o_proj.biases, at.o_proj.bias, self.attn, self.o))
+            if self.fuse:
+                out.append((*self.gu_w[i], self.hn, self.gate_up))
+            else:
+                for lin, o in ((mlp.gate_proj, self.gate), (mlp.up_proj, self.up)):
+                    out.append((lin.weight, lin.scales, lin.biases, lin.bias, self.hn, o))
+            out.append((mlp.down_proj.weight, mlp.down_proj.scales, mlp.down_proj.biases,
+                        mlp.down_proj.bias, self.act, self.down))
+        head = m.model.embed_tokens if self.args.tie_word_embeddings else m.lm_head
+        out.append((head.weight, head.scales, head.biases, None, self.hn, self.logits))
+        return out
 
     def set_tree(self, tokens, tree_position_ids, mask_index, mask_bits):
         self.tokens.copy_(tokens.reshape(-1))
@@ -245,12 +303,20 @@ class TreeVerifier:
         ops.rms_norm(self.h, layers[0].input_layernorm.weight, args.rms_norm_eps, out=self.hn)
         for i, layer in enumerate(layers):
             at = layer.self_attn
-            for lin, out in ((at.q_proj, self.q), (at.k_proj, self.k), (at.v_proj, self.v)):
-                ops.quantized_matmul(self.hn, lin.weight, lin.scales, lin.biases, bias=lin.bias, out=out)
             c = self.cache[i]
-            ops.rope_kv_append(self.q, self.k, self.v, self.positions, at._inv_freqs,
-                               at._scaling_factor, self.q_rot, c.keys[0], c.values[0],
-                               self.len_dev, H, G, hd)
+            if self.fuse:
+                w, sc, bi, b = self.qkv_w[i]
+                ops.quantized_matmul(self.hn, w, sc, bi, bias=b, out=self.qkv)
+                ops.rope_kv_append(self.qkv, self.qkv[:, H * hd:], self.qkv[:, (H + G) * hd:],
+                                   self.positions, at._inv_freqs, at._scaling_factor, self.q_rot,
+                                   c.keys[0], c.values[0], self.len_dev, H, G, hd,
+                                   row_stride=(H + 2 * G) * hd)
+            else:
+                for lin, out in ((at.q_proj, self.q), (at.k_proj, self.k), (at.v_proj, self.v)):
+                    ops.quantized_matmul(self.hn, lin.weight, lin.scales, lin.biases, bias=lin.bias, out=out)
+                ops.rope_kv_append(self.q, self.k, self.v, self.positions, at._inv_freqs,
+                                   at._scaling_factor, self.q_rot, c.keys[0], c.values[0],
+                                   self.len_dev, H, G, hd)
             ops.tree_attention(self.q_rot, c.keys[0], c.values[0], self.mask_bits, self.len_dev,
                                at.scale, max_len=self.max_len, out=self.attn)
             ops.quantized_matmul(self.attn, at.o_proj.weight, at.o_proj.scales, at.o_proj.biases,
@@ -258,11 +324,16 @@ class TreeVerifier:
             ops.rms_norm(self.o, layer.post_attention_layernorm.weight, args.rms_norm_eps,
                          residual=self.h, out=self.hn, h_out=self.h)
             mlp = layer.mlp
-            ops.quantized_matmul(self.hn, mlp.gate_proj.weight, mlp.gate_proj.scales,
-                                 mlp.gate_proj.biases, bias=mlp.gate_proj.bias, out=self.gate)
-            ops.quantized_matmul(self.hn, mlp.up_proj.weight, mlp.up_proj.scales,
-                                 mlp.up_proj.biases, bias=mlp.up_proj.bias, out=self.up)
-            ops.silu_mul(self.gate, self.up, out=self.act)
+            if self.fuse:
+                w, sc, bi, b = self.gu_w[i]
+                ops.quantized_matmul(self.hn, w, sc, bi, bias=b, out=self.gate_up)
+                ops.silu_mul(self.gate_up, None, out=self.act)
+            else:
+                ops.quantized_matmul(self.hn, mlp.gate_proj.weight, mlp.gate_proj.scales,
+                                     mlp.gate_proj.biases, bias=mlp.gate_proj.bias, out=self.gate)
+                ops.quantized_matmul(self.hn, mlp.up_proj.weight, mlp.up_proj.scales,
+                                     mlp.up_proj.biases, bias=mlp.up_proj.bias, out=self.up)
+                ops.silu_mul(self.gate, self.up, out=self.act)
             ops.quantized_matmul(self.act, mlp.down_proj.weight, mlp.down_proj.scales,
                                  mlp.down_proj.biases, bias=mlp.down_proj.bias, out=self.down)
             nxt = layers[i + 1].input_layernorm.weight if i + 1 < len(layers) else m.model.norm.weight

@@ -64,7 +64,8 @@ def test_other_entry_points_reject_bad_arguments():
     p = (ctypes.addressof(buf) + 15) & ~15
     assert L.eagle_rope_arrayed_f16(None, p, p, 1.0, p, 1, 1, 1, 64, None) == 1
     assert L.eagle_rope_arrayed_f16(p, p, p, 1.0, p, 1, 1, 1, 63, None) == 2
-    assert L.eagle_rope_kv_append_f16(p, p, p, p, p, 1.0, p, p, p, p, 33, 4, 2, 64, 100, None) == 2
+    assert L.eagle_rope_kv_append_f16(p, p, p, p, p, 1.0, p, p, p, p, 33, 4, 2, 64, 100, 0, None) == 2
+    assert L.eagle_rope_kv_append_f16(p, p, p, p, p, 1.0, p, p, p, p, 8, 4, 2, 64, 100, 100, None) == 2
     assert L.eagle_tree_attention_f16(p, p, p, p, p, p, 32, 28, 4, 96, 4096, 2080, 0.1, p, 1 << 30, None) == 2
     assert L.eagle_tree_attention_f16(p, p, p, p, p, p, 32, 28, 4, 128, 4096, 2080, 0.1, None, 0, None) == 5
     assert L.eagle_rmsnorm_f16(p, None, p, 1e-6, None, p, 4, 100, None) == 2
