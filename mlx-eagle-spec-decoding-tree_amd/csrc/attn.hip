@@ -51,9 +51,6 @@ __global__ __launch_bounds__(512) void tree_attn_split_kernel(
   const int P = *len_dev;
   const int Ltot = P + T;
   const int ntiles = (Ltot + KT - 1) / KT;
-  const int t0 = split * tiles_per_split;
-  const int t1 = min(t0 + tiles_per_split, ntiles);
-
   half8_t qreg[KSTEPS];
 #pragma unroll
   for (int kk = 0; kk < KSTEPS; ++kk) {
@@ -73,22 +70,47 @@ __global__ __launch_bounds__(512) void tree_attn_split_kernel(
   const half_t* kbase_ptr = kc + (long)g * cap * HD;
   const half_t* vbase_ptr = vc + (long)g * cap * HD;
 
-  for (int tile = t0; tile < t1; ++tile) {
+  // This workgroup's tiles are split, split + nsplit, ...: all workgroups share the live part
+  // of the cache however short it is.  The next tile is fetched into registers while the
+  // current one is being used.
+  constexpr int NVEC = KT * VEC_ROW;                 // 16-byte vectors per K (or V) tile
+  constexpr int NV = NVEC / 64;                      // per thread, for as little as one wave
+  half8_t kreg[NV], vreg[NV];
+  auto fetch = [&](int tile) {
     const int kb = tile * KT;
-    __syncthreads();   // every wave is done with the previous tile
-    for (int v = tid; v < KT * VEC_ROW; v += nthr) {
+#pragma unroll
+    for (int it = 0; it < NV; ++it) {
+      if (it * nthr >= NVEC) break;
+      int v = tid + it * nthr;
+      if (v > NVEC - 1) v = NVEC - 1;
       const int row = v / VEC_ROW;
       const int c = v % VEC_ROW;
-      const int kidx = kb + row;
-      half8_t kv = half8_t{0, 0, 0, 0, 0, 0, 0, 0};
-      half8_t vv = kv;
-      if (kidx < Ltot) {
-        kv = *reinterpret_cast<const half8_t*>(kbase_ptr + (long)kidx * HD + c * 8);
-        vv = *reinterpret_cast<const half8_t*>(vbase_ptr + (long)kidx * HD + c * 8);
-      }
-      *reinterpret_cast<half8_t*>(ldsK + row * STR + c * 16) = kv;
-      *reinterpret_cast<half8_t*>(ldsV + row * STR + c * 16) = vv;
+      int kidx = kb + row;
+      if (kidx > Ltot - 1) kidx = Ltot - 1;          // rows past the end are masked out below
+      kreg[it] = *reinterpret_cast<const half8_t*>(kbase_ptr + (long)kidx * HD + c * 8);
+      vreg[it] = *reinterpret_cast<const half8_t*>(vbase_ptr + (long)kidx * HD + c * 8);
     }
+  };
+  auto stash = [&]() {
+#pragma unroll
+    for (int it = 0; it < NV; ++it) {
+      if (it * nthr >= NVEC) break;
+      const int v = tid + it * nthr;
+      if (v < NVEC) {
+        const int row = v / VEC_ROW;
+        const int c = v % VEC_ROW;
+        *reinterpret_cast<half8_t*>(ldsK + row * STR + c * 16) = kreg[it];
+        *reinterpret_cast<half8_t*>(ldsV + row * STR + c * 16) = vreg[it];
+      }
+    }
+  };
+
+  if (split < ntiles) fetch(split);
+  for (int tile = split; tile < ntiles; tile += nsplit) {
+    const int kb = tile * KT;
+    __syncthreads();   // every wave is done with the previous tile
+    stash();
+    if (tile + nsplit < ntiles) fetch(tile + nsplit);
     __syncthreads();
 
     // S^T[key][token] = sum_d K[key][d] Q[token][d]
@@ -176,48 +198,72 @@ __global__ __launch_bounds__(512) void tree_attn_split_kernel(
     }
 }
 
-// Merge the splits: grid (T, H), HD/2 threads... one thread per two output elements.
+// Merge the splits.  Grid (H, T / 4): a workgroup owns four tree tokens of one head; one
+// thread per four output elements.  The softmax weights of the splits are computed once per
+// token with one split per lane, then every thread adds its slice of the partial outputs.
+constexpr int MERGE_TOK = 4;
+
 template <int HD>
 __global__ void tree_attn_merge_kernel(const float* __restrict__ part_o,
                                        const float* __restrict__ part_ml,
                                        half_t* __restrict__ out, int T, int H, int nsplit) {
-  const int t = blockIdx.x;
-  const int head = blockIdx.y;
-  const int d = threadIdx.x * 2;
-  float mx = -INFINITY;
-  for (int s = 0; s < nsplit; ++s)
-    mx = fmaxf(mx, part_ml[(((long)head * nsplit + s) * 32 + t) * 2]);
-  float den = 0.f, a0 = 0.f, a1 = 0.f;
-  for (int s = 0; s < nsplit; ++s) {
-    const long slot = ((long)head * nsplit + s) * 32 + t;
-    const float m = part_ml[slot * 2];
-    if (m == -INFINITY) continue;
-    const float wgt = exp2f(m - mx);
-    den += wgt * part_ml[slot * 2 + 1];
-    a0 += wgt * part_o[slot * HD + d];
-    a1 += wgt * part_o[slot * HD + d + 1];
+  constexpr int QW = HD / 4;                       // threads per token
+  __shared__ float wts[MERGE_TOK][64];
+  const int head = blockIdx.x;
+  const int tid = threadIdx.x;
+  const int lane = tid & 63;
+  const int wave = tid >> 6;
+  const int nwave = blockDim.x >> 6;
+  for (int tl = wave; tl < MERGE_TOK; tl += nwave) {
+    const int t = blockIdx.y * MERGE_TOK + tl;
+    float m = -INFINITY, l = 0.f;
+    if (lane < nsplit && t < T) {
+      const long slot = ((long)head * nsplit + lane) * 32 + t;
+      m = part_ml[slot * 2];
+      l = part_ml[slot * 2 + 1];
+    }
+    const float mx = wave_max(m);
+    const float w = m == -INFINITY ? 0.f : exp2f(m - mx);
+    const float den = wave_sum(w * l);
+    wts[tl][lane] = den > 0.f ? w / den : 0.f;
   }
-  half2_t o = half2_t{(half_t)(a0 / den), (half_t)(a1 / den)};
-  *reinterpret_cast<half2_t*>(out + ((long)t * H + head) * HD + d) = o;
+  __syncthreads();
+  const int tl = tid / QW;
+  const int dq = tid % QW;
+  const int t = blockIdx.y * MERGE_TOK + tl;
+  if (t >= T) return;
+  float4_t acc = float4_t{0.f, 0.f, 0.f, 0.f};
+  const float* src = part_o + ((long)head * nsplit * 32 + t) * HD + dq * 4;
+  for (int s0 = 0; s0 < nsplit; s0 += 8) {
+    float4_t v[8];
+#pragma unroll
+    for (int k = 0; k < 8; ++k) {
+      const int sp = s0 + k < nsplit ? s0 + k : nsplit - 1;
+      v[k] = *reinterpret_cast<const float4_t*>(src + (long)sp * 32 * HD);
+    }
+#pragma unroll
+    for (int k = 0; k < 8; ++k)
+      if (s0 + k < nsplit) acc += wts[tl][s0 + k] * v[k];
+  }
+  half4_t o = half4_t{(half_t)acc[0], (half_t)acc[1], (half_t)acc[2], (half_t)acc[3]};
+  *reinterpret_cast<half4_t*>(out + ((long)t * H + head) * HD + dq * 4) = o;
 }
 
-int tiles_per_split_for(int max_len, int G) {
+// Key splits (gridDim.y): about one workgroup per compute unit, never more than tiles.
+int splits_for(int max_len, int G) {
   const int ntiles = (max_len + KT - 1) / KT;
-  int want_splits = 256 / (G > 0 ? G : 1);   // about one workgroup per compute unit
-  if (want_splits < 1) want_splits = 1;
-  int tps = (ntiles + want_splits - 1) / want_splits;
-  if (tps < 4) tps = 4;                      // keep the partial traffic below the KV traffic
-  return tps;
+  int n = 256 / (G > 0 ? G : 1);
+  if (n < 1) n = 1;
+  if (n > ntiles) n = ntiles;
+  if (n > 64) n = 64;                  // the merge holds one split per lane
+  return n;
 }
 
 }  // namespace
 
 EAGLE_EXPORT size_t eagle_tree_attention_workspace_bytes(int H, int hd, int max_len) {
   if (H < 1 || hd < 1 || max_len < 1) return 0;
-  // worst case split count: tiles_per_split >= 4
-  const int ntiles = (max_len + KT - 1) / KT;
-  const int nsplit = (ntiles + 3) / 4;
-  return (size_t)H * nsplit * 32 * (hd + 2) * sizeof(float);
+  return (size_t)H * 64 * 32 * (hd + 2) * sizeof(float);   // at most 64 key splits
 }
 
 EAGLE_EXPORT int eagle_tree_attention_f16(const void* q, const void* k_cache, const void* v_cache,
@@ -236,9 +282,8 @@ EAGLE_EXPORT int eagle_tree_attention_f16(const void* q, const void* k_cache, co
   if (!workspace || !eagle_aligned16(workspace) ||
       workspace_bytes < eagle_tree_attention_workspace_bytes(H, hd, max_len))
     return EAGLE_ERR_WORKSPACE;
-  const int tps = tiles_per_split_for(max_len, G);
-  const int ntiles = (max_len + KT - 1) / KT;
-  const int nsplit = (ntiles + tps - 1) / tps;
+  const int nsplit = splits_for(max_len, G);
+  const int tps = 0;
   float* part_ml = static_cast<float*>(workspace);
   float* part_o = part_ml + (size_t)H * nsplit * 32 * 2;
   const float sl2 = scale * 1.4426950408889634f;
@@ -249,14 +294,14 @@ EAGLE_EXPORT int eagle_tree_attention_f16(const void* q, const void* k_cache, co
     hipLaunchKernelGGL(tree_attn_split_kernel<128>, dim3(G, nsplit), dim3(rep * 64), lds, st,
                        (const half_t*)q, (const half_t*)k_cache, (const half_t*)v_cache,
                        tree_mask_bits, cache_len_dev, part_o, part_ml, T, H, G, capacity, tps, sl2);
-    hipLaunchKernelGGL(tree_attn_merge_kernel<128>, dim3(T, H), dim3(64), 0, st, part_o, part_ml,
-                       (half_t*)out, T, H, nsplit);
+    hipLaunchKernelGGL(tree_attn_merge_kernel<128>, dim3(H, (T + MERGE_TOK - 1) / MERGE_TOK),
+                       dim3(MERGE_TOK * 32), 0, st, part_o, part_ml, (half_t*)out, T, H, nsplit);
   } else {
     hipLaunchKernelGGL(tree_attn_split_kernel<64>, dim3(G, nsplit), dim3(rep * 64), lds, st,
                        (const half_t*)q, (const half_t*)k_cache, (const half_t*)v_cache,
                        tree_mask_bits, cache_len_dev, part_o, part_ml, T, H, G, capacity, tps, sl2);
-    hipLaunchKernelGGL(tree_attn_merge_kernel<64>, dim3(T, H), dim3(32), 0, st, part_o, part_ml,
-                       (half_t*)out, T, H, nsplit);
+    hipLaunchKernelGGL(tree_attn_merge_kernel<64>, dim3(H, (T + MERGE_TOK - 1) / MERGE_TOK),
+                       dim3(MERGE_TOK * 16), 0, st, part_o, part_ml, (half_t*)out, T, H, nsplit);
   }
   return eagle_launch_status();
 }
