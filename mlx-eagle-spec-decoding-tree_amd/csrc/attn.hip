@@ -26,7 +26,7 @@ template <int HD>
 __global__ __launch_bounds__(512) void tree_attn_split_kernel(
     const half_t* __restrict__ q, const half_t* __restrict__ kc, const half_t* __restrict__ vc,
     const uint32_t* __restrict__ mask_bits, const int32_t* __restrict__ len_dev,
-    float* __restrict__ part_o, float* __restrict__ part_ml, int T, int H, int G, long cap,
+    half_t* __restrict__ part_o, float* __restrict__ part_ml, int T, int H, int G, long cap,
     int tiles_per_split, float scale_log2e) {
   constexpr int KSTEPS = HD / 16;       // MFMA steps over the head dimension for S
   constexpr int DB = HD / 32;           // 32-wide blocks of the head dimension for O
@@ -186,15 +186,15 @@ __global__ __launch_bounds__(512) void tree_attn_split_kernel(
     part_ml[slot * 2 + 0] = m_run;
     part_ml[slot * 2 + 1] = l_run;
   }
-  float* po = part_o + slot * HD;
+  half_t* po = part_o + slot * HD;     // fp16: |O| <= keys per split, relative error 2^-11
 #pragma unroll
   for (int db = 0; db < DB; ++db)
 #pragma unroll
     for (int i4 = 0; i4 < 4; ++i4) {
       const int d0 = db * 32 + 8 * i4 + 4 * hb;
-      float4_t v = float4_t{o_acc[db][4 * i4 + 0], o_acc[db][4 * i4 + 1], o_acc[db][4 * i4 + 2],
-                            o_acc[db][4 * i4 + 3]};
-      *reinterpret_cast<float4_t*>(po + d0) = v;
+      half4_t v = half4_t{(half_t)o_acc[db][4 * i4 + 0], (half_t)o_acc[db][4 * i4 + 1],
+                          (half_t)o_acc[db][4 * i4 + 2], (half_t)o_acc[db][4 * i4 + 3]};
+      *reinterpret_cast<half4_t*>(po + d0) = v;
     }
 }
 
@@ -204,7 +204,7 @@ __global__ __launch_bounds__(512) void tree_attn_split_kernel(
 constexpr int MERGE_TOK = 4;
 
 template <int HD>
-__global__ void tree_attn_merge_kernel(const float* __restrict__ part_o,
+__global__ void tree_attn_merge_kernel(const half_t* __restrict__ part_o,
                                        const float* __restrict__ part_ml,
                                        half_t* __restrict__ out, int T, int H, int nsplit) {
   constexpr int QW = HD / 4;                       // threads per token
@@ -233,17 +233,21 @@ __global__ void tree_attn_merge_kernel(const float* __restrict__ part_o,
   const int t = blockIdx.y * MERGE_TOK + tl;
   if (t >= T) return;
   float4_t acc = float4_t{0.f, 0.f, 0.f, 0.f};
-  const float* src = part_o + ((long)head * nsplit * 32 + t) * HD + dq * 4;
+  const half_t* src = part_o + ((long)head * nsplit * 32 + t) * HD + dq * 4;
   for (int s0 = 0; s0 < nsplit; s0 += 8) {
-    float4_t v[8];
+    half4_t v[8];
 #pragma unroll
     for (int k = 0; k < 8; ++k) {
       const int sp = s0 + k < nsplit ? s0 + k : nsplit - 1;
-      v[k] = *reinterpret_cast<const float4_t*>(src + (long)sp * 32 * HD);
+      v[k] = *reinterpret_cast<const half4_t*>(src + (long)sp * 32 * HD);
     }
 #pragma unroll
     for (int k = 0; k < 8; ++k)
-      if (s0 + k < nsplit) acc += wts[tl][s0 + k] * v[k];
+      if (s0 + k < nsplit) {
+        const float wk = wts[tl][s0 + k];
+#pragma unroll
+        for (int e = 0; e < 4; ++e) acc[e] += wk * (float)v[k][e];
+      }
   }
   half4_t o = half4_t{(half_t)acc[0], (half_t)acc[1], (half_t)acc[2], (half_t)acc[3]};
   *reinterpret_cast<half4_t*>(out + ((long)t * H + head) * HD + dq * 4) = o;
@@ -255,7 +259,7 @@ int splits_for(int max_len, int G) {
   int n = 256 / (G > 0 ? G : 1);
   if (n < 1) n = 1;
   if (n > ntiles) n = ntiles;
-  if (n > 64) n = 64;                  // the merge holds one split per lane
+  if (n > 32) n = 32;                  // partial traffic grows with the split count
   return n;
 }
 
@@ -285,7 +289,7 @@ EAGLE_EXPORT int eagle_tree_attention_f16(const void* q, const void* k_cache, co
   const int nsplit = splits_for(max_len, G);
   const int tps = 0;
   float* part_ml = static_cast<float*>(workspace);
-  float* part_o = part_ml + (size_t)H * nsplit * 32 * 2;
+  half_t* part_o = reinterpret_cast<half_t*>(part_ml + (size_t)H * nsplit * 32 * 2);
   const float sl2 = scale * 1.4426950408889634f;
   const int rep = H / G;
   hipStream_t st = static_cast<hipStream_t>(stream);

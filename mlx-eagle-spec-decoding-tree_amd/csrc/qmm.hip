@@ -172,6 +172,14 @@ __global__ __launch_bounds__(1024) void qmm_w4g64_kernel(
       for (int ld = 0; ld < C::NL; ++ld) dst[ld] = *reinterpret_cast<const uint4_t*>(p + o[ld]);
     };
 
+    // The weight stream starts before anything else: the first tiles need several
+    // microseconds to arrive, and the rest of the prologue fits inside that wait.
+    uint32_t woff[C::NL];
+    unit_woff(unit0, woff);
+    uint4_t ring[C::RING][C::NL];
+#pragma unroll
+    for (int p = 0; p < C::RING; ++p) load_w(t_lo + p, woff, ring[p]);
+
     // ---- scale / bias staging: this thread's units of a batch (16*B rows x nw units x 2 arrays)
     const int nthr_s = nw * 64;
     int su_row[C::NSU], su_c[C::NSU], su_lds[C::NSU];
@@ -291,17 +299,12 @@ __global__ __launch_bounds__(1024) void qmm_w4g64_kernel(
     };
     const half2_t kmul = h == 0 ? half2_t{(half_t)1.f, (half_t)1.f} : half2_t{(half_t)64.f, (half_t)64.f};
 
-    // ---- prologue: first tiles of the weight stream, batch 0 of scales / biases, x
-    uint32_t woff[C::NL];
-    unit_woff(unit0, woff);
+    // ---- prologue: batch 0 of scales / biases, x
     stage_load(t_lo, 0, su_vals[0]);
     if (NT == 2) {
 #pragma unroll
       for (int q = 1; q < NSET; ++q) stage_load(t_lo + q * B < t_hi ? t_lo + q * B : t_lo, 0, su_vals[q]);
     }
-    uint4_t ring[C::RING][C::NL];
-#pragma unroll
-    for (int p = 0; p < C::RING; ++p) load_w(t_lo + p, woff, ring[p]);
     load_x(unit0);
     stage_store(0, su_vals[0]);
     lds_barrier();
@@ -564,6 +567,9 @@ void choose(int M, int N, int K, Launch* out) {
   int fill = tiles >= 160 ? 1 : (NUM_CU + tiles - 1) / tiles;
   if (fill > 4) fill = 4;
   if (splits < fill) splits = fill;
+  // With only a few tiles per workgroup a second phase is mostly start-up latency (new x, a
+  // cold ring); two K slabs on twice the workgroups finish sooner.
+  if (splits == 1 && units > MAX_STREAM_WAVES && tiles < 4 * NUM_CU) splits = 2;
   if (splits > units) splits = units;
   int per_slab = (units + splits - 1) / splits;
   L.phases = (per_slab + MAX_STREAM_WAVES - 1) / MAX_STREAM_WAVES;
