@@ -412,54 +412,81 @@ __global__ __launch_bounds__(1024) void qmm_w4g64_kernel(
     }
   } else {
     // ------------------------------------------------------------------ reducing wave
+    // A lane owns the same two float4 slots of every batch: slot l4 = (tile j of the batch,
+    // x block t, MFMA lane ln) holds out[16 t + 4 (ln / 16) + i][tile * 16 + ln % 16], i = 0..3.
     const int wl = tid - nw * 64;     // 0 .. 127
+    int sl_l4[2], sl_j[2];
+    half_t* sl_out[2];
+    float* sl_part[2];
+    int sl_rows[2];
+#pragma unroll
+    for (int it = 0; it < 2; ++it) {
+      const int l4 = wl + it * 128;            // 0 .. 255
+      const int jt = l4 >> 6;
+      const int t = jt % NT;
+      const int ln = l4 & 63;
+      const int m0 = 16 * t + 4 * (ln >> 4);
+      sl_l4[it] = l4;
+      sl_j[it] = jt / NT;
+      sl_out[it] = out + (size_t)m0 * N + (ln & 15);
+      sl_rows[it] = M - m0;                    // rows m0 .. m0+3 exist while i < sl_rows
+      // partial[slab][tile][t][i][64]
+      sl_part[it] = partial + (((size_t)slab * tiles_total * NT + t) * 4) * 64 + ln;
+    }
     lds_barrier();
     for (int ph = 0; ph < phases; ++ph) {
       for (int bi = 0; bi < nbp; ++bi) {
         lds_barrier();
         const int buf = (ph * nbp + bi) & 1;
         const int tile0 = t_lo + bi * B;
+        const float4_t* pb = pbuf4 + buf * nw * 256;
 #pragma unroll
         for (int it = 0; it < 2; ++it) {
-          const int l4 = wl + it * 128;            // 0 .. 255
-          const int jt = l4 >> 6;
-          const int j = jt / NT, t = jt % NT;
-          const int tile = tile0 + j;
+          const int tile = tile0 + sl_j[it];
           if (tile >= t_hi) continue;
-          // all partials are fetched before the first add; waves beyond nw re-read the last one
-          float4_t v[MAX_STREAM_WAVES];
+          const float4_t* src = pb + sl_l4[it];
+          float4_t sum;
+          if (nw == MAX_STREAM_WAVES) {
+            // the common shape: all partials fetched with immediate offsets before the adds
+            float4_t v[MAX_STREAM_WAVES];
 #pragma unroll
-          for (int wv = 0; wv < MAX_STREAM_WAVES; ++wv)
-            v[wv] = pbuf4[(buf * nw + (wv < nw ? wv : nw - 1)) * 256 + l4];
-          float4_t sum = v[0];
+            for (int wv = 0; wv < MAX_STREAM_WAVES; ++wv) v[wv] = src[wv * 256];
+            sum = v[0];
 #pragma unroll
-          for (int wv = 1; wv < MAX_STREAM_WAVES; ++wv)
-            if (wv < nw) sum += v[wv];
+            for (int wv = 1; wv < MAX_STREAM_WAVES; ++wv) sum += v[wv];
+          } else {
+            float4_t v[MAX_STREAM_WAVES];
+#pragma unroll
+            for (int wv = 0; wv < MAX_STREAM_WAVES; ++wv)
+              if (wv < nw) v[wv] = src[wv * 256];
+            sum = v[0];
+#pragma unroll
+            for (int wv = 1; wv < MAX_STREAM_WAVES; ++wv)
+              if (wv < nw) sum += v[wv];
+          }
           if (phases > 1) {
-            if (ph > 0) sum += accl4[bi * 256 + l4];
+            float4_t* a = accl4 + bi * 256 + sl_l4[it];
+            if (ph > 0) sum += *a;
             if (ph + 1 < phases) {
-              accl4[bi * 256 + l4] = sum;
+              *a = sum;
               continue;
             }
           }
-          const int ln = l4 & 63;
-          const int n = tile * 16 + (ln & 15);
-          const int m0 = 16 * t + 4 * (ln >> 4);
           if (to_out) {
-            if (n < N) {
+            half_t* o = sl_out[it] + tile * 16;
+            if (tile * 16 + (sl_l4[it] & 15) < N) {
               half_t bn = (half_t)0.f;
-              if (bias) bn = bias[n];
+              if (bias) bn = bias[tile * 16 + (sl_l4[it] & 15)];
 #pragma unroll
               for (int i = 0; i < 4; ++i)
-                if (m0 + i < M) {
-                  half_t o = (half_t)sum[i];
-                  if (bias) o = o + bn;
-                  out[(size_t)(m0 + i) * N + n] = o;
+                if (i < sl_rows[it]) {
+                  half_t r = (half_t)sum[i];
+                  if (bias) r = r + bn;
+                  o[(size_t)i * N] = r;
                 }
             }
           } else {
-            // partial[slab][tile][t][i][64]
-            float* dst = partial + ((((size_t)slab * tiles_total + tile) * NT + t) * 4) * 64 + ln;
+            float* dst = sl_part[it] + (size_t)tile * (NT * 256);
 #pragma unroll
             for (int i = 0; i < 4; ++i)
               __hip_atomic_store(dst + i * 64, sum[i], __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
