@@ -455,14 +455,8 @@ __global__ __launch_bounds__(1024) void qmm_w4g64_kernel(
 #pragma unroll
             for (int wv = 1; wv < MAX_STREAM_WAVES; ++wv) sum += v[wv];
           } else {
-            float4_t v[MAX_STREAM_WAVES];
-#pragma unroll
-            for (int wv = 0; wv < MAX_STREAM_WAVES; ++wv)
-              if (wv < nw) v[wv] = src[wv * 256];
-            sum = v[0];
-#pragma unroll
-            for (int wv = 1; wv < MAX_STREAM_WAVES; ++wv)
-              if (wv < nw) sum += v[wv];
+            sum = src[0];
+            for (int wv = 1; wv < nw; ++wv) sum += src[wv * 256];
           }
           if (phases > 1) {
             float4_t* a = accl4 + bi * 256 + sl_l4[it];
