@@ -30,10 +30,11 @@ PREFIX = 2048
 NODES = 32
 
 
-def qmm_bytes(M, N, K):
+def qmm_bytes(M, N, K, n_out=None):
     """Algorithmic bytes of one 4-bit group-64 QMM: packed weights + fp16 scale and bias per
-    64 weights (0.5625 B per weight) + fp16 activations in and out."""
-    return 0.5625 * N * K + 2.0 * M * (K + N)
+    64 weights (0.5625 B per weight) + fp16 activations in and out (the SwiGLU form writes
+    n_out = N / 2 columns)."""
+    return 0.5625 * N * K + 2.0 * M * (K + (N if n_out is None else n_out))
 
 
 def qmm_shapes(args):
@@ -163,13 +164,16 @@ def main():
     ver.act.normal_()
 
     def qmm_only():
-        for wq, sc, bi, bias, x, out in launches:
-            ops.quantized_matmul(x, wq, sc, bi, bias=bias, out=out)
+        for wq, sc, bi, bias, x, out, swiglu in launches:
+            if swiglu:
+                ops.quantized_matmul_swiglu(x, wq, sc, bi, bias=bias, out=out)
+            else:
+                ops.quantized_matmul(x, wq, sc, bi, bias=bias, out=out)
 
     qt, _ = graph_time_ms(torch, qmm_only, reps=10)
     qmm_ms = float(np.median(qt))
     n_launch = len(launches)
-    alg = sum(qmm_bytes(NODES, wq.shape[0], wq.shape[1] * 8) for wq, *_ in launches)
+    alg = sum(qmm_bytes(NODES, l[0].shape[0], l[0].shape[1] * 8, l[5].shape[-1]) for l in launches)
     kv_bytes = 2 * L * G * (PREFIX + NODES) * hd * 2
     achieved = alg / (qmm_ms * 1e-3) / 1e9
     traffic = QMM_TRAFFIC_BYTES_PER_LAUNCH

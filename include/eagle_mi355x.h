@@ -28,7 +28,7 @@ enum eagle_status {
   EAGLE_ERR_NULL = 1,        /* required pointer is NULL */
   EAGLE_ERR_SHAPE = 2,       /* a dimension is out of the supported range */
   EAGLE_ERR_ALIGN = 3,       /* pointer not 16-byte aligned */
-  EAGLE_ERR_UNSUPPORTED = 4, /* group_size != 64 or bits != 4 */
+  EAGLE_ERR_UNSUPPORTED = 4, /* group_size != 64, bits != 4, or a form the shape does not allow */
   EAGLE_ERR_WORKSPACE = 5,   /* workspace missing or too small */
   EAGLE_ERR_HIP = 6,         /* the HIP runtime reported a launch error */
   EAGLE_ERR_ARCH = 7         /* current device is not gfx950 */
@@ -76,6 +76,17 @@ int eagle_qmm_w4g64_f16_tuned(const void* x, const uint32_t* wq, const void* sca
                               const void* biases, const void* bias, void* out,
                               int M, int N, int K, int nw, int phases, int splits, int ranges,
                               void* workspace, size_t workspace_bytes, eagle_stream_t stream);
+
+/* SwiGLU form of the same matmul for the MLP gate and up projections (mlx_llama.py:214-215:
+ * down(silu(gate(x)) * up(x))).  wq / scales / biases / bias hold both projections with their
+ * rows interleaved in 16-row tiles: gate rows 0..15, up rows 0..15, gate rows 16..31, ...
+ * (N = 2 * intermediate size, N % 32 == 0).  out [M, N/2] = fp16(fp16(silu(g)) * u) with
+ * g, u the fp16 results of the two projections, i.e. the values the separate launches and
+ * eagle_silu_mul_f16 produce.  EAGLE_ERR_UNSUPPORTED when the shape would need K slabs. */
+int eagle_qmm_swiglu_w4g64_f16(const void* x, const uint32_t* wq, const void* scales,
+                               const void* biases, const void* bias, void* out,
+                               int M, int N, int K, int group_size, int bits,
+                               void* workspace, size_t workspace_bytes, eagle_stream_t stream);
 
 /* Quantised embedding gather: out[t,:] = fp16(scales*q + biases) of row ids[t].
  * ids [T] int32, out [T,D] fp16, D % 64 == 0.  Replaces the quantised

@@ -123,7 +123,7 @@ __global__ __launch_bounds__(1024) void qmm_w4g64_kernel(
     const half_t* __restrict__ s, const half_t* __restrict__ b,
     const half_t* __restrict__ bias, half_t* __restrict__ out,
     float* __restrict__ partial, unsigned* __restrict__ counters,
-    int M, int N, int K, int nw, int phases, int t_q, int t_r) {
+    int M, int N, int K, int nw, int phases, int t_q, int t_r, int swiglu) {
   using C = Cfg<NT, GW>;
   constexpr int B = C::B;
   extern __shared__ __attribute__((aligned(16))) unsigned char lds[];
@@ -142,8 +142,10 @@ __global__ __launch_bounds__(1024) void qmm_w4g64_kernel(
   const int slab = blockIdx.y;
   const int tiles_total = (N + 15) >> 4;
   const int bx = blockIdx.x;
-  const int t_lo = bx * t_q + (bx < t_r ? bx : t_r);
-  const int t_hi = t_lo + t_q + (bx < t_r ? 1 : 0);
+  // ranges are counted in tiles, or in (gate, up) tile pairs for the SwiGLU form
+  const int gran = swiglu ? 2 : 1;
+  const int t_lo = gran * (bx * t_q + (bx < t_r ? bx : t_r));
+  const int t_hi = t_lo + gran * (t_q + (bx < t_r ? 1 : 0));
   const int nss = (t_hi - t_lo + C::RING - 1) / C::RING;   // super-steps per phase
   const int nbp = nss * C::BPS;                             // batches per phase
   const bool to_out = nsplit == 1;
@@ -414,6 +416,8 @@ __global__ __launch_bounds__(1024) void qmm_w4g64_kernel(
     // ------------------------------------------------------------------ reducing wave
     // A lane owns the same two float4 slots of every batch: slot l4 = (tile j of the batch,
     // x block t, MFMA lane ln) holds out[16 t + 4 (ln / 16) + i][tile * 16 + ln % 16], i = 0..3.
+    // In the SwiGLU form the weight tiles alternate gate, up, gate, up ...; a lane then owns
+    // the two slots of one (gate, up) pair and stores fp16(fp16(silu(gate)) * up) instead.
     const int wl = tid - nw * 64;     // 0 .. 127
     int sl_l4[2], sl_j[2];
     half_t* sl_out[2];
@@ -421,14 +425,15 @@ __global__ __launch_bounds__(1024) void qmm_w4g64_kernel(
     int sl_rows[2];
 #pragma unroll
     for (int it = 0; it < 2; ++it) {
-      const int l4 = wl + it * 128;            // 0 .. 255
+      int l4 = wl + it * 128;                  // 0 .. 255
+      if (swiglu && NT == 1) l4 = ((2 * (wl >> 6) + it) << 6) | (wl & 63);
       const int jt = l4 >> 6;
       const int t = jt % NT;
       const int ln = l4 & 63;
       const int m0 = 16 * t + 4 * (ln >> 4);
       sl_l4[it] = l4;
       sl_j[it] = jt / NT;
-      sl_out[it] = out + (size_t)m0 * N + (ln & 15);
+      sl_out[it] = out + (size_t)m0 * (swiglu ? N >> 1 : N) + (ln & 15);
       sl_rows[it] = M - m0;                    // rows m0 .. m0+3 exist while i < sl_rows
       // partial[slab][tile][t][i][64]
       sl_part[it] = partial + (((size_t)slab * tiles_total * NT + t) * 4) * 64 + ln;
@@ -440,10 +445,13 @@ __global__ __launch_bounds__(1024) void qmm_w4g64_kernel(
         const int buf = (ph * nbp + bi) & 1;
         const int tile0 = t_lo + bi * B;
         const float4_t* pb = pbuf4 + buf * nw * 256;
+        float4_t sums[2];
+        bool live[2];
 #pragma unroll
         for (int it = 0; it < 2; ++it) {
           const int tile = tile0 + sl_j[it];
-          if (tile >= t_hi) continue;
+          live[it] = tile < t_hi;
+          if (!live[it]) continue;
           const float4_t* src = pb + sl_l4[it];
           float4_t sum;
           if (nw == MAX_STREAM_WAVES) {
@@ -463,9 +471,45 @@ __global__ __launch_bounds__(1024) void qmm_w4g64_kernel(
             if (ph > 0) sum += *a;
             if (ph + 1 < phases) {
               *a = sum;
-              continue;
+              live[it] = false;
             }
           }
+          sums[it] = sum;
+        }
+        if (swiglu) {
+          // slots 0 and 1 of this lane are the gate tile and the up tile of one pair
+          if (live[0] && live[1]) {
+            const int pair = (tile0 + sl_j[0]) >> 1;
+            const int n_out = pair * 16 + (sl_l4[0] & 15);
+            const int n_g = (tile0 + sl_j[0]) * 16 + (sl_l4[0] & 15);
+            half_t* o = sl_out[0] + pair * 16;
+            if (n_g + 16 < N + 1 && n_out < (N >> 1)) {
+              half_t bg = (half_t)0.f, bu = (half_t)0.f;
+              if (bias) {
+                bg = bias[n_g];
+                bu = bias[n_g + 16];
+              }
+#pragma unroll
+              for (int i = 0; i < 4; ++i)
+                if (i < sl_rows[0]) {
+                  half_t g = (half_t)sums[0][i], u = (half_t)sums[1][i];
+                  if (bias) {
+                    g = g + bg;
+                    u = u + bu;
+                  }
+                  const float gf = (float)g;
+                  const half_t a = (half_t)(gf / (1.0f + expf(-gf)));
+                  o[(size_t)i * (N >> 1)] = (half_t)((float)a * (float)u);
+                }
+            }
+          }
+          continue;
+        }
+#pragma unroll
+        for (int it = 0; it < 2; ++it) {
+          if (!live[it]) continue;
+          const int tile = tile0 + sl_j[it];
+          const float4_t sum = sums[it];
           if (to_out) {
             half_t* o = sl_out[it] + tile * 16;
             if (tile * 16 + (sl_l4[it] & 15) < N) {
@@ -545,27 +589,28 @@ inline int nt_of(int M) { return M <= 16 ? 1 : 2; }
 inline int cw_of(int M) { return M <= 16 ? 256 : 128; }
 constexpr int MAX_PHASES = 8;
 
-int lds_bytes(int M, int N, const Launch& L) {
+// gran = 1: ranges are counted in tiles; gran = 2: in (gate, up) tile pairs
+int lds_bytes(int M, int N, const Launch& L, int gran = 1) {
   const int sb = M <= 16 ? 2 * Cfg<1, 4>::SB_BUF : 2 * Cfg<2, 2>::SB_BUF;
   int acc = 0;
   if (L.phases > 1) {
-    const int tiles = (N + 15) / 16;
-    const int per_range = (tiles + L.ranges - 1) / L.ranges;
+    const int tiles = (N + 15) / 16 / gran;
+    const int per_range = gran * ((tiles + L.ranges - 1) / L.ranges);
     acc = (per_range + 3) / 4 * 4 * nt_of(M) * 1024;        // fp32 16 x M per tile, whole super-steps
   }
   return pbuf_bytes(L.nw) + sb + acc;
 }
 
-int validate_launch(int M, int N, int K, const Launch& L) {
+int validate_launch(int M, int N, int K, const Launch& L, int gran = 1) {
   if (L.nw < 1 || L.nw > MAX_STREAM_WAVES || L.splits < 1 || L.splits > MAX_SPLITS ||
       L.phases < 1 || L.phases > MAX_PHASES)
     return EAGLE_ERR_SHAPE;
   const int units = (K + cw_of(M) - 1) / cw_of(M);
   const long per_slab = (long)L.nw * L.phases;
   if (per_slab * L.splits < units || per_slab * (L.splits - 1) >= units) return EAGLE_ERR_SHAPE;
-  const int tiles = (N + 15) / 16;
+  const int tiles = (N + 15) / 16 / gran;
   if (L.ranges < 1 || L.ranges > tiles || L.ranges > MAX_RANGES) return EAGLE_ERR_SHAPE;
-  if (lds_bytes(M, N, L) > LDS_MAX) return EAGLE_ERR_SHAPE;
+  if (lds_bytes(M, N, L, gran) > LDS_MAX) return EAGLE_ERR_SHAPE;
   return EAGLE_OK;
 }
 
@@ -612,8 +657,8 @@ void choose(int M, int N, int K, Launch* out) {
 template <int NT, int GW, bool SLOWSB>
 int launch(const void* x, const uint32_t* wq, const void* s, const void* b, const void* bias,
            void* out, float* partial, unsigned* counters, int M, int N, int K, const Launch& L,
-           hipStream_t stream) {
-  const int lds = lds_bytes(M, N, L);
+           int swiglu, hipStream_t stream) {
+  const int lds = lds_bytes(M, N, L, swiglu ? 2 : 1);
   static bool attr_set = false;   // more than 64 KB of LDS needs an explicit opt-in, once
   if (lds > 65536 && !attr_set) {
     if (hipFuncSetAttribute(reinterpret_cast<const void*>(&qmm_w4g64_kernel<NT, GW, SLOWSB>),
@@ -621,11 +666,11 @@ int launch(const void* x, const uint32_t* wq, const void* s, const void* b, cons
       return EAGLE_ERR_HIP;
     attr_set = true;
   }
-  const int tiles = (N + 15) / 16;
+  const int tiles = ((N + 15) / 16) / (swiglu ? 2 : 1);      // range units: tiles or tile pairs
   hipLaunchKernelGGL((qmm_w4g64_kernel<NT, GW, SLOWSB>), dim3(L.ranges, L.splits),
                      dim3(64 * (L.nw + NWR)), lds, stream, (const half_t*)x, wq,
                      (const half_t*)s, (const half_t*)b, (const half_t*)bias, (half_t*)out,
-                     partial, counters, M, N, K, L.nw, L.phases, tiles / L.ranges, tiles % L.ranges);
+                     partial, counters, M, N, K, L.nw, L.phases, tiles / L.ranges, tiles % L.ranges, swiglu);
   return eagle_launch_status();
 }
 
@@ -644,8 +689,8 @@ int validate(const void* x, const uint32_t* wq, const void* s, const void* b, co
 }
 
 int run(const void* x, const uint32_t* wq, const void* scales, const void* biases,
-        const void* bias, void* out, int M, int N, int K, const Launch& L, void* workspace,
-        size_t workspace_bytes, hipStream_t st) {
+        const void* bias, void* out, int M, int N, int K, const Launch& L, int swiglu,
+        void* workspace, size_t workspace_bytes, hipStream_t st) {
   float* partial = nullptr;
   unsigned* counters = nullptr;
   if (L.splits > 1) {
@@ -663,10 +708,10 @@ int run(const void* x, const uint32_t* wq, const void* scales, const void* biase
   const bool slow = (G % gw) != 0 || (reinterpret_cast<uintptr_t>(scales) & amask) ||
                     (reinterpret_cast<uintptr_t>(biases) & amask);
   if (M <= 16)
-    return slow ? launch<1, 4, true>(x, wq, scales, biases, bias, out, partial, counters, M, N, K, L, st)
-                : launch<1, 4, false>(x, wq, scales, biases, bias, out, partial, counters, M, N, K, L, st);
-  return slow ? launch<2, 2, true>(x, wq, scales, biases, bias, out, partial, counters, M, N, K, L, st)
-              : launch<2, 2, false>(x, wq, scales, biases, bias, out, partial, counters, M, N, K, L, st);
+    return slow ? launch<1, 4, true>(x, wq, scales, biases, bias, out, partial, counters, M, N, K, L, swiglu, st)
+                : launch<1, 4, false>(x, wq, scales, biases, bias, out, partial, counters, M, N, K, L, swiglu, st);
+  return slow ? launch<2, 2, true>(x, wq, scales, biases, bias, out, partial, counters, M, N, K, L, swiglu, st)
+              : launch<2, 2, false>(x, wq, scales, biases, bias, out, partial, counters, M, N, K, L, swiglu, st);
 }
 
 }  // namespace
@@ -702,7 +747,7 @@ EAGLE_EXPORT int eagle_qmm_w4g64_f16_tuned(const void* x, const uint32_t* wq, co
   Launch L{nw, phases, splits, ranges};
   rc = validate_launch(M, N, K, L);
   if (rc != EAGLE_OK) return rc;
-  return run(x, wq, scales, biases, bias, out, M, N, K, L, workspace, workspace_bytes,
+  return run(x, wq, scales, biases, bias, out, M, N, K, L, 0, workspace, workspace_bytes,
              static_cast<hipStream_t>(stream));
 }
 
@@ -717,6 +762,25 @@ EAGLE_EXPORT int eagle_qmm_w4g64_f16(const void* x, const uint32_t* wq, const vo
   choose(M, N, K, &L);
   rc = validate_launch(M, N, K, L);
   if (rc != EAGLE_OK) return rc;
-  return run(x, wq, scales, biases, bias, out, M, N, K, L, workspace, workspace_bytes,
+  return run(x, wq, scales, biases, bias, out, M, N, K, L, 0, workspace, workspace_bytes,
+             static_cast<hipStream_t>(stream));
+}
+
+EAGLE_EXPORT int eagle_qmm_swiglu_w4g64_f16(const void* x, const uint32_t* wq, const void* scales,
+                                            const void* biases, const void* bias, void* out,
+                                            int M, int N, int K, int group_size, int bits,
+                                            void* workspace, size_t workspace_bytes,
+                                            eagle_stream_t stream) {
+  if (group_size != 64 || bits != 4) return EAGLE_ERR_UNSUPPORTED;
+  int rc = validate(x, wq, scales, biases, bias, out, M, N, K);
+  if (rc != EAGLE_OK) return rc;
+  if ((N % 32) != 0) return EAGLE_ERR_SHAPE;             // whole (gate, up) tile pairs
+  Launch L;
+  choose(M, N, K, &L);
+  if (L.splits != 1) return EAGLE_ERR_UNSUPPORTED;       // the activation needs the complete sum
+  if (L.ranges > N / 32) L.ranges = N / 32;
+  rc = validate_launch(M, N, K, L, 2);
+  if (rc != EAGLE_OK) return rc;
+  return run(x, wq, scales, biases, bias, out, M, N, K, L, 1, workspace, workspace_bytes,
              static_cast<hipStream_t>(stream));
 }

@@ -170,7 +170,8 @@ class TreeVerifier:
     accept_indices...) and `accepted_tokens`; the cache length advances on the device.
     Same kernels and operator order as Model.__call__ + the host functions above."""
 
-    def __init__(self, model, cache, total_tokens=31, max_len=None, compact=True, fuse=True):
+    def __init__(self, model, cache, total_tokens=31, max_len=None, compact=True, fuse=True,
+                 swiglu=True):
         args = model.args
         self.model, self.cache, self.args = model, cache, args
         self.V = total_tokens
@@ -183,6 +184,8 @@ class TreeVerifier:
         self.max_len = max_len or self.capacity
         self.compact = compact
         self.fuse = fuse
+        # gate|up with the SwiGLU epilogue when the matmul covers the shape in one K slab
+        self.swiglu = bool(fuse and swiglu and ops.swiglu_supported(T, I, D))
         if fuse:
             self._fuse_projections()
         i32 = dict(dtype=torch.int32, device=dev)
@@ -234,6 +237,17 @@ class TreeVerifier:
         the three (two) projections; memory use is unchanged."""
         self.qkv_w, self.gu_w = [], []
 
+        def interleave(lins):
+            g, u = lins
+            fused = [ops.interleave_gate_up(getattr(g, k), getattr(u, k))
+                     for k in ("weight", "scales", "biases")]
+            bias = None
+            if g.bias is not None or u.bias is not None:
+                z = torch.zeros(g.weight.shape[0], dtype=torch.float16, device=g.weight.device)
+                bias = ops.interleave_gate_up(g.bias if g.bias is not None else z,
+                                              u.bias if u.bias is not None else z)
+            return (*fused, bias)
+
         def fuse(lins):
             parts = [[l.weight, l.scales, l.biases] for l in lins]
             fused = [torch.cat([p[k] for p in parts], dim=0).contiguous() for k in range(3)]
@@ -254,29 +268,36 @@ class TreeVerifier:
         for layer in self.model.model.layers:
             at, mlp = layer.self_attn, layer.mlp
             self.qkv_w.append(fuse([at.q_proj, at.k_proj, at.v_proj]))
-            self.gu_w.append(fuse([mlp.gate_proj, mlp.up_proj]))
+            if self.swiglu:
+                # a tile-interleaved copy: the layers keep their own tensors for the module path
+                self.gu_w.append(interleave([mlp.gate_proj, mlp.up_proj]))
+            else:
+                self.gu_w.append(fuse([mlp.gate_proj, mlp.up_proj]))
 
     def qmm_launches(self):
-        """(weight, scales, biases, bias, x, out) of every quantised matmul of one step, in order."""
+        """(weight, scales, biases, bias, x, out, swiglu) of every quantised matmul of one step,
+        in order; `swiglu` marks the launches that go through `quantized_matmul_swiglu`."""
         m = self.model
         out = []
         for i, layer in enumerate(m.model.layers):
             at, mlp = layer.self_attn, layer.mlp
             if self.fuse:
-                out.append((*self.qkv_w[i], self.hn, self.qkv))
+                out.append((*self.qkv_w[i], self.hn, self.qkv, False))
             else:
                 for lin, o in ((at.q_proj, self.q), (at.k_proj, self.k), (at.v_proj, self.v)):
-                    out.append((lin.weight, lin.scales, lin.biases, lin.bias, self.hn, o))
-            out.append((at.o_proj.weight, at.o_proj.scales, at.o_proj.biases, at.o_proj.bias, self.attn, self.o))
+                    out.append((lin.weight, lin.scales, lin.biases, lin.bias, self.hn, o, False))
+            out.append((at.o_proj.weight, at.o_proj.scales, at.o_proj.biases, at.o_proj.bias,
+                        self.attn, self.o, False))
             if self.fuse:
-                out.append((*self.gu_w[i], self.hn, self.gate_up))
+                out.append((*self.gu_w[i], self.hn, self.act if self.swiglu else self.gate_up,
+                            self.swiglu))
             else:
                 for lin, o in ((mlp.gate_proj, self.gate), (mlp.up_proj, self.up)):
-                    out.append((lin.weight, lin.scales, lin.biases, lin.bias, self.hn, o))
+                    out.append((lin.weight, lin.scales, lin.biases, lin.bias, self.hn, o, False))
             out.append((mlp.down_proj.weight, mlp.down_proj.scales, mlp.down_proj.biases,
-                        mlp.down_proj.bias, self.act, self.down))
+                        mlp.down_proj.bias, self.act, self.down, False))
         head = m.model.embed_tokens if self.args.tie_word_embeddings else m.lm_head
-        out.append((head.weight, head.scales, head.biases, None, self.hn, self.logits))
+        out.append((head.weight, head.scales, head.biases, None, self.hn, self.logits, False))
         return out
 
     def set_tree(self, tokens, tree_position_ids, mask_index, mask_bits):
@@ -326,8 +347,11 @@ class TreeVerifier:
             mlp = layer.mlp
             if self.fuse:
                 w, sc, bi, b = self.gu_w[i]
-                ops.quantized_matmul(self.hn, w, sc, bi, bias=b, out=self.gate_up)
-                ops.silu_mul(self.gate_up, None, out=self.act)
+                if self.swiglu:
+                    ops.quantized_matmul_swiglu(self.hn, w, sc, bi, bias=b, out=self.act)
+                else:
+                    ops.quantized_matmul(self.hn, w, sc, bi, bias=b, out=self.gate_up)
+                    ops.silu_mul(self.gate_up, None, out=self.act)
             else:
                 ops.quantized_matmul(self.hn, mlp.gate_proj.weight, mlp.gate_proj.scales,
                                      mlp.gate_proj.biases, bias=mlp.gate_proj.bias, out=self.gate)

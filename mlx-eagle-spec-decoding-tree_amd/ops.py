@@ -107,6 +107,50 @@ def qmm_plan(M, N, K):
     return tuple(plan)
 
 
+def interleave_gate_up(gate, up):
+    """Rows of two [N, ...] tensors interleaved in 16-row tiles (gate 0..15, up 0..15, gate
+    16..31, ...): the weight layout `quantized_matmul_swiglu` reads."""
+    n = gate.shape[0]
+    if up.shape != gate.shape or n % 16:
+        raise ValueError("gate and up must have the same shape with rows a multiple of 16")
+    g = gate.reshape(n // 16, 1, 16, *gate.shape[1:])
+    u = up.reshape(n // 16, 1, 16, *up.shape[1:])
+    return torch.cat([g, u], dim=1).reshape(2 * n, *gate.shape[1:]).contiguous()
+
+
+def swiglu_supported(M, I, K):
+    """True when the SwiGLU matmul covers this shape (whole tile pairs, no K slabs)."""
+    return I % 16 == 0 and 1 <= M <= 32 and qmm_plan(M, 2 * I, K)[2] == 1
+
+
+def quantized_matmul_swiglu(x, w_q, scales, biases, bias=None, out=None):
+    """silu(x @ Wg.T) * (x @ Wu.T) (mlx_llama.py:214-215) in one launch: w_q / scales / biases
+    / bias hold the gate and up projections interleaved by `interleave_gate_up`.  The result
+    equals `silu_mul(quantized_matmul(x, gate...), quantized_matmul(x, up...))` bit for bit."""
+    _need_cuda(x, w_q, scales, biases, bias)
+    x = _f16(x, "x")
+    w_q = as_packed_u32(w_q)
+    scales, biases = _f16(scales, "scales"), _f16(biases, "biases")
+    *lead, K = x.shape
+    M = reduce(lambda a, b: a * b, lead, 1)
+    N = w_q.shape[0]
+    if w_q.shape[1] * 8 != K or tuple(scales.shape) != (N, K // 64) or tuple(biases.shape) != (N, K // 64):
+        raise ValueError(f"shape mismatch: x {tuple(x.shape)}, w {tuple(w_q.shape)}, "
+                         f"scales {tuple(scales.shape)}, biases {tuple(biases.shape)}")
+    if bias is not None:
+        bias = _f16(bias, "bias")
+        if tuple(bias.shape) != (N,):
+            raise ValueError("bias must have shape [N]")
+    if out is None:
+        out = torch.empty((*lead, N // 2), dtype=torch.float16, device=x.device)
+    L = _lib.lib()
+    ws = workspace("qmm", L.eagle_qmm_workspace_bytes(M, N, K), x.device)
+    rc = L.eagle_qmm_swiglu_w4g64_f16(_ptr(x), _ptr(w_q), _ptr(scales), _ptr(biases), _ptr(bias),
+                                      _ptr(out), M, N, K, 64, 4, _ptr(ws), ws.numel(), _stream())
+    _lib.check(rc, "quantized_matmul_swiglu")
+    return out
+
+
 def matmul(x, w, s, b, group_size, **_ignored):
     """Same contract as the reference's `qmm_kernel.matmul` (qmm_kernel.py:84-164):
     returns a one-element list.  The Metal tuning keywords are accepted and ignored."""

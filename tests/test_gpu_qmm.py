@@ -138,3 +138,44 @@ def test_argument_errors(dev):
         ops.quantized_matmul(x[:8], w, s, s, group_size=32)
     with pytest.raises(ValueError):
         ops.quantized_matmul(x[:8], w, s, s, bits=8)
+
+
+@pytest.mark.parametrize("I,K,bias", [(16, 64, False), (48, 128, True), (272, 256, True), (4864, 896, False),
+                                      (18944, 3584, True), (1024, 7168, False)])
+def test_swiglu_form_equals_separate_launches(dev, I, K, bias):
+    """gate|up in tile-interleaved rows with the activation in the matmul's epilogue: bit-identical
+    to the concatenated launch followed by silu_mul (same launch shape, so the same fp32 sums), and
+    within tolerance of the oracle's qmm -> silu_mul."""
+    for M in (1, 8, 16, 17, 32):
+        if not ops.swiglu_supported(M, I, K):
+            continue
+        print(f"qmm swiglu I={I} K={K} M={M}", flush=True)
+        rng = np.random.default_rng(I + K + M)
+        g = synth.make_qlinear(rng, I, K, bias=bias, gain=1.0)
+        u = synth.make_qlinear(rng, I, K, bias=bias, gain=1.0)
+        x = synth.make_x(rng, M, K)
+        want = oracle.silu_mul(oracle.qmm(x, g["weight"], g["scales"], g["biases"], g.get("bias")),
+                               oracle.qmm(x, u["weight"], u["scales"], u["biases"], u.get("bias")))
+        gd, ud = layer_to_dev(g, dev), layer_to_dev(u, dev)
+        keys = ["weight", "scales", "biases"] + (["bias"] if bias else [])
+        inter = {k: ops.interleave_gate_up(gd[k], ud[k]) for k in keys}
+        cat = {k: torch.cat([gd[k], ud[k]]).contiguous() for k in keys}
+        xd = to_dev(x, dev)
+        got = ops.quantized_matmul_swiglu(xd, inter["weight"], inter["scales"], inter["biases"],
+                                          bias=inter.get("bias"))
+        two = ops.silu_mul(ops.quantized_matmul(xd, cat["weight"], cat["scales"], cat["biases"],
+                                                bias=cat.get("bias")))
+        torch.cuda.synchronize()
+        assert tuple(got.shape) == (M, I)
+        assert torch.equal(got, two), f"I={I} K={K} M={M}: swiglu form differs from matmul + silu_mul"
+        assert rel_err(got.cpu().numpy(), want) <= TOL
+
+
+def test_swiglu_form_refuses_k_slabs(dev):
+    rng = np.random.default_rng(1)
+    g = layer_to_dev(synth.make_qlinear(rng, 32, 8192), dev)
+    assert not ops.swiglu_supported(8, 32, 8192)
+    w = {k: ops.interleave_gate_up(g[k], g[k]) for k in ("weight", "scales", "biases")}
+    with pytest.raises(ValueError):
+        ops.quantized_matmul_swiglu(to_dev(synth.make_x(rng, 8, 8192), dev), w["weight"], w["scales"],
+                                    w["biases"])
