@@ -151,6 +151,31 @@ int eagle_silu_mul_f16(const void* gate, const void* up, void* out, int T, int I
 /* out = fp16(a + b), n elements (residual add, mlx_llama.py:246,248). */
 int eagle_add_f16(const void* a, const void* b, void* out, long n, eagle_stream_t stream);
 
+/* cos/sin table for eagle_tree_attention_rope_f16: out[t][i] = (cos, sin)(positions[t] *
+ * scaling_factor * inv_freqs[i]), fp32 [T, half_dim, 2]; the same angles as
+ * eagle_rope_arrayed_f16 (mlx_arrayed_rope_kernel.py:60-123).  The table depends on the tree
+ * positions only, so one call serves every layer of a step. */
+int eagle_rope_table_f32(const int32_t* positions, const float* inv_freqs, float scaling_factor,
+                         int T, int half_dim, float* out, eagle_stream_t stream);
+
+/* The attention block of one layer in one launch (mlx_llama.py:166-195: rope of q and k with
+ * per-token positions, cache update, masked SDPA).  q_lin / k_lin / v_lin are the token-major
+ * projection outputs ([T, H*hd], [T, G*hd], [T, G*hd]) with a common row stride in elements
+ * (columns of one fused q|k|v matrix, or row_stride = the width of each when separate and
+ * equal).  Rotated keys and the values of the T tree tokens are written to cache rows
+ * P .. P+T-1 (P = *cache_len_dev) and attended to together with the prefix under
+ * tree_mask_bits, exactly as eagle_rope_kv_append_f16 followed by eagle_tree_attention_f16.
+ * out [T, H*hd].  The first 256-byte multiple covering 4*H bytes of the workspace holds
+ * arrival counters: zero before the first call, left zero by every call; calls sharing a
+ * workspace must be stream ordered. */
+size_t eagle_tree_attention_rope_workspace_bytes(int H, int hd, int max_len);
+int eagle_tree_attention_rope_f16(const void* q_lin, const void* k_lin, const void* v_lin,
+                                  long row_stride, const float* rope_cs, void* k_cache,
+                                  void* v_cache, const uint32_t* tree_mask_bits,
+                                  const int32_t* cache_len_dev, void* out, int T, int H, int G,
+                                  int hd, long capacity, int max_len, float scale, void* workspace,
+                                  size_t workspace_bytes, eagle_stream_t stream);
+
 /* Row argmax of fp16 logits [R,V], lowest index among equal maxima
  * (mx.argmax at mlx_eagle.py:316,534,596).  out [R] int32. */
 size_t eagle_argmax_workspace_bytes(int R, long V);

@@ -32,6 +32,10 @@ SIGNATURES = {
     "eagle_tree_attention_workspace_bytes": (c_size_t, [c_int, c_int, c_int]),
     "eagle_tree_attention_f16": (c_int, [c_void_p] * 6 + [c_int] * 4 + [c_long, c_int, c_float,
                                                                        c_void_p, c_size_t, c_void_p]),
+    "eagle_rope_table_f32": (c_int, [c_void_p, c_void_p, c_float, c_int, c_int, c_void_p, c_void_p]),
+    "eagle_tree_attention_rope_workspace_bytes": (c_size_t, [c_int, c_int, c_int]),
+    "eagle_tree_attention_rope_f16": (c_int, [c_void_p] * 3 + [c_long] + [c_void_p] * 6 + [c_int] * 4
+                                      + [c_long, c_int, c_float, c_void_p, c_size_t, c_void_p]),
     "eagle_rmsnorm_f16": (c_int, [c_void_p] * 3 + [c_float] + [c_void_p] * 2 + [c_int] * 2 + [c_void_p]),
     "eagle_silu_mul_f16": (c_int, [c_void_p] * 3 + [c_int] * 2 + [c_void_p]),
     "eagle_add_f16": (c_int, [c_void_p] * 3 + [c_long, c_void_p]),

@@ -640,6 +640,9 @@ void choose(int M, int N, int K, Launch* out) {
   int per_slab = (units + splits - 1) / splits;
   L.phases = (per_slab + MAX_STREAM_WAVES - 1) / MAX_STREAM_WAVES;
   L.nw = (per_slab + L.phases - 1) / L.phases;
+  // 64-byte units (M > 16): two neighbouring waves share each 128-byte line of a weight row,
+  // so an even wave count keeps every line inside one phase
+  if (M > 16 && (L.nw & 1) && L.nw < MAX_STREAM_WAVES) ++L.nw;
   per_slab = L.nw * L.phases;
   L.splits = (units + per_slab - 1) / per_slab;
   int ranges = NUM_CU / L.splits;

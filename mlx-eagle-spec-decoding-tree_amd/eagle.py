@@ -171,7 +171,7 @@ class TreeVerifier:
     Same kernels and operator order as Model.__call__ + the host functions above."""
 
     def __init__(self, model, cache, total_tokens=31, max_len=None, compact=True, fuse=True,
-                 swiglu=True):
+                 swiglu=True, one_launch_attention=False):
         args = model.args
         self.model, self.cache, self.args = model, cache, args
         self.V = total_tokens
@@ -186,6 +186,9 @@ class TreeVerifier:
         self.fuse = fuse
         # gate|up with the SwiGLU epilogue when the matmul covers the shape in one K slab
         self.swiglu = bool(fuse and swiglu and ops.swiglu_supported(T, I, D))
+        # rope + KV append + attention + split merge as one launch instead of three: as fast
+        # inside a graph for prefixes of a few thousand rows, fewer launches outside one
+        self.one_launch_attention = bool(fuse and one_launch_attention)
         if fuse:
             self._fuse_projections()
         i32 = dict(dtype=torch.int32, device=dev)
@@ -208,6 +211,7 @@ class TreeVerifier:
         self.k = torch.empty((T, G * hd), **f16)
         self.v = torch.empty((T, G * hd), **f16)
         self.q_rot = torch.empty((H, T, hd), **f16)
+        self.rope_cs = torch.empty((T, hd // 2, 2), dtype=torch.float32, device=dev)
         self.attn = torch.empty((T, H * hd), **f16)
         self.o = torch.empty((T, D), **f16)
         self.gate_up = torch.empty((T, 2 * I), **f16)        # gate | up of a token side by side
@@ -229,6 +233,7 @@ class TreeVerifier:
                     (D, I), (head.weight.shape[0], D)))
         ops.workspace("qmm", need, dev)
         ops.workspace("attn", L.eagle_tree_attention_workspace_bytes(H, hd, self.max_len), dev)
+        ops.workspace("attn_rope", L.eagle_tree_attention_rope_workspace_bytes(H, hd, self.max_len), dev)
         ops.workspace("argmax", L.eagle_argmax_workspace_bytes(T, args.vocab_size), dev)
 
     def _fuse_projections(self):
@@ -322,24 +327,34 @@ class TreeVerifier:
         ops.embed(self.tokens, emb.weight, emb.scales, emb.biases, out=self.h)
         layers = m.model.layers
         ops.rms_norm(self.h, layers[0].input_layernorm.weight, args.rms_norm_eps, out=self.hn)
+        if self.one_launch_attention:   # one cos/sin table per step: the positions are the same in every layer
+            at0 = layers[0].self_attn
+            ops.rope_table(self.positions, at0._inv_freqs, at0._scaling_factor, out=self.rope_cs)
         for i, layer in enumerate(layers):
             at = layer.self_attn
             c = self.cache[i]
             if self.fuse:
                 w, sc, bi, b = self.qkv_w[i]
                 ops.quantized_matmul(self.hn, w, sc, bi, bias=b, out=self.qkv)
-                ops.rope_kv_append(self.qkv, self.qkv[:, H * hd:], self.qkv[:, (H + G) * hd:],
-                                   self.positions, at._inv_freqs, at._scaling_factor, self.q_rot,
-                                   c.keys[0], c.values[0], self.len_dev, H, G, hd,
-                                   row_stride=(H + 2 * G) * hd)
+                q_lin, k_lin, v_lin = self.qkv, self.qkv[:, H * hd:], self.qkv[:, (H + G) * hd:]
+                if self.one_launch_attention:
+                    ops.tree_attention_rope(q_lin, k_lin, v_lin, self.rope_cs, c.keys[0], c.values[0],
+                                            self.mask_bits, self.len_dev, at.scale, H, G, hd,
+                                            row_stride=(H + 2 * G) * hd, max_len=self.max_len,
+                                            out=self.attn)
+                else:
+                    ops.rope_kv_append(q_lin, k_lin, v_lin, self.positions, at._inv_freqs,
+                                       at._scaling_factor, self.q_rot, c.keys[0], c.values[0],
+                                       self.len_dev, H, G, hd, row_stride=(H + 2 * G) * hd)
             else:
                 for lin, out in ((at.q_proj, self.q), (at.k_proj, self.k), (at.v_proj, self.v)):
                     ops.quantized_matmul(self.hn, lin.weight, lin.scales, lin.biases, bias=lin.bias, out=out)
                 ops.rope_kv_append(self.q, self.k, self.v, self.positions, at._inv_freqs,
                                    at._scaling_factor, self.q_rot, c.keys[0], c.values[0],
                                    self.len_dev, H, G, hd)
-            ops.tree_attention(self.q_rot, c.keys[0], c.values[0], self.mask_bits, self.len_dev,
-                               at.scale, max_len=self.max_len, out=self.attn)
+            if not self.one_launch_attention:
+                ops.tree_attention(self.q_rot, c.keys[0], c.values[0], self.mask_bits, self.len_dev,
+                                   at.scale, max_len=self.max_len, out=self.attn)
             ops.quantized_matmul(self.attn, at.o_proj.weight, at.o_proj.scales, at.o_proj.biases,
                                  bias=at.o_proj.bias, out=self.o)
             ops.rms_norm(self.o, layer.post_attention_layernorm.weight, args.rms_norm_eps,

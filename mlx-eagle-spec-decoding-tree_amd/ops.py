@@ -239,6 +239,46 @@ def tree_attention(q, k_cache, v_cache, tree_mask_bits, cache_len_dev, scale, ma
     return out
 
 
+def rope_table(positions, inv_freqs, scaling_factor=1.0, out=None):
+    """fp32 [T, hd/2, 2] table of (cos, sin)(positions[t] * scaling_factor * inv_freqs[i]) for
+    `tree_attention_rope`; the angles are those of `arrayed_rope`."""
+    _need_cuda(positions, inv_freqs)
+    T, half = positions.numel(), inv_freqs.numel()
+    if out is None:
+        out = torch.empty((T, half, 2), dtype=torch.float32, device=positions.device)
+    rc = _lib.lib().eagle_rope_table_f32(_ptr(positions), _ptr(inv_freqs), float(scaling_factor),
+                                         T, half, _ptr(out), _stream())
+    _lib.check(rc, "rope_table")
+    return out
+
+
+def tree_attention_rope(q_lin, k_lin, v_lin, rope_cs, k_cache, v_cache, tree_mask_bits,
+                        cache_len_dev, scale, H, G, hd, row_stride=0, max_len=None, out=None):
+    """`rope_kv_append` + `tree_attention` in one launch: q_lin [T,H*hd], k_lin / v_lin [T,G*hd]
+    (row_stride > 0: column blocks of one [T,row_stride] matrix), rope_cs from `rope_table`.
+    Appends the rotated keys and the values to cache rows P..P+T-1 and returns [T, H*hd]."""
+    _need_cuda(q_lin, k_lin, v_lin, rope_cs, k_cache, v_cache, tree_mask_bits, cache_len_dev)
+    T = q_lin.shape[0]
+    cap = k_cache.shape[1]
+    if row_stride == 0:
+        if H != G:
+            raise ValueError("separate q and k/v matrices of different widths need row_stride")
+        row_stride = H * hd
+    if max_len is None:
+        max_len = cap
+    if out is None:
+        out = torch.empty((T, H * hd), dtype=torch.float16, device=q_lin.device)
+    L = _lib.lib()
+    need = L.eagle_tree_attention_rope_workspace_bytes(H, hd, max_len)
+    ws = workspace("attn_rope", need, q_lin.device)
+    rc = L.eagle_tree_attention_rope_f16(
+        _ptr(q_lin), _ptr(k_lin), _ptr(v_lin), int(row_stride), _ptr(rope_cs), _ptr(k_cache),
+        _ptr(v_cache), _ptr(tree_mask_bits), _ptr(cache_len_dev), _ptr(out), T, H, G, hd, cap,
+        max_len, float(scale), _ptr(ws), ws.numel(), _stream())
+    _lib.check(rc, "tree_attention_rope")
+    return out
+
+
 def scaled_dot_product_attention(queries, keys, values, cache=None, scale=None, mask=None):
     """Drop-in for the call at mlx_llama.py:185-192 on the tree path:
     queries [1,H,T,hd], keys/values [1,G,S,hd] (prefix then the T tree rows),

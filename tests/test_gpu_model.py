@@ -73,10 +73,10 @@ def test_tree_decoding_matches_oracle(dev, name, P, T):
         assert rel_err(c.values[0, :, P:P + T].cpu().numpy(), ov[:, P:P + T]) <= TOL
 
 
-def run_verifier(s, dev, graph, fuse=True):
+def run_verifier(s, dev, graph, fuse=True, **kw):
     T = s["T"]
     ver = eagle.TreeVerifier(s["model"], s["cache"], total_tokens=T - 1, max_len=s["cache"][0].capacity,
-                             fuse=fuse)
+                             fuse=fuse, **kw)
     ver.set_tree(to_dev(s["tokens"], dev), to_dev(s["depth"], dev), to_dev(s["parents"], dev),
                  to_dev(tree_oracle.mask_bits(s["anc"]).view(np.int32), dev))
     if graph:
@@ -119,6 +119,37 @@ def test_fused_step_equals_module_path_and_oracle(dev, name):
     err = np.abs(ver.logits.cpu().numpy().astype(np.float32) - want["logits"].astype(np.float32)).max()
     if (margins(want["logits"]) > 2 * err).all():
         assert (best, al, am[bonus]) == (want["best"], want["accept_length"], want["next_token"])
+
+
+@pytest.mark.parametrize("name", list(CONFIGS))
+def test_one_launch_attention_step(dev, name):
+    """The step with rope + append + attention + merge as one launch per layer: logits and
+    appended cache rows within tolerance of the three-launch step and of the oracle; a
+    captured graph of it replays to the same bits."""
+    P, T = 200, 32
+    s = build(dev, name, P, T, seed=7)
+    base = run_verifier(s, dev, graph=False)
+    base.step()
+    s2 = build(dev, name, P, T, seed=7)
+    one = run_verifier(s2, dev, graph=False, one_launch_attention=True)
+    one.step()
+    torch.cuda.synchronize()
+    assert rel_err(one.logits.cpu().numpy(), base.logits.cpu().numpy()) <= TOL
+    want = model_oracle.verify_step(s["args"], s["weights"], s["inv"], s["sc"], s["tokens"], s["depth"],
+                                    s["parents"], s["anc"], s["ocache"], P)
+    assert rel_err(one.logits.cpu().numpy(), want["logits"]) <= TOL
+    s3 = build(dev, name, P, T, seed=7)
+    g = run_verifier(s3, dev, graph=True, one_launch_attention=True)
+    for rep in range(3):
+        s3["cache"][0].offset = P
+        s3["cache"][0].sync_len()
+        torch.cuda.synchronize()
+        g.step()
+        torch.cuda.synchronize()
+        assert torch.equal(g.logits, one.logits), f"replay {rep}"
+        assert torch.equal(g.result, one.result), f"replay {rep}"
+    for c, c2 in zip(s2["cache"], s3["cache"]):
+        assert torch.equal(c.keys, c2.keys) and torch.equal(c.values, c2.values)
 
 
 @pytest.mark.parametrize("name", list(CONFIGS))
