@@ -414,30 +414,50 @@ __global__ __launch_bounds__(1024) void qmm_w4g64_kernel(
     }
   } else {
     // ------------------------------------------------------------------ reducing wave
-    // A lane owns the same two float4 slots of every batch: slot l4 = (tile j of the batch,
-    // x block t, MFMA lane ln) holds out[16 t + 4 (ln / 16) + i][tile * 16 + ln % 16], i = 0..3.
-    // In the SwiGLU form the weight tiles alternate gate, up, gate, up ...; a lane then owns
-    // the two slots of one (gate, up) pair and stores fp16(fp16(silu(gate)) * up) instead.
-    const int wl = tid - nw * 64;     // 0 .. 127
+    // A batch is four 16 x 16 blocks (tile j of the batch, x block t), block jt = j * NT + t;
+    // MFMA lane ln of a block holds out[16 t + 4 (ln / 16) + i][tile * 16 + ln % 16], i = 0..3.
+    // Reducing wave ww owns MFMA lanes 32 ww .. 32 ww + 31 of every block, i.e. rows
+    // 16 t + 8 ww .. + 7 of all tiles of the batch: after a transpose through 1 KiB of LDS
+    // each of its lanes stores eight consecutive columns of one row (16 bytes), and the lanes
+    // of a row cover all tiles of the batch.  A lane sums two blocks per batch: with one x
+    // block (NT == 1) tiles it and it + 2 for the lane halves, with two (NT == 2) tile it of
+    // x block = lane half.  Either way a lane's two blocks are neighbouring tiles, which is
+    // what the SwiGLU form needs: gate in slot 0, up in slot 1.
+    const int ww = wave - nw;                 // 0 .. 1
+    const int hi = lane >> 5;
+    const int ln = (lane & 31) + 32 * ww;     // MFMA lane
+    const int rr0 = 4 * ((ln >> 4) & 1);      // first of this lane's four rows inside the wave's eight
+    const int cc = ln & 15;
     int sl_l4[2], sl_j[2];
-    half_t* sl_out[2];
     float* sl_part[2];
-    int sl_rows[2];
 #pragma unroll
     for (int it = 0; it < 2; ++it) {
-      int l4 = wl + it * 128;                  // 0 .. 255
-      if (swiglu && NT == 1) l4 = ((2 * (wl >> 6) + it) << 6) | (wl & 63);
-      const int jt = l4 >> 6;
-      const int t = jt % NT;
-      const int ln = l4 & 63;
-      const int m0 = 16 * t + 4 * (ln >> 4);
-      sl_l4[it] = l4;
-      sl_j[it] = jt / NT;
-      sl_out[it] = out + (size_t)m0 * (swiglu ? N >> 1 : N) + (ln & 15);
-      sl_rows[it] = M - m0;                    // rows m0 .. m0+3 exist while i < sl_rows
+      const int j = NT == 1 ? (swiglu ? 2 * hi + it : it + 2 * hi) : it;
+      const int t = NT == 1 ? 0 : hi;
+      sl_j[it] = j;
+      sl_l4[it] = (j * NT + t) * 64 + ln;
       // partial[slab][tile][t][i][64]
       sl_part[it] = partial + (((size_t)slab * tiles_total * NT + t) * 4) * 64 + ln;
     }
+    // Output staging of this wave: rows (t, rr) x the columns of the batch, fp16, 1 KiB.  It
+    // reuses the slots this wave has just summed: the halves (MFMA lanes 32 ww ..) of blocks
+    // 0 and 1 of the first streaming wave's partial, 512 bytes each, which nobody else reads
+    // and the streaming waves do not write again before the next barrier.
+    const int ocols = swiglu ? 8 * B : 16 * B;               // output columns per batch
+    constexpr int RPR = 4 * NT;                              // staged rows per 512-byte region
+    auto ost = [&](const float4_t* pb, int row, int col) -> half_t* {
+      unsigned char* base = reinterpret_cast<unsigned char*>(const_cast<float4_t*>(pb)) +
+                            ((row / RPR) * 64 + 32 * ww) * 16;
+      return reinterpret_cast<half_t*>(base) + (row % RPR) * ocols + col;
+    };
+    const int st_t = NT == 1 ? 0 : hi;
+    // where this lane's 16-byte piece of the staged rows goes
+    const int lpr = ocols / 8;                               // lanes per row
+    const int o_row = lane / lpr;                            // 0 .. 8 NT - 1 (when active)
+    const int o_col = (lane % lpr) * 8;
+    const bool o_active = lane < 8 * NT * lpr;
+    const int o_m = 16 * (o_row >> 3) + 8 * ww + (o_row & 7);
+    const int ldo = swiglu ? N >> 1 : N;
     lds_barrier();
     for (int ph = 0; ph < phases; ++ph) {
       for (int bi = 0; bi < nbp; ++bi) {
@@ -476,58 +496,66 @@ __global__ __launch_bounds__(1024) void qmm_w4g64_kernel(
           }
           sums[it] = sum;
         }
-        if (swiglu) {
-          // slots 0 and 1 of this lane are the gate tile and the up tile of one pair
-          if (live[0] && live[1]) {
-            const int pair = (tile0 + sl_j[0]) >> 1;
-            const int n_out = pair * 16 + (sl_l4[0] & 15);
-            const int n_g = (tile0 + sl_j[0]) * 16 + (sl_l4[0] & 15);
-            half_t* o = sl_out[0] + pair * 16;
-            if (n_g + 16 < N + 1 && n_out < (N >> 1)) {
-              half_t bg = (half_t)0.f, bu = (half_t)0.f;
-              if (bias) {
-                bg = bias[n_g];
-                bu = bias[n_g + 16];
-              }
+        if (!to_out) {
 #pragma unroll
-              for (int i = 0; i < 4; ++i)
-                if (i < sl_rows[0]) {
-                  half_t g = (half_t)sums[0][i], u = (half_t)sums[1][i];
-                  if (bias) {
-                    g = g + bg;
-                    u = u + bu;
-                  }
-                  const float gf = (float)g;
-                  const half_t a = (half_t)(gf / (1.0f + expf(-gf)));
-                  o[(size_t)i * (N >> 1)] = (half_t)((float)a * (float)u);
-                }
-            }
+          for (int it = 0; it < 2; ++it) {
+            if (!live[it]) continue;
+            float* dst = sl_part[it] + (size_t)(tile0 + sl_j[it]) * (NT * 256);
+#pragma unroll
+            for (int i = 0; i < 4; ++i)
+              __hip_atomic_store(dst + i * 64, sums[it][i], __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
           }
           continue;
         }
-#pragma unroll
-        for (int it = 0; it < 2; ++it) {
-          if (!live[it]) continue;
-          const int tile = tile0 + sl_j[it];
-          const float4_t sum = sums[it];
-          if (to_out) {
-            half_t* o = sl_out[it] + tile * 16;
-            if (tile * 16 + (sl_l4[it] & 15) < N) {
-              half_t bn = (half_t)0.f;
-              if (bias) bn = bias[tile * 16 + (sl_l4[it] & 15)];
-#pragma unroll
-              for (int i = 0; i < 4; ++i)
-                if (i < sl_rows[it]) {
-                  half_t r = (half_t)sum[i];
-                  if (bias) r = r + bn;
-                  o[(size_t)i * N] = r;
-                }
+        if (ph + 1 < phases) continue;
+        // fp16 results into the staging rows
+        if (swiglu) {
+          // slots 0 and 1 of this lane are the gate tile and the up tile of one pair
+          if (live[0] && live[1]) {
+            const int n_g = (tile0 + sl_j[0]) * 16 + cc;
+            half_t bg = (half_t)0.f, bu = (half_t)0.f;
+            if (bias && n_g + 16 < N) {
+              bg = bias[n_g];
+              bu = bias[n_g + 16];
             }
-          } else {
-            float* dst = sl_part[it] + (size_t)tile * (NT * 256);
+            const int pcol = (sl_j[0] >> 1) * 16 + cc;       // pair inside the batch
 #pragma unroll
-            for (int i = 0; i < 4; ++i)
-              __hip_atomic_store(dst + i * 64, sum[i], __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+            for (int i = 0; i < 4; ++i) {
+              half_t g = (half_t)sums[0][i], u = (half_t)sums[1][i];
+              if (bias) {
+                g = g + bg;
+                u = u + bu;
+              }
+              const float gf = (float)g;
+              const half_t a = (half_t)(gf / (1.0f + expf(-gf)));
+              *ost(pb, st_t * 8 + rr0 + i, pcol) = (half_t)((float)a * (float)u);
+            }
+          }
+        } else {
+#pragma unroll
+          for (int it = 0; it < 2; ++it) {
+            if (!live[it]) continue;
+            const int n = (tile0 + sl_j[it]) * 16 + cc;
+            half_t bn = (half_t)0.f;
+            if (bias && n < N) bn = bias[n];
+#pragma unroll
+            for (int i = 0; i < 4; ++i) {
+              half_t r = (half_t)sums[it][i];
+              if (bias) r = r + bn;
+              *ost(pb, st_t * 8 + rr0 + i, sl_j[it] * 16 + cc) = r;
+            }
+          }
+        }
+        // the staged rows are private to this wave: its own LDS writes are enough to wait for
+        asm volatile("s_waitcnt lgkmcnt(0)" ::: "memory");
+        if (o_active && o_m < M) {
+          // column of the piece in the output: tiles (or pairs) of the batch side by side
+          const int unit0 = swiglu ? tile0 >> 1 : tile0;
+          const int n0 = unit0 * 16 + o_col;
+          const int t_of = swiglu ? tile0 + 2 * (o_col >> 4) + 1 : tile0 + (o_col >> 4);
+          if (t_of < t_hi && n0 < ldo) {
+            const half8_t v = *reinterpret_cast<const half8_t*>(ost(pb, o_row, o_col));
+            *reinterpret_cast<half8_t*>(out + (size_t)o_m * ldo + n0) = v;
           }
         }
       }
@@ -548,34 +576,54 @@ __global__ __launch_bounds__(1024) void qmm_w4g64_kernel(
     }
     __syncthreads();
     if (*flag) {
+      // one thread per (tile, x block, row, half of the 16 columns): its eight values are
+      // consecutive floats of every slab's partial and become one 16-byte store
       const int per_tile = NT * 256;                       // floats
-      const int total = (t_hi - t_lo) * per_tile;
+      const int items = (t_hi - t_lo) * NT * 32;
       const size_t slab_stride = (size_t)tiles_total * per_tile;
-      for (int idx = tid; idx < total; idx += blockDim.x) {
-        const int tile = t_lo + idx / per_tile;
-        const int rem = idx % per_tile;                    // (t*4 + i)*64 + ln
-        const int ln = rem & 63;
-        const int ti = rem >> 6;
-        const int t = ti >> 2, i = ti & 3;
-        const float* src = partial + (size_t)tile * per_tile + rem;
-        float v = 0.f;
-        for (int sp0 = 0; sp0 < nsplit; sp0 += 8) {       // eight loads in flight, added in slab order
-          float pv[8];
+      for (int idx = tid; idx < items; idx += blockDim.x) {
+        const int tile = t_lo + idx / (NT * 32);
+        const int rem = idx % (NT * 32);
+        const int t = rem >> 5;
+        const int row = (rem >> 1) & 15;                   // row of the x block
+        const int hc = rem & 1;
+        const int m = 16 * t + row;
+        const int n0 = tile * 16 + 8 * hc;
+        // floats (t*4 + i)*64 + 16*rg + c with row = 4 rg + i, c = 8 hc .. 8 hc + 7
+        const float* src = partial + (size_t)tile * per_tile + (t * 4 + (row & 3)) * 64 + 16 * (row >> 2) + 8 * hc;
+        float v[8];
 #pragma unroll
-          for (int k = 0; k < 8; ++k) {
+        for (int e = 0; e < 8; ++e) v[e] = 0.f;
+        for (int sp0 = 0; sp0 < nsplit; sp0 += 4) {        // sixteen loads in flight, added in slab order
+          uint64_t pv[4][4];
+#pragma unroll
+          for (int k = 0; k < 4; ++k) {
             const int sp = sp0 + k < nsplit ? sp0 + k : nsplit - 1;
-            pv[k] = __hip_atomic_load(src + sp * slab_stride, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+            const uint64_t* q = reinterpret_cast<const uint64_t*>(src + sp * slab_stride);
+#pragma unroll
+            for (int e2 = 0; e2 < 4; ++e2)
+              pv[k][e2] = __hip_atomic_load(q + e2, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
           }
 #pragma unroll
-          for (int k = 0; k < 8; ++k)
-            if (sp0 + k < nsplit) v += pv[k];
+          for (int k = 0; k < 4; ++k)
+            if (sp0 + k < nsplit) {
+#pragma unroll
+              for (int e2 = 0; e2 < 4; ++e2) {
+                union { uint64_t u; float f[2]; } cv;
+                cv.u = pv[k][e2];
+                v[2 * e2] += cv.f[0];
+                v[2 * e2 + 1] += cv.f[1];
+              }
+            }
         }
-        const int n = tile * 16 + (ln & 15);
-        const int m = 16 * t + 4 * (ln >> 4) + i;
-        if (n < N && m < M) {
-          half_t o = (half_t)v;
-          if (bias) o = o + bias[n];
-          out[(size_t)m * N + n] = o;
+        if (n0 < N && m < M) {
+          half8_t o;
+#pragma unroll
+          for (int e = 0; e < 8; ++e) {
+            o[e] = (half_t)v[e];
+            if (bias) o[e] = o[e] + bias[n0 + e];
+          }
+          *reinterpret_cast<half8_t*>(out + (size_t)m * N + n0) = o;
         }
       }
     }
