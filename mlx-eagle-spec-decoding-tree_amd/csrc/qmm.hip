@@ -174,14 +174,6 @@ __global__ __launch_bounds__(1024) void qmm_w4g64_kernel(
       for (int ld = 0; ld < C::NL; ++ld) dst[ld] = *reinterpret_cast<const uint4_t*>(p + o[ld]);
     };
 
-    // The weight stream starts before anything else: the first tiles need several
-    // microseconds to arrive, and the rest of the prologue fits inside that wait.
-    uint32_t woff[C::NL];
-    unit_woff(unit0, woff);
-    uint4_t ring[C::RING][C::NL];
-#pragma unroll
-    for (int p = 0; p < C::RING; ++p) load_w(t_lo + p, woff, ring[p]);
-
     // ---- scale / bias staging: this thread's units of a batch (16*B rows x nw units x 2 arrays)
     const int nthr_s = nw * 64;
     int su_row[C::NSU], su_c[C::NSU], su_lds[C::NSU];
@@ -251,7 +243,23 @@ __global__ __launch_bounds__(1024) void qmm_w4g64_kernel(
     half8_t xop[NT][C::NMF];
     half8_t xaux[NT];
     const int hperm = ((h & 1) << 2) | (h & 2);          // 0, 4, 2, 6
-    auto load_x = [&](int unit) {
+    uint4_t xraw[NT][C::NMF];
+    auto x_issue = [&](int unit) {
+      const int col0 = unit * C::CW;
+#pragma unroll
+      for (int t = 0; t < NT; ++t)
+#pragma unroll
+        for (int j = 0; j < C::NMF; ++j) {
+          const int wi = 16 * (j >> 2) + 8 * ((j >> 1) & 1) + (j & 1) + hperm;
+          // out-of-range rows and columns read a valid address and are zeroed afterwards
+          int col = col0 + 8 * wi;
+          if (col > K - 8) col = K - 8;
+          int m = 16 * t + r;
+          if (m > M - 1) m = M - 1;
+          xraw[t][j] = *reinterpret_cast<const uint4_t*>(x + (size_t)m * K + col);
+        }
+    };
+    auto x_finish = [&](int unit) {
       const int col0 = unit * C::CW;
       float sE[NT][GW], sO[NT][GW];
 #pragma unroll
@@ -265,8 +273,8 @@ __global__ __launch_bounds__(1024) void qmm_w4g64_kernel(
           const int wi = 16 * (j >> 2) + 8 * ((j >> 1) & 1) + (j & 1) + hperm;
           const int col = col0 + 8 * wi;
           const int m = 16 * t + r;
-          uint4_t u = uint4_t{0u, 0u, 0u, 0u};
-          if (m < M && col < K) u = *reinterpret_cast<const uint4_t*>(x + (size_t)m * K + col);
+          uint4_t u = xraw[t][j];
+          if (!(m < M && col < K)) u = uint4_t{0u, 0u, 0u, 0u};
           uint4_t o;
           o[0] = __builtin_amdgcn_perm(u[2], u[0], 0x05040100u);   // (x0, x4)
           o[1] = __builtin_amdgcn_perm(u[2], u[0], 0x07060302u);   // (x1, x5)
@@ -299,15 +307,29 @@ __global__ __launch_bounds__(1024) void qmm_w4g64_kernel(
         xaux[t] = a;
       }
     };
+    auto load_x = [&](int unit) {
+      x_issue(unit);
+      x_finish(unit);
+    };
     const half2_t kmul = h == 0 ? half2_t{(half_t)1.f, (half_t)1.f} : half2_t{(half_t)64.f, (half_t)64.f};
 
-    // ---- prologue: batch 0 of scales / biases, x
+    // ---- prologue.  Loads retire in issue order, so the small ones go first: x (cached, it
+    // was just written) and the first scales / biases arrive while the weight ring, which
+    // takes microseconds to fill, is in flight, and the x operands are built in that shadow.
     stage_load(t_lo, 0, su_vals[0]);
     if (NT == 2) {
 #pragma unroll
       for (int q = 1; q < NSET; ++q) stage_load(t_lo + q * B < t_hi ? t_lo + q * B : t_lo, 0, su_vals[q]);
     }
-    load_x(unit0);
+    x_issue(unit0);
+    uint32_t woff[C::NL];
+    unit_woff(unit0, woff);
+    uint4_t ring[C::RING][C::NL];
+    __builtin_amdgcn_sched_barrier(0);      // keep the issue order: the scheduler would sink the ring
+#pragma unroll
+    for (int p = 0; p < C::RING; ++p) load_w(t_lo + p, woff, ring[p]);
+    __builtin_amdgcn_sched_barrier(0);
+    x_finish(unit0);
     stage_store(0, su_vals[0]);
     lds_barrier();
 
@@ -372,9 +394,11 @@ __global__ __launch_bounds__(1024) void qmm_w4g64_kernel(
     // ---- main loop over super-steps of RING tiles (ring slots are compile-time indices) and
     // phases.  Every load of the loop is unconditional: targets beyond the work are
     // redirected to addresses that are already cached.
+    // (the host guarantees at least one tile per workgroup and one phase: a loop that always
+    // runs once keeps the ring loads of the prologue where they are, before the x operands)
     const int nvs = phases * nss;
-    int ph = 0, ss = 0;
-    for (int vs = 0; vs < nvs; ++vs) {
+    int ph = 0, ss = 0, vs = 0;
+    do {
       const bool last_ss = ss == nss - 1;
       const bool more_phases = ph + 1 < phases;
       if (ss == 0 && ph > 0) load_x(unit0 + ph * nw);
@@ -411,7 +435,7 @@ __global__ __launch_bounds__(1024) void qmm_w4g64_kernel(
         ss = 0;
         ++ph;
       }
-    }
+    } while (++vs < nvs);
   } else {
     // ------------------------------------------------------------------ reducing wave
     // A batch is four 16 x 16 blocks (tile j of the batch, x block t), block jt = j * NT + t;
