@@ -701,9 +701,14 @@ void choose(int M, int N, int K, Launch* out) {
   const int units = (K + cw_of(M) - 1) / cw_of(M);
   const int tiles = (N + 15) / 16;
   Launch L;
-  int splits = (units + 2 * MAX_STREAM_WAVES - 1) / (2 * MAX_STREAM_WAVES);
+  // M <= 16: one phase only (a phase switch costs more than a K slab there)
+  const int phase_cap = M <= 16 ? 1 : 2;
+  int splits = (units + phase_cap * MAX_STREAM_WAVES - 1) / (phase_cap * MAX_STREAM_WAVES);
   int fill = tiles >= 160 ? 1 : (NUM_CU + tiles - 1) / tiles;
   if (fill > 4) fill = 4;
+  // M <= 16 with about one tile per compute unit: four slabs of a few waves, each walking
+  // several tiles, beat one slab of many waves that touches a single tile
+  if (M <= 16 && tiles < 3 * NUM_CU / 2 && units >= 8) fill = 4;
   if (splits < fill) splits = fill;
   // With only a few tiles per workgroup a second phase is mostly start-up latency (new x, a
   // cold ring); two K slabs on twice the workgroups finish sooner.
