@@ -158,15 +158,15 @@ int eagle_add_f16(const void* a, const void* b, void* out, long n, eagle_stream_
 int eagle_rope_table_f32(const int32_t* positions, const float* inv_freqs, float scaling_factor,
                          int T, int half_dim, float* out, eagle_stream_t stream);
 
-/* The attention block of one layer in one launch (mlx_llama.py:166-195: rope of q and k with
+/* The attention block of one layer without a separate rope launch (mlx_llama.py:166-195: rope of q and k with
  * per-token positions, cache update, masked SDPA).  q_lin / k_lin / v_lin are the token-major
  * projection outputs ([T, H*hd], [T, G*hd], [T, G*hd]) with a common row stride in elements
  * (columns of one fused q|k|v matrix, or row_stride = the width of each when separate and
  * equal).  Rotated keys and the values of the T tree tokens are written to cache rows
  * P .. P+T-1 (P = *cache_len_dev) and attended to together with the prefix under
- * tree_mask_bits, exactly as eagle_rope_kv_append_f16 followed by eagle_tree_attention_f16.
- * out [T, H*hd].  The first 256-byte multiple covering 4*H bytes of the workspace holds
- * arrival counters: zero before the first call, left zero by every call; calls sharing a
+ * tree_mask_bits, exactly as eagle_rope_kv_append_f16 followed by eagle_tree_attention_f16
+ * (one launch less: tree rows are read from the projections, rotated on the way, and stored
+ * to the cache by the workgroup that owns their key tile).  out [T, H*hd].  Calls sharing a
  * workspace must be stream ordered. */
 size_t eagle_tree_attention_rope_workspace_bytes(int H, int hd, int max_len);
 int eagle_tree_attention_rope_f16(const void* q_lin, const void* k_lin, const void* v_lin,

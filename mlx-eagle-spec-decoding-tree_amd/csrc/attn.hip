@@ -14,6 +14,10 @@
 // its partner lane+32 the other half of the keys), and feeds exp(S^T) straight back as
 // the B operand of O^T += V^T P^T; only V needs a transposed (16-bit) read from LDS.
 // Partial (m, l, O) per split go to a workspace and a second kernel merges them.
+//
+// A second form of the split kernel takes the un-rotated projection outputs instead
+// (mlx_llama.py:166-183): it rotates q and the tree keys itself and appends the tree rows to
+// the cache, which saves the separate rope / append launch.
 #include "common.h"
 
 #include <math.h>
@@ -22,19 +26,42 @@ namespace {
 
 constexpr int KT = 32;   // keys per tile
 
-template <int HD>
+// (lo, hi) = elements i0..i0+7 and i0+half..i0+half+7 of a head vector; cs = 8 (cos, sin) pairs
+__device__ inline void rotate_pair(half8_t& lo, half8_t& hi, const float* cs) {
+  float4_t c[4];
+#pragma unroll
+  for (int k = 0; k < 4; ++k) c[k] = *reinterpret_cast<const float4_t*>(cs + 4 * k);
+#pragma unroll
+  for (int j = 0; j < 8; ++j) {
+    const float co = c[j >> 1][(j & 1) * 2], sn = c[j >> 1][(j & 1) * 2 + 1];
+    const float x1 = (float)lo[j], x2 = (float)hi[j];
+    lo[j] = (half_t)(x1 * co - x2 * sn);
+    hi[j] = (half_t)(x1 * sn + x2 * co);
+  }
+}
+
+// ROPE = false: q [H,T,hd] is rotated already and the cache holds the tree rows.
+// ROPE = true: q, k_lin, v_lin are the token-major projection outputs (row stride ld); q and
+// the tree keys are rotated here with the cos/sin table rope_cs [T][hd/2][2], tree rows are
+// taken from k_lin / v_lin instead of the cache, and the workgroup that owns a tile with tree
+// rows appends them to the cache (every tile has exactly one owner per KV group, and no
+// workgroup reads a cache row at or beyond P, so the append races with nothing).
+template <int HD, bool ROPE>
 __global__ __launch_bounds__(512) void tree_attn_split_kernel(
-    const half_t* __restrict__ q, const half_t* __restrict__ kc, const half_t* __restrict__ vc,
+    const half_t* __restrict__ q, half_t* kc, half_t* vc,
     const uint32_t* __restrict__ mask_bits, const int32_t* __restrict__ len_dev,
     half_t* __restrict__ part_o, float* __restrict__ part_ml, int T, int H, int G, long cap,
-    int tiles_per_split, float scale_log2e) {
+    int tiles_per_split, float scale_log2e, const half_t* __restrict__ k_lin,
+    const half_t* __restrict__ v_lin, long ld, const float* __restrict__ rope_cs) {
   constexpr int KSTEPS = HD / 16;       // MFMA steps over the head dimension for S
   constexpr int DB = HD / 32;           // 32-wide blocks of the head dimension for O
   constexpr int STR = HD * 2 + 16;      // LDS row stride in bytes (pad: conflict-free reads)
   constexpr int VEC_ROW = HD / 8;       // 16-byte vectors per K/V row
   extern __shared__ __attribute__((aligned(16))) unsigned char lds[];
+  constexpr int HALF = HD / 2;
   unsigned char* ldsK = lds;
   unsigned char* ldsV = lds + KT * STR;
+  float* cs_lds = reinterpret_cast<float*>(lds + 2 * KT * STR);   // ROPE: [T][HALF][2]
 
   const int g = blockIdx.x;
   const int split = blockIdx.y;
@@ -48,15 +75,21 @@ __global__ __launch_bounds__(512) void tree_attn_split_kernel(
   const int hb = lane >> 5;             // which half of the k / key index this lane holds
   const int head = g * rep + wave;
 
-  const int P = *len_dev;
+  int P = *len_dev;
+  if (ROPE) {                           // never index past the cache, whatever the counter says
+    if (P > cap - T) P = (int)(cap - T);
+    if (P < 0) P = 0;
+  }
   const int Ltot = P + T;
   const int ntiles = (Ltot + KT - 1) / KT;
   half8_t qreg[KSTEPS];
 #pragma unroll
   for (int kk = 0; kk < KSTEPS; ++kk) {
     qreg[kk] = half8_t{0, 0, 0, 0, 0, 0, 0, 0};
-    if (ql < T)
-      qreg[kk] = *reinterpret_cast<const half8_t*>(q + ((long)head * T + ql) * HD + kk * 16 + hb * 8);
+    if (ql < T) {
+      const half_t* qp = ROPE ? q + (long)ql * ld + (long)head * HD : q + ((long)head * T + ql) * HD;
+      qreg[kk] = *reinterpret_cast<const half8_t*>(qp + kk * 16 + hb * 8);
+    }
   }
   const uint32_t mybits = ql < T ? mask_bits[ql] : 0u;
 
@@ -69,6 +102,8 @@ __global__ __launch_bounds__(512) void tree_attn_split_kernel(
 
   const half_t* kbase_ptr = kc + (long)g * cap * HD;
   const half_t* vbase_ptr = vc + (long)g * cap * HD;
+  const half_t* klin = ROPE ? k_lin + (long)g * HD : nullptr;
+  const half_t* vlin = ROPE ? v_lin + (long)g * HD : nullptr;
 
   // This workgroup's tiles are split, split + nsplit, ...: all workgroups share the live part
   // of the cache however short it is.  The next tile is fetched into registers while the
@@ -87,8 +122,14 @@ __global__ __launch_bounds__(512) void tree_attn_split_kernel(
       const int c = v % VEC_ROW;
       int kidx = kb + row;
       if (kidx > Ltot - 1) kidx = Ltot - 1;          // rows past the end are masked out below
-      kreg[it] = *reinterpret_cast<const half8_t*>(kbase_ptr + (long)kidx * HD + c * 8);
-      vreg[it] = *reinterpret_cast<const half8_t*>(vbase_ptr + (long)kidx * HD + c * 8);
+      const half_t* kp = kbase_ptr + (long)kidx * HD;
+      const half_t* vp = vbase_ptr + (long)kidx * HD;
+      if (ROPE && kidx >= P) {
+        kp = klin + (long)(kidx - P) * ld;
+        vp = vlin + (long)(kidx - P) * ld;
+      }
+      kreg[it] = *reinterpret_cast<const half8_t*>(kp + c * 8);
+      vreg[it] = *reinterpret_cast<const half8_t*>(vp + c * 8);
     }
   };
   auto stash = [&]() {
@@ -106,12 +147,52 @@ __global__ __launch_bounds__(512) void tree_attn_split_kernel(
   };
 
   if (split < ntiles) fetch(split);
+  if (ROPE) {
+    for (int v = tid; v < T * HALF / 2; v += nthr)
+      *reinterpret_cast<float4_t*>(cs_lds + 4 * v) = *reinterpret_cast<const float4_t*>(rope_cs + 4 * v);
+    __syncthreads();
+    if (ql < T) {
+#pragma unroll
+      for (int kk = 0; kk < KSTEPS / 2; ++kk)
+        rotate_pair(qreg[kk], qreg[kk + KSTEPS / 2], cs_lds + (ql * HALF + kk * 16 + hb * 8) * 2);
+    }
+  }
   for (int tile = split; tile < ntiles; tile += nsplit) {
     const int kb = tile * KT;
     __syncthreads();   // every wave is done with the previous tile
+    if (ROPE && kb + KT > P) {
+      // tree rows: append the values as they are
+#pragma unroll
+      for (int it = 0; it < NV; ++it) {
+        if (it * nthr >= NVEC) break;
+        const int v = tid + it * nthr;
+        const int kidx = kb + v / VEC_ROW;
+        if (v < NVEC && kidx >= P && kidx < Ltot)
+          *reinterpret_cast<half8_t*>(vc + ((long)g * cap + kidx) * HD + (v % VEC_ROW) * 8) = vreg[it];
+      }
+    }
     stash();
     if (tile + nsplit < ntiles) fetch(tile + nsplit);
     __syncthreads();
+    if (ROPE && kb + KT > P) {
+      // rotate the tree keys in LDS (one thread per pair of 16-byte pieces) and append them
+      for (int v = tid; v < KT * (VEC_ROW / 2); v += nthr) {
+        const int row = v / (VEC_ROW / 2);
+        const int c = v % (VEC_ROW / 2);
+        const int kidx = kb + row;
+        if (kidx >= P && kidx < Ltot) {
+          half8_t lo = *reinterpret_cast<const half8_t*>(ldsK + row * STR + c * 16);
+          half8_t hi = *reinterpret_cast<const half8_t*>(ldsK + row * STR + (c + VEC_ROW / 2) * 16);
+          rotate_pair(lo, hi, cs_lds + ((kidx - P) * HALF + c * 8) * 2);
+          *reinterpret_cast<half8_t*>(ldsK + row * STR + c * 16) = lo;
+          *reinterpret_cast<half8_t*>(ldsK + row * STR + (c + VEC_ROW / 2) * 16) = hi;
+          half_t* dst = kc + ((long)g * cap + kidx) * HD;
+          *reinterpret_cast<half8_t*>(dst + c * 8) = lo;
+          *reinterpret_cast<half8_t*>(dst + HALF + c * 8) = hi;
+        }
+      }
+      __syncthreads();
+    }
 
     // S^T[key][token] = sum_d K[key][d] Q[token][d]
     float16_t sacc;
@@ -263,6 +344,37 @@ int splits_for(int max_len, int G) {
   return n;
 }
 
+template <int HD, bool ROPE>
+int launch_attention(const half_t* q, half_t* kc, half_t* vc, const uint32_t* bits, const int32_t* len,
+                     void* out, int T, int H, int G, long cap, int max_len, float scale, void* workspace,
+                     const half_t* k_lin, const half_t* v_lin, long ld, const float* cs, hipStream_t st) {
+  const int nsplit = splits_for(max_len, G);
+  float* part_ml = static_cast<float*>(workspace);
+  half_t* part_o = reinterpret_cast<half_t*>(part_ml + (size_t)H * nsplit * 32 * 2);
+  const float sl2 = scale * 1.4426950408889634f;
+  const int rep = H / G;
+  const size_t lds = 2 * KT * (HD * 2 + 16) + (ROPE ? (size_t)EAGLE_MAX_TREE * HD * 4 : 0);
+  hipLaunchKernelGGL((tree_attn_split_kernel<HD, ROPE>), dim3(G, nsplit), dim3(rep * 64), lds, st, q, kc,
+                     vc, bits, len, part_o, part_ml, T, H, G, cap, 0, sl2, k_lin, v_lin, ld, cs);
+  hipLaunchKernelGGL(tree_attn_merge_kernel<HD>, dim3(H, (T + MERGE_TOK - 1) / MERGE_TOK),
+                     dim3(MERGE_TOK * HD / 4), 0, st, part_o, part_ml, (half_t*)out, T, H, nsplit);
+  return eagle_launch_status();
+}
+
+__global__ void rope_table_kernel(const int32_t* __restrict__ pos, const float* __restrict__ inv_freq,
+                                  float scale, float* __restrict__ out, int T, int half) {
+  const int idx = blockIdx.x * blockDim.x + threadIdx.x;
+  if (idx >= T * half) return;
+  const int i = idx % half;
+  const int t = idx / half;
+  const float lf = scale * inv_freq[i];
+  const float theta = lf * (float)pos[t];
+  float sn, cs;
+  sincosf(theta, &sn, &cs);
+  out[2 * idx] = cs;
+  out[2 * idx + 1] = sn;
+}
+
 }  // namespace
 
 EAGLE_EXPORT size_t eagle_tree_attention_workspace_bytes(int H, int hd, int max_len) {
@@ -286,26 +398,64 @@ EAGLE_EXPORT int eagle_tree_attention_f16(const void* q, const void* k_cache, co
   if (!workspace || !eagle_aligned16(workspace) ||
       workspace_bytes < eagle_tree_attention_workspace_bytes(H, hd, max_len))
     return EAGLE_ERR_WORKSPACE;
-  const int nsplit = splits_for(max_len, G);
-  const int tps = 0;
-  float* part_ml = static_cast<float*>(workspace);
-  half_t* part_o = reinterpret_cast<half_t*>(part_ml + (size_t)H * nsplit * 32 * 2);
-  const float sl2 = scale * 1.4426950408889634f;
-  const int rep = H / G;
   hipStream_t st = static_cast<hipStream_t>(stream);
-  const size_t lds = 2 * KT * (hd * 2 + 16);
-  if (hd == 128) {
-    hipLaunchKernelGGL(tree_attn_split_kernel<128>, dim3(G, nsplit), dim3(rep * 64), lds, st,
-                       (const half_t*)q, (const half_t*)k_cache, (const half_t*)v_cache,
-                       tree_mask_bits, cache_len_dev, part_o, part_ml, T, H, G, capacity, tps, sl2);
-    hipLaunchKernelGGL(tree_attn_merge_kernel<128>, dim3(H, (T + MERGE_TOK - 1) / MERGE_TOK),
-                       dim3(MERGE_TOK * 32), 0, st, part_o, part_ml, (half_t*)out, T, H, nsplit);
-  } else {
-    hipLaunchKernelGGL(tree_attn_split_kernel<64>, dim3(G, nsplit), dim3(rep * 64), lds, st,
-                       (const half_t*)q, (const half_t*)k_cache, (const half_t*)v_cache,
-                       tree_mask_bits, cache_len_dev, part_o, part_ml, T, H, G, capacity, tps, sl2);
-    hipLaunchKernelGGL(tree_attn_merge_kernel<64>, dim3(H, (T + MERGE_TOK - 1) / MERGE_TOK),
-                       dim3(MERGE_TOK * 16), 0, st, part_o, part_ml, (half_t*)out, T, H, nsplit);
-  }
+  // the kernel only reads the caches in this form
+  half_t* kc = const_cast<half_t*>(static_cast<const half_t*>(k_cache));
+  half_t* vc = const_cast<half_t*>(static_cast<const half_t*>(v_cache));
+  if (hd == 128)
+    return launch_attention<128, false>((const half_t*)q, kc, vc, tree_mask_bits, cache_len_dev, out, T, H,
+                                        G, capacity, max_len, scale, workspace, nullptr, nullptr, 0,
+                                        nullptr, st);
+  return launch_attention<64, false>((const half_t*)q, kc, vc, tree_mask_bits, cache_len_dev, out, T, H, G,
+                                     capacity, max_len, scale, workspace, nullptr, nullptr, 0, nullptr, st);
+}
+
+EAGLE_EXPORT int eagle_rope_table_f32(const int32_t* positions, const float* inv_freqs,
+                                      float scaling_factor, int T, int half_dim, float* out,
+                                      eagle_stream_t stream) {
+  if (!positions || !inv_freqs || !out) return EAGLE_ERR_NULL;
+  if (T < 1 || T > EAGLE_MAX_TREE || half_dim < 1) return EAGLE_ERR_SHAPE;
+  if (!eagle_aligned16(out)) return EAGLE_ERR_ALIGN;
+  const int total = T * half_dim;
+  hipLaunchKernelGGL(rope_table_kernel, dim3((total + 255) / 256), dim3(256), 0,
+                     static_cast<hipStream_t>(stream), positions, inv_freqs, scaling_factor, out, T,
+                     half_dim);
   return eagle_launch_status();
+}
+
+EAGLE_EXPORT size_t eagle_tree_attention_rope_workspace_bytes(int H, int hd, int max_len) {
+  return eagle_tree_attention_workspace_bytes(H, hd, max_len);
+}
+
+EAGLE_EXPORT int eagle_tree_attention_rope_f16(const void* q_lin, const void* k_lin, const void* v_lin,
+                                               long row_stride, const float* rope_cs, void* k_cache,
+                                               void* v_cache, const uint32_t* tree_mask_bits,
+                                               const int32_t* cache_len_dev, void* out, int T, int H,
+                                               int G, int hd, long capacity, int max_len, float scale,
+                                               void* workspace, size_t workspace_bytes,
+                                               eagle_stream_t stream) {
+  if (!q_lin || !k_lin || !v_lin || !rope_cs || !k_cache || !v_cache || !tree_mask_bits ||
+      !cache_len_dev || !out)
+    return EAGLE_ERR_NULL;
+  if (T < 1 || T > EAGLE_MAX_TREE || H < 1 || G < 1 || (H % G) != 0 || (H / G) > 8 ||
+      (hd != 64 && hd != 128) || max_len < T || max_len > capacity || row_stride < hd ||
+      (row_stride % 8) != 0)
+    return EAGLE_ERR_SHAPE;
+  if (!eagle_aligned16(q_lin) || !eagle_aligned16(k_lin) || !eagle_aligned16(v_lin) ||
+      !eagle_aligned16(rope_cs) || !eagle_aligned16(k_cache) || !eagle_aligned16(v_cache) ||
+      !eagle_aligned16(out))
+    return EAGLE_ERR_ALIGN;
+  if (!workspace || !eagle_aligned16(workspace) ||
+      workspace_bytes < eagle_tree_attention_rope_workspace_bytes(H, hd, max_len))
+    return EAGLE_ERR_WORKSPACE;
+  hipStream_t st = static_cast<hipStream_t>(stream);
+  if (hd == 128)
+    return launch_attention<128, true>((const half_t*)q_lin, (half_t*)k_cache, (half_t*)v_cache,
+                                       tree_mask_bits, cache_len_dev, out, T, H, G, capacity, max_len, scale,
+                                       workspace, (const half_t*)k_lin, (const half_t*)v_lin, row_stride,
+                                       rope_cs, st);
+  return launch_attention<64, true>((const half_t*)q_lin, (half_t*)k_cache, (half_t*)v_cache,
+                                    tree_mask_bits, cache_len_dev, out, T, H, G, capacity, max_len, scale,
+                                    workspace, (const half_t*)k_lin, (const half_t*)v_lin, row_stride,
+                                    rope_cs, st);
 }

@@ -186,8 +186,8 @@ class TreeVerifier:
         self.fuse = fuse
         # gate|up with the SwiGLU epilogue when the matmul covers the shape in one K slab
         self.swiglu = bool(fuse and swiglu and ops.swiglu_supported(T, I, D))
-        # rope + KV append + attention + split merge as one launch instead of three: as fast
-        # inside a graph for prefixes of a few thousand rows, fewer launches outside one
+        # rope and KV append inside the attention launch instead of a launch of their own (as
+        # fast inside a captured graph, one launch less per layer outside one)
         self.one_launch_attention = bool(fuse and one_launch_attention)
         if fuse:
             self._fuse_projections()

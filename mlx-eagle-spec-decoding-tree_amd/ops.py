@@ -254,7 +254,7 @@ def rope_table(positions, inv_freqs, scaling_factor=1.0, out=None):
 
 def tree_attention_rope(q_lin, k_lin, v_lin, rope_cs, k_cache, v_cache, tree_mask_bits,
                         cache_len_dev, scale, H, G, hd, row_stride=0, max_len=None, out=None):
-    """`rope_kv_append` + `tree_attention` in one launch: q_lin [T,H*hd], k_lin / v_lin [T,G*hd]
+    """`rope_kv_append` + `tree_attention` without the rope launch: q_lin [T,H*hd], k_lin / v_lin [T,G*hd]
     (row_stride > 0: column blocks of one [T,row_stride] matrix), rope_cs from `rope_table`.
     Appends the rotated keys and the values to cache rows P..P+T-1 and returns [T, H*hd]."""
     _need_cuda(q_lin, k_lin, v_lin, rope_cs, k_cache, v_cache, tree_mask_bits, cache_len_dev)

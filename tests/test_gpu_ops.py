@@ -159,8 +159,8 @@ def test_sdpa_signature(dev):
                                         (14, 2, 64, 515, 32), (32, 8, 128, 100, 8), (4, 2, 64, 0, 16),
                                         (8, 8, 128, 31, 24), (4, 4, 64, 7, 1)])
 def test_tree_attention_rope_one_launch(dev, H, G, hd, P, T):
-    """rope(q, k) + cache append + tree attention + split merge in one launch: against the
-    oracle's rope -> append -> attention, and against the two-launch device path."""
+    """rope(q, k) + cache append inside the attention launch: against the oracle's
+    rope -> append -> attention, and against the device path with a separate rope launch."""
     print(f"attn+rope H={H} G={G} hd={hd} P={P} T={T}", flush=True)
     rng = np.random.default_rng(H + P + T + 1)
     cap = P + T + 13
@@ -216,8 +216,7 @@ def test_tree_attention_rope_one_launch(dev, H, G, hd, P, T):
 
 
 def test_tree_attention_rope_repeated_calls_share_workspace(dev):
-    """The arrival counters in the workspace return to zero: a second call with another
-    length gives the right answer too."""
+    """Calls with different lengths share one workspace."""
     rng = np.random.default_rng(5)
     H, G, hd, T = 8, 2, 64, 32
     cap = 700
