@@ -156,22 +156,31 @@ __global__ __launch_bounds__(1024) void qmm_w4g64_kernel(
     const uint32_t row_bytes = (uint32_t)K8 * 4u;
     const int unit0 = slab * phases * nw + wave;            // this wave's unit in phase 0
 
-    // byte offset of this lane's words inside a weight row, clamped into the row
-    auto unit_woff = [&](int unit, uint32_t (&o)[C::NL]) {
+    // Weight addresses are (uniform tile base) + (32-bit lane offset), which the loads take as
+    // scalar base + vector offset: no per-tile address arithmetic in the vector unit.  The lane
+    // offset is row-in-tile * row bytes + the byte offset of this lane's words inside the row
+    // (clamped into the row); it changes only with the column unit.  Rows past N in a last,
+    // partial tile read the last row instead.
+    const int rows_last = N - 16 * (tiles_total - 1);                 // 8 or 16
+    const uint32_t r_last = (uint32_t)(r < rows_last ? r : rows_last - 1);
+    auto unit_woff = [&](int unit, uint32_t (&o)[2 * C::NL]) {
 #pragma unroll
       for (int ld = 0; ld < C::NL; ++ld) {
         int word = unit * (C::CW / 8) + ld * 16 + h * 4;
         if (word > K8 - 4) word = K8 - 4;
-        o[ld] = (uint32_t)word * 4u;
+        o[ld] = (uint32_t)r * row_bytes + (uint32_t)word * 4u;
+        o[C::NL + ld] = r_last * row_bytes + (uint32_t)word * 4u;
       }
     };
-    auto load_w = [&](int tile, const uint32_t (&o)[C::NL], uint4_t (&dst)[C::NL]) {
-      int t = tile < t_hi ? tile : t_hi - 1;
-      int row = t * 16 + r;
-      if (row > N - 1) row = N - 1;
-      const unsigned char* p = reinterpret_cast<const unsigned char*>(w) + (uint32_t)row * row_bytes;
+    const unsigned char* wbytes = reinterpret_cast<const unsigned char*>(w);
+    const size_t tile_bytes = (size_t)16 * row_bytes;
+    auto load_w = [&](int tile, const uint32_t (&o)[2 * C::NL], uint4_t (&dst)[C::NL]) {
+      const int t = tile < t_hi ? tile : t_hi - 1;
+      const unsigned char* tb = wbytes + (size_t)t * tile_bytes;      // uniform
+      const bool last = t == tiles_total - 1;                         // uniform
 #pragma unroll
-      for (int ld = 0; ld < C::NL; ++ld) dst[ld] = *reinterpret_cast<const uint4_t*>(p + o[ld]);
+      for (int ld = 0; ld < C::NL; ++ld)
+        dst[ld] = *reinterpret_cast<const uint4_t*>(tb + (last ? o[C::NL + ld] : o[ld]));
     };
 
     // ---- scale / bias staging: this thread's units of a batch (16*B rows x nw units x 2 arrays)
@@ -322,7 +331,7 @@ __global__ __launch_bounds__(1024) void qmm_w4g64_kernel(
       for (int q = 1; q < NSET; ++q) stage_load(t_lo + q * B < t_hi ? t_lo + q * B : t_lo, 0, su_vals[q]);
     }
     x_issue(unit0);
-    uint32_t woff[C::NL];
+    uint32_t woff[2 * C::NL];
     unit_woff(unit0, woff);
     uint4_t ring[C::RING][C::NL];
     __builtin_amdgcn_sched_barrier(0);      // keep the issue order: the scheduler would sink the ring
