@@ -82,7 +82,7 @@ int eagle_qmm_w4g64_f16_tuned(const void* x, const uint32_t* wq, const void* sca
  * rows interleaved in 16-row tiles: gate rows 0..15, up rows 0..15, gate rows 16..31, ...
  * (N = 2 * intermediate size, N % 32 == 0).  out [M, N/2] = fp16(fp16(silu(g)) * u) with
  * g, u the fp16 results of the two projections, i.e. the values the separate launches and
- * eagle_silu_mul_f16 produce.  EAGLE_ERR_UNSUPPORTED when the shape would need K slabs. */
+ * eagle_silu_mul_f16 produce.  Workspace as for eagle_qmm_w4g64_f16 with the same M, N, K. */
 int eagle_qmm_swiglu_w4g64_f16(const void* x, const uint32_t* wq, const void* scales,
                                const void* biases, const void* bias, void* out,
                                int M, int N, int K, int group_size, int bits,

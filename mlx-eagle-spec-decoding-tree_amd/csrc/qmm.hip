@@ -610,21 +610,12 @@ __global__ __launch_bounds__(1024) void qmm_w4g64_kernel(
     __syncthreads();
     if (*flag) {
       // one thread per (tile, x block, row, half of the 16 columns): its eight values are
-      // consecutive floats of every slab's partial and become one 16-byte store
+      // consecutive floats of every slab's partial and become one 16-byte store.  In the
+      // SwiGLU form an item is a (gate, up) tile pair and the store is the activation.
       const int per_tile = NT * 256;                       // floats
-      const int items = (t_hi - t_lo) * NT * 32;
+      const int items = ((t_hi - t_lo) / gran) * NT * 32;
       const size_t slab_stride = (size_t)tiles_total * per_tile;
-      for (int idx = tid; idx < items; idx += blockDim.x) {
-        const int tile = t_lo + idx / (NT * 32);
-        const int rem = idx % (NT * 32);
-        const int t = rem >> 5;
-        const int row = (rem >> 1) & 15;                   // row of the x block
-        const int hc = rem & 1;
-        const int m = 16 * t + row;
-        const int n0 = tile * 16 + 8 * hc;
-        // floats (t*4 + i)*64 + 16*rg + c with row = 4 rg + i, c = 8 hc .. 8 hc + 7
-        const float* src = partial + (size_t)tile * per_tile + (t * 4 + (row & 3)) * 64 + 16 * (row >> 2) + 8 * hc;
-        float v[8];
+      auto sum_slabs = [&](const float* src, float (&v)[8]) {
 #pragma unroll
         for (int e = 0; e < 8; ++e) v[e] = 0.f;
         for (int sp0 = 0; sp0 < nsplit; sp0 += 4) {        // sixteen loads in flight, added in slab order
@@ -649,7 +640,38 @@ __global__ __launch_bounds__(1024) void qmm_w4g64_kernel(
               }
             }
         }
-        if (n0 < N && m < M) {
+      };
+      for (int idx = tid; idx < items; idx += blockDim.x) {
+        const int tile = t_lo + gran * (idx / (NT * 32));
+        const int rem = idx % (NT * 32);
+        const int t = rem >> 5;
+        const int row = (rem >> 1) & 15;                   // row of the x block
+        const int hc = rem & 1;
+        const int m = 16 * t + row;
+        const int n0 = tile * 16 + 8 * hc;
+        // floats (t*4 + i)*64 + 16*rg + c with row = 4 rg + i, c = 8 hc .. 8 hc + 7
+        const float* src = partial + (size_t)tile * per_tile + (t * 4 + (row & 3)) * 64 + 16 * (row >> 2) + 8 * hc;
+        float v[8];
+        sum_slabs(src, v);
+        if (swiglu) {
+          float u[8];
+          sum_slabs(src + per_tile, u);                    // the up tile follows the gate tile
+          if (n0 + 16 < N + 8 && m < M) {
+            half8_t o;
+#pragma unroll
+            for (int e = 0; e < 8; ++e) {
+              half_t g = (half_t)v[e], uu = (half_t)u[e];
+              if (bias) {
+                g = g + bias[n0 + e];
+                uu = uu + bias[n0 + 16 + e];
+              }
+              const float gf = (float)g;
+              const half_t a = (half_t)(gf / (1.0f + expf(-gf)));
+              o[e] = (half_t)((float)a * (float)uu);
+            }
+            *reinterpret_cast<half8_t*>(out + (size_t)m * (N >> 1) + (tile >> 1) * 16 + 8 * hc) = o;
+          }
+        } else if (n0 < N && m < M) {
           half8_t o;
 #pragma unroll
           for (int e = 0; e < 8; ++e) {
@@ -719,9 +741,9 @@ void choose(int M, int N, int K, Launch* out) {
   // several tiles, beat one slab of many waves that touches a single tile
   if (M <= 16 && tiles < 3 * NUM_CU / 2 && units >= 8) fill = 4;
   if (splits < fill) splits = fill;
-  // With only a few tiles per workgroup a second phase is mostly start-up latency (new x, a
-  // cold ring); two K slabs on twice the workgroups finish sooner.
-  if (splits == 1 && units > MAX_STREAM_WAVES && tiles < 4 * NUM_CU) splits = 2;
+  // A second phase costs a drained ring and a reload of x; unless the partials would be a
+  // large matrix of their own (very many tiles), two K slabs finish sooner.
+  if (splits == 1 && units > MAX_STREAM_WAVES && tiles < 16 * NUM_CU) splits = 2;
   if (splits > units) splits = units;
   int per_slab = (units + splits - 1) / splits;
   L.phases = (per_slab + MAX_STREAM_WAVES - 1) / MAX_STREAM_WAVES;
@@ -866,7 +888,6 @@ EAGLE_EXPORT int eagle_qmm_swiglu_w4g64_f16(const void* x, const uint32_t* wq, c
   if ((N % 32) != 0) return EAGLE_ERR_SHAPE;             // whole (gate, up) tile pairs
   Launch L;
   choose(M, N, K, &L);
-  if (L.splits != 1) return EAGLE_ERR_UNSUPPORTED;       // the activation needs the complete sum
   if (L.ranges > N / 32) L.ranges = N / 32;
   rc = validate_launch(M, N, K, L, 2);
   if (rc != EAGLE_OK) return rc;

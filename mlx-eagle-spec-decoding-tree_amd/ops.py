@@ -119,8 +119,8 @@ def interleave_gate_up(gate, up):
 
 
 def swiglu_supported(M, I, K):
-    """True when the SwiGLU matmul covers this shape (whole tile pairs, no K slabs)."""
-    return I % 16 == 0 and 1 <= M <= 32 and qmm_plan(M, 2 * I, K)[2] == 1
+    """True when the SwiGLU matmul covers this shape (whole (gate, up) tile pairs)."""
+    return I % 16 == 0 and 1 <= M <= 32 and K % 64 == 0
 
 
 def quantized_matmul_swiglu(x, w_q, scales, biases, bias=None, out=None):

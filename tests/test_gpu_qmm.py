@@ -171,11 +171,22 @@ def test_swiglu_form_equals_separate_launches(dev, I, K, bias):
         assert rel_err(got.cpu().numpy(), want) <= TOL
 
 
-def test_swiglu_form_refuses_k_slabs(dev):
+def test_swiglu_form_with_k_slabs(dev):
+    """Shapes whose launch uses K slabs: the last workgroup of a tile range applies the activation."""
     rng = np.random.default_rng(1)
-    g = layer_to_dev(synth.make_qlinear(rng, 32, 8192), dev)
-    assert not ops.swiglu_supported(8, 32, 8192)
-    w = {k: ops.interleave_gate_up(g[k], g[k]) for k in ("weight", "scales", "biases")}
-    with pytest.raises(ValueError):
-        ops.quantized_matmul_swiglu(to_dev(synth.make_x(rng, 8, 8192), dev), w["weight"], w["scales"],
-                                    w["biases"])
+    for M, I, K in ((8, 32, 8192), (32, 48, 7168), (17, 1024, 3584)):
+        assert ops.qmm_plan(M, 2 * I, K)[2] > 1
+        g = synth.make_qlinear(rng, I, K, bias=True, gain=1.0)
+        u = synth.make_qlinear(rng, I, K, bias=True, gain=1.0)
+        x = synth.make_x(rng, M, K)
+        want = oracle.silu_mul(oracle.qmm(x, g["weight"], g["scales"], g["biases"], g["bias"]),
+                               oracle.qmm(x, u["weight"], u["scales"], u["biases"], u["bias"]))
+        gd, ud = layer_to_dev(g, dev), layer_to_dev(u, dev)
+        inter = {k: ops.interleave_gate_up(gd[k], ud[k]) for k in ("weight", "scales", "biases", "bias")}
+        cat = {k: torch.cat([gd[k], ud[k]]).contiguous() for k in ("weight", "scales", "biases", "bias")}
+        xd = to_dev(x, dev)
+        got = ops.quantized_matmul_swiglu(xd, inter["weight"], inter["scales"], inter["biases"], bias=inter["bias"])
+        two = ops.silu_mul(ops.quantized_matmul(xd, cat["weight"], cat["scales"], cat["biases"], bias=cat["bias"]))
+        torch.cuda.synchronize()
+        assert torch.equal(got, two), f"M={M} I={I} K={K}"
+        assert rel_err(got.cpu().numpy(), want) <= TOL
