@@ -46,7 +46,7 @@ __device__ inline void rotate_pair(half8_t& lo, half8_t& hi, const float* cs) {
 // taken from k_lin / v_lin instead of the cache, and the workgroup that owns a tile with tree
 // rows appends them to the cache (every tile has exactly one owner per KV group, and no
 // workgroup reads a cache row at or beyond P, so the append races with nothing).
-template <int HD, bool ROPE, int NV>
+template <int HD, bool ROPE>
 __global__ __launch_bounds__(512) void tree_attn_split_kernel(
     const half_t* __restrict__ q, half_t* kc, half_t* vc,
     const uint32_t* __restrict__ mask_bits, const int32_t* __restrict__ len_dev,
@@ -109,13 +109,13 @@ __global__ __launch_bounds__(512) void tree_attn_split_kernel(
   // of the cache however short it is.  The next tile is fetched into registers while the
   // current one is being used.
   constexpr int NVEC = KT * VEC_ROW;                 // 16-byte vectors per K (or V) tile
-  // NV (template): vectors per thread, NV * blockDim.x >= NVEC
-  constexpr bool TWO = NV <= 4;                      // a second tile in flight when it fits the registers
-  half8_t kregA[NV], vregA[NV], kregB[TWO ? NV : 1], vregB[TWO ? NV : 1];
-  auto fetch = [&](int tile, auto& kreg, auto& vreg) {
+  constexpr int NV = NVEC / 64;                      // per thread, for as little as one wave
+  half8_t kreg[NV], vreg[NV];
+  auto fetch = [&](int tile) {
     const int kb = tile * KT;
 #pragma unroll
     for (int it = 0; it < NV; ++it) {
+      if (it * nthr >= NVEC) break;
       int v = tid + it * nthr;
       if (v > NVEC - 1) v = NVEC - 1;
       const int row = v / VEC_ROW;
@@ -132,9 +132,10 @@ __global__ __launch_bounds__(512) void tree_attn_split_kernel(
       vreg[it] = *reinterpret_cast<const half8_t*>(vp + c * 8);
     }
   };
-  auto stash = [&](const auto& kreg, const auto& vreg) {
+  auto stash = [&]() {
 #pragma unroll
     for (int it = 0; it < NV; ++it) {
+      if (it * nthr >= NVEC) break;
       const int v = tid + it * nthr;
       if (v < NVEC) {
         const int row = v / VEC_ROW;
@@ -145,11 +146,7 @@ __global__ __launch_bounds__(512) void tree_attn_split_kernel(
     }
   };
 
-  // two tiles in flight: sets A and B are refilled as soon as their tile sits in LDS
-  if (split < ntiles) fetch(split, kregA, vregA);
-  if constexpr (TWO) {
-    if (split + nsplit < ntiles) fetch(split + nsplit, kregB, vregB);
-  }
+  if (split < ntiles) fetch(split);
   if (ROPE) {
     for (int v = tid; v < T * HALF / 2; v += nthr)
       *reinterpret_cast<float4_t*>(cs_lds + 4 * v) = *reinterpret_cast<const float4_t*>(rope_cs + 4 * v);
@@ -160,22 +157,22 @@ __global__ __launch_bounds__(512) void tree_attn_split_kernel(
         rotate_pair(qreg[kk], qreg[kk + KSTEPS / 2], cs_lds + (ql * HALF + kk * 16 + hb * 8) * 2);
     }
   }
-  constexpr int AHEAD = TWO ? 2 : 1;
-  auto process = [&](int tile, auto& kreg, auto& vreg) {
+  for (int tile = split; tile < ntiles; tile += nsplit) {
     const int kb = tile * KT;
     __syncthreads();   // every wave is done with the previous tile
     if (ROPE && kb + KT > P) {
       // tree rows: append the values as they are
 #pragma unroll
       for (int it = 0; it < NV; ++it) {
-          const int v = tid + it * nthr;
+        if (it * nthr >= NVEC) break;
+        const int v = tid + it * nthr;
         const int kidx = kb + v / VEC_ROW;
         if (v < NVEC && kidx >= P && kidx < Ltot)
           *reinterpret_cast<half8_t*>(vc + ((long)g * cap + kidx) * HD + (v % VEC_ROW) * 8) = vreg[it];
       }
     }
-    stash(kreg, vreg);
-    if (tile + AHEAD * nsplit < ntiles) fetch(tile + AHEAD * nsplit, kreg, vreg);
+    stash();
+    if (tile + nsplit < ntiles) fetch(tile + nsplit);
     __syncthreads();
     if (ROPE && kb + KT > P) {
       // rotate the tree keys in LDS (one thread per pair of 16-byte pieces) and append them
@@ -262,12 +259,6 @@ __global__ __launch_bounds__(512) void tree_attn_split_kernel(
         o_acc[db] = __builtin_amdgcn_mfma_f32_32x32x16_f16(a, bp, o_acc[db], 0, 0, 0);
       }
     }
-  };
-  for (int tile = split; tile < ntiles; tile += AHEAD * nsplit) {
-    process(tile, kregA, vregA);
-    if constexpr (TWO) {
-      if (tile + nsplit < ntiles) process(tile + nsplit, kregB, vregB);
-    }
   }
 
   // partials: part_ml [H][nsplit][32][2], part_o [H][nsplit][32][HD]
@@ -276,12 +267,7 @@ __global__ __launch_bounds__(512) void tree_attn_split_kernel(
     part_ml[slot * 2 + 0] = m_run;
     part_ml[slot * 2 + 1] = l_run;
   }
-  // fp16 partial outputs (|O| <= keys per split, relative error 2^-11).  The accumulators hold
-  // O^T; they go through this wave's LDS rows so that a lane stores 16 contiguous bytes of one
-  // token's row and a store instruction covers whole rows.
-  __syncthreads();                       // the K/V tiles are dead
-  constexpr int OSTR = HD * 2 + 16;      // bytes per staged token row
-  unsigned char* ost = lds + wave * (32 * OSTR);
+  half_t* po = part_o + slot * HD;     // fp16: |O| <= keys per split, relative error 2^-11
 #pragma unroll
   for (int db = 0; db < DB; ++db)
 #pragma unroll
@@ -289,17 +275,8 @@ __global__ __launch_bounds__(512) void tree_attn_split_kernel(
       const int d0 = db * 32 + 8 * i4 + 4 * hb;
       half4_t v = half4_t{(half_t)o_acc[db][4 * i4 + 0], (half_t)o_acc[db][4 * i4 + 1],
                           (half_t)o_acc[db][4 * i4 + 2], (half_t)o_acc[db][4 * i4 + 3]};
-      *reinterpret_cast<half4_t*>(ost + ql * OSTR + d0 * 2) = v;
+      *reinterpret_cast<half4_t*>(po + d0) = v;
     }
-  half_t* po = part_o + ((long)head * nsplit + split) * 32 * HD;
-#pragma unroll
-  for (int it = 0; it < 32 * VEC_ROW / 64; ++it) {
-    const int v = lane + it * 64;
-    const int tok = v / VEC_ROW;
-    const int c = v % VEC_ROW;
-    *reinterpret_cast<half8_t*>(po + tok * HD + c * 8) =
-        *reinterpret_cast<const half8_t*>(ost + tok * OSTR + c * 16);
-  }
 }
 
 // Merge the splits.  Grid (H, T / 4): a workgroup owns four tree tokens of one head; one
@@ -318,20 +295,6 @@ __global__ void tree_attn_merge_kernel(const half_t* __restrict__ part_o,
   const int lane = tid & 63;
   const int wave = tid >> 6;
   const int nwave = blockDim.x >> 6;
-  // this thread's output slice; its first partial outputs are requested before the weights
-  // are worked out, so that both round trips to memory overlap
-  const int tl_o = tid / QW;
-  const int dq = tid % QW;
-  const int t_o = blockIdx.y * MERGE_TOK + tl_o;
-  const int t_c = t_o < T ? t_o : T - 1;
-  const half_t* src = part_o + ((long)head * nsplit * 32 + t_c) * HD + dq * 4;
-  constexpr int PRE = 16;
-  half4_t pre[PRE];
-#pragma unroll
-  for (int k = 0; k < PRE; ++k) {
-    const int sp = k < nsplit ? k : nsplit - 1;
-    pre[k] = *reinterpret_cast<const half4_t*>(src + (long)sp * 32 * HD);
-  }
   for (int tl = wave; tl < MERGE_TOK; tl += nwave) {
     const int t = blockIdx.y * MERGE_TOK + tl;
     float m = -INFINITY, l = 0.f;
@@ -346,16 +309,13 @@ __global__ void tree_attn_merge_kernel(const half_t* __restrict__ part_o,
     wts[tl][lane] = den > 0.f ? w / den : 0.f;
   }
   __syncthreads();
-  if (t_o >= T) return;
+  const int tl = tid / QW;
+  const int dq = tid % QW;
+  const int t = blockIdx.y * MERGE_TOK + tl;
+  if (t >= T) return;
   float4_t acc = float4_t{0.f, 0.f, 0.f, 0.f};
-#pragma unroll
-  for (int k = 0; k < PRE; ++k)
-    if (k < nsplit) {
-      const float wk = wts[tl_o][k];
-#pragma unroll
-      for (int e = 0; e < 4; ++e) acc[e] += wk * (float)pre[k][e];
-    }
-  for (int s0 = PRE; s0 < nsplit; s0 += 8) {
+  const half_t* src = part_o + ((long)head * nsplit * 32 + t) * HD + dq * 4;
+  for (int s0 = 0; s0 < nsplit; s0 += 8) {
     half4_t v[8];
 #pragma unroll
     for (int k = 0; k < 8; ++k) {
@@ -365,12 +325,11 @@ __global__ void tree_attn_merge_kernel(const half_t* __restrict__ part_o,
 #pragma unroll
     for (int k = 0; k < 8; ++k)
       if (s0 + k < nsplit) {
-        const float wk = wts[tl_o][s0 + k];
+        const float wk = wts[tl][s0 + k];
 #pragma unroll
         for (int e = 0; e < 4; ++e) acc[e] += wk * (float)v[k][e];
       }
   }
-  const int t = t_o;
   half4_t o = half4_t{(half_t)acc[0], (half_t)acc[1], (half_t)acc[2], (half_t)acc[3]};
   *reinterpret_cast<half4_t*>(out + ((long)t * H + head) * HD + dq * 4) = o;
 }
@@ -380,11 +339,8 @@ int splits_for(int max_len, int G) {
   const int ntiles = (max_len + KT - 1) / KT;
   int n = 256 / (G > 0 ? G : 1);
   if (n < 1) n = 1;
-  // at least two key tiles per workgroup: below that the partials written and merged outweigh
-  // the key/value rows read
-  if (n > (ntiles + 1) / 2) n = (ntiles + 1) / 2;
-  if (n > 64) n = 64;                  // one split per lane in the merge
-  if (n < 1) n = 1;
+  if (n > ntiles) n = ntiles;
+  if (n > 32) n = 32;                  // partial traffic grows with the split count
   return n;
 }
 
@@ -397,33 +353,9 @@ int launch_attention(const half_t* q, half_t* kc, half_t* vc, const uint32_t* bi
   half_t* part_o = reinterpret_cast<half_t*>(part_ml + (size_t)H * nsplit * 32 * 2);
   const float sl2 = scale * 1.4426950408889634f;
   const int rep = H / G;
-  size_t lds = 2 * KT * (HD * 2 + 16) + (ROPE ? (size_t)EAGLE_MAX_TREE * HD * 4 : 0);
-  const size_t stage = (size_t)rep * 32 * (HD * 2 + 16);   // per-wave rows of the partial output
-  if (lds < stage) lds = stage;
-  const int nvec = KT * HD / 8;                        // 16-byte vectors per K (or V) tile
-  const int per_thread = (nvec + rep * 64 - 1) / (rep * 64);
-#define EAGLE_ATTN_LAUNCH(NVS)                                                                      \
-  if (lds > 65536) {                                                                                \
-    static bool raised = false; /* more than 64 KiB of LDS has to be requested once */              \
-    if (!raised && hipFuncSetAttribute((const void*)tree_attn_split_kernel<HD, ROPE, NVS>,          \
-                                       hipFuncAttributeMaxDynamicSharedMemorySize,                  \
-                                       160 * 1024) != hipSuccess)                                   \
-      return EAGLE_ERR_HIP;                                                                         \
-    raised = true;                                                                                  \
-  }                                                                                                 \
-  hipLaunchKernelGGL((tree_attn_split_kernel<HD, ROPE, NVS>), dim3(G, nsplit), dim3(rep * 64), lds, \
-                     st, q, kc, vc, bits, len, part_o, part_ml, T, H, G, cap, 0, sl2, k_lin, v_lin, \
-                     ld, cs)
-  if (per_thread <= 1) {
-    EAGLE_ATTN_LAUNCH(1);
-  } else if (per_thread <= 2) {
-    EAGLE_ATTN_LAUNCH(2);
-  } else if (per_thread <= 4) {
-    EAGLE_ATTN_LAUNCH(4);
-  } else {
-    EAGLE_ATTN_LAUNCH(8);
-  }
-#undef EAGLE_ATTN_LAUNCH
+  const size_t lds = 2 * KT * (HD * 2 + 16) + (ROPE ? (size_t)EAGLE_MAX_TREE * HD * 4 : 0);
+  hipLaunchKernelGGL((tree_attn_split_kernel<HD, ROPE>), dim3(G, nsplit), dim3(rep * 64), lds, st, q, kc,
+                     vc, bits, len, part_o, part_ml, T, H, G, cap, 0, sl2, k_lin, v_lin, ld, cs);
   hipLaunchKernelGGL(tree_attn_merge_kernel<HD>, dim3(H, (T + MERGE_TOK - 1) / MERGE_TOK),
                      dim3(MERGE_TOK * HD / 4), 0, st, part_o, part_ml, (half_t*)out, T, H, nsplit);
   return eagle_launch_status();
