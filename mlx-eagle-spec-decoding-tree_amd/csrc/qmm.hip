@@ -741,9 +741,10 @@ void choose(int M, int N, int K, Launch* out) {
   // several tiles, beat one slab of many waves that touches a single tile
   if (M <= 16 && tiles < 3 * NUM_CU / 2 && units >= 8) fill = 4;
   if (splits < fill) splits = fill;
-  // A second phase costs a drained ring and a reload of x; unless the partials would be a
-  // large matrix of their own (very many tiles), two K slabs finish sooner.
-  if (splits == 1 && units > MAX_STREAM_WAVES && tiles < 16 * NUM_CU) splits = 2;
+  // With only a few tiles per workgroup a second phase is mostly start-up latency (new x, a
+  // drained ring); two K slabs on twice the workgroups finish sooner.  (With more tiles the
+  // two forms time alike in isolation and the phases win inside a verify step.)
+  if (splits == 1 && units > MAX_STREAM_WAVES && tiles < 4 * NUM_CU) splits = 2;
   if (splits > units) splits = units;
   int per_slab = (units + splits - 1) / splits;
   L.phases = (per_slab + MAX_STREAM_WAVES - 1) / MAX_STREAM_WAVES;
