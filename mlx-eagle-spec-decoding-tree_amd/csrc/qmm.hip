@@ -737,9 +737,9 @@ void choose(int M, int N, int K, Launch* out) {
   int splits = (units + phase_cap * MAX_STREAM_WAVES - 1) / (phase_cap * MAX_STREAM_WAVES);
   int fill = tiles >= 160 ? 1 : (NUM_CU + tiles - 1) / tiles;
   if (fill > 4) fill = 4;
-  // M <= 16 with about one tile per compute unit: four slabs of a few waves, each walking
-  // several tiles, beat one slab of many waves that touches a single tile
-  if (M <= 16 && tiles < 3 * NUM_CU / 2 && units >= 8) fill = 4;
+  // About one tile per compute unit: four slabs of a few waves, each walking several tiles,
+  // beat fewer slabs of many waves that touch one or two tiles
+  if (tiles < 3 * NUM_CU / 2 && units >= (M <= 16 ? 8 : 16)) fill = 4;
   if (splits < fill) splits = fill;
   // With only a few tiles per workgroup a second phase is mostly start-up latency (new x, a
   // drained ring); two K slabs on twice the workgroups finish sooner.  (With more tiles the
@@ -750,8 +750,9 @@ void choose(int M, int N, int K, Launch* out) {
   L.phases = (per_slab + MAX_STREAM_WAVES - 1) / MAX_STREAM_WAVES;
   L.nw = (per_slab + L.phases - 1) / L.phases;
   // 64-byte units (M > 16): two neighbouring waves share each 128-byte line of a weight row,
-  // so an even wave count keeps every line inside one phase
-  if (M > 16 && (L.nw & 1) && L.nw < MAX_STREAM_WAVES) ++L.nw;
+  // so an even wave count keeps every line inside one phase (left alone when the slabs divide
+  // the units exactly)
+  if (M > 16 && (L.nw & 1) && L.nw < MAX_STREAM_WAVES && (units % splits) != 0) ++L.nw;
   per_slab = L.nw * L.phases;
   L.splits = (units + per_slab - 1) / per_slab;
   int ranges = NUM_CU / L.splits;
