@@ -13,7 +13,9 @@
 // tree tokens), runs the online softmax on its accumulator (a lane owns one tree token,
 // its partner lane+32 the other half of the keys), and feeds exp(S^T) straight back as
 // the B operand of O^T += V^T P^T; only V needs a transposed (16-bit) read from LDS.
-// Partial (m, l, O) per split go to a workspace and a second kernel merges them.
+// Partial (m, l, O) per split go to a workspace and a second kernel merges them.  The key
+// tiles of the live length are dealt evenly to as many splits as give each at most
+// max(2, tiles / grid splits) tiles; the busiest workgroup sets the time.
 //
 // A second form of the split kernel takes the un-rotated projection outputs instead
 // (mlx_llama.py:166-183): it rotates q and the tree keys itself and appends the tree rows to
@@ -25,6 +27,13 @@
 namespace {
 
 constexpr int KT = 32;   // keys per tile
+
+// splits that get work when `ntiles` key tiles are dealt to a grid of `nsplit` splits
+__host__ __device__ inline int active_splits(int ntiles, int nsplit) {
+  int tpw = (ntiles + nsplit - 1) / nsplit;
+  if (tpw < 2) tpw = 2;
+  return (ntiles + tpw - 1) / tpw;
+}
 
 // (lo, hi) = elements i0..i0+7 and i0+half..i0+half+7 of a head vector; cs = 8 (cos, sin) pairs
 __device__ inline void rotate_pair(half8_t& lo, half8_t& hi, const float* cs) {
@@ -82,6 +91,12 @@ __global__ __launch_bounds__(512) void tree_attn_split_kernel(
   }
   const int Ltot = P + T;
   const int ntiles = (Ltot + KT - 1) / KT;
+  // Splits in use for this length: every workgroup gets at most `tpw` key tiles, two at
+  // least (with one, writing and merging the partials costs more than reading the keys).
+  // The tile count of the busiest workgroup sets the time, so the tiles are spread evenly
+  // over exactly as many workgroups as that takes; the rest of the grid leaves at once.
+  const int nactive = active_splits(ntiles, nsplit);
+  if (split >= nactive) return;
   half8_t qreg[KSTEPS];
 #pragma unroll
   for (int kk = 0; kk < KSTEPS; ++kk) {
@@ -146,7 +161,7 @@ __global__ __launch_bounds__(512) void tree_attn_split_kernel(
     }
   };
 
-  if (split < ntiles) fetch(split);
+  fetch(split);
   if (ROPE) {
     for (int v = tid; v < T * HALF / 2; v += nthr)
       *reinterpret_cast<float4_t*>(cs_lds + 4 * v) = *reinterpret_cast<const float4_t*>(rope_cs + 4 * v);
@@ -157,7 +172,7 @@ __global__ __launch_bounds__(512) void tree_attn_split_kernel(
         rotate_pair(qreg[kk], qreg[kk + KSTEPS / 2], cs_lds + (ql * HALF + kk * 16 + hb * 8) * 2);
     }
   }
-  for (int tile = split; tile < ntiles; tile += nsplit) {
+  for (int tile = split; tile < ntiles; tile += nactive) {
     const int kb = tile * KT;
     __syncthreads();   // every wave is done with the previous tile
     if (ROPE && kb + KT > P) {
@@ -172,7 +187,7 @@ __global__ __launch_bounds__(512) void tree_attn_split_kernel(
       }
     }
     stash();
-    if (tile + nsplit < ntiles) fetch(tile + nsplit);
+    if (tile + nactive < ntiles) fetch(tile + nactive);
     __syncthreads();
     if (ROPE && kb + KT > P) {
       // rotate the tree keys in LDS (one thread per pair of 16-byte pieces) and append them
@@ -287,7 +302,8 @@ constexpr int MERGE_TOK = 4;
 template <int HD>
 __global__ void tree_attn_merge_kernel(const half_t* __restrict__ part_o,
                                        const float* __restrict__ part_ml,
-                                       half_t* __restrict__ out, int T, int H, int nsplit) {
+                                       half_t* __restrict__ out, int T, int H, int nsplit,
+                                       const int32_t* __restrict__ len_dev, long cap, int clamp_len) {
   constexpr int QW = HD / 4;                       // threads per token
   __shared__ float wts[MERGE_TOK][64];
   const int head = blockIdx.x;
@@ -295,10 +311,16 @@ __global__ void tree_attn_merge_kernel(const half_t* __restrict__ part_o,
   const int lane = tid & 63;
   const int wave = tid >> 6;
   const int nwave = blockDim.x >> 6;
+  int P = *len_dev;
+  if (clamp_len) {
+    if (P > cap - T) P = (int)(cap - T);
+    if (P < 0) P = 0;
+  }
+  const int nact = active_splits((P + T + KT - 1) / KT, nsplit);   // as in the split kernel
   for (int tl = wave; tl < MERGE_TOK; tl += nwave) {
     const int t = blockIdx.y * MERGE_TOK + tl;
     float m = -INFINITY, l = 0.f;
-    if (lane < nsplit && t < T) {
+    if (lane < nact && t < T) {
       const long slot = ((long)head * nsplit + lane) * 32 + t;
       m = part_ml[slot * 2];
       l = part_ml[slot * 2 + 1];
@@ -315,16 +337,16 @@ __global__ void tree_attn_merge_kernel(const half_t* __restrict__ part_o,
   if (t >= T) return;
   float4_t acc = float4_t{0.f, 0.f, 0.f, 0.f};
   const half_t* src = part_o + ((long)head * nsplit * 32 + t) * HD + dq * 4;
-  for (int s0 = 0; s0 < nsplit; s0 += 8) {
+  for (int s0 = 0; s0 < nact; s0 += 8) {
     half4_t v[8];
 #pragma unroll
     for (int k = 0; k < 8; ++k) {
-      const int sp = s0 + k < nsplit ? s0 + k : nsplit - 1;
+      const int sp = s0 + k < nact ? s0 + k : nact - 1;
       v[k] = *reinterpret_cast<const half4_t*>(src + (long)sp * 32 * HD);
     }
 #pragma unroll
     for (int k = 0; k < 8; ++k)
-      if (s0 + k < nsplit) {
+      if (s0 + k < nact) {
         const float wk = wts[tl][s0 + k];
 #pragma unroll
         for (int e = 0; e < 4; ++e) acc[e] += wk * (float)v[k][e];
@@ -334,13 +356,14 @@ __global__ void tree_attn_merge_kernel(const half_t* __restrict__ part_o,
   *reinterpret_cast<half4_t*>(out + ((long)t * H + head) * HD + dq * 4) = o;
 }
 
-// Key splits (gridDim.y): about one workgroup per compute unit, never more than tiles.
+// Key splits of the grid (gridDim.y), sized for the longest length; how many of them get work
+// follows the live length inside the kernels (active_splits).
 int splits_for(int max_len, int G) {
+  (void)G;
   const int ntiles = (max_len + KT - 1) / KT;
-  int n = 256 / (G > 0 ? G : 1);
+  int n = (ntiles + 1) / 2;            // two tiles per workgroup at the longest length
+  if (n > 64) n = 64;                  // one split per lane in the merge
   if (n < 1) n = 1;
-  if (n > ntiles) n = ntiles;
-  if (n > 32) n = 32;                  // partial traffic grows with the split count
   return n;
 }
 
@@ -357,7 +380,8 @@ int launch_attention(const half_t* q, half_t* kc, half_t* vc, const uint32_t* bi
   hipLaunchKernelGGL((tree_attn_split_kernel<HD, ROPE>), dim3(G, nsplit), dim3(rep * 64), lds, st, q, kc,
                      vc, bits, len, part_o, part_ml, T, H, G, cap, 0, sl2, k_lin, v_lin, ld, cs);
   hipLaunchKernelGGL(tree_attn_merge_kernel<HD>, dim3(H, (T + MERGE_TOK - 1) / MERGE_TOK),
-                     dim3(MERGE_TOK * HD / 4), 0, st, part_o, part_ml, (half_t*)out, T, H, nsplit);
+                     dim3(MERGE_TOK * HD / 4), 0, st, part_o, part_ml, (half_t*)out, T, H, nsplit,
+                     len, cap, ROPE ? 1 : 0);
   return eagle_launch_status();
 }
 
