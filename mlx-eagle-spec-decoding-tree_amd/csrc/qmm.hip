@@ -728,6 +728,13 @@ size_t partial_bytes(int M, int N, int splits) {
 // it takes to give every compute unit a workgroup when there are few row tiles.  Tile ranges:
 // about one workgroup per compute unit, more when the per-range accumulators of a
 // multi-phase launch would not fit LDS.
+// The busiest workgroup sets the time: no more ranges than it takes to keep its share
+// (items = tiles, or tile pairs in the SwiGLU form).
+inline int balanced_ranges(int items, int ranges) {
+  const int most = (items + ranges - 1) / ranges;
+  return (items + most - 1) / most;
+}
+
 void choose(int M, int N, int K, Launch* out) {
   const int units = (K + cw_of(M) - 1) / cw_of(M);
   const int tiles = (N + 15) / 16;
@@ -764,6 +771,7 @@ void choose(int M, int N, int K, Launch* out) {
     L.ranges += NUM_CU / L.splits > 0 ? NUM_CU / L.splits : 1;
     if (L.ranges > tiles) L.ranges = tiles;
   }
+  L.ranges = balanced_ranges(tiles, L.ranges);
   *out = L;
 }
 
@@ -891,6 +899,7 @@ EAGLE_EXPORT int eagle_qmm_swiglu_w4g64_f16(const void* x, const uint32_t* wq, c
   Launch L;
   choose(M, N, K, &L);
   if (L.ranges > N / 32) L.ranges = N / 32;
+  L.ranges = balanced_ranges(N / 32, L.ranges);
   rc = validate_launch(M, N, K, L, 2);
   if (rc != EAGLE_OK) return rc;
   return run(x, wq, scales, biases, bias, out, M, N, K, L, 1, workspace, workspace_bytes,
