@@ -456,6 +456,9 @@ __global__ __launch_bounds__(1024) void qmm_w4g64_kernel(
     // block (NT == 1) tiles it and it + 2 for the lane halves, with two (NT == 2) tile it of
     // x block = lane half.  Either way a lane's two blocks are neighbouring tiles, which is
     // what the SwiGLU form needs: gate in slot 0, up in slot 1.
+    // The whole workgroup waits at the next barrier for these two waves: they go first
+    // whenever they have something to issue.
+    __builtin_amdgcn_s_setprio(3);
     const int ww = wave - nw;                 // 0 .. 1
     const int hi = lane >> 5;
     const int ln = (lane & 31) + 32 * ww;     // MFMA lane
