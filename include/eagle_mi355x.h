@@ -64,18 +64,19 @@ int eagle_qmm_w4g64_f16(const void* x, const uint32_t* wq, const void* scales,
                         const void* biases, const void* bias, void* out,
                         int M, int N, int K, int group_size, int bits,
                         void* workspace, size_t workspace_bytes, eagle_stream_t stream);
-/* The launch shape the library would pick: plan4 = {streaming waves per workgroup,
- * phases (column units each streaming wave owns, one after the other; a unit is 256
- * columns for M <= 16, 128 above), K slabs, tile ranges (workgroups per slab)}. */
-int eagle_qmm_plan(int M, int N, int K, int* plan4);
-/* Same matmul with the launch shape forced (tuning sweeps and tests).  nw <= 14,
- * phases <= 8, nw * phases * splits must cover K with no empty slab,
- * 1 <= ranges <= ceil(N / 16), and the shape must fit LDS, else EAGLE_ERR_SHAPE. */
+/* The launch shape the library would pick: plan5 = {streaming waves per workgroup,
+ * phases (column units each streaming wave owns, one after the other), K slabs, tile
+ * ranges (workgroups per slab), columns per unit (256 for M <= 16; 128 or 256 above)}. */
+int eagle_qmm_plan(int M, int N, int K, int* plan5);
+/* Same matmul with the launch shape forced (tuning sweeps and tests).  nw <= 14 (<= 10
+ * with 256-column units at M > 16), phases <= 8, nw * phases * splits must cover K with no
+ * empty slab, 1 <= ranges <= ceil(N / 16), unit_cols 0 (the default for M), 128 or 256,
+ * and the shape must fit LDS, else EAGLE_ERR_SHAPE. */
 size_t eagle_qmm_workspace_bytes_tuned(int M, int N, int splits);
 int eagle_qmm_w4g64_f16_tuned(const void* x, const uint32_t* wq, const void* scales,
                               const void* biases, const void* bias, void* out,
                               int M, int N, int K, int nw, int phases, int splits, int ranges,
-                              void* workspace, size_t workspace_bytes, eagle_stream_t stream);
+                              int unit_cols, void* workspace, size_t workspace_bytes, eagle_stream_t stream);
 
 /* SwiGLU form of the same matmul for the MLP gate and up projections (mlx_llama.py:214-215:
  * down(silu(gate(x)) * up(x))).  wq / scales / biases / bias hold both projections with their

@@ -44,6 +44,7 @@ namespace {
 
 constexpr int MAX_STREAM_WAVES = 14;   // + 2 reducing waves = 1024 threads
 constexpr int NWR = 2;                 // reducing waves per workgroup
+constexpr int MAX_WIDE_WAVES = 10;     // 32 rows x 256 columns of x need 168 registers: 12 waves per CU
 constexpr int MAX_SPLITS = 64;
 constexpr int MAX_RANGES = EAGLE_QMM_COUNTER_BYTES / 4;
 constexpr int LDS_MAX = 160 * 1024;
@@ -106,6 +107,7 @@ struct Launch {
   int phases;   // column units a streaming wave owns, one after the other
   int splits;   // K slabs (gridDim.y); a slab is nw * phases units
   int ranges;   // tile ranges (gridDim.x)
+  int wide = 0; // M > 16 only: 256-column units, at most MAX_WIDE_WAVES streaming waves
 };
 
 template <int V>
@@ -118,7 +120,7 @@ constexpr int STEP_LAST = 2;   // last super-step of the last phase: nothing to 
 // SLOWSB: scales / biases are fetched element by element (odd group counts, rows shorter
 // than a unit, unaligned arrays).
 template <int NT, int GW, bool SLOWSB>
-__global__ __launch_bounds__(1024) void qmm_w4g64_kernel(
+__global__ __launch_bounds__(NT == 2 && GW == 4 ? 768 : 1024) void qmm_w4g64_kernel(
     const half_t* __restrict__ x, const uint32_t* __restrict__ w,
     const half_t* __restrict__ s, const half_t* __restrict__ b,
     const half_t* __restrict__ bias, half_t* __restrict__ out,
@@ -692,12 +694,13 @@ __global__ __launch_bounds__(1024) void qmm_w4g64_kernel(
 // host side
 // ------------------------------------------------------------------------------------------
 inline int nt_of(int M) { return M <= 16 ? 1 : 2; }
-inline int cw_of(int M) { return M <= 16 ? 256 : 128; }
+inline int cw_of(int M, int wide = 0) { return (M <= 16 || wide) ? 256 : 128; }
 constexpr int MAX_PHASES = 8;
 
 // gran = 1: ranges are counted in tiles; gran = 2: in (gate, up) tile pairs
 int lds_bytes(int M, int N, const Launch& L, int gran = 1) {
-  const int sb = M <= 16 ? 2 * Cfg<1, 4>::SB_BUF : 2 * Cfg<2, 2>::SB_BUF;
+  const int sb = M <= 16 ? 2 * Cfg<1, 4>::SB_BUF
+                         : (L.wide ? 2 * Cfg<2, 4>::SB_BUF : 2 * Cfg<2, 2>::SB_BUF);
   int acc = 0;
   if (L.phases > 1) {
     const int tiles = (N + 15) / 16 / gran;
@@ -711,7 +714,8 @@ int validate_launch(int M, int N, int K, const Launch& L, int gran = 1) {
   if (L.nw < 1 || L.nw > MAX_STREAM_WAVES || L.splits < 1 || L.splits > MAX_SPLITS ||
       L.phases < 1 || L.phases > MAX_PHASES)
     return EAGLE_ERR_SHAPE;
-  const int units = (K + cw_of(M) - 1) / cw_of(M);
+  if (L.wide && (M <= 16 || L.nw > MAX_WIDE_WAVES)) return EAGLE_ERR_SHAPE;
+  const int units = (K + cw_of(M, L.wide) - 1) / cw_of(M, L.wide);
   const long per_slab = (long)L.nw * L.phases;
   if (per_slab * L.splits < units || per_slab * (L.splits - 1) >= units) return EAGLE_ERR_SHAPE;
   const int tiles = (N + 15) / 16 / gran;
@@ -739,9 +743,39 @@ inline int balanced_ranges(int items, int ranges) {
 }
 
 void choose(int M, int N, int K, Launch* out) {
-  const int units = (K + cw_of(M) - 1) / cw_of(M);
   const int tiles = (N + 15) / 16;
   Launch L;
+  if (M > 16) {
+    // 256-column units on fewer, fatter waves (A/B runs of a whole verify step): when K needs
+    // slabs anyway (K > 3584) they remove the second phase; with very many tiles they halve
+    // the per-tile overhead of the two phases.  Smaller shapes are faster on 14 narrow waves.
+    const int uw = (K + 255) / 256;
+    const int un = (K + 127) / 128;
+    if (tiles >= 16 * NUM_CU && uw > MAX_WIDE_WAVES / 2 && uw <= 2 * MAX_WIDE_WAVES) {
+      L.wide = 1;                        // very many tiles: partials would be a large matrix
+      L.phases = 2;
+      L.nw = (uw + 1) / 2;
+      L.splits = 1;
+    } else if (un > 2 * MAX_STREAM_WAVES) {
+      L.wide = 1;
+      L.phases = 1;
+      L.splits = (uw + MAX_WIDE_WAVES - 1) / MAX_WIDE_WAVES;
+      L.nw = (uw + L.splits - 1) / L.splits;
+      L.splits = (uw + L.nw - 1) / L.nw;
+    }
+    if (L.wide) {
+      int ranges = NUM_CU / L.splits;
+      if (ranges < 1) ranges = 1;
+      if (ranges > tiles) ranges = tiles;
+      if (ranges > MAX_RANGES) ranges = MAX_RANGES;
+      L.ranges = ranges;
+      while (lds_bytes(M, N, L) > LDS_MAX && L.ranges < tiles && L.ranges < MAX_RANGES) ++L.ranges;
+      L.ranges = balanced_ranges(tiles, L.ranges);
+      *out = L;
+      return;
+    }
+  }
+  const int units = (K + cw_of(M) - 1) / cw_of(M);
   // M <= 16: one phase only (a phase switch costs more than a K slab there)
   const int phase_cap = M <= 16 ? 1 : 2;
   int splits = (units + phase_cap * MAX_STREAM_WAVES - 1) / (phase_cap * MAX_STREAM_WAVES);
@@ -827,13 +861,16 @@ int run(const void* x, const uint32_t* wq, const void* scales, const void* biase
   }
   // vector fetches of scales / biases need whole, aligned units in every row
   const int G = K / 64;
-  const int gw = M <= 16 ? 4 : 2;
+  const int gw = (M <= 16 || L.wide) ? 4 : 2;
   const uintptr_t amask = gw == 4 ? 7u : 3u;
   const bool slow = (G % gw) != 0 || (reinterpret_cast<uintptr_t>(scales) & amask) ||
                     (reinterpret_cast<uintptr_t>(biases) & amask);
   if (M <= 16)
     return slow ? launch<1, 4, true>(x, wq, scales, biases, bias, out, partial, counters, M, N, K, L, swiglu, st)
                 : launch<1, 4, false>(x, wq, scales, biases, bias, out, partial, counters, M, N, K, L, swiglu, st);
+  if (L.wide)
+    return slow ? launch<2, 4, true>(x, wq, scales, biases, bias, out, partial, counters, M, N, K, L, swiglu, st)
+                : launch<2, 4, false>(x, wq, scales, biases, bias, out, partial, counters, M, N, K, L, swiglu, st);
   return slow ? launch<2, 2, true>(x, wq, scales, biases, bias, out, partial, counters, M, N, K, L, swiglu, st)
               : launch<2, 2, false>(x, wq, scales, biases, bias, out, partial, counters, M, N, K, L, swiglu, st);
 }
@@ -852,23 +889,27 @@ EAGLE_EXPORT size_t eagle_qmm_workspace_bytes_tuned(int M, int N, int splits) {
   return (size_t)EAGLE_QMM_COUNTER_BYTES + partial_bytes(M, N, splits);
 }
 
-EAGLE_EXPORT int eagle_qmm_plan(int M, int N, int K, int* plan4) {
-  if (!plan4) return EAGLE_ERR_NULL;
+EAGLE_EXPORT int eagle_qmm_plan(int M, int N, int K, int* plan5) {
+  if (!plan5) return EAGLE_ERR_NULL;
   if (M < 1 || M > EAGLE_MAX_M || N < 8 || K < 64 || (K % 64) != 0) return EAGLE_ERR_SHAPE;
   Launch L;
   choose(M, N, K, &L);
-  plan4[0] = L.nw; plan4[1] = L.phases; plan4[2] = L.splits; plan4[3] = L.ranges;
+  plan5[0] = L.nw; plan5[1] = L.phases; plan5[2] = L.splits; plan5[3] = L.ranges;
+  plan5[4] = cw_of(M, L.wide);
   return EAGLE_OK;
 }
 
 EAGLE_EXPORT int eagle_qmm_w4g64_f16_tuned(const void* x, const uint32_t* wq, const void* scales,
                                            const void* biases, const void* bias, void* out, int M,
                                            int N, int K, int nw, int phases, int splits, int ranges,
-                                           void* workspace, size_t workspace_bytes,
+                                           int unit_cols, void* workspace, size_t workspace_bytes,
                                            eagle_stream_t stream) {
   int rc = validate(x, wq, scales, biases, bias, out, M, N, K);
   if (rc != EAGLE_OK) return rc;
+  if (unit_cols != 0 && unit_cols != 128 && unit_cols != 256) return EAGLE_ERR_SHAPE;
+  if (unit_cols == 128 && M <= 16) return EAGLE_ERR_SHAPE;
   Launch L{nw, phases, splits, ranges};
+  L.wide = (unit_cols == 256 && M > 16) ? 1 : 0;
   rc = validate_launch(M, N, K, L);
   if (rc != EAGLE_OK) return rc;
   return run(x, wq, scales, biases, bias, out, M, N, K, L, 0, workspace, workspace_bytes,

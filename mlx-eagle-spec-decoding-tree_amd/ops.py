@@ -86,23 +86,25 @@ def quantized_matmul(x, w_q, scales, biases, transpose=True, group_size=64, bits
                                    _ptr(out), M, N, K, group_size, bits, _ptr(ws), ws.numel(),
                                    _stream())
     else:
-        # tuned = (nw, phases, splits, ranges): forced launch shape
+        # tuned = (nw, phases, splits, ranges[, unit_cols]): forced launch shape
         if group_size != 64 or bits != 4:
             raise ValueError("only group_size=64, bits=4 is supported")
-        nw, phases, splits, ranges = (int(v) for v in tuned)
+        nw, phases, splits, ranges = (int(v) for v in tuned[:4])
+        unit_cols = int(tuned[4]) if len(tuned) > 4 else 0
         need = L.eagle_qmm_workspace_bytes_tuned(M, N, splits)
         ws = workspace("qmm", need, x.device)
         rc = L.eagle_qmm_w4g64_f16_tuned(_ptr(x), _ptr(w_q), _ptr(scales), _ptr(biases),
                                          _ptr(bias), _ptr(out), M, N, K, nw, phases, splits, ranges,
-                                         _ptr(ws), ws.numel(), _stream())
+                                         unit_cols, _ptr(ws), ws.numel(), _stream())
     _lib.check(rc, "quantized_matmul")
     return out
 
 
 def qmm_plan(M, N, K):
-    """The launch shape the library picks: (streaming waves, phases, K slabs, tile ranges)."""
+    """The launch shape the library picks: (streaming waves, phases, K slabs, tile ranges,
+    columns per unit)."""
     import ctypes
-    plan = (ctypes.c_int * 4)()
+    plan = (ctypes.c_int * 5)()
     _lib.check(_lib.lib().eagle_qmm_plan(M, N, K, plan), "qmm_plan")
     return tuple(plan)
 

@@ -10,24 +10,25 @@ from util import TOL, layer_to_dev, rel_err, to_dev
 pytestmark = pytest.mark.gpu
 
 
-def shape_for(M, N, K, nw, phases, ranges):
+def shape_for(M, N, K, nw, phases, ranges, wide=False):
     """A forced launch shape: `nw` streaming waves per workgroup, each owning `phases` column
-    units in turn (the K slabs follow from both), `ranges` workgroups per slab; None if it
-    cannot be launched."""
-    cw = 256 if M <= 16 else 128
+    units in turn (the K slabs follow from both), `ranges` workgroups per slab, `wide`:
+    256-column units at M > 16; None if it cannot be launched."""
+    wide = wide and M > 16
+    cw = 256 if M <= 16 or wide else 128
     nt = 1 if M <= 16 else 2
     units = -(-K // cw)
     per_slab = nw * phases
     splits = -(-units // per_slab)
     tiles = -(-N // 16)
-    if nw > 14 or phases > 8 or per_slab * (splits - 1) >= units or ranges > tiles or splits > 64:
+    if nw > (10 if wide else 14) or phases > 8 or per_slab * (splits - 1) >= units or ranges > tiles or splits > 64:
         return None
-    lds = 2 * nw * 4096 + (32768 if nt == 1 else 8192)
+    lds = 2 * nw * 4096 + (32768 if nt == 1 else (16384 if wide else 8192))
     if phases > 1:
         lds += -(-(-(-tiles // ranges)) // 4) * 4 * nt * 1024
     if lds > 160 * 1024:
         return None
-    return (nw, phases, splits, ranges)
+    return (nw, phases, splits, ranges, cw)
 
 
 def run_case(dev, M, N, K, seed=0, bias=False, tuned=None):
@@ -63,6 +64,19 @@ def test_forced_launch_shapes(dev, nw, phases, ranges, M):
     run_case(dev, M, N, K, seed=nw * 100 + ranges + phases, tuned=tuned)
 
 
+@pytest.mark.parametrize("nw,phases", [(1, 1), (2, 1), (3, 2), (5, 3), (7, 1), (7, 2), (10, 1), (10, 2), (4, 4)])
+@pytest.mark.parametrize("ranges", [1, 7, 96])
+@pytest.mark.parametrize("M", [17, 32])
+def test_forced_launch_shapes_wide_units(dev, nw, phases, ranges, M):
+    """M > 16 with 256-column units (the form picked for K > 3584 and for very many tiles)."""
+    N, K = 1536, 3584
+    tuned = shape_for(M, N, K, nw, phases, ranges, wide=True)
+    if tuned is None:
+        pytest.skip("shape cannot be launched")
+    print(f"qmm tuned={tuned} M={M}", flush=True)
+    run_case(dev, M, N, K, seed=nw * 100 + ranges + phases, tuned=tuned, bias=(nw & 1) == 1)
+
+
 @pytest.mark.parametrize("N,K", [(8, 64), (8, 128), (24, 192), (40, 896), (136, 2944), (512, 3584),
                                  (64, 18944)])
 def test_edge_shapes(dev, N, K):
@@ -70,9 +84,10 @@ def test_edge_shapes(dev, N, K):
         print(f"qmm edge N={N} K={K} M={M}", flush=True)
         run_case(dev, M, N, K, seed=N + K + M)
         for cfg in ((1, 1, 1), (3, 2, 2), (14, 1, 3), (2, 3, 1)):
-            tuned = shape_for(M, N, K, *cfg)
-            if tuned is not None:
-                run_case(dev, M, N, K, seed=N + K + M, tuned=tuned)
+            for wide in (False, True):
+                tuned = shape_for(M, N, K, *cfg, wide=wide)
+                if tuned is not None and (wide is False or M > 16):
+                    run_case(dev, M, N, K, seed=N + K + M, tuned=tuned)
 
 
 def test_bias_and_leading_dims(dev):
@@ -122,10 +137,10 @@ def test_plan_covers_benchmark_shapes(dev):
         for N, K in ((3584, 3584), (512, 3584), (18944, 3584), (3584, 18944), (152064, 3584),
                      (8192, 2048), (896, 896), (128, 896), (4864, 896), (896, 4864),
                      (4096, 4096), (1024, 4096), (14336, 4096), (4096, 14336), (128256, 4096)):
-            nw, phases, splits, ranges = ops.qmm_plan(M, N, K)
-            cw = 256 if M <= 16 else 128
+            nw, phases, splits, ranges, cw = ops.qmm_plan(M, N, K)
+            assert cw == 256 if M <= 16 else cw in (128, 256)
             assert nw * phases * splits * cw >= K > nw * phases * (splits - 1) * cw
-            assert 1 <= nw <= 14 and 1 <= ranges <= -(-N // 16)
+            assert 1 <= nw <= (14 if M <= 16 or cw == 128 else 10) and 1 <= ranges <= -(-N // 16)
 
 
 def test_argument_errors(dev):

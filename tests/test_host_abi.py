@@ -87,10 +87,11 @@ def test_plan_is_consistent_for_benchmark_shapes():
         for N, K in ((3584, 3584), (512, 3584), (18944, 3584), (3584, 18944), (152064, 3584),
                      (8192, 2048), (896, 896), (128, 896), (4864, 896), (896, 4864), (151936, 896),
                      (4096, 4096), (1024, 4096), (14336, 4096), (4096, 14336), (128256, 4096)):
-            nw, phases, splits, ranges = ops.qmm_plan(M, N, K)
-            cw = 256 if M <= 16 else 128
+            nw, phases, splits, ranges, cw = ops.qmm_plan(M, N, K)
+            assert cw == 256 if M <= 16 else cw in (128, 256)
             assert nw * phases * splits * cw >= K > nw * phases * (splits - 1) * cw
-            assert 1 <= nw <= 14 and 1 <= phases <= 2 and 1 <= ranges <= -(-N // 16)
+            assert 1 <= nw <= (14 if M <= 16 or cw == 128 else 10) and 1 <= phases <= 2
+            assert 1 <= ranges <= -(-N // 16)
             assert ranges * splits <= 1024
 
 
