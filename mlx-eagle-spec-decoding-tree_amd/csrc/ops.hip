@@ -122,22 +122,27 @@ __global__ void rope_kv_append_kernel(const half_t* __restrict__ q_lin,
 // ------------------------------------------------------------------------------------
 constexpr int RMS_MAXV = 4;
 
-__global__ __launch_bounds__(256) void rmsnorm_kernel(const half_t* __restrict__ x,
-                                                      const half_t* __restrict__ res,
-                                                      const half_t* __restrict__ w, float eps,
-                                                      half_t* __restrict__ h_out,
-                                                      half_t* __restrict__ out, int D) {
-  __shared__ float red[4];
+// BLOCK threads per row; the norm weights are requested together with the row, before the
+// reduction, so that their latency is not added to it.
+template <int BLOCK>
+__global__ __launch_bounds__(BLOCK) void rmsnorm_kernel(const half_t* __restrict__ x,
+                                                        const half_t* __restrict__ res,
+                                                        const half_t* __restrict__ w, float eps,
+                                                        half_t* __restrict__ h_out,
+                                                        half_t* __restrict__ out, int D) {
+  constexpr int NV = 256 * RMS_MAXV / BLOCK;     // vectors per thread
+  __shared__ float red[BLOCK / 64];
   const int t = blockIdx.x;
   const int nvec = D >> 3;
   const half_t* xr = x + (long)t * D;
-  half8_t v[RMS_MAXV];
+  half8_t v[NV], w8[NV];
   float ss = 0.f;
 #pragma unroll
-  for (int i = 0; i < RMS_MAXV; ++i) {
-    const int c = threadIdx.x + i * 256;
+  for (int i = 0; i < NV; ++i) {
+    const int c = threadIdx.x + i * BLOCK;
     if (c < nvec) {
       half8_t a = *reinterpret_cast<const half8_t*>(xr + c * 8);
+      w8[i] = *reinterpret_cast<const half8_t*>(w + c * 8);
       if (res) {
         const half8_t r8 = *reinterpret_cast<const half8_t*>(res + (long)t * D + c * 8);
 #pragma unroll
@@ -152,16 +157,17 @@ __global__ __launch_bounds__(256) void rmsnorm_kernel(const half_t* __restrict__
   ss = wave_sum(ss);
   if ((threadIdx.x & 63) == 0) red[threadIdx.x >> 6] = ss;
   __syncthreads();
-  const float tot = red[0] + red[1] + red[2] + red[3];
+  float tot = 0.f;
+#pragma unroll
+  for (int k = 0; k < BLOCK / 64; ++k) tot += red[k];
   const float rinv = 1.0f / sqrtf(tot / (float)D + eps);
 #pragma unroll
-  for (int i = 0; i < RMS_MAXV; ++i) {
-    const int c = threadIdx.x + i * 256;
+  for (int i = 0; i < NV; ++i) {
+    const int c = threadIdx.x + i * BLOCK;
     if (c < nvec) {
-      const half8_t w8 = *reinterpret_cast<const half8_t*>(w + c * 8);
       half8_t o;
 #pragma unroll
-      for (int j = 0; j < 8; ++j) o[j] = (half_t)((float)w8[j] * ((float)v[i][j] * rinv));
+      for (int j = 0; j < 8; ++j) o[j] = (half_t)((float)w8[i][j] * ((float)v[i][j] * rinv));
       *reinterpret_cast<half8_t*>(out + (long)t * D + c * 8) = o;
     }
   }
@@ -344,9 +350,14 @@ EAGLE_EXPORT int eagle_rmsnorm_f16(const void* x, const void* residual, const vo
   if (!eagle_aligned16(x) || !eagle_aligned16(w) || !eagle_aligned16(out) ||
       (residual && (!eagle_aligned16(residual) || !eagle_aligned16(h_out))))
     return EAGLE_ERR_ALIGN;
-  hipLaunchKernelGGL(rmsnorm_kernel, dim3(T), dim3(256), 0, static_cast<hipStream_t>(stream),
-                     (const half_t*)x, (const half_t*)residual, (const half_t*)w, eps,
-                     (half_t*)h_out, (half_t*)out, D);
+  if (D > 256 * 8)   // one vector per thread while the row is short enough
+    hipLaunchKernelGGL(rmsnorm_kernel<512>, dim3(T), dim3(512), 0, static_cast<hipStream_t>(stream),
+                       (const half_t*)x, (const half_t*)residual, (const half_t*)w, eps,
+                       (half_t*)h_out, (half_t*)out, D);
+  else
+    hipLaunchKernelGGL(rmsnorm_kernel<256>, dim3(T), dim3(256), 0, static_cast<hipStream_t>(stream),
+                       (const half_t*)x, (const half_t*)residual, (const half_t*)w, eps,
+                       (half_t*)h_out, (half_t*)out, D);
   return eagle_launch_status();
 }
 
