@@ -305,39 +305,60 @@ __global__ void tree_attn_merge_kernel(const half_t* __restrict__ part_o,
                                        half_t* __restrict__ out, int T, int H, int nsplit,
                                        const int32_t* __restrict__ len_dev, long cap, int clamp_len) {
   constexpr int QW = HD / 4;                       // threads per token
+  constexpr int TPW = 256 / HD;                    // tokens per wave: MERGE_TOK tokens on HD / 64 waves
+  constexpr int PRE = 8;
   __shared__ float wts[MERGE_TOK][64];
   const int head = blockIdx.x;
   const int tid = threadIdx.x;
   const int lane = tid & 63;
   const int wave = tid >> 6;
-  const int nwave = blockDim.x >> 6;
+  // Everything that does not depend on the live length is requested first: the (m, l) pairs
+  // of every split of the grid and the first partial outputs.  Splits beyond the active
+  // ones hold stale values; they are masked (m) or skipped (O) below, never multiplied.
+  float2_t ml[TPW];
+#pragma unroll
+  for (int k = 0; k < TPW; ++k) {
+    int t = blockIdx.y * MERGE_TOK + wave * TPW + k;
+    if (t > T - 1) t = T - 1;
+    const int sp = lane < nsplit ? lane : nsplit - 1;
+    ml[k] = *reinterpret_cast<const float2_t*>(part_ml + (((long)head * nsplit + sp) * 32 + t) * 2);
+  }
+  const int tl = tid / QW;
+  const int dq = tid % QW;
+  const int t = blockIdx.y * MERGE_TOK + tl;
+  const int t_c = t < T ? t : T - 1;
+  const half_t* src = part_o + ((long)head * nsplit * 32 + t_c) * HD + dq * 4;
+  half4_t pre[PRE];
+#pragma unroll
+  for (int k = 0; k < PRE; ++k)
+    pre[k] = *reinterpret_cast<const half4_t*>(src + (long)(k < nsplit ? k : nsplit - 1) * 32 * HD);
+
   int P = *len_dev;
   if (clamp_len) {
     if (P > cap - T) P = (int)(cap - T);
     if (P < 0) P = 0;
   }
   const int nact = active_splits((P + T + KT - 1) / KT, nsplit);   // as in the split kernel
-  for (int tl = wave; tl < MERGE_TOK; tl += nwave) {
-    const int t = blockIdx.y * MERGE_TOK + tl;
-    float m = -INFINITY, l = 0.f;
-    if (lane < nact && t < T) {
-      const long slot = ((long)head * nsplit + lane) * 32 + t;
-      m = part_ml[slot * 2];
-      l = part_ml[slot * 2 + 1];
-    }
+#pragma unroll
+  for (int k = 0; k < TPW; ++k) {
+    const float m = lane < nact ? ml[k][0] : -INFINITY;
+    const float l = lane < nact ? ml[k][1] : 0.f;
     const float mx = wave_max(m);
     const float w = m == -INFINITY ? 0.f : exp2f(m - mx);
     const float den = wave_sum(w * l);
-    wts[tl][lane] = den > 0.f ? w / den : 0.f;
+    wts[wave * TPW + k][lane] = den > 0.f ? w / den : 0.f;
   }
   __syncthreads();
-  const int tl = tid / QW;
-  const int dq = tid % QW;
-  const int t = blockIdx.y * MERGE_TOK + tl;
   if (t >= T) return;
   float4_t acc = float4_t{0.f, 0.f, 0.f, 0.f};
-  const half_t* src = part_o + ((long)head * nsplit * 32 + t) * HD + dq * 4;
-  for (int s0 = 0; s0 < nact; s0 += 8) {
+#pragma unroll
+  for (int k = 0; k < PRE; ++k)
+    if (k < nact) {
+      const float wk = wts[tl][k];
+#pragma unroll
+      for (int e = 0; e < 4; ++e) acc[e] += wk * (float)pre[k][e];
+    }
+  for (int s0 = PRE; s0 < nact; s0 += 8) {
     half4_t v[8];
 #pragma unroll
     for (int k = 0; k < 8; ++k) {
