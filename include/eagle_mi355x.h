@@ -152,7 +152,16 @@ int eagle_silu_mul_f16(const void* gate, const void* up, void* out, int T, int I
 /* out = fp16(a + b), n elements (residual add, mlx_llama.py:246,248). */
 int eagle_add_f16(const void* a, const void* b, void* out, long n, eagle_stream_t stream);
 
-/* cos/sin table for eagle_tree_attention_rope_f16: out[t][i] = (cos, sin)(positions[t] *
+/* eagle_rope_kv_append_f16 with the angles taken from a table of eagle_rope_table_f32
+ * (below) instead of positions and frequencies: one table per verify step serves every
+ * layer, and the per-layer launch no longer evaluates sincos.  Same angles; the rotated
+ * values agree with eagle_rope_kv_append_f16 to one fp16 ulp. */
+int eagle_rope_kv_append_table_f16(const void* q_lin, const void* k_lin, const void* v_lin,
+                                   const float* rope_cs, void* q_out, void* k_cache, void* v_cache,
+                                   const int32_t* cache_len_dev, int T, int H, int G, int hd,
+                                   long capacity, long row_stride, eagle_stream_t stream);
+
+/* cos/sin table for eagle_rope_kv_append_table_f16 and eagle_tree_attention_rope_f16: out[t][i] = (cos, sin)(positions[t] *
  * scaling_factor * inv_freqs[i]), fp32 [T, half_dim, 2]; the same angles as
  * eagle_rope_arrayed_f16 (mlx_arrayed_rope_kernel.py:60-123).  The table depends on the tree
  * positions only, so one call serves every layer of a step. */

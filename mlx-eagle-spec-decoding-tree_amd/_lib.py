@@ -29,6 +29,7 @@ SIGNATURES = {
     "eagle_rope_arrayed_f16": (c_int, [c_void_p] * 3 + [c_float, c_void_p] + [c_int] * 4 + [c_void_p]),
     "eagle_rope_kv_append_f16": (c_int, [c_void_p] * 5 + [c_float] + [c_void_p] * 4 + [c_int] * 4
                                  + [c_long, c_long, c_void_p]),
+    "eagle_rope_kv_append_table_f16": (c_int, [c_void_p] * 8 + [c_int] * 4 + [c_long, c_long, c_void_p]),
     "eagle_tree_attention_workspace_bytes": (c_size_t, [c_int, c_int, c_int]),
     "eagle_tree_attention_f16": (c_int, [c_void_p] * 6 + [c_int] * 4 + [c_long, c_int, c_float,
                                                                        c_void_p, c_size_t, c_void_p]),

@@ -44,8 +44,8 @@ __device__ inline void rotate_pair(half8_t& lo, half8_t& hi, const float* cs) {
   for (int j = 0; j < 8; ++j) {
     const float co = c[j >> 1][(j & 1) * 2], sn = c[j >> 1][(j & 1) * 2 + 1];
     const float x1 = (float)lo[j], x2 = (float)hi[j];
-    lo[j] = (half_t)(x1 * co - x2 * sn);
-    hi[j] = (half_t)(x1 * sn + x2 * co);
+    lo[j] = (half_t)__builtin_fmaf(x1, co, -(x2 * sn));
+    hi[j] = (half_t)__builtin_fmaf(x1, sn, x2 * co);
   }
 }
 

@@ -21,8 +21,10 @@ __device__ inline void rotate8(const half8_t lo, const half8_t hi, const float* 
     sincosf(theta, &sn, &cs);
     const float x1 = (float)lo[j];
     const float x2 = (float)hi[j];
-    (*olo)[j] = (half_t)(x1 * cs - x2 * sn);
-    (*ohi)[j] = (half_t)(x1 * sn + x2 * cs);
+    // one fused multiply-add on an explicitly rounded product: every rotation in the library
+    // uses this form, so that they agree bit for bit
+    (*olo)[j] = (half_t)__builtin_fmaf(x1, cs, -(x2 * sn));
+    (*ohi)[j] = (half_t)__builtin_fmaf(x1, sn, x2 * cs);
   }
 }
 
@@ -69,8 +71,8 @@ __global__ void rope_arrayed_scalar_kernel(const half_t* __restrict__ x,
   sincosf(theta, &sn, &cs);
   const float x1 = (float)x[row * hd + i];
   const float x2 = (float)x[row * hd + i + half];
-  out[row * hd + i] = (half_t)(x1 * cs - x2 * sn);
-  out[row * hd + i + half] = (half_t)(x1 * sn + x2 * cs);
+  out[row * hd + i] = (half_t)__builtin_fmaf(x1, cs, -(x2 * sn));
+  out[row * hd + i + half] = (half_t)__builtin_fmaf(x1, sn, x2 * cs);
 }
 
 // Token-major projections -> rotated q [H,T,hd] and K/V cache rows P + t.
@@ -83,7 +85,8 @@ __global__ void rope_kv_append_kernel(const half_t* __restrict__ q_lin,
                                       half_t* __restrict__ q_out, half_t* __restrict__ k_cache,
                                       half_t* __restrict__ v_cache,
                                       const int32_t* __restrict__ len_dev, int T, int H, int G,
-                                      int hd, long cap, long ld_q, long ld_kv) {
+                                      int hd, long cap, long ld_q, long ld_kv,
+                                      const float* __restrict__ rope_cs) {
   const int half = hd >> 1;
   const int per_row = half >> 3;
   const int heads = H + 2 * G;
@@ -103,7 +106,24 @@ __global__ void rope_kv_append_kernel(const half_t* __restrict__ q_lin,
     const half8_t lo = *reinterpret_cast<const half8_t*>(src + c * 8);
     const half8_t hi = *reinterpret_cast<const half8_t*>(src + half + c * 8);
     half8_t olo, ohi;
-    rotate8(lo, hi, inv_freq, c * 8, scale, (float)pos[t], &olo, &ohi);
+    if (rope_cs) {
+      // (cos, sin) of this token's angles from the per-step table: the same values, no sincosf
+      const float4_t* cs = reinterpret_cast<const float4_t*>(rope_cs + ((long)t * half + c * 8) * 2);
+#pragma unroll
+      for (int j2 = 0; j2 < 4; ++j2) {
+        const float4_t v = cs[j2];
+#pragma unroll
+        for (int e = 0; e < 2; ++e) {
+          const int j = 2 * j2 + e;
+          const float co = v[2 * e], sn = v[2 * e + 1];
+          const float x1 = (float)lo[j], x2 = (float)hi[j];
+          olo[j] = (half_t)__builtin_fmaf(x1, co, -(x2 * sn));
+          ohi[j] = (half_t)__builtin_fmaf(x1, sn, x2 * co);
+        }
+      }
+    } else {
+      rotate8(lo, hi, inv_freq, c * 8, scale, (float)pos[t], &olo, &ohi);
+    }
     *reinterpret_cast<half8_t*>(dst + c * 8) = olo;
     *reinterpret_cast<half8_t*>(dst + half + c * 8) = ohi;
   } else {
@@ -339,7 +359,34 @@ EAGLE_EXPORT int eagle_rope_kv_append_f16(const void* q_lin, const void* k_lin, 
                      static_cast<hipStream_t>(stream), (const half_t*)q_lin, (const half_t*)k_lin,
                      (const half_t*)v_lin, positions, inv_freqs, scaling_factor, (half_t*)q_out,
                      (half_t*)k_cache, (half_t*)v_cache, cache_len_dev, T, H, G, hd, capacity,
-                     row_stride ? row_stride : (long)H * hd, row_stride ? row_stride : (long)G * hd);
+                     row_stride ? row_stride : (long)H * hd, row_stride ? row_stride : (long)G * hd,
+                     (const float*)nullptr);
+  return eagle_launch_status();
+}
+
+EAGLE_EXPORT int eagle_rope_kv_append_table_f16(const void* q_lin, const void* k_lin,
+                                                const void* v_lin, const float* rope_cs,
+                                                void* q_out, void* k_cache, void* v_cache,
+                                                const int32_t* cache_len_dev, int T, int H, int G,
+                                                int hd, long capacity, long row_stride,
+                                                eagle_stream_t stream) {
+  if (!q_lin || !k_lin || !v_lin || !rope_cs || !q_out || !k_cache || !v_cache || !cache_len_dev)
+    return EAGLE_ERR_NULL;
+  if (T < 1 || T > EAGLE_MAX_TREE || H < 1 || G < 1 || (H % G) != 0 || hd < 16 || (hd % 16) != 0 ||
+      capacity < T || row_stride < 0 || (row_stride % 8) != 0 ||
+      (row_stride > 0 && row_stride < (long)H * hd))
+    return EAGLE_ERR_SHAPE;
+  if (!eagle_aligned16(q_lin) || !eagle_aligned16(k_lin) || !eagle_aligned16(v_lin) ||
+      !eagle_aligned16(rope_cs) || !eagle_aligned16(q_out) || !eagle_aligned16(k_cache) ||
+      !eagle_aligned16(v_cache))
+    return EAGLE_ERR_ALIGN;
+  const long total = (long)T * (H + 2 * G) * (hd / 16);
+  hipLaunchKernelGGL(rope_kv_append_kernel, dim3(blocks_for(total, 256)), dim3(256), 0,
+                     static_cast<hipStream_t>(stream), (const half_t*)q_lin, (const half_t*)k_lin,
+                     (const half_t*)v_lin, (const int32_t*)nullptr, (const float*)nullptr, 1.0f,
+                     (half_t*)q_out, (half_t*)k_cache, (half_t*)v_cache, cache_len_dev, T, H, G, hd,
+                     capacity, row_stride ? row_stride : (long)H * hd,
+                     row_stride ? row_stride : (long)G * hd, rope_cs);
   return eagle_launch_status();
 }
 

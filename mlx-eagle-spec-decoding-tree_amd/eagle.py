@@ -327,7 +327,7 @@ class TreeVerifier:
         ops.embed(self.tokens, emb.weight, emb.scales, emb.biases, out=self.h)
         layers = m.model.layers
         ops.rms_norm(self.h, layers[0].input_layernorm.weight, args.rms_norm_eps, out=self.hn)
-        if self.one_launch_attention:   # one cos/sin table per step: the positions are the same in every layer
+        if self.fuse:   # one cos/sin table per step: the positions are the same in every layer
             at0 = layers[0].self_attn
             ops.rope_table(self.positions, at0._inv_freqs, at0._scaling_factor, out=self.rope_cs)
         for i, layer in enumerate(layers):
@@ -345,7 +345,8 @@ class TreeVerifier:
                 else:
                     ops.rope_kv_append(q_lin, k_lin, v_lin, self.positions, at._inv_freqs,
                                        at._scaling_factor, self.q_rot, c.keys[0], c.values[0],
-                                       self.len_dev, H, G, hd, row_stride=(H + 2 * G) * hd)
+                                       self.len_dev, H, G, hd, row_stride=(H + 2 * G) * hd,
+                                       rope_cs=self.rope_cs)
             else:
                 for lin, out in ((at.q_proj, self.q), (at.k_proj, self.k), (at.v_proj, self.v)):
                     ops.quantized_matmul(self.hn, lin.weight, lin.scales, lin.biases, bias=lin.bias, out=out)

@@ -196,10 +196,17 @@ def rope_positions(inp, offsets, inv_freqs, scaling_factor, verbose=False):
 
 
 def rope_kv_append(q_lin, k_lin, v_lin, positions, inv_freqs, scaling_factor, q_out, k_cache,
-                   v_cache, cache_len_dev, H, G, hd, row_stride=0):
+                   v_cache, cache_len_dev, H, G, hd, row_stride=0, rope_cs=None):
     """Rotate q and k at `positions`, write q as [H,T,hd] and append k, v to the caches.
-    row_stride > 0: q_lin, k_lin, v_lin are column blocks of one [T,row_stride] matrix."""
+    row_stride > 0: q_lin, k_lin, v_lin are column blocks of one [T,row_stride] matrix.
+    rope_cs: the `rope_table` of these positions (then positions / inv_freqs are not read)."""
     T = q_lin.shape[0]
+    if rope_cs is not None:
+        rc = _lib.lib().eagle_rope_kv_append_table_f16(
+            _ptr(q_lin), _ptr(k_lin), _ptr(v_lin), _ptr(rope_cs), _ptr(q_out), _ptr(k_cache),
+            _ptr(v_cache), _ptr(cache_len_dev), T, H, G, hd, k_cache.shape[1], int(row_stride), _stream())
+        _lib.check(rc, "rope_kv_append")
+        return
     rc = _lib.lib().eagle_rope_kv_append_f16(
         _ptr(q_lin), _ptr(k_lin), _ptr(v_lin), _ptr(positions), _ptr(inv_freqs),
         float(scaling_factor), _ptr(q_out), _ptr(k_cache), _ptr(v_cache), _ptr(cache_len_dev),

@@ -243,3 +243,33 @@ def test_tree_attention_rope_repeated_calls_share_workspace(dev):
                                       row_stride=W, max_len=cap)
         torch.cuda.synchronize()
         assert rel_err(got.cpu().numpy(), want_t) <= TOL
+
+
+@pytest.mark.parametrize("H,G,hd,T", [(28, 4, 128, 32), (14, 2, 64, 17), (4, 4, 64, 1)])
+def test_rope_kv_append_from_table(dev, H, G, hd, T):
+    """Angles from the per-step cos/sin table instead of sincos in the launch: the values are
+    copies, the rotated q and k agree to one fp16 ulp in at most a handful of elements (the two
+    sincos evaluations may differ in the last fp32 bit)."""
+    rng = np.random.default_rng(H + T)
+    P, cap = 77, 77 + T + 5
+    W = (H + 2 * G) * hd
+    qkv = to_dev(synth.make_x(rng, T, W), dev)
+    pos = to_dev((P + rng.integers(0, 9, size=T)).astype(np.int32), dev)
+    inv = ops.default_inv_freqs(hd, 1000000.0, device=dev)
+    len_dev = torch.tensor([P], dtype=torch.int32, device=dev)
+    outs = []
+    for table in (False, True):
+        k = torch.zeros((G, cap, hd), dtype=torch.float16, device=dev)
+        v = torch.zeros_like(k)
+        q = torch.empty((H, T, hd), dtype=torch.float16, device=dev)
+        cs = ops.rope_table(pos, inv, 0.5) if table else None
+        ops.rope_kv_append(qkv, qkv[:, H * hd:], qkv[:, (H + G) * hd:], pos, inv, 0.5, q, k, v, len_dev, H, G, hd,
+                           row_stride=W, rope_cs=cs)
+        torch.cuda.synchronize()
+        outs.append((q, k, v))
+    (q0, k0, v0), (q1, k1, v1) = outs
+    assert torch.equal(v0, v1)
+    for a, b in ((q0, q1), (k0, k1)):
+        d = (a.float() - b.float()).abs()
+        assert int((d > 0).sum()) <= max(1, a.numel() // 10000)
+        assert float(d.max()) <= 2.0 ** -10 * float(a.float().abs().max())
