@@ -15,6 +15,9 @@ CONFIGS = {
                       attention_bias=True, tie=False),
     "llama_like_tied": dict(layers=2, hidden=512, inter=768, heads=4, kv_heads=4, head_dim=128, vocab=640,
                             attention_bias=False, tie=True, theta=5e5),
+    # down projection with K = 4608: K slabs of 256-column units at 32 rows
+    "long_mlp": dict(layers=2, hidden=256, inter=4608, heads=4, kv_heads=1, head_dim=64, vocab=512,
+                     attention_bias=True, tie=False),
 }
 
 
