@@ -222,13 +222,22 @@ __global__ __launch_bounds__(512) void tree_attn_split_kernel(
     // accumulator register i of this lane is key 8*(i/4) + 4*hb + i%4 of the tile
     float sv[16];
     float bm = -INFINITY;
+    if (kb + KT <= P) {
+      // a tile of prefix rows: visible to every token, no mask arithmetic
 #pragma unroll
-    for (int i = 0; i < 16; ++i) {
-      const int key = kb + 8 * (i >> 2) + 4 * hb + (i & 3);
-      const int rel = key - P;
-      const bool vis = (key < P) || (key < Ltot && ((mybits >> (rel & 31)) & 1u));
-      sv[i] = vis ? sacc[i] * scale_log2e : -INFINITY;
-      bm = fmaxf(bm, sv[i]);
+      for (int i = 0; i < 16; ++i) {
+        sv[i] = sacc[i] * scale_log2e;
+        bm = fmaxf(bm, sv[i]);
+      }
+    } else {
+#pragma unroll
+      for (int i = 0; i < 16; ++i) {
+        const int key = kb + 8 * (i >> 2) + 4 * hb + (i & 3);
+        const int rel = key - P;
+        const bool vis = (key < P) || (key < Ltot && ((mybits >> (rel & 31)) & 1u));
+        sv[i] = vis ? sacc[i] * scale_log2e : -INFINITY;
+        bm = fmaxf(bm, sv[i]);
+      }
     }
     bm = fmaxf(bm, __shfl_xor(bm, 32, 64));
     const float m_new = fmaxf(m_run, bm);
@@ -239,10 +248,11 @@ __global__ __launch_bounds__(512) void tree_attn_split_kernel(
 #pragma unroll
       for (int i = 0; i < 16; ++i) p[i] = 0.f;
     } else {
-      alpha = exp2f(m_run - m_new);
+      // arguments are <= 0: the bare hardware exp2 (results below 2^-126 flush to zero)
+      alpha = __builtin_amdgcn_exp2f(m_run - m_new);
 #pragma unroll
       for (int i = 0; i < 16; ++i) {
-        p[i] = exp2f(sv[i] - m_new);
+        p[i] = __builtin_amdgcn_exp2f(sv[i] - m_new);
         psum += p[i];
       }
     }
