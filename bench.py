@@ -25,7 +25,7 @@ sys.path.insert(0, ROOT)
 HBM_PEAK_GBS = 8000.0
 # HBM bytes per QMM launch of this workload (FETCH_SIZE + WRITE_SIZE from two rocprofv3 --pmc
 # runs of this script, scaled by a copy kernel of known size); None until measured.
-QMM_TRAFFIC_BYTES_PER_LAUNCH = 49201096
+QMM_TRAFFIC_BYTES_PER_LAUNCH = 47795789
 PREFIX = 2048
 NODES = 32
 
