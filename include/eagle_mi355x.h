@@ -186,6 +186,19 @@ int eagle_tree_attention_rope_f16(const void* q_lin, const void* k_lin, const vo
                                   int hd, long capacity, int max_len, float scale, void* workspace,
                                   size_t workspace_bytes, eagle_stream_t stream);
 
+/* Attention of the draft-side expansion (mlx_eagle.py:143-178,207 through mlx_llama.py:185-192):
+ * T <= 32 query tokens against the P = *cache_len_dev prefix rows (visible to every query) and
+ * the Tk <= 64 cache rows P .. P+Tk-1 that follow them, of which query t sees row j iff bit
+ * (j % 32) of mask_words[2*t + j/32] is set.  With T == Tk <= 32 and the upper words zero this
+ * is eagle_tree_attention_f16; the expansion has T = k queries and Tk = k * (level + 1) rows
+ * (every earlier level's rows plus its own).  q [H,T,hd], out [T, H*hd]; the workspace is the
+ * one of eagle_tree_attention_f16. */
+int eagle_draft_attention_f16(const void* q, const void* k_cache, const void* v_cache,
+                              const uint32_t* mask_words, const int32_t* cache_len_dev, void* out,
+                              int T, int Tk, int H, int G, int hd, long capacity, int max_len,
+                              float scale, void* workspace, size_t workspace_bytes,
+                              eagle_stream_t stream);
+
 /* Row argmax of fp16 logits [R,V], lowest index among equal maxima
  * (mx.argmax at mlx_eagle.py:316,534,596).  out [R] int32. */
 size_t eagle_argmax_workspace_bytes(int R, long V);
@@ -235,6 +248,47 @@ int eagle_greedy_accept(const int32_t* node_argmax, const int32_t* draft_tokens,
 int eagle_kv_compact_f16(void* const* caches_dev, int n_caches, const int32_t* accept,
                          int32_t* cache_len_dev, int G, int hd, long capacity,
                          eagle_stream_t stream);
+
+/* ---------------------------------------------------------------------------
+ * Draft-side tree expansion (generate_draft_tree and its helpers).
+ * ------------------------------------------------------------------------- */
+
+/* The k <= 8 most likely tokens of each of R <= 32 rows of fp16 logits [*, V] and their
+ * log-probabilities in fp16, best first, equal scores lowest index first.  row_index (may be
+ * NULL) selects the rows: row r reads logits row row_index[r] (a device value, e.g. the
+ * accept length of mlx_eagle.py:404).
+ *   mode 0 (mlx_eagle.py:410-412): top-k of the logits, score = fp16(logit - fp16(logsumexp))
+ *   mode 1 (mlx_eagle.py:103-104): score = fp16(log(fp16(softmax))), top-k of the scores
+ * (in fp16 distinct logits can share a score; the order among them is by index).
+ * out_index [R,k] int32, out_score [R,k] fp16. */
+size_t eagle_logsoftmax_topk_workspace_bytes(int R, long V);
+int eagle_logsoftmax_topk_f16(const void* logits, const int32_t* row_index, int R, long V, int k,
+                              int mode, int32_t* out_index, void* out_score, void* workspace,
+                              size_t workspace_bytes, eagle_stream_t stream);
+
+/* State of generate_draft_tree before its loop (mlx_eagle.py:130-155) from the level-0 top-k
+ * (topk_index [k] int32, topk_score [k] fp16):
+ *   saved_scores [k + k*k*depth] fp16 and saved_tokens (same length, int32): entries 0..k-1;
+ *   parents [1 + k*depth] uint32: entry 0 = 0 and the level-0 rows 1..k = 1..k;
+ *   cur_scores [k] fp16, cur_ids [k] int32: scores and input tokens of the first draft forward;
+ *   mask_words [k][2] uint32: the identity block (query r sees expansion row r). */
+int eagle_draft_tree_init(const int32_t* topk_index, const void* topk_score, int k,
+                          void* saved_scores, int32_t* saved_tokens, uint32_t* parents,
+                          void* cur_scores, int32_t* cur_ids, uint32_t* mask_words,
+                          eagle_stream_t stream);
+
+/* One level of the loop after the draft forward and the per-row top-k (mode 1) of its logits:
+ * process_generate_tree_iteration (mlx_eagle.py:97-115) and the bookkeeping around it
+ * (mlx_eagle.py:157-162,171,194-207).  topk_index / topk_score [k,k].  Writes the level's k*k
+ * cumulative scores (fp16 add) and tokens into saved_scores / saved_tokens at k + k*k*level,
+ * selects the k best (descending, ties lowest flat index) into topk_cs_index [k], out_ids [k]
+ * (= topk_cs_index / k), cur_scores, cur_ids; unless it is the last level, parents rows
+ * 1 + k*(level+1) .. and mask_words for the next level (child r inherits the words of query
+ * out_ids[r] and sees expansion row k*(level+1) + r).  Needs k * depth <= 64. */
+int eagle_draft_tree_level(const int32_t* topk_index, const void* topk_score, int level, int k,
+                           int depth, void* saved_scores, int32_t* saved_tokens, uint32_t* parents,
+                           void* cur_scores, int32_t* cur_ids, uint32_t* mask_words,
+                           int32_t* out_ids, int32_t* topk_cs_index, eagle_stream_t stream);
 
 /* Small device-side helpers for graph-replayed steps. */
 int eagle_fill_i32(int32_t* dst, int32_t value, long n, eagle_stream_t stream);

@@ -1,4 +1,4 @@
-// Tree-masked grouped-query attention of T <= 32 tree tokens against a KV cache (gfx950).
+// Tree-masked grouped-query attention of T <= 32 query tokens against a KV cache (gfx950).
 //
 //   out[t, h*hd + d] = sum_j softmax_j( scale * q[h,t,:] . k[g,j,:] + mask[t,j] ) v[g,j,d]
 //
@@ -16,6 +16,10 @@
 // Partial (m, l, O) per split go to a workspace and a second kernel merges them.  The key
 // tiles of the live length are dealt evenly to as many splits as give each at most
 // max(2, tiles / grid splits) tiles; the busiest workgroup sets the time.
+//
+// The draft-side form (mlx_eagle.py:143-178,207) has fewer query rows than masked key rows: T
+// queries see the P prefix rows and, through masks of one or two 32-bit words per query, the
+// Tk <= 64 rows P .. P+Tk-1 written by the earlier expansion levels and this one.
 //
 // A second form of the split kernel takes the un-rotated projection outputs instead
 // (mlx_llama.py:166-183): it rotates q and the tree keys itself and appends the tree rows to
@@ -55,13 +59,13 @@ __device__ inline void rotate_pair(half8_t& lo, half8_t& hi, const float* cs) {
 // taken from k_lin / v_lin instead of the cache, and the workgroup that owns a tile with tree
 // rows appends them to the cache (every tile has exactly one owner per KV group, and no
 // workgroup reads a cache row at or beyond P, so the append races with nothing).
-template <int HD, bool ROPE>
+template <int HD, bool ROPE, bool WIDE = false>
 __global__ __launch_bounds__(512) void tree_attn_split_kernel(
     const half_t* __restrict__ q, half_t* kc, half_t* vc,
     const uint32_t* __restrict__ mask_bits, const int32_t* __restrict__ len_dev,
     half_t* __restrict__ part_o, float* __restrict__ part_ml, int T, int H, int G, long cap,
     int tiles_per_split, float scale_log2e, const half_t* __restrict__ k_lin,
-    const half_t* __restrict__ v_lin, long ld, const float* __restrict__ rope_cs) {
+    const half_t* __restrict__ v_lin, long ld, const float* __restrict__ rope_cs, int Tk) {
   constexpr int KSTEPS = HD / 16;       // MFMA steps over the head dimension for S
   constexpr int DB = HD / 32;           // 32-wide blocks of the head dimension for O
   constexpr int STR = HD * 2 + 16;      // LDS row stride in bytes (pad: conflict-free reads)
@@ -89,7 +93,7 @@ __global__ __launch_bounds__(512) void tree_attn_split_kernel(
     if (P > cap - T) P = (int)(cap - T);
     if (P < 0) P = 0;
   }
-  const int Ltot = P + T;
+  const int Ltot = P + Tk;                // Tk = T unless WIDE
   const int ntiles = (Ltot + KT - 1) / KT;
   // Splits in use for this length: every workgroup gets at most `tpw` key tiles, two at
   // least (with one, writing and merging the partials costs more than reading the keys).
@@ -106,7 +110,9 @@ __global__ __launch_bounds__(512) void tree_attn_split_kernel(
       qreg[kk] = *reinterpret_cast<const half8_t*>(qp + kk * 16 + hb * 8);
     }
   }
-  const uint32_t mybits = ql < T ? mask_bits[ql] : 0u;
+  // WIDE: two mask words per query (masked key rows 0..31 and 32..63)
+  const uint32_t mybits = ql < T ? mask_bits[WIDE ? 2 * ql : ql] : 0u;
+  const uint32_t mybits_hi = (WIDE && ql < T) ? mask_bits[2 * ql + 1] : 0u;
 
   float m_run = -INFINITY, l_run = 0.f;
   float16_t o_acc[DB];
@@ -234,7 +240,8 @@ __global__ __launch_bounds__(512) void tree_attn_split_kernel(
       for (int i = 0; i < 16; ++i) {
         const int key = kb + 8 * (i >> 2) + 4 * hb + (i & 3);
         const int rel = key - P;
-        const bool vis = (key < P) || (key < Ltot && ((mybits >> (rel & 31)) & 1u));
+        const uint32_t word = (WIDE && rel >= 32) ? mybits_hi : mybits;
+        const bool vis = (key < P) || (key < Ltot && ((word >> (rel & 31)) & 1u));
         sv[i] = vis ? sacc[i] * scale_log2e : -INFINITY;
         bm = fmaxf(bm, sv[i]);
       }
@@ -313,7 +320,8 @@ template <int HD>
 __global__ void tree_attn_merge_kernel(const half_t* __restrict__ part_o,
                                        const float* __restrict__ part_ml,
                                        half_t* __restrict__ out, int T, int H, int nsplit,
-                                       const int32_t* __restrict__ len_dev, long cap, int clamp_len) {
+                                       const int32_t* __restrict__ len_dev, long cap, int clamp_len,
+                                       int Tk) {
   constexpr int QW = HD / 4;                       // threads per token
   constexpr int TPW = 256 / HD;                    // tokens per wave: MERGE_TOK tokens on HD / 64 waves
   constexpr int PRE = 8;
@@ -348,7 +356,7 @@ __global__ void tree_attn_merge_kernel(const half_t* __restrict__ part_o,
     if (P > cap - T) P = (int)(cap - T);
     if (P < 0) P = 0;
   }
-  const int nact = active_splits((P + T + KT - 1) / KT, nsplit);   // as in the split kernel
+  const int nact = active_splits((P + Tk + KT - 1) / KT, nsplit);   // as in the split kernel
 #pragma unroll
   for (int k = 0; k < TPW; ++k) {
     const float m = lane < nact ? ml[k][0] : -INFINITY;
@@ -398,21 +406,23 @@ int splits_for(int max_len, int G) {
   return n;
 }
 
-template <int HD, bool ROPE>
+template <int HD, bool ROPE, bool WIDE = false>
 int launch_attention(const half_t* q, half_t* kc, half_t* vc, const uint32_t* bits, const int32_t* len,
                      void* out, int T, int H, int G, long cap, int max_len, float scale, void* workspace,
-                     const half_t* k_lin, const half_t* v_lin, long ld, const float* cs, hipStream_t st) {
+                     const half_t* k_lin, const half_t* v_lin, long ld, const float* cs, hipStream_t st,
+                     int Tk = 0) {
+  if (!WIDE) Tk = T;
   const int nsplit = splits_for(max_len, G);
   float* part_ml = static_cast<float*>(workspace);
   half_t* part_o = reinterpret_cast<half_t*>(part_ml + (size_t)H * nsplit * 32 * 2);
   const float sl2 = scale * 1.4426950408889634f;
   const int rep = H / G;
   const size_t lds = 2 * KT * (HD * 2 + 16) + (ROPE ? (size_t)EAGLE_MAX_TREE * HD * 4 : 0);
-  hipLaunchKernelGGL((tree_attn_split_kernel<HD, ROPE>), dim3(G, nsplit), dim3(rep * 64), lds, st, q, kc,
-                     vc, bits, len, part_o, part_ml, T, H, G, cap, 0, sl2, k_lin, v_lin, ld, cs);
+  hipLaunchKernelGGL((tree_attn_split_kernel<HD, ROPE, WIDE>), dim3(G, nsplit), dim3(rep * 64), lds, st, q,
+                     kc, vc, bits, len, part_o, part_ml, T, H, G, cap, 0, sl2, k_lin, v_lin, ld, cs, Tk);
   hipLaunchKernelGGL(tree_attn_merge_kernel<HD>, dim3(H, (T + MERGE_TOK - 1) / MERGE_TOK),
                      dim3(MERGE_TOK * HD / 4), 0, st, part_o, part_ml, (half_t*)out, T, H, nsplit,
-                     len, cap, ROPE ? 1 : 0);
+                     len, cap, ROPE ? 1 : 0, Tk);
   return eagle_launch_status();
 }
 
@@ -463,6 +473,33 @@ EAGLE_EXPORT int eagle_tree_attention_f16(const void* q, const void* k_cache, co
                                         nullptr, st);
   return launch_attention<64, false>((const half_t*)q, kc, vc, tree_mask_bits, cache_len_dev, out, T, H, G,
                                      capacity, max_len, scale, workspace, nullptr, nullptr, 0, nullptr, st);
+}
+
+EAGLE_EXPORT int eagle_draft_attention_f16(const void* q, const void* k_cache, const void* v_cache,
+                                           const uint32_t* mask_words, const int32_t* cache_len_dev,
+                                           void* out, int T, int Tk, int H, int G, int hd,
+                                           long capacity, int max_len, float scale, void* workspace,
+                                           size_t workspace_bytes, eagle_stream_t stream) {
+  if (!q || !k_cache || !v_cache || !mask_words || !cache_len_dev || !out) return EAGLE_ERR_NULL;
+  if (T < 1 || T > EAGLE_MAX_TREE || Tk < 1 || Tk > 2 * EAGLE_MAX_TREE || H < 1 || G < 1 ||
+      (H % G) != 0 || (H / G) > 8 || (hd != 64 && hd != 128) || max_len < Tk || max_len > capacity)
+    return EAGLE_ERR_SHAPE;
+  if (!eagle_aligned16(q) || !eagle_aligned16(k_cache) || !eagle_aligned16(v_cache) ||
+      !eagle_aligned16(out))
+    return EAGLE_ERR_ALIGN;
+  if (!workspace || !eagle_aligned16(workspace) ||
+      workspace_bytes < eagle_tree_attention_workspace_bytes(H, hd, max_len))
+    return EAGLE_ERR_WORKSPACE;
+  hipStream_t st = static_cast<hipStream_t>(stream);
+  half_t* kc = const_cast<half_t*>(static_cast<const half_t*>(k_cache));
+  half_t* vc = const_cast<half_t*>(static_cast<const half_t*>(v_cache));
+  if (hd == 128)
+    return launch_attention<128, false, true>((const half_t*)q, kc, vc, mask_words, cache_len_dev, out, T,
+                                              H, G, capacity, max_len, scale, workspace, nullptr, nullptr,
+                                              0, nullptr, st, Tk);
+  return launch_attention<64, false, true>((const half_t*)q, kc, vc, mask_words, cache_len_dev, out, T, H,
+                                           G, capacity, max_len, scale, workspace, nullptr, nullptr, 0,
+                                           nullptr, st, Tk);
 }
 
 EAGLE_EXPORT int eagle_rope_table_f32(const int32_t* positions, const float* inv_freqs,

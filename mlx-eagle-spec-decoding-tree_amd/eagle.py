@@ -64,6 +64,84 @@ def bits_to_mask(bits, dtype=torch.bfloat16):
     return torch.where(vis, zero, torch.full((), -math.inf, dtype=dtype, device=bits.device))
 
 
+def _level_buffers(k, depth, dev):
+    C = k + k * k * depth
+    return dict(
+        saved_scores=torch.zeros(C, dtype=torch.float16, device=dev),
+        saved_tokens=torch.zeros(C, dtype=torch.int32, device=dev),
+        parents=torch.zeros(1 + k * depth, dtype=torch.int32, device=dev),
+        cur_scores=torch.zeros(k, dtype=torch.float16, device=dev),
+        cur_ids=torch.zeros(k, dtype=torch.int32, device=dev),
+        mask_words=torch.zeros((k, 2), dtype=torch.int32, device=dev),
+        out_ids=torch.zeros(k, dtype=torch.int32, device=dev),
+        topk_cs_index=torch.zeros(k, dtype=torch.int32, device=dev))
+
+
+def draft_tree_init(topk_index, topk_score, k, b):
+    """State of the expansion before its first level, in the buffers of `_level_buffers`."""
+    rc = _lib.lib().eagle_draft_tree_init(_ptr(topk_index), _ptr(topk_score), k, _ptr(b["saved_scores"]),
+                                          _ptr(b["saved_tokens"]), _ptr(b["parents"]),
+                                          _ptr(b["cur_scores"]), _ptr(b["cur_ids"]),
+                                          _ptr(b["mask_words"]), _stream())
+    _lib.check(rc, "draft_tree_init")
+
+
+def draft_tree_level(topk_index, topk_score, level, k, depth, b):
+    """One level of the expansion on the buffers of `_level_buffers` (no host round trip)."""
+    rc = _lib.lib().eagle_draft_tree_level(_ptr(topk_index), _ptr(topk_score), level, k, depth,
+                                           _ptr(b["saved_scores"]), _ptr(b["saved_tokens"]),
+                                           _ptr(b["parents"]), _ptr(b["cur_scores"]), _ptr(b["cur_ids"]),
+                                           _ptr(b["mask_words"]), _ptr(b["out_ids"]),
+                                           _ptr(b["topk_cs_index"]), _stream())
+    _lib.check(rc, "draft_tree_level")
+
+
+def process_generate_tree_iteration(logits, current_scores, k=8, tokenizer=None):
+    """mlx_eagle.py:97-115.  logits [1,k,V] fp16, current_scores [1,k,1] fp16 ->
+    (next_input_ids [1,k], next_scores [1,k,1], out_ids [k], topk_index [1,k,k],
+    cu_scores [1,k,k], topk_cs_index [k])."""
+    dev = logits.device
+    V = logits.shape[-1]
+    idx, score = ops.logsoftmax_topk(logits.reshape(-1, V), k, mode=1)
+    b = _level_buffers(k, 1, dev)
+    b["cur_scores"].copy_(current_scores.reshape(-1).to(torch.float16))
+    draft_tree_level(idx, score, 0, k, 1, b)
+    cu = b["saved_scores"][k:].reshape(1, k, k)
+    return (b["cur_ids"][None], b["cur_scores"].reshape(1, k, 1), b["out_ids"],
+            idx.reshape(1, k, k), cu, b["topk_cs_index"])
+
+
+def generate_draft_tree(topk_index, topk_p, draft_model, cache, depth=5, k=8, tokenizer=None):
+    """mlx_eagle.py:118-213: `depth` draft forwards of k tokens, all k at one position, each seeing
+    the prefix, its ancestors' rows and its own.  topk_index [1,k], topk_p [1,k,1] ->
+    (parents_list, saved_topk_indices, saved_cu_scores) as lists of per-level tensors."""
+    dev = topk_index.device
+    offset = cache[0].offset
+    current_input_ids = topk_index.to(torch.int32)
+    scores = topk_p.to(torch.float16)
+    ninf = float("-inf")
+    mask = torch.full((1, 1, k, offset + depth * k), ninf, dtype=torch.bfloat16, device=dev)
+    mask[..., :offset] = 0
+    eye = torch.full((k, k), ninf, dtype=torch.bfloat16, device=dev)
+    eye.fill_diagonal_(0)
+    saved_topk_indices = [current_input_ids[:, None]]
+    saved_cu_scores = [scores.transpose(1, 2)]
+    parents_list = [torch.zeros(1, dtype=torch.int32, device=dev)]
+    topk_cs_index = torch.arange(k, dtype=torch.int32, device=dev)
+    for i in range(depth):
+        bias = 1 + k * k * max(0, i - 1) + (k if i > 0 else 0)
+        parents_list.append(topk_cs_index + bias)
+        mask[..., offset + i * k: offset + (i + 1) * k] = eye
+        logits = draft_model(current_input_ids, cache, position_ids=offset + i, flat_rope=True,
+                             mask=mask[..., : offset + (i + 1) * k])
+        (current_input_ids, scores, out_ids, topk_index, cu_scores,
+         topk_cs_index) = process_generate_tree_iteration(logits, scores, k=k)
+        saved_topk_indices.append(topk_index)
+        saved_cu_scores.append(cu_scores)
+        mask = mask[..., out_ids.long(), :]
+    return parents_list, saved_topk_indices, saved_cu_scores
+
+
 def process_draft_tree_device(scores, tokens, parents_list, sampled_token_id, k, total_tokens,
                               out=None):
     """Device-only form: flat fp16 scores [C], int32 tokens [C], parents [C/k] ->
@@ -159,6 +237,91 @@ def accept_candidate(cache, accept_indices, accept_length, offset):
         _lib.check(rc, "accept_candidate")
     for c in cache:
         c.offset = offset + accept_length + 1
+
+
+def spec_step(y, base_model, draft_model, base_cache, draft_cache, offset=None, accept_length=0,
+              k=8, depth=5, verify_num_tokens=31, tokenizer=None):
+    """mlx_eagle.py:379-463 up to its first return: the draft forward of the tokens accepted
+    last step, the level-0 top-k, the expansion, the tree layout and the target forward.
+    y [1, accept_length + 1] int.  Returns (tree_position_ids, mask_index, draft_tokens,
+    base_logits, base_offset, draft_offset)."""
+    base_offset = base_cache[0].offset
+    draft_offset = draft_cache[0].offset + 1 + accept_length
+    _y = y
+    if accept_length > 0:
+        pad_size = 8 - accept_length - 1
+        if pad_size < 0:
+            raise ValueError("accept_length above 7")
+        y = torch.cat((y, torch.zeros((1, pad_size), dtype=y.dtype, device=y.device)), dim=-1)
+    draft_logits = draft_model(y, cache=draft_cache)
+    for c in draft_cache:
+        c.offset = draft_offset
+    row = torch.tensor([accept_length], dtype=torch.int32, device=y.device)
+    topk_index, topk_p = ops.logsoftmax_topk(draft_logits[0], k, mode=0, row_index=row)
+    out_parents, out_tokens, out_scores = generate_draft_tree(
+        topk_index=topk_index, topk_p=topk_p[..., None], draft_model=draft_model, cache=draft_cache,
+        depth=depth, k=k)
+    tree_position_ids, mask_index, draft_tokens, tree_mask = process_draft_tree(
+        scores_list=out_scores, ss_token=out_tokens, parents_list=out_parents,
+        sampled_token_id=_y[:, -1:], k=k, total_tokens=verify_num_tokens)
+    base_logits = tree_decoding(token_ids=draft_tokens, tree_mask=tree_mask, base_model=base_model,
+                                cache=base_cache, tree_position_ids=tree_position_ids)
+    return tree_position_ids, mask_index, draft_tokens, base_logits, base_offset, draft_offset
+
+
+def generate_step(prompt, base_model, draft_model, prefill_step_size=512, k=8, depth=5,
+                  verify_num_tokens=31, max_tokens=128, tokenizer=None, N=20, capacity=None):
+    """mlx_eagle.py:503-606, greedy.  prompt: 1-D int tensor on the models' device.  Instead of
+    printing, returns dict(tokens: every generated token in order, first: the token sampled
+    from the prompt, steps: per step (accept_length, best_candidate, accept_indices, y), n,
+    mean_tokens_per_step)."""
+    from .cache import make_prompt_cache
+
+    if verify_num_tokens + 1 > MAXT:
+        raise ValueError(f"at most {MAXT - 1} draft nodes per verification")
+    y = prompt.reshape(-1).to(torch.int64)
+    if capacity is None:
+        capacity = y.numel() + max_tokens + N + k * depth + MAXT + 16
+    base_cache = make_prompt_cache(base_model, capacity=capacity)
+    draft_cache = make_prompt_cache(draft_model, capacity=capacity)
+    while y.numel() > prefill_step_size:
+        draft_model(y[:prefill_step_size][None], cache=draft_cache)
+        base_model(y[:prefill_step_size][None], cache=base_cache)
+        y = y[prefill_step_size:]
+    draft_model(y[None], cache=draft_cache)
+    base_logits = base_model(y[None], cache=base_cache)
+    y = ops.argmax_rows(base_logits[0, -1:].contiguous()).reshape(1, 1).to(torch.int64)
+    first = int(y.item())
+    tokens, steps = [], []
+    n = 0
+    accept_length = 0
+    i = -1
+    for i in range(N):
+        if n >= max_tokens:
+            break
+        (tree_position_ids, mask_index, draft_tokens, base_logits, base_offset,
+         draft_offset) = spec_step(y, base_model, draft_model, base_cache, draft_cache,
+                                   accept_length=accept_length, k=k, depth=depth,
+                                   verify_num_tokens=verify_num_tokens)
+        retrieve_indices = post_process_draft_tree(tree_position_ids, verify_num_tokens, mask_index)
+        ri = retrieve_indices.long()                  # -1 wraps to the last node (mlx_eagle.py:582)
+        candidates = draft_tokens[0, ri]
+        best, al, sample_p = evaluate_posterior_greedy(base_logits[0, ri], candidates)
+        accept_length = int(al.item())
+        best = int(best.item())
+        accept_indices = retrieve_indices[best, 1:1 + accept_length]
+        accepted_tokens = candidates[best, 1:1 + accept_length]
+        accept_candidate(base_cache, accept_indices, accept_length, base_offset)
+        for c in draft_cache:
+            c.offset = draft_offset
+        next_token = ops.argmax_rows(sample_p[None].contiguous()).reshape(1)
+        y = torch.cat((accepted_tokens.to(torch.int64), next_token.to(torch.int64)))[None]
+        n += 1 + accept_length
+        tokens.extend(int(t) for t in y[0].tolist())
+        steps.append((accept_length, best, [int(v) for v in accept_indices.tolist()],
+                      [int(v) for v in y[0].tolist()]))
+    return dict(tokens=tokens, first=first, steps=steps, n=n,
+                mean_tokens_per_step=n / max(1, len(steps)))
 
 
 class TreeVerifier:

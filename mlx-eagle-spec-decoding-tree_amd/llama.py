@@ -6,8 +6,8 @@ fp16 roundings fall in the same places; every operator runs as a HIP kernel
 behind the C ABI.  `patch_model(model, kernel)` is the plug-in seam of
 mlx_model_fwd_bench.py:43-86.
 
-Only the tree-verification shapes are served: at most 32 rows per linear layer
-and an explicit additive mask; prefill is outside this build.
+The kernels serve at most 32 rows per linear layer.  Passes without a mask are causal
+(mlx_llama.py:275-276); longer ones (the prompt) run as consecutive 32-token passes.
 """
 from functools import reduce
 
@@ -16,6 +16,9 @@ import torch
 
 from . import ops
 from .synth import ModelArgs, inv_freqs
+
+
+CAUSAL_CHUNK = 32
 
 
 class Module:
@@ -175,12 +178,17 @@ class LlamaModel(Module):
         self.norm = RMSNorm(tensors["model.norm.weight"], args.rms_norm_eps)
 
     def __call__(self, inputs, cache=None, mask=None, position_ids=None, flat_rope=False):
+        if cache is None:
+            raise NotImplementedError("the tree path always runs with a KV cache")
+        L = inputs.shape[1]
         h = self.embed_tokens(inputs)
         if mask is None:
-            raise NotImplementedError("causal prefill masks are outside the tree path")
+            # causal over the new tokens, everything in the cache visible (mlx_llama.py:275-276)
+            offset = cache[0].offset
+            mask = torch.zeros((1, 1, L, offset + L), dtype=h.dtype, device=h.device)
+            mask[..., offset:] = torch.triu(
+                torch.full((L, L), float("-inf"), dtype=h.dtype, device=h.device), diagonal=1)
         mask = mask.to(h.dtype)                                    # mlx_llama.py:278
-        if cache is None:
-            cache = [None] * len(self.layers)
         for layer, c in zip(self.layers, cache):
             h = layer(h, mask, cache=c, position_ids=position_ids, flat_rope=flat_rope)
         return self.norm(h)
@@ -208,6 +216,14 @@ class Model(Module):
         return cls(args, tensors, device)
 
     def __call__(self, inputs, cache=None, mask=None, position_ids=None, flat_rope=False):
+        if mask is None and inputs.shape[1] > CAUSAL_CHUNK:
+            # a long causal pass (prompt prefill, mlx_eagle.py:522-533) as consecutive passes of
+            # at most 32 tokens: the kernels of this path take at most 32 rows
+            if position_ids is not None or flat_rope:
+                raise NotImplementedError("chunked causal passes take their positions from the cache")
+            parts = [self(inputs[:, s:s + CAUSAL_CHUNK], cache)
+                     for s in range(0, inputs.shape[1], CAUSAL_CHUNK)]
+            return torch.cat(parts, dim=1)
         out = self.model(inputs, cache, mask=mask, position_ids=position_ids, flat_rope=flat_rope)
         if self.args.tie_word_embeddings:
             return self.model.embed_tokens.as_linear(out)

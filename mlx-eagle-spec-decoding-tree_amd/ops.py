@@ -288,10 +288,48 @@ def tree_attention_rope(q_lin, k_lin, v_lin, rope_cs, k_cache, v_cache, tree_mas
     return out
 
 
+def mask_to_words(mask):
+    """[T,Tk] additive ({0,-inf}) or boolean visibility matrix, Tk <= 64 -> [T,2] int32: bit
+    (j % 32) of word j // 32 says whether query t sees masked row j."""
+    vis = mask if mask.dtype == torch.bool else (mask == 0)
+    T, Tk = vis.shape
+    if Tk > 64:
+        raise ValueError("at most 64 masked rows")
+    v = torch.zeros((T, 64), dtype=torch.int64, device=vis.device)
+    v[:, :Tk] = vis.to(torch.int64)
+    weights = torch.ones(32, dtype=torch.int64, device=vis.device) << torch.arange(32, device=vis.device)
+    words = (v.reshape(T, 2, 32) * weights[None, None, :]).sum(2)
+    words = torch.where(words >= 2 ** 31, words - 2 ** 32, words)
+    return words.to(torch.int32).contiguous()
+
+
+def draft_attention(q, k_cache, v_cache, mask_words, cache_len_dev, Tk, scale, max_len=None, out=None):
+    """q [H,T,hd]; k_cache, v_cache [G,capacity,hd] holding *cache_len_dev prefix rows followed
+    by Tk <= 64 rows that query t sees according to mask_words [T,2].  Returns [T, H*hd]."""
+    _need_cuda(q, k_cache, v_cache, mask_words, cache_len_dev)
+    H, T, hd = q.shape
+    G, cap, _ = k_cache.shape
+    if max_len is None:
+        max_len = cap
+    if out is None:
+        out = torch.empty((T, H * hd), dtype=torch.float16, device=q.device)
+    L = _lib.lib()
+    need = L.eagle_tree_attention_workspace_bytes(H, hd, max_len)
+    ws = workspace("attn", need, q.device)
+    rc = L.eagle_draft_attention_f16(_ptr(q), _ptr(k_cache), _ptr(v_cache), _ptr(mask_words),
+                                     _ptr(cache_len_dev), _ptr(out), T, int(Tk), H, G, hd, cap, max_len,
+                                     float(scale), _ptr(ws), ws.numel(), _stream())
+    _lib.check(rc, "draft_attention")
+    return out
+
+
 def scaled_dot_product_attention(queries, keys, values, cache=None, scale=None, mask=None):
-    """Drop-in for the call at mlx_llama.py:185-192 on the tree path:
-    queries [1,H,T,hd], keys/values [1,G,S,hd] (prefix then the T tree rows),
-    mask [1,1,T,S] additive whose prefix part is zero.  Returns [1,H,T,hd]."""
+    """Drop-in for the call at mlx_llama.py:185-192 on the tree and draft paths:
+    queries [1,H,T,hd] with T <= 32, keys/values [1,G,S,hd], mask [1,1,T,S] additive.  Only
+    the last min(S, 64) columns of the mask are looked at: every earlier column has to be zero
+    (a prefix that all queries see), which holds for the verification mask
+    (mlx_eagle.py:337-338), the expansion masks up to depth 8 (mlx_eagle.py:143-171) and causal
+    masks of up to 32 new tokens.  Returns [1,H,T,hd]."""
     _need_cuda(queries, keys, values, mask)
     B, H, T, hd = queries.shape
     if B != 1:
@@ -299,18 +337,38 @@ def scaled_dot_product_attention(queries, keys, values, cache=None, scale=None, 
     G, S = keys.shape[1], keys.shape[2]
     if scale is None:
         scale = hd ** -0.5
-    P = S - T
     if mask is None:
         raise ValueError("the tree path always passes a mask")
-    m = mask.reshape(T, S)
-    bits = mask_to_bits(m[:, P:])
+    Tk = min(S, 64)
+    P = S - Tk
+    words = mask_to_words(mask.reshape(T, S)[:, P:])
     len_dev = torch.tensor([P], dtype=torch.int32, device=queries.device)
     if cache is not None and keys.data_ptr() == cache.keys.data_ptr():
         k_buf, v_buf = cache.keys[0], cache.values[0]        # the fetched views alias the cache
     else:
         k_buf, v_buf = _f16(keys[0], "k"), _f16(values[0], "v")
-    out = tree_attention(_f16(queries[0], "q"), k_buf, v_buf, bits, len_dev, scale, max_len=S)
+    out = draft_attention(_f16(queries[0], "q"), k_buf, v_buf, words, len_dev, Tk, scale, max_len=S)
     return out.reshape(T, H, hd).permute(1, 0, 2).unsqueeze(0).contiguous()
+
+
+def logsoftmax_topk(logits, k, mode, row_index=None, out=None):
+    """The k most likely tokens per row of fp16 logits [R,V] (or the rows row_index selects)
+    and their fp16 log-probabilities, best first, ties lowest index first.  mode 0: the level-0
+    form of mlx_eagle.py:410-412; mode 1: the form of mlx_eagle.py:103-104.
+    Returns (index [R,k] int32, score [R,k] fp16)."""
+    _need_cuda(logits, row_index)
+    logits = _f16(logits, "logits")
+    V = logits.shape[-1]
+    R = row_index.numel() if row_index is not None else logits.numel() // V
+    if out is None:
+        out = (torch.empty((R, k), dtype=torch.int32, device=logits.device),
+               torch.empty((R, k), dtype=torch.float16, device=logits.device))
+    L = _lib.lib()
+    ws = workspace("topk", L.eagle_logsoftmax_topk_workspace_bytes(R, V), logits.device)
+    rc = L.eagle_logsoftmax_topk_f16(_ptr(logits), _ptr(row_index), R, V, int(k), int(mode),
+                                     _ptr(out[0]), _ptr(out[1]), _ptr(ws), ws.numel(), _stream())
+    _lib.check(rc, "logsoftmax_topk")
+    return out
 
 
 def rms_norm(x, weight, eps, residual=None, out=None, h_out=None):
