@@ -290,6 +290,21 @@ int eagle_draft_tree_level(const int32_t* topk_index, const void* topk_score, in
                            void* cur_scores, int32_t* cur_ids, uint32_t* mask_words,
                            int32_t* out_ids, int32_t* topk_cs_index, eagle_stream_t stream);
 
+/* Loop state of the speculative step on the device, so that consecutive steps need no host
+ * round trip.  `accept` is the result array of eagle_greedy_accept of the previous step
+ * ({best, accept_length, bonus_node, next_token, ...}).
+ * eagle_spec_begin (mlx_eagle.py:393-394): *expand_len = *write_len = *draft_len + 1 +
+ * accept_length, the row at which the expansion starts in the draft cache.
+ * eagle_spec_update (mlx_eagle.py:591-599) after the verification: y [y_len] = the accepted
+ * tokens, the bonus token, zeros; *draft_len = *expand_len; *root_token = the bonus token; the
+ * accept_length + 1 new tokens are appended to out_tokens [max_out] at *out_count, which
+ * advances (tokens beyond max_out are dropped, the count still advances). */
+int eagle_spec_begin(const int32_t* draft_len_dev, const int32_t* accept, int32_t* expand_len_dev,
+                     int32_t* write_len_dev, eagle_stream_t stream);
+int eagle_spec_update(const int32_t* accept, const int32_t* accepted_tokens, int32_t* y, int y_len,
+                      int32_t* draft_len_dev, const int32_t* expand_len_dev, int32_t* root_token_dev,
+                      int32_t* out_tokens, int32_t* out_count_dev, int max_out, eagle_stream_t stream);
+
 /* Small device-side helpers for graph-replayed steps. */
 int eagle_fill_i32(int32_t* dst, int32_t value, long n, eagle_stream_t stream);
 /* positions[t] = *cache_len_dev + tree_position_ids[t] (mlx_eagle.py:343). */

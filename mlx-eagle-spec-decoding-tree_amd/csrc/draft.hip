@@ -254,6 +254,39 @@ __global__ __launch_bounds__(64) void draft_tree_level_kernel(
   }
 }
 
+// Loop state of the speculative step kept on the device (mlx_eagle.py:393-394, 591-599).
+__global__ void spec_begin_kernel(const int32_t* __restrict__ draft_len,
+                                  const int32_t* __restrict__ accept, int32_t* __restrict__ expand_len,
+                                  int32_t* __restrict__ write_len) {
+  if (threadIdx.x == 0) {
+    const int32_t v = *draft_len + 1 + accept[1];     // draft_offset (mlx_eagle.py:394)
+    *expand_len = v;
+    *write_len = v;
+  }
+}
+
+__global__ void spec_update_kernel(const int32_t* __restrict__ accept,
+                                   const int32_t* __restrict__ accepted_tokens, int32_t* __restrict__ y,
+                                   int y_len, int32_t* __restrict__ draft_len,
+                                   const int32_t* __restrict__ expand_len, int32_t* __restrict__ root_token,
+                                   int32_t* __restrict__ out_tokens, int32_t* __restrict__ out_count,
+                                   int max_out) {
+  const int j = threadIdx.x;
+  const int a = accept[1];
+  const int32_t next = accept[3];
+  const int base = *out_count;
+  int32_t v = 0;
+  if (j < a) v = accepted_tokens[j]; else if (j == a) v = next;
+  if (j < y_len) y[j] = v;                            // accepted tokens, bonus token, zero padding
+  if (j <= a && base + j < max_out) out_tokens[base + j] = v;
+  __syncthreads();
+  if (j == 0) {
+    *draft_len = *expand_len;                         // the expansion rows are dropped (:593-594)
+    *root_token = next;
+    *out_count = base + a + 1;
+  }
+}
+
 inline int chunks_for(long V) { return (int)((V + CHUNK - 1) / CHUNK); }
 
 }  // namespace
@@ -326,5 +359,28 @@ EAGLE_EXPORT int eagle_draft_tree_level(const int32_t* topk_index, const void* t
                      topk_index, static_cast<const half_t*>(topk_score), level, k, depth,
                      static_cast<half_t*>(saved_scores), saved_tokens, parents,
                      static_cast<half_t*>(cur_scores), cur_ids, mask_words, out_ids, topk_cs_index);
+  return eagle_launch_status();
+}
+
+EAGLE_EXPORT int eagle_spec_begin(const int32_t* draft_len_dev, const int32_t* accept,
+                                  int32_t* expand_len_dev, int32_t* write_len_dev,
+                                  eagle_stream_t stream) {
+  if (!draft_len_dev || !accept || !expand_len_dev || !write_len_dev) return EAGLE_ERR_NULL;
+  hipLaunchKernelGGL(spec_begin_kernel, dim3(1), dim3(64), 0, static_cast<hipStream_t>(stream),
+                     draft_len_dev, accept, expand_len_dev, write_len_dev);
+  return eagle_launch_status();
+}
+
+EAGLE_EXPORT int eagle_spec_update(const int32_t* accept, const int32_t* accepted_tokens, int32_t* y,
+                                   int y_len, int32_t* draft_len_dev, const int32_t* expand_len_dev,
+                                   int32_t* root_token_dev, int32_t* out_tokens, int32_t* out_count_dev,
+                                   int max_out, eagle_stream_t stream) {
+  if (!accept || !accepted_tokens || !y || !draft_len_dev || !expand_len_dev || !root_token_dev ||
+      !out_tokens || !out_count_dev)
+    return EAGLE_ERR_NULL;
+  if (y_len < 1 || y_len > 64 || max_out < 1) return EAGLE_ERR_SHAPE;
+  hipLaunchKernelGGL(spec_update_kernel, dim3(1), dim3(64), 0, static_cast<hipStream_t>(stream), accept,
+                     accepted_tokens, y, y_len, draft_len_dev, expand_len_dev, root_token_dev, out_tokens,
+                     out_count_dev, max_out);
   return eagle_launch_status();
 }

@@ -324,6 +324,51 @@ def generate_step(prompt, base_model, draft_model, prefill_step_size=512, k=8, d
                 mean_tokens_per_step=n / max(1, len(steps)))
 
 
+def fuse_projections(model, swiglu):
+    """Lay q/k/v and gate/up of every layer out as one matrix each (rows concatenated) and
+    re-point the layers' tensors at row blocks of it, so that one matmul launch serves
+    the three (two) projections; memory use is unchanged."""
+    qkv_w, gu_w = [], []
+
+    def interleave(lins):
+        g, u = lins
+        fused = [ops.interleave_gate_up(getattr(g, k), getattr(u, k))
+                 for k in ("weight", "scales", "biases")]
+        bias = None
+        if g.bias is not None or u.bias is not None:
+            z = torch.zeros(g.weight.shape[0], dtype=torch.float16, device=g.weight.device)
+            bias = ops.interleave_gate_up(g.bias if g.bias is not None else z,
+                                          u.bias if u.bias is not None else z)
+        return (*fused, bias)
+
+    def fuse(lins):
+        parts = [[l.weight, l.scales, l.biases] for l in lins]
+        fused = [torch.cat([p[k] for p in parts], dim=0).contiguous() for k in range(3)]
+        bias = None
+        if any(l.bias is not None for l in lins):
+            bias = torch.cat([l.bias if l.bias is not None
+                              else torch.zeros(l.weight.shape[0], dtype=torch.float16,
+                                               device=l.weight.device) for l in lins]).contiguous()
+        row = 0
+        for l in lins:
+            n = l.weight.shape[0]
+            l.weight, l.scales, l.biases = (f[row:row + n] for f in fused)
+            if l.bias is not None:
+                l.bias = bias[row:row + n]
+            row += n
+        return (*fused, bias)
+
+    for layer in model.model.layers:
+        at, mlp = layer.self_attn, layer.mlp
+        qkv_w.append(fuse([at.q_proj, at.k_proj, at.v_proj]))
+        if swiglu:
+            # a tile-interleaved copy: the layers keep their own tensors for the module path
+            gu_w.append(interleave([mlp.gate_proj, mlp.up_proj]))
+        else:
+            gu_w.append(fuse([mlp.gate_proj, mlp.up_proj]))
+    return qkv_w, gu_w
+
+
 class TreeVerifier:
     """One target-model tree-verification step with static buffers, so that it can be
     captured once in a HIP graph and replayed: embedding, all decoder layers, final norm,
@@ -400,47 +445,7 @@ class TreeVerifier:
         ops.workspace("argmax", L.eagle_argmax_workspace_bytes(T, args.vocab_size), dev)
 
     def _fuse_projections(self):
-        """Lay q/k/v and gate/up of every layer out as one matrix each (rows concatenated) and
-        re-point the layers' tensors at row blocks of it, so that one matmul launch serves
-        the three (two) projections; memory use is unchanged."""
-        self.qkv_w, self.gu_w = [], []
-
-        def interleave(lins):
-            g, u = lins
-            fused = [ops.interleave_gate_up(getattr(g, k), getattr(u, k))
-                     for k in ("weight", "scales", "biases")]
-            bias = None
-            if g.bias is not None or u.bias is not None:
-                z = torch.zeros(g.weight.shape[0], dtype=torch.float16, device=g.weight.device)
-                bias = ops.interleave_gate_up(g.bias if g.bias is not None else z,
-                                              u.bias if u.bias is not None else z)
-            return (*fused, bias)
-
-        def fuse(lins):
-            parts = [[l.weight, l.scales, l.biases] for l in lins]
-            fused = [torch.cat([p[k] for p in parts], dim=0).contiguous() for k in range(3)]
-            bias = None
-            if any(l.bias is not None for l in lins):
-                bias = torch.cat([l.bias if l.bias is not None
-                                  else torch.zeros(l.weight.shape[0], dtype=torch.float16,
-                                                   device=l.weight.device) for l in lins]).contiguous()
-            row = 0
-            for l in lins:
-                n = l.weight.shape[0]
-                l.weight, l.scales, l.biases = (f[row:row + n] for f in fused)
-                if l.bias is not None:
-                    l.bias = bias[row:row + n]
-                row += n
-            return (*fused, bias)
-
-        for layer in self.model.model.layers:
-            at, mlp = layer.self_attn, layer.mlp
-            self.qkv_w.append(fuse([at.q_proj, at.k_proj, at.v_proj]))
-            if self.swiglu:
-                # a tile-interleaved copy: the layers keep their own tensors for the module path
-                self.gu_w.append(interleave([mlp.gate_proj, mlp.up_proj]))
-            else:
-                self.gu_w.append(fuse([mlp.gate_proj, mlp.up_proj]))
+        self.qkv_w, self.gu_w = fuse_projections(self.model, self.swiglu)
 
     def qmm_launches(self):
         """(weight, scales, biases, bias, x, out, swiglu) of every quantised matmul of one step,

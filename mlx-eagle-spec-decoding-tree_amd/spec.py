@@ -1,0 +1,229 @@
+"""The whole speculative step of the reference loop (mlx_eagle.py:379-463, 571-599) enqueued on
+one stream with static buffers and all loop state on the device: draft pass over the tokens
+accepted last step, level-0 top-k, `depth` expansion passes with their bookkeeping, tree layout,
+target verification, greedy acceptance, KV compaction, state update.  Captured once as a HIP
+graph, N steps are N replays and one device-to-host copy of the emitted tokens at the end (the
+reference synchronises at least five times per step).
+
+Differences from the host-driven functions of eagle.py, both invisible in the results: the
+draft pass over the accepted tokens always has 8 rows (the reference pads to 8 only when
+something was accepted, mlx_eagle.py:400-408; row `accept_length` of a causal pass does not
+depend on the rows after it), and the expansion masks travel as two 32-bit words per query.
+"""
+import torch
+
+from . import _lib, ops
+from .eagle import (MAXT, TreeVerifier, _level_buffers, _ptr, _stream, draft_tree_init, draft_tree_level,
+                    fuse_projections, process_draft_tree_device)
+
+Y_LEN = 8
+
+
+class DecoderPass:
+    """One pass of T <= 32 rows through a decoder with static buffers: tokens -> logits [T,V].
+    The rows are written to the cache at *write_len; query t sees the *attn_len rows before
+    them and, of the Tk rows from there on, those its two mask words select."""
+
+    def __init__(self, model, cache, T, max_len=None, swiglu=True):
+        args = model.args
+        self.model, self.cache, self.args, self.T = model, cache, args, T
+        dev = model.device
+        D, I = args.hidden_size, args.intermediate_size
+        H, G, hd = args.num_attention_heads, args.num_key_value_heads, args.head_dim
+        self.max_len = max_len or cache[0].capacity
+        self.swiglu = bool(swiglu and ops.swiglu_supported(T, I, D))
+        self.qkv_w, self.gu_w = fuse_projections(model, self.swiglu)
+        f16 = dict(dtype=torch.float16, device=dev)
+        self.h = torch.empty((T, D), **f16)
+        self.hn = torch.empty((T, D), **f16)
+        self.qkv = torch.empty((T, (H + 2 * G) * hd), **f16)
+        self.q_rot = torch.empty((H, T, hd), **f16)
+        self.rope_cs = torch.empty((T, hd // 2, 2), dtype=torch.float32, device=dev)
+        self.attn = torch.empty((T, H * hd), **f16)
+        self.o = torch.empty((T, D), **f16)
+        self.gate_up = torch.empty((T, 2 * I), **f16)
+        self.act = torch.empty((T, I), **f16)
+        self.down = torch.empty((T, D), **f16)
+        self.logits = torch.empty((T, args.vocab_size), **f16)
+        L = _lib.lib()
+        head = model.lm_head if not args.tie_word_embeddings else model.model.embed_tokens
+        need = max(L.eagle_qmm_workspace_bytes(T, n, k) for n, k in
+                   (((H + 2 * G) * hd, D), (D, H * hd), (2 * I, D), (D, I), (head.weight.shape[0], D)))
+        ops.workspace("qmm", need, dev)
+        ops.workspace("attn", L.eagle_tree_attention_workspace_bytes(H, hd, self.max_len), dev)
+        ops.workspace("topk", L.eagle_logsoftmax_topk_workspace_bytes(T, args.vocab_size), dev)
+
+    def forward(self, tokens, positions, write_len, attn_len, mask_words, Tk):
+        m, args = self.model, self.args
+        H, G, hd = args.num_attention_heads, args.num_key_value_heads, args.head_dim
+        W = (H + 2 * G) * hd
+        emb = m.model.embed_tokens
+        ops.embed(tokens, emb.weight, emb.scales, emb.biases, out=self.h)
+        layers = m.model.layers
+        ops.rms_norm(self.h, layers[0].input_layernorm.weight, args.rms_norm_eps, out=self.hn)
+        at0 = layers[0].self_attn
+        ops.rope_table(positions, at0._inv_freqs, at0._scaling_factor, out=self.rope_cs)
+        for i, layer in enumerate(layers):
+            at, mlp, c = layer.self_attn, layer.mlp, self.cache[i]
+            w, sc, bi, b = self.qkv_w[i]
+            ops.quantized_matmul(self.hn, w, sc, bi, bias=b, out=self.qkv)
+            ops.rope_kv_append(self.qkv, self.qkv[:, H * hd:], self.qkv[:, (H + G) * hd:], positions,
+                               at._inv_freqs, at._scaling_factor, self.q_rot, c.keys[0], c.values[0],
+                               write_len, H, G, hd, row_stride=W, rope_cs=self.rope_cs)
+            ops.draft_attention(self.q_rot, c.keys[0], c.values[0], mask_words, attn_len, Tk, at.scale,
+                                max_len=self.max_len, out=self.attn)
+            ops.quantized_matmul(self.attn, at.o_proj.weight, at.o_proj.scales, at.o_proj.biases,
+                                 bias=at.o_proj.bias, out=self.o)
+            ops.rms_norm(self.o, layer.post_attention_layernorm.weight, args.rms_norm_eps,
+                         residual=self.h, out=self.hn, h_out=self.h)
+            w, sc, bi, b = self.gu_w[i]
+            if self.swiglu:
+                ops.quantized_matmul_swiglu(self.hn, w, sc, bi, bias=b, out=self.act)
+            else:
+                ops.quantized_matmul(self.hn, w, sc, bi, bias=b, out=self.gate_up)
+                ops.silu_mul(self.gate_up, None, out=self.act)
+            ops.quantized_matmul(self.act, mlp.down_proj.weight, mlp.down_proj.scales,
+                                 mlp.down_proj.biases, bias=mlp.down_proj.bias, out=self.down)
+            nxt = layers[i + 1].input_layernorm.weight if i + 1 < len(layers) else m.model.norm.weight
+            ops.rms_norm(self.down, nxt, args.rms_norm_eps, residual=self.h, out=self.hn, h_out=self.h)
+        head = m.model.embed_tokens if args.tie_word_embeddings else m.lm_head
+        ops.quantized_matmul(self.hn, head.weight, head.scales, head.biases, out=self.logits)
+        return self.logits
+
+
+class SpeculativeDecoder:
+    """Greedy tree-speculative generation with the step on the device.
+
+        dec = SpeculativeDecoder(base_model, draft_model, capacity=..., k=8, depth=3,
+                                 verify_num_tokens=31)
+        dec.prefill(prompt)          # both models, chunked causal passes; first token
+        dec.capture()                # optional: one HIP graph per step
+        tokens = dec.generate(n_steps)
+    """
+
+    def __init__(self, base_model, draft_model, capacity, k=8, depth=3, verify_num_tokens=31,
+                 max_out=8192):
+        from .cache import make_prompt_cache
+
+        if k != Y_LEN:
+            raise ValueError("the step is laid out for k = 8 candidates per node")
+        if verify_num_tokens + 1 > MAXT or k * depth > 64 or depth + 2 > Y_LEN:
+            raise ValueError("tree does not fit: at most 31 draft nodes, k * depth <= 64, depth <= 6")
+        if k + k * k * depth < verify_num_tokens:
+            raise ValueError("fewer candidates than draft nodes")
+        self.base_model, self.draft_model = base_model, draft_model
+        self.k, self.depth, self.V = k, depth, verify_num_tokens
+        self.capacity = capacity
+        dev = base_model.device
+        self.dev = dev
+        self.base_cache = make_prompt_cache(base_model, capacity=capacity)
+        self.draft_cache = make_prompt_cache(draft_model, capacity=capacity)
+        self.verifier = TreeVerifier(base_model, self.base_cache, total_tokens=verify_num_tokens,
+                                     max_len=capacity)
+        self.draft = DecoderPass(draft_model, self.draft_cache, k, max_len=capacity)
+        i32 = dict(dtype=torch.int32, device=dev)
+        self.y = torch.zeros(Y_LEN, **i32)
+        self.root_token = torch.zeros(1, **i32)
+        self.draft_len = self.draft_cache[0].len_dev
+        self.expand_len = torch.zeros(1, **i32)
+        self.write_len = torch.zeros(1, **i32)
+        self.positions = torch.zeros(k, **i32)
+        self.arange = torch.arange(k, **i32)
+        self.levels = torch.arange(depth, **i32)[:, None].repeat(1, k).contiguous()
+        causal = torch.tril(torch.ones((k, k), dtype=torch.bool, device=dev))
+        self.causal_words = ops.mask_to_words(causal)
+        self.topk_index = torch.zeros((k, k), **i32)
+        self.topk_score = torch.zeros((k, k), dtype=torch.float16, device=dev)
+        self.buf = _level_buffers(k, depth, dev)
+        self.out_tokens = torch.zeros(max_out, **i32)
+        self.out_count = torch.zeros(1, **i32)
+        self.max_out = max_out
+        self.graph = None
+        self.first = None
+
+    def prefill(self, prompt):
+        """mlx_eagle.py:522-535: both models read the prompt; the first token is the target's
+        argmax at its last position."""
+        ids = prompt.reshape(1, -1).to(torch.int64)
+        self.draft_model(ids, cache=self.draft_cache)
+        logits = self.base_model(ids, cache=self.base_cache)
+        first = ops.argmax_rows(logits[0, -1:].contiguous())
+        self.y.zero_()
+        self.y[:1] = first
+        self.root_token.copy_(first)
+        self.verifier.result.zero_()            # accept_length 0
+        self.out_count.zero_()
+        self.base_cache[0].sync_len()
+        self.draft_cache[0].sync_len()
+        self.first = int(first.item())
+        return self.first
+
+    def enqueue_step(self):
+        L = _lib.lib()
+        st = _stream()
+        k, depth, ver, d, b = self.k, self.depth, self.verifier, self.draft, self.buf
+        accept = ver.result
+        # draft pass over the accepted tokens and the bonus token (mlx_eagle.py:400-408)
+        _lib.check(L.eagle_tree_positions(_ptr(self.arange), _ptr(self.draft_len), _ptr(self.positions),
+                                          k, st), "positions")
+        logits = d.forward(self.y, self.positions, self.draft_len, self.draft_len, self.causal_words, k)
+        _lib.check(L.eagle_spec_begin(_ptr(self.draft_len), _ptr(accept), _ptr(self.expand_len),
+                                      _ptr(self.write_len), st), "spec_begin")
+        # level 0: the k most likely continuations of the bonus token (mlx_eagle.py:410-412)
+        ops.logsoftmax_topk(logits, k, 0, row_index=accept[1:2],
+                            out=(self.topk_index[:1], self.topk_score[:1]))
+        draft_tree_init(self.topk_index, self.topk_score, k, b)
+        for i in range(depth):
+            _lib.check(L.eagle_tree_positions(_ptr(self.levels[i]), _ptr(self.expand_len),
+                                              _ptr(self.positions), k, st), "positions")
+            logits = d.forward(b["cur_ids"], self.positions, self.write_len, self.expand_len,
+                               b["mask_words"], k * (i + 1))
+            ops.logsoftmax_topk(logits, k, 1, out=(self.topk_index, self.topk_score))
+            draft_tree_level(self.topk_index, self.topk_score, i, k, depth, b)
+            _lib.check(L.eagle_advance_len(_ptr(self.write_len), k, st), "advance_len")
+        process_draft_tree_device(b["saved_scores"], b["saved_tokens"], b["parents"], self.root_token, k,
+                                  self.V, out=(ver.tree_position_ids, ver.mask_index, ver.tokens,
+                                               ver.mask_bits))
+        ver.forward()        # target pass, argmax, acceptance, KV compaction, target length
+        _lib.check(L.eagle_spec_update(_ptr(accept), _ptr(ver.accepted_tokens), _ptr(self.y), Y_LEN,
+                                       _ptr(self.draft_len), _ptr(self.expand_len),
+                                       _ptr(self.root_token), _ptr(self.out_tokens),
+                                       _ptr(self.out_count), self.max_out, st), "spec_update")
+
+    def _state(self):
+        return [self.y, self.root_token, self.draft_len, self.verifier.len_dev, self.verifier.result,
+                self.out_count, self.out_tokens]
+
+    def capture(self):
+        """Record one step into a HIP graph (after an eager run on a side stream); the loop
+        state is restored afterwards, cache rows written meanwhile lie beyond the lengths."""
+        saved = [t.clone() for t in self._state()]
+        side = torch.cuda.Stream()
+        side.wait_stream(torch.cuda.current_stream())
+        with torch.cuda.stream(side):
+            self.enqueue_step()
+        torch.cuda.current_stream().wait_stream(side)
+        torch.cuda.synchronize()
+        for t, s in zip(self._state(), saved):
+            t.copy_(s)
+        self.graph = torch.cuda.CUDAGraph()
+        with torch.cuda.graph(self.graph):
+            self.enqueue_step()
+        for t, s in zip(self._state(), saved):
+            t.copy_(s)
+        torch.cuda.synchronize()
+        return self
+
+    def step(self):
+        if self.graph is not None:
+            self.graph.replay()
+        else:
+            self.enqueue_step()
+
+    def generate(self, n_steps):
+        """Run n_steps speculative steps; returns the emitted tokens (without the first one).
+        The caches must have room for n_steps * (depth + 2) + 8 * depth + 40 more rows."""
+        for _ in range(n_steps):
+            self.step()
+        n = int(self.out_count.item())
+        return self.out_tokens[:min(n, self.max_out)].tolist()

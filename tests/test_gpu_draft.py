@@ -262,3 +262,38 @@ def test_generate_step_matches_oracle_loop(dev):
     assert res["first"] == want["first"]
     assert res["tokens"] == want["tokens"]
     assert [s[0] for s in res["steps"]] == [s[0] for s in want["steps"]]
+
+
+@pytest.mark.parametrize("same", [True, False])
+@pytest.mark.parametrize("graph", [False, True])
+def test_device_loop_equals_host_loop(dev, same, graph):
+    """SpeculativeDecoder (state on the device, optionally one HIP graph per step) emits the
+    stream of the host-driven generate_step, which is the target's greedy stream."""
+    from mlx_eagle_spec_decoding_tree_amd import spec
+
+    print(f"device loop same={same} graph={graph}", flush=True)
+    (targs, tw, target), (dargs, dw, draft) = tiny_pair(dev, same=same, seed=5)
+    rng = np.random.default_rng(8)
+    prompt = rng.integers(0, targs.vocab_size, 40).astype(np.int32)
+    N = 6
+    host = eagle.generate_step(to_dev(prompt.astype(np.int64), dev), target, draft, k=8, depth=3,
+                               verify_num_tokens=31, max_tokens=10 ** 6, N=N)
+    # fresh models: the fused passes re-point the layers' tensors
+    (_, _, target2), (_, _, draft2) = tiny_pair(dev, same=same, seed=5)
+    dec = spec.SpeculativeDecoder(target2, draft2, capacity=256, k=8, depth=3, verify_num_tokens=31)
+    first = dec.prefill(to_dev(prompt.astype(np.int64), dev))
+    if graph:
+        dec.capture()
+    tokens = dec.generate(N)
+    assert first == host["first"]
+    want = greedy_reference(target, prompt, len(tokens) + 1, dev)
+    assert [first] + tokens == want
+    assert tokens == host["tokens"]
+    assert int(dec.verifier.len_dev.item()) == len(prompt) + len(tokens)
+    if same:
+        assert len(tokens) >= 3 * N
+    # a second run continues the stream
+    more = dec.generate(2)
+    assert more[:len(tokens)] == tokens and len(more) > len(tokens)
+    want = greedy_reference(target, prompt, len(more) + 1, dev)
+    assert [first] + more == want
