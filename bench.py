@@ -10,6 +10,13 @@ input resident in HBM.  Prints ONE JSON line.
   python bench.py [--gpus 1] [--steps K] [--warmup W] [--no-cpu] [--sweep]
 
 --sweep additionally prints (to stderr) the per-shape QMM table for M in {1,8,16,24,32}.
+
+  python bench.py --loop [--steps 300]
+
+measures the end-to-end greedy tree loop instead (a second workload with a line of its own):
+random-init Qwen2.5-0.5B-shaped drafter, Llama-3-8B-shaped target, 512-token random prompt,
+depth 3, 31 draft nodes; every step (draft pass, expansion, tree layout, verification,
+acceptance, KV compaction) is one HIP-graph replay with the loop state on the device.
 """
 import argparse
 import json
@@ -83,10 +90,17 @@ def main():
     ap.add_argument("--calibrate-copy", action="store_true",
                     help="before anything else run one 1 GiB device copy (a kernel of known traffic: "
                          "1 GiB read + 1 GiB written) so that profiler byte counters can be scaled")
+    ap.add_argument("--loop", action="store_true",
+                    help="measure the end-to-end tree loop (drafter + target) instead of the verify step")
+    ap.add_argument("--self-draft", action="store_true",
+                    help="with --loop: the target drafts for itself (high acceptance; exercises the "
+                         "accept path at full size)")
     opt = ap.parse_args()
     if opt.gpus != 1:
         print("bench.py: this build runs on one GPU only; run with --gpus 1", file=sys.stderr)
         sys.exit(2)
+    if opt.loop:
+        return loop_bench(opt)
 
     import torch
     from mlx_eagle_spec_decoding_tree_amd import _lib, eagle, llama, ops, synth
@@ -234,6 +248,70 @@ def main():
             "roofline": roofline, "cpu_baseline": cpu}
     if parity is not None:
         line["parity"] = parity
+    print(json.dumps(line), flush=True)
+
+
+def loop_bench(opt):
+    """End-to-end greedy tree loop (mlx_eagle.py:503-606) on synthetic models."""
+    import torch
+    from mlx_eagle_spec_decoding_tree_amd import _lib, llama, spec, synth
+
+    if not torch.cuda.is_available():
+        print("bench.py: no GPU visible", file=sys.stderr)
+        sys.exit(2)
+    dev = torch.device("cuda:0")
+    _lib.check(_lib.lib().eagle_check_device(), "device check")
+    steps = opt.steps if opt.steps != 50 else 300
+    k, depth, nodes, prompt_len = 8, 3, 31, 512
+    targs = synth.llama3_8b()
+    t0 = time.time()
+    target = llama.Model.from_numpy(targs, synth.make_model_weights(targs, seed=opt.seed), dev)
+    if opt.self_draft:
+        dargs = targs
+        draft = llama.Model.from_numpy(targs, synth.make_model_weights(targs, seed=opt.seed), dev)
+    else:
+        dargs = synth.qwen25_05b()
+        draft = llama.Model.from_numpy(dargs, synth.make_model_weights(dargs, seed=opt.seed + 1), dev)
+    print(f"[bench] synthetic models in {time.time() - t0:.1f} s", file=sys.stderr, flush=True)
+    rng = np.random.default_rng(opt.seed + 2)
+    prompt = torch.from_numpy(rng.integers(0, min(targs.vocab_size, dargs.vocab_size), prompt_len)).to(dev)
+    capacity = prompt_len + (opt.warmup + steps) * (depth + 2) + k * depth + 64
+    dec = spec.SpeculativeDecoder(target, draft, capacity=capacity, k=k, depth=depth,
+                                  verify_num_tokens=nodes, max_out=(opt.warmup + steps) * (depth + 2) + 8)
+    torch.cuda.synchronize()
+    t0 = time.time()
+    dec.prefill(prompt)
+    torch.cuda.synchronize()
+    prefill_ms = (time.time() - t0) * 1e3
+    dec.capture()
+    for _ in range(opt.warmup):
+        dec.step()
+    torch.cuda.synchronize()
+    n0 = int(dec.out_count.item())
+    e0, e1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+    t0 = time.time()
+    e0.record()
+    for _ in range(steps):
+        dec.step()
+    e1.record()
+    torch.cuda.synchronize()
+    wall_ms = (time.time() - t0) * 1e3
+    gpu_ms = e0.elapsed_time(e1)
+    n = int(dec.out_count.item()) - n0
+    ms = max(wall_ms, gpu_ms)
+    line = {
+        "metric": "end-to-end tree loop, generated tokens per second (greedy)",
+        "value": round(n / ms * 1e3, 2), "unit": "tokens/s", "n_gpus": 1, "steps": steps,
+        "warmup": opt.warmup, "ms_per_step": round(ms / steps, 4), "higher_is_better": True,
+        "scaling": "weak", "vs_baseline": None, "dtype": "f16", "data": "synthetic",
+        "config": {"workload": ("tree loop: " + ("target drafts for itself" if opt.self_draft else
+                                                 "Qwen2.5-0.5B-shaped 4-bit drafter")
+                                + ", Llama-3-8B-shaped 4-bit target, 512-token prompt, k 8, depth 3, "
+                                  "31 draft nodes"),
+                   "prompt_len": prompt_len, "k": k, "depth": depth, "verify_num_tokens": nodes},
+        "tokens": n, "tokens_per_step": round(n / steps, 4), "prefill_ms": round(prefill_ms, 1),
+        "gpu_ms_total": round(gpu_ms, 2), "wall_ms_total": round(wall_ms, 2),
+    }
     print(json.dumps(line), flush=True)
 
 
