@@ -328,6 +328,12 @@ def fuse_projections(model, swiglu):
     """Lay q/k/v and gate/up of every layer out as one matrix each (rows concatenated) and
     re-point the layers' tensors at row blocks of it, so that one matmul launch serves
     the three (two) projections; memory use is unchanged."""
+    # one fused layout per model, shared by every pass object built on it
+    done = getattr(model, "_fused_projections", None)
+    if done is None:
+        done = model._fused_projections = {}
+    if swiglu in done:
+        return done[swiglu]
     qkv_w, gu_w = [], []
 
     def interleave(lins):
@@ -358,14 +364,19 @@ def fuse_projections(model, swiglu):
             row += n
         return (*fused, bias)
 
+    other = done.get(not swiglu)
     for layer in model.model.layers:
         at, mlp = layer.self_attn, layer.mlp
-        qkv_w.append(fuse([at.q_proj, at.k_proj, at.v_proj]))
+        if other is None:
+            qkv_w.append(fuse([at.q_proj, at.k_proj, at.v_proj]))
         if swiglu:
             # a tile-interleaved copy: the layers keep their own tensors for the module path
             gu_w.append(interleave([mlp.gate_proj, mlp.up_proj]))
         else:
             gu_w.append(fuse([mlp.gate_proj, mlp.up_proj]))
+    if other is not None:
+        qkv_w = other[0]
+    done[swiglu] = (qkv_w, gu_w)
     return qkv_w, gu_w
 
 

@@ -53,7 +53,8 @@ class DecoderPass:
         ops.workspace("attn", L.eagle_tree_attention_workspace_bytes(H, hd, self.max_len), dev)
         ops.workspace("topk", L.eagle_logsoftmax_topk_workspace_bytes(T, args.vocab_size), dev)
 
-    def forward(self, tokens, positions, write_len, attn_len, mask_words, Tk):
+    def forward(self, tokens, positions, write_len, attn_len, mask_words, Tk, head=True):
+        """head=False: stop after the last layer (a pass that is only run for its KV rows)."""
         m, args = self.model, self.args
         H, G, hd = args.num_attention_heads, args.num_key_value_heads, args.head_dim
         W = (H + 2 * G) * hd
@@ -86,9 +87,79 @@ class DecoderPass:
                                  mlp.down_proj.biases, bias=mlp.down_proj.bias, out=self.down)
             nxt = layers[i + 1].input_layernorm.weight if i + 1 < len(layers) else m.model.norm.weight
             ops.rms_norm(self.down, nxt, args.rms_norm_eps, residual=self.h, out=self.hn, h_out=self.h)
+        if not head:
+            return None
         head = m.model.embed_tokens if args.tie_word_embeddings else m.lm_head
         ops.quantized_matmul(self.hn, head.weight, head.scales, head.biases, out=self.logits)
         return self.logits
+
+
+class CausalPrefill:
+    """The prompt pass (mlx_eagle.py:522-533) as consecutive causal passes of 32 rows, each one
+    HIP-graph replay; a last piece shorter than 32 is padded (its extra rows land beyond the
+    cache length and no real row sees them)."""
+
+    ROWS = 32
+
+    def __init__(self, model, cache, max_len=None, head=True):
+        self.cache, self.head = cache, head
+        dev = model.device
+        R = self.ROWS
+        self.run = DecoderPass(model, cache, R, max_len=max_len)
+        self.tokens = torch.zeros(R, dtype=torch.int32, device=dev)
+        self.positions = torch.zeros(R, dtype=torch.int32, device=dev)
+        self.arange = torch.arange(R, dtype=torch.int32, device=dev)
+        self.words = ops.mask_to_words(torch.tril(torch.ones((R, R), dtype=torch.bool, device=dev)))
+        self.len_dev = cache[0].len_dev
+        self.graph = None
+
+    def _enqueue(self):
+        L = _lib.lib()
+        st = _stream()
+        _lib.check(L.eagle_tree_positions(_ptr(self.arange), _ptr(self.len_dev), _ptr(self.positions),
+                                          self.ROWS, st), "positions")
+        self.run.forward(self.tokens, self.positions, self.len_dev, self.len_dev, self.words, self.ROWS,
+                         head=self.head)
+        _lib.check(L.eagle_advance_len(_ptr(self.len_dev), self.ROWS, st), "advance_len")
+
+    def capture(self):
+        saved = self.len_dev.clone()
+        side = torch.cuda.Stream()
+        side.wait_stream(torch.cuda.current_stream())
+        with torch.cuda.stream(side):
+            self._enqueue()
+        torch.cuda.current_stream().wait_stream(side)
+        torch.cuda.synchronize()
+        self.len_dev.copy_(saved)
+        self.graph = torch.cuda.CUDAGraph()
+        with torch.cuda.graph(self.graph):
+            self._enqueue()
+        self.len_dev.copy_(saved)
+        torch.cuda.synchronize()
+        return self
+
+    def __call__(self, ids):
+        """Append the tokens `ids` (1-D) to the cache; returns the logits row of the last one
+        ([1,V] view of a static buffer) when the pass has a head."""
+        ids = ids.reshape(-1).to(torch.int32)
+        n = ids.numel()
+        R = self.ROWS
+        start = self.cache[0].offset
+        if start + (n + R - 1) // R * R > self.cache[0].capacity:
+            raise ValueError("KV cache too small for the padded prompt pass")
+        self.cache[0].sync_len()
+        for s in range(0, n, R):
+            part = ids[s:s + R]
+            self.tokens.zero_()
+            self.tokens[:part.numel()] = part
+            if self.graph is not None:
+                self.graph.replay()
+            else:
+                self._enqueue()
+        for c in self.cache:
+            c.offset = start + n
+        self.cache[0].sync_len()
+        return self.run.logits[(n - 1) % R:(n - 1) % R + 1] if self.head else None
 
 
 class SpeculativeDecoder:
@@ -140,14 +211,21 @@ class SpeculativeDecoder:
         self.max_out = max_out
         self.graph = None
         self.first = None
+        self._prefill = None
+
+    def prepare(self):
+        """Build and capture the prompt passes (done by the first prefill otherwise)."""
+        if self._prefill is None:
+            self._prefill = (CausalPrefill(self.draft_model, self.draft_cache, self.capacity, head=False).capture(),
+                             CausalPrefill(self.base_model, self.base_cache, self.capacity).capture())
+        return self
 
     def prefill(self, prompt):
         """mlx_eagle.py:522-535: both models read the prompt; the first token is the target's
         argmax at its last position."""
-        ids = prompt.reshape(1, -1).to(torch.int64)
-        self.draft_model(ids, cache=self.draft_cache)
-        logits = self.base_model(ids, cache=self.base_cache)
-        first = ops.argmax_rows(logits[0, -1:].contiguous())
+        self.prepare()
+        self._prefill[0](prompt)
+        first = ops.argmax_rows(self._prefill[1](prompt))
         self.y.zero_()
         self.y[:1] = first
         self.root_token.copy_(first)
