@@ -784,6 +784,9 @@ void choose(int M, int N, int K, Launch* out) {
   // About one tile per compute unit: four slabs of a few waves, each walking several tiles,
   // beat fewer slabs of many waves that touch one or two tiles
   if (tiles < 3 * NUM_CU / 2 && units >= (M <= 16 ? 8 : 16)) fill = 4;
+  // K of at most 1024: a slab would be one or two waves; the round trip of the partials costs
+  // more than the idle compute units (4.8 us against 6.7 us for 1152 x 896 at 8 rows)
+  if (units <= (M <= 16 ? 4 : 8)) fill = 1;
   if (splits < fill) splits = fill;
   // With only a few tiles per workgroup a second phase is mostly start-up latency (new x, a
   // drained ring); two K slabs on twice the workgroups finish sooner.  (With more tiles the
