@@ -89,8 +89,8 @@ __global__ __launch_bounds__(512) void tree_attn_split_kernel(
   const int head = g * rep + wave;
 
   int P = *len_dev;
-  if (ROPE) {                           // never index past the cache, whatever the counter says
-    if (P > cap - T) P = (int)(cap - T);
+  if (ROPE || WIDE) {                   // never index past the cache, whatever the counter says
+    if (P > cap - Tk) P = (int)(cap - Tk);
     if (P < 0) P = 0;
   }
   const int Ltot = P + Tk;                // Tk = T unless WIDE
@@ -353,7 +353,7 @@ __global__ void tree_attn_merge_kernel(const half_t* __restrict__ part_o,
 
   int P = *len_dev;
   if (clamp_len) {
-    if (P > cap - T) P = (int)(cap - T);
+    if (P > cap - Tk) P = (int)(cap - Tk);
     if (P < 0) P = 0;
   }
   const int nact = active_splits((P + Tk + KT - 1) / KT, nsplit);   // as in the split kernel
@@ -422,7 +422,7 @@ int launch_attention(const half_t* q, half_t* kc, half_t* vc, const uint32_t* bi
                      kc, vc, bits, len, part_o, part_ml, T, H, G, cap, 0, sl2, k_lin, v_lin, ld, cs, Tk);
   hipLaunchKernelGGL(tree_attn_merge_kernel<HD>, dim3(H, (T + MERGE_TOK - 1) / MERGE_TOK),
                      dim3(MERGE_TOK * HD / 4), 0, st, part_o, part_ml, (half_t*)out, T, H, nsplit,
-                     len, cap, ROPE ? 1 : 0, Tk);
+                     len, cap, (ROPE || WIDE) ? 1 : 0, Tk);
   return eagle_launch_status();
 }
 

@@ -234,6 +234,7 @@ class SpeculativeDecoder:
         self.base_cache[0].sync_len()
         self.draft_cache[0].sync_len()
         self.first = int(first.item())
+        self._bound = self.base_cache[0].offset
         return self.first
 
     def enqueue_step(self):
@@ -301,6 +302,13 @@ class SpeculativeDecoder:
     def generate(self, n_steps):
         """Run n_steps speculative steps; returns the emitted tokens (without the first one).
         The caches must have room for n_steps * (depth + 2) + 8 * depth + 40 more rows."""
+        # upper bound of the rows either cache can hold after these steps (the lengths live on
+        # the device; a step adds at most depth + 2 tokens and writes up to 8 * depth + 32 rows
+        # beyond the length)
+        self._bound += n_steps * (self.depth + 2)
+        if self._bound + max(Y_LEN * (self.depth + 1), MAXT) > self.capacity:
+            self._bound -= n_steps * (self.depth + 2)
+            raise ValueError(f"KV caches of {self.capacity} rows are too small for {n_steps} more steps")
         for _ in range(n_steps):
             self.step()
         n = int(self.out_count.item())

@@ -297,3 +297,19 @@ def test_device_loop_equals_host_loop(dev, same, graph):
     assert more[:len(tokens)] == tokens and len(more) > len(tokens)
     want = greedy_reference(target, prompt, len(more) + 1, dev)
     assert [first] + more == want
+
+
+def test_device_loop_refuses_to_overrun_the_caches(dev):
+    from mlx_eagle_spec_decoding_tree_amd import spec
+
+    (targs, tw, target), (dargs, dw, draft) = tiny_pair(dev, same=False, seed=5)
+    prompt = np.random.default_rng(1).integers(0, targs.vocab_size, 40).astype(np.int64)
+    dec = spec.SpeculativeDecoder(target, draft, capacity=128, k=8, depth=3, verify_num_tokens=31)
+    dec.prefill(to_dev(prompt, dev))
+    dec.generate(5)                       # 40 + 5 * 5 + 32 <= 128
+    with pytest.raises(ValueError, match="too small"):
+        dec.generate(10)
+    with pytest.raises(ValueError):
+        spec.SpeculativeDecoder(target, draft, capacity=128, k=8, depth=9)
+    with pytest.raises(ValueError):
+        spec.SpeculativeDecoder(target, draft, capacity=128, k=8, depth=3, verify_num_tokens=32)
