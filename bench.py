@@ -254,7 +254,7 @@ def main():
 def loop_bench(opt):
     """End-to-end greedy tree loop (mlx_eagle.py:503-606) on synthetic models."""
     import torch
-    from mlx_eagle_spec_decoding_tree_amd import _lib, llama, spec, synth
+    from mlx_eagle_spec_decoding_tree_amd import _lib, llama, ops, spec, synth
 
     if not torch.cuda.is_available():
         print("bench.py: no GPU visible", file=sys.stderr)
@@ -300,6 +300,20 @@ def loop_bench(opt):
     gpu_ms = e0.elapsed_time(e1)
     n = int(dec.out_count.item()) - n0
     ms = max(wall_ms, gpu_ms)
+    # full-size parity: whatever was drafted, the emitted stream is the target's own greedy
+    # stream; checked on its first tokens with plain one-token passes of the target
+    n_check = min(24, int(dec.out_count.item()))
+    emitted = [dec.first] + dec.out_tokens[:n_check].tolist()
+    from mlx_eagle_spec_decoding_tree_amd.cache import make_prompt_cache
+    ref_cache = make_prompt_cache(target, capacity=prompt_len + n_check + 40)
+    logits = target(prompt[None], cache=ref_cache)
+    greedy = [int(ops.argmax_rows(logits[0, -1:].contiguous()).item())]
+    for _ in range(n_check):
+        logits = target(torch.tensor([[greedy[-1]]], dtype=torch.int64, device=dev), cache=ref_cache)
+        greedy.append(int(ops.argmax_rows(logits[0, -1:].contiguous()).item()))
+    agree = 0
+    while agree < len(greedy) and greedy[agree] == emitted[agree]:
+        agree += 1
     line = {
         "metric": "end-to-end tree loop, generated tokens per second (greedy)",
         "value": round(n / ms * 1e3, 2), "unit": "tokens/s", "n_gpus": 1, "steps": steps,
@@ -312,6 +326,8 @@ def loop_bench(opt):
                    "prompt_len": prompt_len, "k": k, "depth": depth, "verify_num_tokens": nodes},
         "tokens": n, "tokens_per_step": round(n / steps, 4), "prefill_ms": round(prefill_ms, 1),
         "gpu_ms_total": round(gpu_ms, 2), "wall_ms_total": round(wall_ms, 2),
+        "parity": {"checked_tokens": len(greedy), "equal_to_target_greedy_stream": agree,
+                   "stream_equal": agree == len(greedy)},
     }
     print(json.dumps(line), flush=True)
 
