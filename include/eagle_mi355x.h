@@ -89,6 +89,15 @@ int eagle_qmm_swiglu_w4g64_f16(const void* x, const uint32_t* wq, const void* sc
                                int M, int N, int K, int group_size, int bits,
                                void* workspace, size_t workspace_bytes, eagle_stream_t stream);
 
+/* The same product for any number of rows M, as a tiled MFMA GEMM (128 x 128 output blocks,
+ * weights expanded to fp16 in registers): the form for the prompt pass (mlx_eagle.py:522-533,
+ * where mlx_model_fwd_bench.py:65-73 falls back to mx.quantized_matmul because the row count is
+ * not 8..32).  Bound by the matrix cores, not by the weight stream, from a few hundred rows on.
+ * No workspace.  N % 8 == 0, K % 64 == 0; bias (may be NULL) 8-byte aligned. */
+int eagle_qmm_gemm_w4g64_f16(const void* x, const uint32_t* wq, const void* scales,
+                             const void* biases, const void* bias, void* out, int M, int N, int K,
+                             int group_size, int bits, eagle_stream_t stream);
+
 /* Quantised embedding gather: out[t,:] = fp16(scales*q + biases) of row ids[t].
  * ids [T] int32, out [T,D] fp16, D % 64 == 0.  Replaces the quantised
  * nn.Embedding lookup of mlx_llama.py:273. */

@@ -58,7 +58,8 @@ def as_packed_u32(w_q):
 def quantized_matmul(x, w_q, scales, biases, transpose=True, group_size=64, bits=4, bias=None,
                      out=None, tuned=None):
     """`mx.quantized_matmul(x, w, scales, biases, transpose=True, group_size=64, bits=4)`
-    for 1..32 rows of x (any leading dims, flattened as qmm_kernel.py:99-100,136).
+    (any leading dims, flattened as qmm_kernel.py:99-100,136): the streaming kernel for 1..32
+    rows of x, a tiled GEMM above that.
     `bias` ([N] fp16) is added after rounding, as the patched linear layer does
     (mlx_model_fwd_bench.py:70-71)."""
     if not transpose:
@@ -80,6 +81,14 @@ def quantized_matmul(x, w_q, scales, biases, transpose=True, group_size=64, bits
     if out is None:
         out = torch.empty((*lead, N), dtype=torch.float16, device=x.device)
     L = _lib.lib()
+    if M > 32:
+        # many rows (the prompt pass): the tiled GEMM form
+        if tuned is not None:
+            raise ValueError("launch shapes can be forced for at most 32 rows")
+        rc = L.eagle_qmm_gemm_w4g64_f16(_ptr(x), _ptr(w_q), _ptr(scales), _ptr(biases), _ptr(bias),
+                                        _ptr(out), M, N, K, group_size, bits, _stream())
+        _lib.check(rc, "quantized_matmul")
+        return out
     if tuned is None:
         ws = workspace("qmm", L.eagle_qmm_workspace_bytes(M, N, K), x.device)
         rc = L.eagle_qmm_w4g64_f16(_ptr(x), _ptr(w_q), _ptr(scales), _ptr(biases), _ptr(bias),

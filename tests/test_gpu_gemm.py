@@ -1,0 +1,53 @@
+"""Many-row form of the 4-bit group-64 matmul (the prompt pass) against the oracle."""
+import numpy as np
+import pytest
+import torch
+
+from mlx_eagle_spec_decoding_tree_amd import ops, synth
+from oracle import oracle
+from util import TOL, layer_to_dev, rel_err, to_dev
+
+pytestmark = pytest.mark.gpu
+
+
+@pytest.mark.parametrize("M,N,K,bias", [(512, 1152, 896, True), (512, 896, 4864, False), (33, 64, 64, True),
+                                        (128, 128, 128, False), (129, 200, 192, True), (300, 4096, 1024, False),
+                                        (512, 3584, 3584, True), (64, 1000, 640, False)])
+def test_gemm_form_matches_oracle(dev, M, N, K, bias):
+    print(f"gemm M={M} N={N} K={K}", flush=True)
+    rng = np.random.default_rng(M + N + K)
+    layer = synth.make_qlinear(rng, N, K, bias=bias)
+    x = synth.make_x(rng, M, K)
+    want = oracle.qmm(x, layer["weight"], layer["scales"], layer["biases"], layer.get("bias"))
+    d = layer_to_dev(layer, dev)
+    got = ops.quantized_matmul(to_dev(x, dev), d["weight"], d["scales"], d["biases"], bias=d.get("bias"))
+    got = got.cpu().numpy()
+    assert got.shape == (M, N) and np.isfinite(got.astype(np.float32)).all()
+    assert rel_err(got, want) <= TOL
+    # rows are independent: the first 32 rows agree with the streaming kernel to rounding of the weights
+    small = ops.quantized_matmul(to_dev(x[:32], dev), d["weight"], d["scales"], d["biases"],
+                                 bias=d.get("bias")).cpu().numpy()
+    assert rel_err(got[:32], small) <= TOL
+
+
+def test_gemm_form_integer_exact(dev):
+    """Integer-valued x, scales 1 and integer biases: every product and sum is exact in fp16/fp32."""
+    rng = np.random.default_rng(5)
+    M, N, K = 96, 192, 128
+    w = rng.integers(0, 1 << 32, size=(N, K // 8), dtype=np.uint32)
+    s = np.ones((N, K // 64), np.float16)
+    b = rng.integers(-8, 1, (N, K // 64)).astype(np.float16)
+    x = rng.integers(-2, 3, (M, K)).astype(np.float16)
+    q = synth.unpack_nibbles(w).astype(np.int64)
+    wd = q + np.repeat(b.astype(np.int64), 64, axis=1)
+    want = x.astype(np.int64) @ wd.T
+    got = ops.quantized_matmul(to_dev(x, dev), to_dev(w, dev), to_dev(s, dev), to_dev(b, dev)).cpu().numpy()
+    assert np.array_equal(got.astype(np.int64), want)
+
+
+def test_gemm_form_rejects_bad_shapes(dev):
+    x = torch.zeros((64, 96), dtype=torch.float16, device=dev)
+    w = torch.zeros((64, 12), dtype=torch.int32, device=dev)
+    s = torch.zeros((64, 1), dtype=torch.float16, device=dev)
+    with pytest.raises(ValueError):
+        ops.quantized_matmul(x, w, s, s)
