@@ -278,7 +278,7 @@ def loop_bench(opt):
     capacity = prompt_len + (opt.warmup + steps) * (depth + 2) + k * depth + 64
     dec = spec.SpeculativeDecoder(target, draft, capacity=capacity, k=k, depth=depth,
                                   verify_num_tokens=nodes, max_out=(opt.warmup + steps) * (depth + 2) + 8)
-    dec.prepare()
+    dec.prepare(prompt_len)
     torch.cuda.synchronize()
     t0 = time.time()
     dec.prefill(prompt)

@@ -94,48 +94,149 @@ class DecoderPass:
         return self.logits
 
 
-class CausalPrefill:
-    """The prompt pass (mlx_eagle.py:522-533) as consecutive causal passes of 32 rows, each one
-    HIP-graph replay; a last piece shorter than 32 is padded (its extra rows land beyond the
-    cache length and no real row sees them)."""
+class ChunkPass:
+    """A causal pass of R rows (a multiple of 32, at most 1024) through a decoder: the linear
+    layers see all R rows at once (the tiled GEMM form of the matmul above 32 rows), rope /
+    cache append / attention run per piece of 32 rows, every piece seeing the cache rows before
+    it and its own rows causally.  Rows are appended at the cache length, which advances by R."""
 
-    ROWS = 32
+    PIECE = 32
 
-    def __init__(self, model, cache, max_len=None, head=True):
-        self.cache, self.head = cache, head
+    def __init__(self, model, cache, R, max_len=None, head=True):
+        args = model.args
+        self.model, self.cache, self.args, self.R, self.head = model, cache, args, R, head
         dev = model.device
-        R = self.ROWS
-        self.run = DecoderPass(model, cache, R, max_len=max_len)
-        self.tokens = torch.zeros(R, dtype=torch.int32, device=dev)
-        self.positions = torch.zeros(R, dtype=torch.int32, device=dev)
-        self.arange = torch.arange(R, dtype=torch.int32, device=dev)
-        self.words = ops.mask_to_words(torch.tril(torch.ones((R, R), dtype=torch.bool, device=dev)))
+        P = self.PIECE
+        if R % P or R < P or R > 32 * P:
+            raise ValueError("rows must be a multiple of 32 between 32 and 1024")
+        self.pieces = R // P
+        D, I = args.hidden_size, args.intermediate_size
+        H, G, hd = args.num_attention_heads, args.num_key_value_heads, args.head_dim
+        self.max_len = max_len or cache[0].capacity
+        self.qkv_w, self.gu_w = fuse_projections(model, False)
+        f16 = dict(dtype=torch.float16, device=dev)
+        i32 = dict(dtype=torch.int32, device=dev)
+        self.tokens = torch.zeros(R, **i32)
+        self.h = torch.empty((R, D), **f16)
+        self.hn = torch.empty((R, D), **f16)
+        self.qkv = torch.empty((R, (H + 2 * G) * hd), **f16)
+        self.q_rot = torch.empty((H, P, hd), **f16)
+        self.rope_cs = torch.empty((R, hd // 2, 2), dtype=torch.float32, device=dev)
+        self.attn = torch.empty((R, H * hd), **f16)
+        self.o = torch.empty((R, D), **f16)
+        self.gate_up = torch.empty((R, 2 * I), **f16)
+        self.act = torch.empty((R, I), **f16)
+        self.down = torch.empty((R, D), **f16)
+        self.logits = torch.empty((P, args.vocab_size), **f16)      # of the last piece only
+        self.piece_off = (torch.arange(self.pieces, **i32) * P).contiguous()
+        self.piece_len = torch.zeros(self.pieces, **i32)
+        self.arange = torch.arange(P, **i32)
+        self.positions = torch.zeros(R, **i32)
+        self.words = ops.mask_to_words(torch.tril(torch.ones((P, P), dtype=torch.bool, device=dev)))
         self.len_dev = cache[0].len_dev
+        L = _lib.lib()
+        hw = model.lm_head if not args.tie_word_embeddings else model.model.embed_tokens
+        ops.workspace("qmm", L.eagle_qmm_workspace_bytes(P, hw.weight.shape[0], D), dev)
+        ops.workspace("attn", L.eagle_tree_attention_workspace_bytes(H, hd, self.max_len), dev)
         self.graph = None
 
-    def _enqueue(self):
+    def enqueue(self):
         L = _lib.lib()
         st = _stream()
-        _lib.check(L.eagle_tree_positions(_ptr(self.arange), _ptr(self.len_dev), _ptr(self.positions),
-                                          self.ROWS, st), "positions")
-        self.run.forward(self.tokens, self.positions, self.len_dev, self.len_dev, self.words, self.ROWS,
-                         head=self.head)
-        _lib.check(L.eagle_advance_len(_ptr(self.len_dev), self.ROWS, st), "advance_len")
+        m, args, P = self.model, self.args, self.PIECE
+        H, G, hd = args.num_attention_heads, args.num_key_value_heads, args.head_dim
+        W = (H + 2 * G) * hd
+        layers = m.model.layers
+        at0 = layers[0].self_attn
+        # cache length, positions and rotary table of every piece, once for all layers
+        _lib.check(L.eagle_tree_positions(_ptr(self.piece_off), _ptr(self.len_dev), _ptr(self.piece_len),
+                                          self.pieces, st), "piece lengths")
+        for j in range(self.pieces):
+            pos = self.positions[j * P:(j + 1) * P]
+            _lib.check(L.eagle_tree_positions(_ptr(self.arange), _ptr(self.piece_len[j:j + 1]), _ptr(pos),
+                                              P, st), "positions")
+            ops.rope_table(pos, at0._inv_freqs, at0._scaling_factor, out=self.rope_cs[j * P:(j + 1) * P])
+        emb = m.model.embed_tokens
+        ops.embed(self.tokens, emb.weight, emb.scales, emb.biases, out=self.h)
+        ops.rms_norm(self.h, layers[0].input_layernorm.weight, args.rms_norm_eps, out=self.hn)
+        for i, layer in enumerate(layers):
+            at, mlp, c = layer.self_attn, layer.mlp, self.cache[i]
+            w, sc, bi, b = self.qkv_w[i]
+            ops.quantized_matmul(self.hn, w, sc, bi, bias=b, out=self.qkv)
+            for j in range(self.pieces):
+                rows = slice(j * P, (j + 1) * P)
+                qkv = self.qkv[rows]
+                plen = self.piece_len[j:j + 1]
+                ops.rope_kv_append(qkv, qkv[:, H * hd:], qkv[:, (H + G) * hd:], None, at._inv_freqs,
+                                   at._scaling_factor, self.q_rot, c.keys[0], c.values[0], plen, H, G, hd,
+                                   row_stride=W, rope_cs=self.rope_cs[rows])
+                ops.draft_attention(self.q_rot, c.keys[0], c.values[0], self.words, plen, P, at.scale,
+                                    max_len=self.max_len, out=self.attn[rows])
+            ops.quantized_matmul(self.attn, at.o_proj.weight, at.o_proj.scales, at.o_proj.biases,
+                                 bias=at.o_proj.bias, out=self.o)
+            ops.rms_norm(self.o, layer.post_attention_layernorm.weight, args.rms_norm_eps,
+                         residual=self.h, out=self.hn, h_out=self.h)
+            w, sc, bi, b = self.gu_w[i]
+            ops.quantized_matmul(self.hn, w, sc, bi, bias=b, out=self.gate_up)
+            ops.silu_mul(self.gate_up, None, out=self.act)
+            ops.quantized_matmul(self.act, mlp.down_proj.weight, mlp.down_proj.scales,
+                                 mlp.down_proj.biases, bias=mlp.down_proj.bias, out=self.down)
+            nxt = layers[i + 1].input_layernorm.weight if i + 1 < len(layers) else m.model.norm.weight
+            ops.rms_norm(self.down, nxt, args.rms_norm_eps, residual=self.h, out=self.hn, h_out=self.h)
+        if self.head:
+            hw = m.model.embed_tokens if args.tie_word_embeddings else m.lm_head
+            ops.quantized_matmul(self.hn[self.R - P:], hw.weight, hw.scales, hw.biases, out=self.logits)
+        _lib.check(L.eagle_advance_len(_ptr(self.len_dev), self.R, st), "advance_len")
 
     def capture(self):
         saved = self.len_dev.clone()
         side = torch.cuda.Stream()
         side.wait_stream(torch.cuda.current_stream())
         with torch.cuda.stream(side):
-            self._enqueue()
+            self.enqueue()
         torch.cuda.current_stream().wait_stream(side)
         torch.cuda.synchronize()
         self.len_dev.copy_(saved)
         self.graph = torch.cuda.CUDAGraph()
         with torch.cuda.graph(self.graph):
-            self._enqueue()
+            self.enqueue()
         self.len_dev.copy_(saved)
         torch.cuda.synchronize()
+        return self
+
+    def run(self):
+        if self.graph is not None:
+            self.graph.replay()
+        else:
+            self.enqueue()
+
+
+class CausalPrefill:
+    """The prompt pass (mlx_eagle.py:522-533) as causal passes of up to `chunk` rows (512, the
+    reference's prefill_step_size), each one HIP-graph replay; a last piece that is not a
+    multiple of 32 is padded (its extra rows land beyond the cache length and no real row sees
+    them).  One captured pass per distinct row count."""
+
+    def __init__(self, model, cache, max_len=None, head=True, chunk=512, graphs=True):
+        self.model, self.cache, self.head, self.max_len = model, cache, head, max_len
+        self.chunk, self.graphs = chunk, graphs
+        self.passes = {}
+
+    def _pass(self, R):
+        p = self.passes.get(R)
+        if p is None:
+            p = ChunkPass(self.model, self.cache, R, max_len=self.max_len, head=self.head)
+            if self.graphs:
+                p.capture()
+            self.passes[R] = p
+        return p
+
+    def prepare(self, n):
+        """Build (and capture) the passes a prompt of n tokens needs."""
+        while n > 0:
+            R = min(self.chunk, (n + 31) // 32 * 32)
+            self._pass(R)
+            n -= R
         return self
 
     def __call__(self, ids):
@@ -143,23 +244,29 @@ class CausalPrefill:
         ([1,V] view of a static buffer) when the pass has a head."""
         ids = ids.reshape(-1).to(torch.int32)
         n = ids.numel()
-        R = self.ROWS
         start = self.cache[0].offset
-        if start + (n + R - 1) // R * R > self.cache[0].capacity:
+        if start + (n + 31) // 32 * 32 > self.cache[0].capacity:
             raise ValueError("KV cache too small for the padded prompt pass")
         self.cache[0].sync_len()
-        for s in range(0, n, R):
+        s, last = 0, None
+        while s < n:
+            R = min(self.chunk, (n - s + 31) // 32 * 32)
+            p = self._pass(R)
             part = ids[s:s + R]
-            self.tokens.zero_()
-            self.tokens[:part.numel()] = part
-            if self.graph is not None:
-                self.graph.replay()
-            else:
-                self._enqueue()
+            p.tokens.zero_()
+            p.tokens[:part.numel()] = part
+            p.run()
+            last, last_rows = p, part.numel()
+            s += R
         for c in self.cache:
             c.offset = start + n
         self.cache[0].sync_len()
-        return self.run.logits[(n - 1) % R:(n - 1) % R + 1] if self.head else None
+        if not self.head:
+            return None
+        row = last_rows - (last.R - ChunkPass.PIECE) - 1     # within the last piece
+        if row < 0:
+            raise RuntimeError("the last token does not lie in the last piece")
+        return last.logits[row:row + 1]
 
 
 class SpeculativeDecoder:
@@ -213,11 +320,15 @@ class SpeculativeDecoder:
         self.first = None
         self._prefill = None
 
-    def prepare(self):
-        """Build and capture the prompt passes (done by the first prefill otherwise)."""
+    def prepare(self, prompt_len=0):
+        """Build and capture the prompt passes for a prompt of this length (done by the first
+        prefill otherwise)."""
         if self._prefill is None:
-            self._prefill = (CausalPrefill(self.draft_model, self.draft_cache, self.capacity, head=False).capture(),
-                             CausalPrefill(self.base_model, self.base_cache, self.capacity).capture())
+            self._prefill = (CausalPrefill(self.draft_model, self.draft_cache, self.capacity, head=False),
+                             CausalPrefill(self.base_model, self.base_cache, self.capacity))
+        if prompt_len:
+            for p in self._prefill:
+                p.prepare(prompt_len)
         return self
 
     def prefill(self, prompt):

@@ -313,3 +313,33 @@ def test_device_loop_refuses_to_overrun_the_caches(dev):
         spec.SpeculativeDecoder(target, draft, capacity=128, k=8, depth=9)
     with pytest.raises(ValueError):
         spec.SpeculativeDecoder(target, draft, capacity=128, k=8, depth=3, verify_num_tokens=32)
+
+
+@pytest.mark.parametrize("n,chunk,graphs", [(75, 512, True), (200, 64, False), (32, 512, True)])
+def test_chunked_prompt_pass_matches_oracle(dev, n, chunk, graphs):
+    """spec.CausalPrefill: linear layers over the whole chunk (tiled GEMM form above 32 rows),
+    attention per 32-row piece; cache rows and the last token's logits against the oracle."""
+    from mlx_eagle_spec_decoding_tree_amd import spec
+
+    (args, w, model), _ = tiny_pair(dev, same=True, seed=3)
+    rng = np.random.default_rng(n)
+    ids = rng.integers(0, args.vocab_size, n).astype(np.int32)
+    inv, sc = synth.inv_freqs(args)
+    side = draft_oracle.Side(args, w, inv, sc, 320)
+    want = side.causal(ids)
+    cache = make_prompt_cache(model, capacity=320)
+    pre = spec.CausalPrefill(model, cache, head=True, chunk=chunk, graphs=graphs)
+    got = pre(to_dev(ids, dev)).cpu().numpy()
+    assert cache[0].offset == n and int(cache[0].len_dev.item()) == n
+    assert got.shape == (1, args.vocab_size)
+    assert rel_err(got, want[-1:]) <= 2 * TOL
+    assert got.argmax() == want[-1].argmax() or np.sort(want[-1])[-1] - np.sort(want[-1])[-2] < 0.05
+    for (ok, ov), c in zip(side.cache, cache):
+        assert rel_err(c.keys[0, :, :n].cpu().numpy(), ok[:, :n]) <= 2 * TOL
+        assert rel_err(c.values[0, :, :n].cpu().numpy(), ov[:, :n]) <= 2 * TOL
+    # a second call continues from the cache
+    more = rng.integers(0, args.vocab_size, 40).astype(np.int32)
+    want2 = side.causal(more)
+    got2 = pre(to_dev(more, dev)).cpu().numpy()
+    assert cache[0].offset == n + 40
+    assert rel_err(got2, want2[-1:]) <= 2 * TOL
