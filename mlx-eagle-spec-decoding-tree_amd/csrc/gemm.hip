@@ -10,9 +10,10 @@
 //     two steps ahead into registers;
 //   * every lane loads the 16 bytes (four packed words = 32 weights) of its weight row that its
 //     half of the MFMA K range needs, two steps ahead, and expands them in registers:
-//     w & 0x000f000f | 0x64006400 is the fp16 pair (1024 + q0, 1024 + q4) (v_and_or_b32); minus
-//     1024 (exact) and one packed fp16 fma with (s, b) gives the weights rounded to fp16, as
-//     the reference kernels hold them.  That yields the eight weights of a word in the order
+//     a shift and v_and_or_b32 make the fp16 pair (16 + q_i, 16 + q_{i+4}); one packed fp16
+//     fma with (s, b - 16 s) gives the weights in fp16, as the reference kernels hold them (the
+//     expansion is what bounds this kernel, so it is four packed instructions per word, not
+//     eight).  That yields the eight weights of a word in the order
 //     q0 q4 q1 q5 q2 q6 q3 q7; x is stored to LDS in the same order within every group of
 //     eight, so both MFMA operands agree on which K index sits where.
 // fp32 accumulation, one fp16 rounding, optional fp16 bias added after the rounding.
@@ -20,7 +21,8 @@
 
 namespace {
 
-constexpr int BM = 128, BN = 128, BK = 64;
+constexpr int BN = 128, BK = 64;
+constexpr long SMALL_BLOCKS = 256;       // compute units    // set from measurements
 constexpr int XS = BK + 8;                  // LDS row stride in halves (144 bytes: conflict-free 16-byte reads)
 
 __device__ inline half8_t permute8(half8_t v) {
@@ -34,141 +36,203 @@ __device__ inline uint32_t and_or(uint32_t v, uint32_t mask, uint32_t bits) {
 }
 
 // eight weights of one packed word, order q0 q4 q1 q5 q2 q6 q3 q7, as fp16(s*q + b).
-// Even nibbles land in the low mantissa bits of 1024.0 (0x6400: one ulp = 1), odd nibbles four
-// bits higher in 64.0 (0x5400: one ulp = 1/16), so only one shift is needed per word.
-__device__ inline half8_t dequant_word(uint32_t w, half2_t s2, half2_t b2) {
-  const half2_t k1024 = half2_t{(half_t)1024.f, (half_t)1024.f};
-  const half2_t k64 = half2_t{(half_t)64.f, (half_t)64.f};
+// Every nibble is moved to the top four mantissa bits of 16.0 (0x4c00), where one step is 1:
+// the fp16 pair is (16 + q_i, 16 + q_{i+4}) and one packed fma with (s, b - 16 s) gives the
+// weights.  (Nibbles left in the low mantissa bits would need an offset of 1024 s, which does
+// not leave b enough bits; with 16 s the rounding of b - 16 s is below 1e-3 of a weight.)
+__device__ inline half8_t dequant_word(uint32_t w, half2_t s2, half2_t b16) {
   union { uint32_t u; half2_t h; } c[4];
-  const uint32_t w8 = w >> 8;
-  c[0].u = and_or(w, 0x000f000fu, 0x64006400u);
-  c[1].u = and_or(w, 0x00f000f0u, 0x54005400u);
-  c[2].u = and_or(w8, 0x000f000fu, 0x64006400u);
-  c[3].u = and_or(w8, 0x00f000f0u, 0x54005400u);
+  c[0].u = and_or(w << 6, 0x03c003c0u, 0x4c004c00u);
+  c[1].u = and_or(w << 2, 0x03c003c0u, 0x4c004c00u);
+  c[2].u = and_or(w >> 2, 0x03c003c0u, 0x4c004c00u);
+  c[3].u = and_or(w >> 6, 0x03c003c0u, 0x4c004c00u);
   half8_t o;
 #pragma unroll
   for (int i = 0; i < 4; ++i) {
-    const half2_t q = c[i].h - ((i & 1) ? k64 : k1024);      // exact
-    const half2_t v = __builtin_elementwise_fma(q, s2, b2);
+    const half2_t v = __builtin_elementwise_fma(c[i].h, s2, b16);
     o[2 * i] = v[0];
     o[2 * i + 1] = v[1];
   }
   return o;
 }
 
+// MT = 32-row x tiles per wave: 2 (128-row blocks) or 4 (256-row blocks: twice the matrix work
+// per expanded weight and per byte read from LDS).
+template <int E>
+struct StepIndex {
+  static constexpr int value = E;
+};
+
+// SB8: K is a multiple of 512, so that scales and biases can be fetched eight groups (16 bytes)
+// at a time, one fetch per eight K steps, instead of one 2-byte load per row and step (the
+// loads of one instruction go to 32 or 64 different cache lines either way, and the rate of
+// such requests, not their bytes, is what the kernel runs up against).
+template <int NTW, int MT, bool SB8>
 __global__ __launch_bounds__(256) void qmm_gemm_w4g64_kernel(
     const half_t* __restrict__ x, const uint32_t* __restrict__ w, const half_t* __restrict__ s,
     const half_t* __restrict__ b, const half_t* __restrict__ bias, half_t* __restrict__ out, int M,
     int N, int K) {
-  __shared__ __attribute__((aligned(16))) half_t xs[2][BM * XS];
+  // NTW = 32-row weight tiles per wave: 2 (waves 2 x 2 over the block) or 1 (four waves side by
+  // side, each over all x rows of the block: no weight row is loaded or expanded twice)
+  constexpr int WN = 128 / (32 * NTW);       // waves along the weight rows
+  constexpr int WM = 4 / WN;                 // waves along the x rows
+  constexpr int BMT = 32 * MT * WM;          // rows of x per workgroup
+  constexpr int TPR = 256 / BMT;             // threads per x row in the block load (2 or 1)
+  constexpr int PP = 8 / TPR;                // 16-byte pieces per thread
+  extern __shared__ __attribute__((aligned(16))) half_t xs_all[];
+  half_t* xs[2] = {xs_all, xs_all + BMT * XS};
   const int tid = threadIdx.x;
   const int wave = tid >> 6, lane = tid & 63;
   const int ql = lane & 31, hb = lane >> 5;
-  const int wn = wave & 1, wm = wave >> 1;
-  const int n0 = blockIdx.x * BN + wn * 64;
-  const int m0 = blockIdx.y * BM;
+  const int wn = wave % WN, wm = wave / WN;
+  const int n0 = blockIdx.x * BN + wn * 32 * NTW;
+  const int m0 = blockIdx.y * BMT;
   const int KW = K >> 3;                    // packed words per weight row
   const int KG = K >> 6;                    // groups per weight row
   const int steps = K / BK;
 
-  // x block loads: thread -> (row, 32-column half), four 16-byte pieces
-  const int xr = tid >> 1, xh = tid & 1;
+  const int xr = tid / TPR, xh = tid % TPR;
   int xrow = m0 + xr;
   if (xrow > M - 1) xrow = M - 1;           // rows past the end are never stored
-  const half_t* xp = x + (long)xrow * K + xh * 32;
-  // weight rows of this lane's two 32-row tiles
-  int nrow[2];
+  const half_t* xp = x + (long)xrow * K + xh * (BK / TPR);
+  int nrow[NTW];
 #pragma unroll
-  for (int nt = 0; nt < 2; ++nt) {
+  for (int nt = 0; nt < NTW; ++nt) {
     nrow[nt] = n0 + nt * 32 + ql;
     if (nrow[nt] > N - 1) nrow[nt] = N - 1;
   }
 
-  // two register sets: the loads of step ks + 2 are issued while step ks is computed, so every
-  // load has two steps to arrive even with a single wave per SIMD
-  half8_t xreg[2][4];
-  uint4_t wreg[2][2];
-  half_t sreg[2][2], breg[2][2];
-  auto fetch = [&](int ks, int p) {
+  half8_t xreg[PP];                         // x of the next step
+  uint4_t wreg[2][NTW];                     // packed weights, two steps in flight
+  half_t sreg[2][NTW], breg[2][NTW];        // !SB8: scale and bias of those steps
+  half8_t s8[2][NTW], b8[2][NTW];           // SB8: of this chunk of eight steps and of the next
+  half8_t af[2][NTW][4];                    // expanded weights of this step and the next
+  auto fetch_x = [&](int ks) {
 #pragma unroll
-    for (int g = 0; g < 4; ++g) xreg[p][g] = *reinterpret_cast<const half8_t*>(xp + (long)ks * BK + g * 8);
+    for (int g = 0; g < PP; ++g) xreg[g] = *reinterpret_cast<const half8_t*>(xp + (long)ks * BK + g * 8);
+  };
+  auto fetch_w = [&](int ks, int p) {
 #pragma unroll
-    for (int nt = 0; nt < 2; ++nt) {
+    for (int nt = 0; nt < NTW; ++nt) {
       wreg[p][nt] = *reinterpret_cast<const uint4_t*>(w + (long)nrow[nt] * KW + ks * 8 + hb * 4);
-      sreg[p][nt] = s[(long)nrow[nt] * KG + ks];
-      breg[p][nt] = b[(long)nrow[nt] * KG + ks];
+      if (!SB8) {
+        sreg[p][nt] = s[(long)nrow[nt] * KG + ks];
+        breg[p][nt] = b[(long)nrow[nt] * KG + ks];
+      }
     }
   };
-  auto stash = [&](int buf, int p) {
+  auto fetch_sb = [&](int chunk, int q) {
 #pragma unroll
-    for (int g = 0; g < 4; ++g)
-      *reinterpret_cast<half8_t*>(&xs[buf][xr * XS + xh * 32 + g * 8]) = permute8(xreg[p][g]);
+    for (int nt = 0; nt < NTW; ++nt) {
+      s8[q][nt] = *reinterpret_cast<const half8_t*>(s + (long)nrow[nt] * KG + chunk * 8);
+      b8[q][nt] = *reinterpret_cast<const half8_t*>(b + (long)nrow[nt] * KG + chunk * 8);
+    }
+  };
+  auto stash = [&](int buf) {
+#pragma unroll
+    for (int g = 0; g < PP; ++g)
+      *reinterpret_cast<half8_t*>(&xs[buf][xr * XS + xh * (BK / TPR) + g * 8]) = permute8(xreg[g]);
+  };
+  // word j of the weight tiles of register set p; e = index of their step within the chunk of
+  // eight (8 = first step of the next chunk)
+  auto expand = [&](int p, int j, int e) {
+#pragma unroll
+    for (int nt = 0; nt < NTW; ++nt) {
+      const half_t sc = SB8 ? s8[e >> 3][nt][e & 7] : sreg[p][nt];
+      const half_t bi = SB8 ? b8[e >> 3][nt][e & 7] : breg[p][nt];
+      const half_t b16 = (half_t)((float)bi - 16.f * (float)sc);
+      af[p][nt][j] = dequant_word(wreg[p][nt][j], half2_t{sc, sc}, half2_t{b16, b16});
+    }
   };
 
-  float16_t acc[2][2];                      // [weight tile][x tile]
+  float16_t acc[NTW][MT];                   // [weight tile][x tile]
 #pragma unroll
-  for (int nt = 0; nt < 2; ++nt)
+  for (int nt = 0; nt < NTW; ++nt)
 #pragma unroll
-    for (int mt = 0; mt < 2; ++mt)
+    for (int mt = 0; mt < MT; ++mt)
 #pragma unroll
       for (int i = 0; i < 16; ++i) acc[nt][mt][i] = 0.f;
 
-  fetch(0, 0);
-  fetch(steps > 1 ? 1 : 0, 1);
-  stash(0, 0);
+  const int chunks = steps >> 3;
+  fetch_x(0);
+  fetch_w(0, 0);
+  fetch_w(steps > 1 ? 1 : 0, 1);
+  if (SB8) {
+    fetch_sb(0, 0);
+    fetch_sb(chunks > 1 ? 1 : 0, 1);
+  }
+  stash(0);
+#pragma unroll
+  for (int j = 0; j < 4; ++j) expand(0, j, 0);
   __syncthreads();
 
-  // One K step.  Register set p = ks & 1 holds the weights of step ks (its x part went to LDS
-  // during the previous step); once they are expanded the set is free for step ks + 2.  The
-  // loaded values are used where they were loaded: a copy of a register with a load in flight
-  // would wait for the load.
-  auto body = [&](int ks, int p) {
-    half8_t af[2][4];
+  // One K step, p = ks & 1: LDS buffer p holds x of this step and af[p] its expanded weights;
+  // register set p ^ 1 holds the packed weights of the next step, which are expanded between
+  // this step's matrix instructions; set p is free for the loads of step ks + 2.  Loaded
+  // values are used where they were loaded (a copy of a register with a load in flight would
+  // wait for the load), and the loads are issued first (left alone, the scheduler sinks them
+  // to the end of the step, where the in-order counter waits for them at once).
+  auto body = [&](int ks, auto E) {
+    constexpr int e = decltype(E)::value;   // step within its chunk (SB8) / parity of the step
+    constexpr int p = e & 1;
+    fetch_x(ks + 1 < steps ? ks + 1 : steps - 1);
+    fetch_w(ks + 2 < steps ? ks + 2 : steps - 1, p);
+    __builtin_amdgcn_sched_barrier(0);
 #pragma unroll
-    for (int nt = 0; nt < 2; ++nt) {
-      const half2_t s2 = half2_t{sreg[p][nt], sreg[p][nt]}, b2 = half2_t{breg[p][nt], breg[p][nt]};
+    for (int j = 0; j < 4; ++j) {
+      half8_t bf[MT];
 #pragma unroll
-      for (int j = 0; j < 4; ++j) af[nt][j] = dequant_word(wreg[p][nt][j], s2, b2);
+      for (int mt = 0; mt < MT; ++mt)
+        bf[mt] = *reinterpret_cast<const half8_t*>(&xs[p][(wm * 32 * MT + mt * 32 + ql) * XS + hb * 32 + j * 8]);
+      expand(p ^ 1, j, e + 1);
+#pragma unroll
+      for (int nt = 0; nt < NTW; ++nt)
+#pragma unroll
+        for (int mt = 0; mt < MT; ++mt)
+          acc[nt][mt] = __builtin_amdgcn_mfma_f32_32x32x16_f16(af[p][nt][j], bf[mt], acc[nt][mt], 0, 0, 0);
     }
     __builtin_amdgcn_sched_barrier(0);
-    // unconditional (the last steps load their own data again): no branches in the loop body;
-    // issued here, ahead of the matrix work (left alone, the scheduler sinks the loads to the
-    // end of the step, where the in-order counter then waits for them at once)
-    fetch(ks + 2 < steps ? ks + 2 : steps - 1, p);
-    __builtin_amdgcn_sched_barrier(0);
-    // all eight x operands of the step are requested at once: one LDS wait per step
-    half8_t bf[4][2];
+    stash(p ^ 1);
+    if (SB8 && e == 7) {
+      // the next chunk becomes the current one (its loads were issued eight steps ago)
 #pragma unroll
-    for (int j = 0; j < 4; ++j)
-#pragma unroll
-      for (int mt = 0; mt < 2; ++mt)
-        bf[j][mt] = *reinterpret_cast<const half8_t*>(&xs[p][(wm * 64 + mt * 32 + ql) * XS + hb * 32 + j * 8]);
-#pragma unroll
-    for (int j = 0; j < 4; ++j)
-#pragma unroll
-      for (int nt = 0; nt < 2; ++nt)
-#pragma unroll
-        for (int mt = 0; mt < 2; ++mt)
-          acc[nt][mt] = __builtin_amdgcn_mfma_f32_32x32x16_f16(af[nt][j], bf[j][mt], acc[nt][mt], 0, 0, 0);
-    __builtin_amdgcn_sched_barrier(0);
-    stash(p ^ 1, p ^ 1);
+      for (int nt = 0; nt < NTW; ++nt) {
+        s8[0][nt] = s8[1][nt];
+        b8[0][nt] = b8[1][nt];
+      }
+      const int c = (ks >> 3) + 2;
+      fetch_sb(c < chunks ? c : chunks - 1, 1);
+    }
     __syncthreads();
   };
-  int ks = 0;
-  for (; ks + 1 < steps; ks += 2) {
-    body(ks, 0);
-    body(ks + 1, 1);
+  if (SB8) {
+    for (int ks = 0; ks < steps; ks += 8) {
+      body(ks, StepIndex<0>{});
+      body(ks + 1, StepIndex<1>{});
+      body(ks + 2, StepIndex<2>{});
+      body(ks + 3, StepIndex<3>{});
+      body(ks + 4, StepIndex<4>{});
+      body(ks + 5, StepIndex<5>{});
+      body(ks + 6, StepIndex<6>{});
+      body(ks + 7, StepIndex<7>{});
+    }
+  } else {
+    int ks = 0;
+    for (; ks + 1 < steps; ks += 2) {
+      body(ks, StepIndex<0>{});
+      body(ks + 1, StepIndex<1>{});
+    }
+    if (ks < steps) body(ks, StepIndex<0>{});
   }
-  if (ks < steps) body(ks, 0);
 
   // accumulator register i of a lane: weight row (output column) 8*(i/4) + 4*hb + i%4 of the
   // tile, x row (output row) ql
 #pragma unroll
-  for (int mt = 0; mt < 2; ++mt) {
-    const int m = m0 + wm * 64 + mt * 32 + ql;
+  for (int mt = 0; mt < MT; ++mt) {
+    const int m = m0 + wm * 32 * MT + mt * 32 + ql;
     if (m >= M) continue;
 #pragma unroll
-    for (int nt = 0; nt < 2; ++nt) {
+    for (int nt = 0; nt < NTW; ++nt) {
 #pragma unroll
       for (int i4 = 0; i4 < 4; ++i4) {
         const int n = n0 + nt * 32 + 8 * i4 + 4 * hb;
@@ -182,6 +246,24 @@ __global__ __launch_bounds__(256) void qmm_gemm_w4g64_kernel(
   }
 }
 
+template <int NTW, int MT, bool SB8>
+int launch_gemm(const half_t* x, const uint32_t* w, const half_t* s, const half_t* b, const half_t* bias,
+                half_t* out, int M, int N, int K, hipStream_t st) {
+  constexpr int BMT = 32 * MT * (NTW == 2 ? 2 : 1);
+  static_assert(256 % BMT == 0 && BMT >= 32, "block load mapping");
+  const size_t lds = 2 * (size_t)BMT * XS * sizeof(half_t);
+  static bool configured = false;
+  if (!configured) {
+    if (hipFuncSetAttribute(reinterpret_cast<const void*>(&qmm_gemm_w4g64_kernel<NTW, MT, SB8>),
+                            hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds) != hipSuccess)
+      return EAGLE_ERR_HIP;
+    configured = true;
+  }
+  const dim3 grid((N + BN - 1) / BN, (M + BMT - 1) / BMT);
+  hipLaunchKernelGGL((qmm_gemm_w4g64_kernel<NTW, MT, SB8>), grid, dim3(256), lds, st, x, w, s, b, bias, out, M, N, K);
+  return eagle_launch_status();
+}
+
 }  // namespace
 
 EAGLE_EXPORT int eagle_qmm_gemm_w4g64_f16(const void* x, const uint32_t* wq, const void* scales,
@@ -193,10 +275,20 @@ EAGLE_EXPORT int eagle_qmm_gemm_w4g64_f16(const void* x, const uint32_t* wq, con
   if (!eagle_aligned16(x) || !eagle_aligned16(wq) || !eagle_aligned16(out) ||
       (bias && (reinterpret_cast<uintptr_t>(bias) & 7u)))
     return EAGLE_ERR_ALIGN;
-  const dim3 grid((N + BN - 1) / BN, (M + BM - 1) / BM);
-  hipLaunchKernelGGL(qmm_gemm_w4g64_kernel, grid, dim3(256), 0, static_cast<hipStream_t>(stream),
-                     static_cast<const half_t*>(x), wq, static_cast<const half_t*>(scales),
-                     static_cast<const half_t*>(biases), static_cast<const half_t*>(bias),
-                     static_cast<half_t*>(out), M, N, K);
-  return eagle_launch_status();
+  hipStream_t st = static_cast<hipStream_t>(stream);
+  const half_t* xh = static_cast<const half_t*>(x);
+  const half_t* sh = static_cast<const half_t*>(scales);
+  const half_t* bh = static_cast<const half_t*>(biases);
+  const half_t* bi = static_cast<const half_t*>(bias);
+  half_t* oh = static_cast<half_t*>(out);
+  // 64-row blocks when 128-row blocks would leave compute units without a workgroup
+  const long blocks128 = (long)((N + BN - 1) / BN) * ((M + 127) / 128);
+  const bool small = blocks128 < SMALL_BLOCKS && M > 64;
+  const bool sb8 = (K % 512) == 0 && eagle_aligned16(scales) && eagle_aligned16(biases);
+  if (small) {
+    if (sb8) return launch_gemm<1, 2, true>(xh, wq, sh, bh, bi, oh, M, N, K, st);
+    return launch_gemm<1, 2, false>(xh, wq, sh, bh, bi, oh, M, N, K, st);
+  }
+  if (sb8) return launch_gemm<1, 4, true>(xh, wq, sh, bh, bi, oh, M, N, K, st);
+  return launch_gemm<1, 4, false>(xh, wq, sh, bh, bi, oh, M, N, K, st);
 }
