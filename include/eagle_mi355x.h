@@ -35,6 +35,7 @@ enum eagle_status {
 };
 
 #define EAGLE_MAX_TREE 32    /* tree tokens per verify step (root + 31 nodes) */
+#define EAGLE_MAX_CHUNK 1024 /* rows of one causal pass over a prompt chunk */
 #define EAGLE_MAX_M 32       /* rows of x accepted by the quantised matmul */
 
 const char* eagle_status_string(int status);
@@ -176,6 +177,8 @@ int eagle_rope_kv_append_table_f16(const void* q_lin, const void* k_lin, const v
  * positions only, so one call serves every layer of a step. */
 int eagle_rope_table_f32(const int32_t* positions, const float* inv_freqs, float scaling_factor,
                          int T, int half_dim, float* out, eagle_stream_t stream);
+/* Both table forms take up to EAGLE_MAX_CHUNK rows (a prompt chunk); the other tree entry
+ * points take at most EAGLE_MAX_TREE. */
 
 /* The attention block of one layer without a separate rope launch (mlx_llama.py:166-195: rope of q and k with
  * per-token positions, cache update, masked SDPA).  q_lin / k_lin / v_lin are the token-major
@@ -207,6 +210,17 @@ int eagle_draft_attention_f16(const void* q, const void* k_cache, const void* v_
                               int T, int Tk, int H, int G, int hd, long capacity, int max_len,
                               float scale, void* workspace, size_t workspace_bytes,
                               eagle_stream_t stream);
+
+/* Causal attention of a prompt chunk (mlx_llama.py:185-192 with the causal mask of
+ * mlx_llama.py:275-276; mlx_eagle.py:522-533): R query rows (a multiple of 32, at most
+ * EAGLE_MAX_CHUNK) in pieces of 32.  Piece j has its rows at cache rows piece_len_dev[j] ..
+ * piece_len_dev[j] + 31 (already appended), sees every cache row before them and its own rows
+ * causally.  q [H,R,hd] (rotated), out [R, H*hd].  One launch pair for all pieces. */
+size_t eagle_causal_attention_workspace_bytes(int R, int H, int hd, int max_len);
+int eagle_causal_attention_f16(const void* q, const void* k_cache, const void* v_cache,
+                               const int32_t* piece_len_dev, void* out, int R, int H, int G, int hd,
+                               long capacity, int max_len, float scale, void* workspace,
+                               size_t workspace_bytes, eagle_stream_t stream);
 
 /* Row argmax of fp16 logits [R,V], lowest index among equal maxima
  * (mx.argmax at mlx_eagle.py:316,534,596).  out [R] int32. */

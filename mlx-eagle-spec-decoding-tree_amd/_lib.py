@@ -43,6 +43,9 @@ SIGNATURES = {
     "eagle_draft_tree_level": (c_int, [c_void_p] * 2 + [c_int] * 3 + [c_void_p] * 9),
     "eagle_spec_begin": (c_int, [c_void_p] * 5),
     "eagle_spec_update": (c_int, [c_void_p] * 3 + [c_int] + [c_void_p] * 5 + [c_int, c_void_p]),
+    "eagle_causal_attention_workspace_bytes": (c_size_t, [c_int] * 4),
+    "eagle_causal_attention_f16": (c_int, [c_void_p] * 5 + [c_int] * 4 + [c_long, c_int, c_float,
+                                                                         c_void_p, c_size_t, c_void_p]),
     "eagle_rope_table_f32": (c_int, [c_void_p, c_void_p, c_float, c_int, c_int, c_void_p, c_void_p]),
     "eagle_tree_attention_rope_workspace_bytes": (c_size_t, [c_int, c_int, c_int]),
     "eagle_tree_attention_rope_f16": (c_int, [c_void_p] * 3 + [c_long] + [c_void_p] * 6 + [c_int] * 4

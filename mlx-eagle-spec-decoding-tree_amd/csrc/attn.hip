@@ -65,7 +65,7 @@ __global__ __launch_bounds__(512) void tree_attn_split_kernel(
     const uint32_t* __restrict__ mask_bits, const int32_t* __restrict__ len_dev,
     half_t* __restrict__ part_o, float* __restrict__ part_ml, int T, int H, int G, long cap,
     int tiles_per_split, float scale_log2e, const half_t* __restrict__ k_lin,
-    const half_t* __restrict__ v_lin, long ld, const float* __restrict__ rope_cs, int Tk) {
+    const half_t* __restrict__ v_lin, long ld, const float* __restrict__ rope_cs, int Tk, int q_rows) {
   constexpr int KSTEPS = HD / 16;       // MFMA steps over the head dimension for S
   constexpr int DB = HD / 32;           // 32-wide blocks of the head dimension for O
   constexpr int STR = HD * 2 + 16;      // LDS row stride in bytes (pad: conflict-free reads)
@@ -88,7 +88,10 @@ __global__ __launch_bounds__(512) void tree_attn_split_kernel(
   const int hb = lane >> 5;             // which half of the k / key index this lane holds
   const int head = g * rep + wave;
 
-  int P = *len_dev;
+  // blockIdx.z: piece of a causal pass (32 query rows each, its own cache length, queries at
+  // rows 32 * piece of q [H, q_rows, hd]); a single piece otherwise
+  const int piece = blockIdx.z;
+  int P = len_dev[piece];
   if (ROPE || WIDE) {                   // never index past the cache, whatever the counter says
     if (P > cap - Tk) P = (int)(cap - Tk);
     if (P < 0) P = 0;
@@ -106,13 +109,15 @@ __global__ __launch_bounds__(512) void tree_attn_split_kernel(
   for (int kk = 0; kk < KSTEPS; ++kk) {
     qreg[kk] = half8_t{0, 0, 0, 0, 0, 0, 0, 0};
     if (ql < T) {
-      const half_t* qp = ROPE ? q + (long)ql * ld + (long)head * HD : q + ((long)head * T + ql) * HD;
+      const half_t* qp = ROPE ? q + (long)ql * ld + (long)head * HD
+                              : q + ((long)head * q_rows + piece * 32 + ql) * HD;
       qreg[kk] = *reinterpret_cast<const half8_t*>(qp + kk * 16 + hb * 8);
     }
   }
   // WIDE: two mask words per query (masked key rows 0..31 and 32..63)
-  const uint32_t mybits = ql < T ? mask_bits[WIDE ? 2 * ql : ql] : 0u;
-  const uint32_t mybits_hi = (WIDE && ql < T) ? mask_bits[2 * ql + 1] : 0u;
+  // no mask array: causal among the T rows
+  const uint32_t mybits = ql < T ? (mask_bits ? mask_bits[WIDE ? 2 * ql : ql] : (2u << ql) - 1u) : 0u;
+  const uint32_t mybits_hi = (WIDE && ql < T && mask_bits) ? mask_bits[2 * ql + 1] : 0u;
 
   float m_run = -INFINITY, l_run = 0.f;
   float16_t o_acc[DB];
@@ -294,7 +299,7 @@ __global__ __launch_bounds__(512) void tree_attn_split_kernel(
   }
 
   // partials: part_ml [H][nsplit][32][2], part_o [H][nsplit][32][HD]
-  const long slot = ((long)head * nsplit + split) * 32 + ql;
+  const long slot = (((long)piece * H + head) * nsplit + split) * 32 + ql;
   if (hb == 0) {
     part_ml[slot * 2 + 0] = m_run;
     part_ml[slot * 2 + 1] = l_run;
@@ -322,6 +327,10 @@ __global__ void tree_attn_merge_kernel(const half_t* __restrict__ part_o,
                                        half_t* __restrict__ out, int T, int H, int nsplit,
                                        const int32_t* __restrict__ len_dev, long cap, int clamp_len,
                                        int Tk) {
+  const int piece = blockIdx.z;                     // as in the split kernel
+  part_o += (long)piece * H * nsplit * 32 * HD;
+  part_ml += (long)piece * H * nsplit * 32 * 2;
+  out += (long)piece * 32 * H * HD;
   constexpr int QW = HD / 4;                       // threads per token
   constexpr int TPW = 256 / HD;                    // tokens per wave: MERGE_TOK tokens on HD / 64 waves
   constexpr int PRE = 8;
@@ -351,7 +360,7 @@ __global__ void tree_attn_merge_kernel(const half_t* __restrict__ part_o,
   for (int k = 0; k < PRE; ++k)
     pre[k] = *reinterpret_cast<const half4_t*>(src + (long)(k < nsplit ? k : nsplit - 1) * 32 * HD);
 
-  int P = *len_dev;
+  int P = len_dev[piece];
   if (clamp_len) {
     if (P > cap - Tk) P = (int)(cap - Tk);
     if (P < 0) P = 0;
@@ -410,17 +419,19 @@ template <int HD, bool ROPE, bool WIDE = false>
 int launch_attention(const half_t* q, half_t* kc, half_t* vc, const uint32_t* bits, const int32_t* len,
                      void* out, int T, int H, int G, long cap, int max_len, float scale, void* workspace,
                      const half_t* k_lin, const half_t* v_lin, long ld, const float* cs, hipStream_t st,
-                     int Tk = 0) {
+                     int Tk = 0, int pieces = 1) {
   if (!WIDE) Tk = T;
+  const int q_rows = pieces * T;
   const int nsplit = splits_for(max_len, G);
   float* part_ml = static_cast<float*>(workspace);
-  half_t* part_o = reinterpret_cast<half_t*>(part_ml + (size_t)H * nsplit * 32 * 2);
+  half_t* part_o = reinterpret_cast<half_t*>(part_ml + (size_t)pieces * H * nsplit * 32 * 2);
   const float sl2 = scale * 1.4426950408889634f;
   const int rep = H / G;
   const size_t lds = 2 * KT * (HD * 2 + 16) + (ROPE ? (size_t)EAGLE_MAX_TREE * HD * 4 : 0);
-  hipLaunchKernelGGL((tree_attn_split_kernel<HD, ROPE, WIDE>), dim3(G, nsplit), dim3(rep * 64), lds, st, q,
-                     kc, vc, bits, len, part_o, part_ml, T, H, G, cap, 0, sl2, k_lin, v_lin, ld, cs, Tk);
-  hipLaunchKernelGGL(tree_attn_merge_kernel<HD>, dim3(H, (T + MERGE_TOK - 1) / MERGE_TOK),
+  hipLaunchKernelGGL((tree_attn_split_kernel<HD, ROPE, WIDE>), dim3(G, nsplit, pieces), dim3(rep * 64), lds,
+                     st, q, kc, vc, bits, len, part_o, part_ml, T, H, G, cap, 0, sl2, k_lin, v_lin, ld, cs, Tk,
+                     q_rows);
+  hipLaunchKernelGGL(tree_attn_merge_kernel<HD>, dim3(H, (T + MERGE_TOK - 1) / MERGE_TOK, pieces),
                      dim3(MERGE_TOK * HD / 4), 0, st, part_o, part_ml, (half_t*)out, T, H, nsplit,
                      len, cap, (ROPE || WIDE) ? 1 : 0, Tk);
   return eagle_launch_status();
@@ -502,11 +513,44 @@ EAGLE_EXPORT int eagle_draft_attention_f16(const void* q, const void* k_cache, c
                                            nullptr, st, Tk);
 }
 
+EAGLE_EXPORT size_t eagle_causal_attention_workspace_bytes(int R, int H, int hd, int max_len) {
+  if (R < 32 || (R % 32) != 0) return 0;
+  return (size_t)(R / 32) * eagle_tree_attention_workspace_bytes(H, hd, max_len);
+}
+
+EAGLE_EXPORT int eagle_causal_attention_f16(const void* q, const void* k_cache, const void* v_cache,
+                                            const int32_t* piece_len_dev, void* out, int R, int H, int G,
+                                            int hd, long capacity, int max_len, float scale,
+                                            void* workspace, size_t workspace_bytes,
+                                            eagle_stream_t stream) {
+  if (!q || !k_cache || !v_cache || !piece_len_dev || !out) return EAGLE_ERR_NULL;
+  if (R < 32 || (R % 32) != 0 || R > EAGLE_MAX_CHUNK || H < 1 || G < 1 || (H % G) != 0 ||
+      (H / G) > 8 || (hd != 64 && hd != 128) || max_len < 32 || max_len > capacity)
+    return EAGLE_ERR_SHAPE;
+  if (!eagle_aligned16(q) || !eagle_aligned16(k_cache) || !eagle_aligned16(v_cache) ||
+      !eagle_aligned16(out))
+    return EAGLE_ERR_ALIGN;
+  if (!workspace || !eagle_aligned16(workspace) ||
+      workspace_bytes < eagle_causal_attention_workspace_bytes(R, H, hd, max_len))
+    return EAGLE_ERR_WORKSPACE;
+  hipStream_t st = static_cast<hipStream_t>(stream);
+  half_t* kc = const_cast<half_t*>(static_cast<const half_t*>(k_cache));
+  half_t* vc = const_cast<half_t*>(static_cast<const half_t*>(v_cache));
+  // the two-word form of the kernel: it keeps the cache length inside the buffer
+  if (hd == 128)
+    return launch_attention<128, false, true>((const half_t*)q, kc, vc, nullptr, piece_len_dev, out, 32, H,
+                                              G, capacity, max_len, scale, workspace, nullptr, nullptr, 0,
+                                              nullptr, st, 32, R / 32);
+  return launch_attention<64, false, true>((const half_t*)q, kc, vc, nullptr, piece_len_dev, out, 32, H, G,
+                                           capacity, max_len, scale, workspace, nullptr, nullptr, 0, nullptr,
+                                           st, 32, R / 32);
+}
+
 EAGLE_EXPORT int eagle_rope_table_f32(const int32_t* positions, const float* inv_freqs,
                                       float scaling_factor, int T, int half_dim, float* out,
                                       eagle_stream_t stream) {
   if (!positions || !inv_freqs || !out) return EAGLE_ERR_NULL;
-  if (T < 1 || T > EAGLE_MAX_TREE || half_dim < 1) return EAGLE_ERR_SHAPE;
+  if (T < 1 || T > EAGLE_MAX_CHUNK || half_dim < 1) return EAGLE_ERR_SHAPE;
   if (!eagle_aligned16(out)) return EAGLE_ERR_ALIGN;
   const int total = T * half_dim;
   hipLaunchKernelGGL(rope_table_kernel, dim3((total + 255) / 256), dim3(256), 0,

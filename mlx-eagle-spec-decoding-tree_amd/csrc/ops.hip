@@ -372,7 +372,7 @@ EAGLE_EXPORT int eagle_rope_kv_append_table_f16(const void* q_lin, const void* k
                                                 eagle_stream_t stream) {
   if (!q_lin || !k_lin || !v_lin || !rope_cs || !q_out || !k_cache || !v_cache || !cache_len_dev)
     return EAGLE_ERR_NULL;
-  if (T < 1 || T > EAGLE_MAX_TREE || H < 1 || G < 1 || (H % G) != 0 || hd < 16 || (hd % 16) != 0 ||
+  if (T < 1 || T > EAGLE_MAX_CHUNK || H < 1 || G < 1 || (H % G) != 0 || hd < 16 || (hd % 16) != 0 ||
       capacity < T || row_stride < 0 || (row_stride % 8) != 0 ||
       (row_stride > 0 && row_stride < (long)H * hd))
     return EAGLE_ERR_SHAPE;

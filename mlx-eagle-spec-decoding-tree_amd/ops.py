@@ -12,7 +12,8 @@ import torch
 
 from . import _lib
 
-_WS = {}  # (device index, tag) -> workspace tensor
+_WS = {}        # (device index, tag) -> workspace tensor
+_RETIRED = []   # outgrown workspaces, kept allocated (see workspace())
 
 
 def _stream():
@@ -42,6 +43,12 @@ def workspace(tag, nbytes, device):
     key = (device.index, tag)
     buf = _WS.get(key)
     if buf is None or buf.numel() < nbytes:
+        if buf is not None:
+            # a captured graph may still hold the old address, and beginning the next capture
+            # returns every free block to the driver (torch.cuda.graph empties the allocator's
+            # cache): a replay would then write to unmapped memory.  Outgrown buffers therefore
+            # stay allocated until the process ends.
+            _RETIRED.append(buf)
         buf = torch.zeros(max(int(nbytes), 1 << 16), dtype=torch.uint8, device=device)
         _WS[key] = buf
     return buf
@@ -358,6 +365,26 @@ def scaled_dot_product_attention(queries, keys, values, cache=None, scale=None, 
         k_buf, v_buf = _f16(keys[0], "k"), _f16(values[0], "v")
     out = draft_attention(_f16(queries[0], "q"), k_buf, v_buf, words, len_dev, Tk, scale, max_len=S)
     return out.reshape(T, H, hd).permute(1, 0, 2).unsqueeze(0).contiguous()
+
+
+def causal_attention(q, k_cache, v_cache, piece_len_dev, scale, max_len=None, out=None):
+    """Causal attention of a prompt chunk in pieces of 32 rows, one launch pair for all pieces:
+    q [H,R,hd] (R a multiple of 32); piece j sits at cache rows piece_len_dev[j] .. +31.
+    Returns [R, H*hd]."""
+    _need_cuda(q, k_cache, v_cache, piece_len_dev)
+    H, R, hd = q.shape
+    G, cap, _ = k_cache.shape
+    if max_len is None:
+        max_len = cap
+    if out is None:
+        out = torch.empty((R, H * hd), dtype=torch.float16, device=q.device)
+    L = _lib.lib()
+    ws = workspace("attn_chunk", L.eagle_causal_attention_workspace_bytes(R, H, hd, max_len), q.device)
+    rc = L.eagle_causal_attention_f16(_ptr(q), _ptr(k_cache), _ptr(v_cache), _ptr(piece_len_dev), _ptr(out),
+                                      R, H, G, hd, cap, max_len, float(scale), _ptr(ws), ws.numel(),
+                                      _stream())
+    _lib.check(rc, "causal_attention")
+    return out
 
 
 def logsoftmax_topk(logits, k, mode, row_index=None, out=None):

@@ -96,9 +96,9 @@ class DecoderPass:
 
 class ChunkPass:
     """A causal pass of R rows (a multiple of 32, at most 1024) through a decoder: the linear
-    layers see all R rows at once (the tiled GEMM form of the matmul above 32 rows), rope /
-    cache append / attention run per piece of 32 rows, every piece seeing the cache rows before
-    it and its own rows causally.  Rows are appended at the cache length, which advances by R."""
+    layers see all R rows at once (the tiled GEMM form of the matmul above 32 rows), so do rope
+    and the cache append; attention runs per piece of 32 rows (all pieces in one launch), every
+    piece seeing the cache rows before it and its own rows causally.  Rows are appended at the cache length, which advances by R."""
 
     PIECE = 32
 
@@ -120,7 +120,7 @@ class ChunkPass:
         self.h = torch.empty((R, D), **f16)
         self.hn = torch.empty((R, D), **f16)
         self.qkv = torch.empty((R, (H + 2 * G) * hd), **f16)
-        self.q_rot = torch.empty((H, P, hd), **f16)
+        self.q_rot = torch.empty((H, R, hd), **f16)
         self.rope_cs = torch.empty((R, hd // 2, 2), dtype=torch.float32, device=dev)
         self.attn = torch.empty((R, H * hd), **f16)
         self.o = torch.empty((R, D), **f16)
@@ -132,12 +132,11 @@ class ChunkPass:
         self.piece_len = torch.zeros(self.pieces, **i32)
         self.arange = torch.arange(P, **i32)
         self.positions = torch.zeros(R, **i32)
-        self.words = ops.mask_to_words(torch.tril(torch.ones((P, P), dtype=torch.bool, device=dev)))
         self.len_dev = cache[0].len_dev
         L = _lib.lib()
         hw = model.lm_head if not args.tie_word_embeddings else model.model.embed_tokens
         ops.workspace("qmm", L.eagle_qmm_workspace_bytes(P, hw.weight.shape[0], D), dev)
-        ops.workspace("attn", L.eagle_tree_attention_workspace_bytes(H, hd, self.max_len), dev)
+        ops.workspace("attn_chunk", L.eagle_causal_attention_workspace_bytes(R, H, hd, self.max_len), dev)
         self.graph = None
 
     def enqueue(self):
@@ -155,7 +154,7 @@ class ChunkPass:
             pos = self.positions[j * P:(j + 1) * P]
             _lib.check(L.eagle_tree_positions(_ptr(self.arange), _ptr(self.piece_len[j:j + 1]), _ptr(pos),
                                               P, st), "positions")
-            ops.rope_table(pos, at0._inv_freqs, at0._scaling_factor, out=self.rope_cs[j * P:(j + 1) * P])
+        ops.rope_table(self.positions, at0._inv_freqs, at0._scaling_factor, out=self.rope_cs)
         emb = m.model.embed_tokens
         ops.embed(self.tokens, emb.weight, emb.scales, emb.biases, out=self.h)
         ops.rms_norm(self.h, layers[0].input_layernorm.weight, args.rms_norm_eps, out=self.hn)
@@ -163,15 +162,13 @@ class ChunkPass:
             at, mlp, c = layer.self_attn, layer.mlp, self.cache[i]
             w, sc, bi, b = self.qkv_w[i]
             ops.quantized_matmul(self.hn, w, sc, bi, bias=b, out=self.qkv)
-            for j in range(self.pieces):
-                rows = slice(j * P, (j + 1) * P)
-                qkv = self.qkv[rows]
-                plen = self.piece_len[j:j + 1]
-                ops.rope_kv_append(qkv, qkv[:, H * hd:], qkv[:, (H + G) * hd:], None, at._inv_freqs,
-                                   at._scaling_factor, self.q_rot, c.keys[0], c.values[0], plen, H, G, hd,
-                                   row_stride=W, rope_cs=self.rope_cs[rows])
-                ops.draft_attention(self.q_rot, c.keys[0], c.values[0], self.words, plen, P, at.scale,
-                                    max_len=self.max_len, out=self.attn[rows])
+            # all rows at once: rotate and append, then attention with one 32-row piece per
+            # workgroup column
+            ops.rope_kv_append(self.qkv, self.qkv[:, H * hd:], self.qkv[:, (H + G) * hd:], None,
+                               at._inv_freqs, at._scaling_factor, self.q_rot, c.keys[0], c.values[0],
+                               self.len_dev, H, G, hd, row_stride=W, rope_cs=self.rope_cs)
+            ops.causal_attention(self.q_rot, c.keys[0], c.values[0], self.piece_len, at.scale,
+                                 max_len=self.max_len, out=self.attn)
             ops.quantized_matmul(self.attn, at.o_proj.weight, at.o_proj.scales, at.o_proj.biases,
                                  bias=at.o_proj.bias, out=self.o)
             ops.rms_norm(self.o, layer.post_attention_layernorm.weight, args.rms_norm_eps,
@@ -222,20 +219,21 @@ class CausalPrefill:
         self.chunk, self.graphs = chunk, graphs
         self.passes = {}
 
-    def _pass(self, R):
+    def _pass(self, R, capture=True):
         p = self.passes.get(R)
         if p is None:
-            p = ChunkPass(self.model, self.cache, R, max_len=self.max_len, head=self.head)
-            if self.graphs:
-                p.capture()
-            self.passes[R] = p
+            p = self.passes[R] = ChunkPass(self.model, self.cache, R, max_len=self.max_len, head=self.head)
+        if capture and self.graphs and p.graph is None:
+            p.capture()
         return p
 
-    def prepare(self, n):
-        """Build (and capture) the passes a prompt of n tokens needs."""
+    def prepare(self, n, capture=True):
+        """Build (and, with capture, record) the passes a prompt of n tokens needs.  Several
+        models sharing the workspaces should all be built before any of them is captured, so
+        that no workspace is outgrown after an address went into a graph."""
         while n > 0:
             R = min(self.chunk, (n + 31) // 32 * 32)
-            self._pass(R)
+            self._pass(R, capture)
             n -= R
         return self
 
@@ -328,13 +326,15 @@ class SpeculativeDecoder:
                              CausalPrefill(self.base_model, self.base_cache, self.capacity))
         if prompt_len:
             for p in self._prefill:
+                p.prepare(prompt_len, capture=False)     # every workspace at its final size first
+            for p in self._prefill:
                 p.prepare(prompt_len)
         return self
 
     def prefill(self, prompt):
         """mlx_eagle.py:522-535: both models read the prompt; the first token is the target's
         argmax at its last position."""
-        self.prepare()
+        self.prepare(prompt.numel())
         self._prefill[0](prompt)
         first = ops.argmax_rows(self._prefill[1](prompt))
         self.y.zero_()

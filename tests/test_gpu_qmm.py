@@ -147,8 +147,10 @@ def test_argument_errors(dev):
     x = torch.zeros(33, 128, dtype=torch.float16, device=dev)
     w = torch.zeros(8, 16, dtype=torch.int32, device=dev)
     s = torch.zeros(8, 2, dtype=torch.float16, device=dev)
+    # more than 32 rows go to the tiled GEMM form; the streaming kernel itself refuses them
+    assert tuple(ops.quantized_matmul(x, w, s, s).shape) == (33, 8)
     with pytest.raises(ValueError):
-        ops.quantized_matmul(x, w, s, s)              # M > 32
+        ops.quantized_matmul(x, w, s, s, tuned=(1, 1, 1, 1))
     with pytest.raises(ValueError):
         ops.quantized_matmul(x[:8], w, s, s, group_size=32)
     with pytest.raises(ValueError):

@@ -113,3 +113,17 @@ def test_mask_bit_helpers_round_trip():
     back = eagle.bits_to_mask(bits, torch.float32)
     assert torch.equal(back == 0, vis)
     assert torch.equal(ops.mask_to_bits(back), bits)
+
+
+def test_outgrown_workspaces_stay_allocated():
+    """A captured graph may hold a workspace address, and beginning a later capture hands every
+    free block back to the driver: a workspace that is outgrown must not be released."""
+    import torch
+    from mlx_eagle_spec_decoding_tree_amd import ops
+
+    cpu = torch.device("cpu")
+    a = ops.workspace("test_outgrown", 100_000, cpu)
+    assert ops.workspace("test_outgrown", 50_000, cpu) is a          # large enough: reused
+    b = ops.workspace("test_outgrown", 300_000, cpu)
+    assert b is not a and b.numel() >= 300_000
+    assert any(t is a for t in ops._RETIRED)
