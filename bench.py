@@ -92,6 +92,8 @@ def main():
                          "1 GiB read + 1 GiB written) so that profiler byte counters can be scaled")
     ap.add_argument("--loop", action="store_true",
                     help="measure the end-to-end tree loop (drafter + target) instead of the verify step")
+    ap.add_argument("--gemm", action="store_true",
+                    help="measure the many-row (prompt pass) form of the quantised matmul instead")
     ap.add_argument("--self-draft", action="store_true",
                     help="with --loop: the target drafts for itself (high acceptance; exercises the "
                          "accept path at full size)")
@@ -101,6 +103,8 @@ def main():
         sys.exit(2)
     if opt.loop:
         return loop_bench(opt)
+    if opt.gemm:
+        return gemm_bench(opt)
 
     import torch
     from mlx_eagle_spec_decoding_tree_amd import _lib, eagle, llama, ops, synth
@@ -248,6 +252,49 @@ def main():
             "roofline": roofline, "cpu_baseline": cpu}
     if parity is not None:
         line["parity"] = parity
+    print(json.dumps(line), flush=True)
+
+
+def gemm_bench(opt):
+    """The linear layers of one Llama-3-8B-shaped decoder layer over a 512-row prompt chunk
+    (mlx_eagle.py:522-533): tiled MFMA GEMM with in-register dequantisation.  Bound by the matrix
+    cores: 2*M*N*K flops per launch against 2.5 PFLOP/s dense fp16."""
+    import torch
+    from mlx_eagle_spec_decoding_tree_amd import _lib, ops
+
+    if not torch.cuda.is_available():
+        print("bench.py: no GPU visible", file=sys.stderr)
+        sys.exit(2)
+    dev = torch.device("cuda:0")
+    _lib.check(_lib.lib().eagle_check_device(), "device check")
+    M = 512
+    shapes = [("q|k|v", 6144, 4096), ("o", 4096, 4096), ("gate|up", 28672, 4096), ("down", 4096, 14336)]
+    gen = torch.Generator(device=dev).manual_seed(opt.seed)
+    rows, total_us, total_flop = [], 0.0, 0.0
+    for name, N, K in shapes:
+        w = torch.randint(-2 ** 31, 2 ** 31 - 1, (N, K // 8), dtype=torch.int32, device=dev, generator=gen)
+        sc = (torch.rand(N, K // 64, device=dev, generator=gen) * 0.015 + 0.005).half()
+        bi = (-8 * sc.float()).half()
+        x = torch.randn(M, K, device=dev, generator=gen).half()
+        out = torch.empty(M, N, dtype=torch.float16, device=dev)
+        ms, _ = graph_time_ms(torch, lambda: ops.quantized_matmul(x, w, sc, bi, out=out), opt.steps, opt.warmup)
+        us = 1e3 * sorted(ms)[len(ms) // 2]
+        flop = 2.0 * M * N * K
+        rows.append({"name": name, "N": N, "K": K, "us": round(us, 2), "tflops": round(flop / us / 1e6, 1)})
+        total_us += us
+        total_flop += flop
+    achieved = total_flop / total_us / 1e6
+    line = {
+        "metric": "prompt-pass quantised matmul, TFLOP/s over the linear layers of one decoder layer",
+        "value": round(achieved, 1), "unit": "TFLOP/s", "n_gpus": 1, "steps": opt.steps, "warmup": opt.warmup,
+        "ms_per_step": round(total_us / 1e3, 4), "higher_is_better": True, "scaling": "weak",
+        "vs_baseline": None, "dtype": "f16", "data": "synthetic",
+        "config": {"workload": "Llama-3-8B-shaped 4-bit g64 layer, 512-row prompt chunk: q|k|v, o, gate|up, "
+                               "down as tiled MFMA GEMMs", "rows": M},
+        "roofline": {"bound": "mfma", "kernel": "qmm_gemm_w4g64_kernel", "achieved": round(achieved, 1),
+                     "peak": 2500.0, "unit": "TFLOP/s", "frac": round(achieved / 2500.0, 4), "traffic": None},
+        "shapes": rows,
+    }
     print(json.dumps(line), flush=True)
 
 
