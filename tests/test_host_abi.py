@@ -127,3 +127,45 @@ def test_outgrown_workspaces_stay_allocated():
     b = ops.workspace("test_outgrown", 300_000, cpu)
     assert b is not a and b.numel() >= 300_000
     assert any(t is a for t in ops._RETIRED)
+
+
+def test_draft_side_entry_points_reject_bad_arguments():
+    L = _lib.lib()
+    buf = (ctypes.c_char * 4096)()
+    p = (ctypes.addressof(buf) + 15) & ~15
+    big = 1 << 30
+    # draft attention: T <= 32 queries, Tk <= 64 masked rows
+    assert L.eagle_draft_attention_f16(p, p, p, None, p, p, 8, 24, 14, 2, 64, 4096, 2048, 0.1, p, big, None) == 1
+    assert L.eagle_draft_attention_f16(p, p, p, p, p, p, 33, 24, 14, 2, 64, 4096, 2048, 0.1, p, big, None) == 2
+    assert L.eagle_draft_attention_f16(p, p, p, p, p, p, 8, 65, 14, 2, 64, 4096, 2048, 0.1, p, big, None) == 2
+    assert L.eagle_draft_attention_f16(p, p, p, p, p, p, 8, 24, 14, 2, 64, 4096, 8192, 0.1, p, big, None) == 2
+    assert L.eagle_draft_attention_f16(p, p, p, p, p, p, 8, 24, 14, 2, 64, 4096, 2048, 0.1, None, 0, None) == 5
+    # causal chunk attention: rows a multiple of 32, at most 1024
+    assert L.eagle_causal_attention_f16(p, p, p, p, p, 48, 14, 2, 64, 4096, 2048, 0.1, p, big, None) == 2
+    assert L.eagle_causal_attention_f16(p, p, p, p, p, 2048, 14, 2, 64, 4096, 2048, 0.1, p, big, None) == 2
+    assert L.eagle_causal_attention_f16(p, p, p, p, p, 512, 14, 2, 64, 4096, 2048, 0.1, p, 1024, None) == 5
+    assert (L.eagle_causal_attention_workspace_bytes(512, 14, 64, 2048)
+            == 16 * L.eagle_tree_attention_workspace_bytes(14, 64, 2048))
+    # log-softmax + top-k: k <= 8, k <= V, modes 0 and 1
+    assert L.eagle_logsoftmax_topk_f16(None, None, 8, 1000, 8, 0, p, p, p, big, None) == 1
+    assert L.eagle_logsoftmax_topk_f16(p, None, 8, 1000, 9, 0, p, p, p, big, None) == 2
+    assert L.eagle_logsoftmax_topk_f16(p, None, 8, 4, 8, 0, p, p, p, big, None) == 2
+    assert L.eagle_logsoftmax_topk_f16(p, None, 33, 1000, 8, 0, p, p, p, big, None) == 2
+    assert L.eagle_logsoftmax_topk_f16(p, None, 8, 1000, 8, 2, p, p, p, big, None) == 4
+    assert L.eagle_logsoftmax_topk_f16(p, None, 8, 152064, 8, 1, p, p, p, 1024, None) == 5
+    assert L.eagle_logsoftmax_topk_workspace_bytes(8, 152064) == 8 * 38 * 18 * 4
+    # tree bookkeeping: k <= 8, k * depth <= 64, level < depth
+    assert L.eagle_draft_tree_init(p, p, 9, p, p, p, p, p, p, None) == 2
+    assert L.eagle_draft_tree_init(p, None, 8, p, p, p, p, p, p, None) == 1
+    assert L.eagle_draft_tree_level(p, p, 3, 8, 3, p, p, p, p, p, p, p, p, None) == 2
+    assert L.eagle_draft_tree_level(p, p, 0, 8, 9, p, p, p, p, p, p, p, p, None) == 2
+    assert L.eagle_draft_tree_level(p, p, 0, 8, 3, p, p, p, p, p, p, None, p, None) == 1
+    assert L.eagle_spec_begin(p, None, p, p, None) == 1
+    assert L.eagle_spec_update(p, p, p, 0, p, p, p, p, p, 16, None) == 2
+    assert L.eagle_spec_update(p, p, p, 8, p, p, p, p, p, 0, None) == 2
+    # many-row matmul
+    assert L.eagle_qmm_gemm_w4g64_f16(p, p, p, p, None, None, 512, 128, 128, 64, 4, None) == 1
+    assert L.eagle_qmm_gemm_w4g64_f16(p, p, p, p, None, p, 512, 100, 128, 64, 4, None) == 2
+    assert L.eagle_qmm_gemm_w4g64_f16(p, p, p, p, None, p, 512, 128, 100, 64, 4, None) == 2
+    assert L.eagle_qmm_gemm_w4g64_f16(p, p, p, p, None, p, 512, 128, 128, 32, 4, None) == 4
+    assert L.eagle_qmm_gemm_w4g64_f16(p + 2, p, p, p, None, p, 512, 128, 128, 64, 4, None) == 3
