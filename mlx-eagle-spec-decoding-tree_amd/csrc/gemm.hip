@@ -21,8 +21,8 @@
 
 namespace {
 
-constexpr int BN = 128, BK = 64;
-constexpr long SMALL_BLOCKS = 256;       // compute units    // set from measurements
+constexpr int BK = 64;
+constexpr long NUM_CU = 256;
 constexpr int XS = BK + 8;                  // LDS row stride in halves (144 bytes: conflict-free 16-byte reads)
 
 __device__ inline half8_t permute8(half8_t v) {
@@ -72,10 +72,12 @@ __global__ __launch_bounds__(256) void qmm_gemm_w4g64_kernel(
     const half_t* __restrict__ x, const uint32_t* __restrict__ w, const half_t* __restrict__ s,
     const half_t* __restrict__ b, const half_t* __restrict__ bias, half_t* __restrict__ out, int M,
     int N, int K) {
-  // NTW = 32-row weight tiles per wave: 2 (waves 2 x 2 over the block) or 1 (four waves side by
-  // side, each over all x rows of the block: no weight row is loaded or expanded twice)
-  constexpr int WN = 128 / (32 * NTW);       // waves along the weight rows
-  constexpr int WM = 4 / WN;                 // waves along the x rows
+  // NTW = 32-row weight tiles per wave (1 or 2); the four waves sit side by side along the
+  // weight rows, each over all x rows of the block: no weight row is loaded or expanded twice,
+  // and with NTW = 2 every x operand read from LDS serves two matrix instructions
+  constexpr int WN = 4;                      // waves along the weight rows (side by side)
+  constexpr int WM = 1;                      // waves along the x rows
+  constexpr int BN = 32 * NTW * WN;          // weight rows per workgroup (128 or 256)
   constexpr int BMT = 32 * MT * WM;          // rows of x per workgroup
   constexpr int TPR = 256 / BMT;             // threads per x row in the block load (2 or 1)
   constexpr int PP = 8 / TPR;                // 16-byte pieces per thread
@@ -249,7 +251,8 @@ __global__ __launch_bounds__(256) void qmm_gemm_w4g64_kernel(
 template <int NTW, int MT, bool SB8>
 int launch_gemm(const half_t* x, const uint32_t* w, const half_t* s, const half_t* b, const half_t* bias,
                 half_t* out, int M, int N, int K, hipStream_t st) {
-  constexpr int BMT = 32 * MT * (NTW == 2 ? 2 : 1);
+  constexpr int BMT = 32 * MT;
+  constexpr int BN = 128 * NTW;
   static_assert(256 % BMT == 0 && BMT >= 32, "block load mapping");
   const size_t lds = 2 * (size_t)BMT * XS * sizeof(half_t);
   static bool configured = false;
@@ -281,13 +284,25 @@ EAGLE_EXPORT int eagle_qmm_gemm_w4g64_f16(const void* x, const uint32_t* wq, con
   const half_t* bh = static_cast<const half_t*>(biases);
   const half_t* bi = static_cast<const half_t*>(bias);
   half_t* oh = static_cast<half_t*>(out);
-  // 64-row blocks when 128-row blocks would leave compute units without a workgroup
-  const long blocks128 = (long)((N + BN - 1) / BN) * ((M + 127) / 128);
-  const bool small = blocks128 < SMALL_BLOCKS && M > 64;
+  // Block shape: 64 x 128, 128 x 128 or 128 x 256 (x rows x weight rows).  The compute unit with
+  // the most workgroups sets the time, and a workgroup's work goes with its block (bigger
+  // blocks do a little less per output: 0.55 / 1 / 1.85); the estimate below reproduced the
+  // faster choice for every projection shape of the 7B / 8B / 0.5B models at 512 and 2048 rows.
+  auto most = [](long blocks) { return (double)((blocks + NUM_CU - 1) / NUM_CU); };
+  const long nb = (N + 127) / 128;
+  const double cost_norm = most(nb * ((M + 127) / 128));
+  const double cost_small = M > 64 ? 0.55 * most(nb * ((M + 63) / 64)) : 1e30;
+  const double cost_big = 1.85 * most(((N + 255) / 256) * (long)((M + 127) / 128));
+  const bool small = cost_small < cost_norm && cost_small <= cost_big;
+  const bool big = !small && cost_big < cost_norm;
   const bool sb8 = (K % 512) == 0 && eagle_aligned16(scales) && eagle_aligned16(biases);
   if (small) {
     if (sb8) return launch_gemm<1, 2, true>(xh, wq, sh, bh, bi, oh, M, N, K, st);
     return launch_gemm<1, 2, false>(xh, wq, sh, bh, bi, oh, M, N, K, st);
+  }
+  if (big) {
+    if (sb8) return launch_gemm<2, 4, true>(xh, wq, sh, bh, bi, oh, M, N, K, st);
+    return launch_gemm<2, 4, false>(xh, wq, sh, bh, bi, oh, M, N, K, st);
   }
   if (sb8) return launch_gemm<1, 4, true>(xh, wq, sh, bh, bi, oh, M, N, K, st);
   return launch_gemm<1, 4, false>(xh, wq, sh, bh, bi, oh, M, N, K, st);
