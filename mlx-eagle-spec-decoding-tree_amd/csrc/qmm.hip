@@ -756,10 +756,25 @@ void choose(int M, int N, int K, Launch* out) {
       L.phases = 2;
       L.nw = (uw + 1) / 2;
       L.splits = 1;
-    } else if (un > 2 * MAX_STREAM_WAVES) {
+    } else if (un > 2 * MAX_STREAM_WAVES && !(tiles < 3 * NUM_CU / 2 && un <= 4 * MAX_STREAM_WAVES)) {
+      // (few tiles and K up to 7168: four narrow slabs, below)
       L.wide = 1;
       L.phases = 1;
-      L.splits = (uw + MAX_WIDE_WAVES - 1) / MAX_WIDE_WAVES;
+      const int least = (uw + MAX_WIDE_WAVES - 1) / MAX_WIDE_WAVES;
+      // of the slab counts close to the least possible, the one that gives the most workgroups
+      // (tile ranges x slabs) up to one per compute unit
+      int best = least, best_wgs = 0;
+      for (int sp = least; sp <= least + 2 && sp <= uw; ++sp) {
+        int r = NUM_CU / sp;
+        if (r < 1) r = 1;
+        if (r > tiles) r = tiles;
+        const int wgs = sp * balanced_ranges(tiles, r);
+        if (wgs > best_wgs) {
+          best_wgs = wgs;
+          best = sp;
+        }
+      }
+      L.splits = best;
       L.nw = (uw + L.splits - 1) / L.splits;
       L.splits = (uw + L.nw - 1) / L.nw;
     }
