@@ -10,7 +10,6 @@ import math
 import torch
 
 from . import _lib, ops
-from .cache import KVCache
 
 MAXT = 32
 

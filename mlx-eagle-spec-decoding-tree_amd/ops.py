@@ -5,7 +5,6 @@ torch only supplies device memory and the current stream.  There is no eager
 or CPU fallback: every function raises if the library is missing or the tensor
 is not on a GPU.
 """
-import math
 from functools import reduce
 
 import torch

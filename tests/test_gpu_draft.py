@@ -7,7 +7,7 @@ import torch
 
 from mlx_eagle_spec_decoding_tree_amd import eagle, llama, ops, synth
 from mlx_eagle_spec_decoding_tree_amd.cache import make_prompt_cache
-from oracle import draft_oracle, model_oracle, oracle, tree_oracle
+from oracle import draft_oracle, oracle, tree_oracle
 from util import TOL, rel_err, to_dev
 
 pytestmark = pytest.mark.gpu
