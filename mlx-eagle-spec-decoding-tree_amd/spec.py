@@ -335,6 +335,10 @@ class SpeculativeDecoder:
         """mlx_eagle.py:522-535: both models read the prompt; the first token is the target's
         argmax at its last position."""
         self.prepare(prompt.numel())
+        for cache in (self.base_cache, self.draft_cache):     # a new sequence: empty caches
+            for c in cache:
+                c.offset = 0
+            cache[0].sync_len()
         self._prefill[0](prompt)
         first = ops.argmax_rows(self._prefill[1](prompt))
         self.y.zero_()

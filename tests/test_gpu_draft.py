@@ -297,6 +297,11 @@ def test_device_loop_equals_host_loop(dev, same, graph):
     assert more[:len(tokens)] == tokens and len(more) > len(tokens)
     want = greedy_reference(target, prompt, len(more) + 1, dev)
     assert [first] + more == want
+    # a new prompt starts from empty caches, with the graphs already captured
+    prompt2 = rng.integers(0, targs.vocab_size, 33).astype(np.int32)
+    first2 = dec.prefill(to_dev(prompt2.astype(np.int64), dev))
+    tokens2 = dec.generate(3)
+    assert [first2] + tokens2 == greedy_reference(target, prompt2, len(tokens2) + 1, dev)
 
 
 def test_device_loop_refuses_to_overrun_the_caches(dev):
