@@ -217,15 +217,20 @@ def test_generate_draft_tree_matches_oracle(dev, depth):
         assert rel_err(c.values[0, :, :P + k * depth].cpu().numpy(), ov[:, :P + k * depth]) <= 2 * TOL
 
 
-def greedy_reference(model, prompt, n, dev):
-    """Plain greedy decoding of the target, one token per pass."""
-    cache = make_prompt_cache(model, capacity=len(prompt) + n + 8)
-    logits = model(to_dev(prompt.astype(np.int64), dev)[None], cache=cache)
-    out = [int(logits[0, -1].float().argmax())]
-    for _ in range(n - 1):
-        logits = model(torch.tensor([[out[-1]]], dtype=torch.int64, device=dev), cache=cache)
-        out.append(int(logits[0, -1].float().argmax()))
-    return out
+def assert_greedy_stream(model, prompt, stream, dev, tol=0.06):
+    """Every token of `stream` is the target's argmax given the prompt and the tokens before it,
+    up to `tol` in logit units: the verification pass and a one-token pass round differently, so
+    at a near-tie they may pick different maxima (then both are valid greedy streams)."""
+    cache = make_prompt_cache(model, capacity=len(prompt) + len(stream) + 8)
+    logits = model(to_dev(prompt.astype(np.int64), dev)[None], cache=cache)[0, -1].float()
+    exact = 0
+    for i, tok in enumerate(stream):
+        deficit = float(logits.max() - logits[tok])
+        assert deficit <= tol, (i, tok, int(logits.argmax()), deficit)
+        exact += int(logits.argmax()) == tok
+        logits = model(torch.tensor([[tok]], dtype=torch.int64, device=dev), cache=cache)[0, -1].float()
+    assert exact >= len(stream) - 2      # near-ties are rare
+    return exact
 
 
 @pytest.mark.parametrize("same", [True, False])
@@ -239,8 +244,7 @@ def test_generate_step_stream_equals_target_greedy(dev, same):
                               verify_num_tokens=31, max_tokens=64, N=6)
     n = res["n"]
     assert n == len(res["tokens"]) == sum(1 + s[0] for s in res["steps"])
-    want = greedy_reference(target, prompt, n + 1, dev)
-    assert [res["first"]] + res["tokens"] == want
+    assert_greedy_stream(target, prompt, [res["first"]] + res["tokens"], dev)
     if same:
         assert res["mean_tokens_per_step"] >= 3.0
     for al, best, acc, y in res["steps"]:
@@ -286,22 +290,21 @@ def test_device_loop_equals_host_loop(dev, same, graph):
         dec.capture()
     tokens = dec.generate(N)
     assert first == host["first"]
-    want = greedy_reference(target, prompt, len(tokens) + 1, dev)
-    assert [first] + tokens == want
-    assert tokens == host["tokens"]
+    assert_greedy_stream(target, prompt, [first] + tokens, dev)
+    if tokens != host["tokens"]:          # only possible after a near-tie: then both are greedy streams
+        assert_greedy_stream(target, prompt, [host["first"]] + host["tokens"], dev)
     assert int(dec.verifier.len_dev.item()) == len(prompt) + len(tokens)
     if same:
         assert len(tokens) >= 3 * N
     # a second run continues the stream
     more = dec.generate(2)
     assert more[:len(tokens)] == tokens and len(more) > len(tokens)
-    want = greedy_reference(target, prompt, len(more) + 1, dev)
-    assert [first] + more == want
+    assert_greedy_stream(target, prompt, [first] + more, dev)
     # a new prompt starts from empty caches, with the graphs already captured
     prompt2 = rng.integers(0, targs.vocab_size, 33).astype(np.int32)
     first2 = dec.prefill(to_dev(prompt2.astype(np.int64), dev))
     tokens2 = dec.generate(3)
-    assert [first2] + tokens2 == greedy_reference(target, prompt2, len(tokens2) + 1, dev)
+    assert_greedy_stream(target, prompt2, [first2] + tokens2, dev)
 
 
 def test_device_loop_refuses_to_overrun_the_caches(dev):
@@ -348,3 +351,19 @@ def test_chunked_prompt_pass_matches_oracle(dev, n, chunk, graphs):
     got2 = pre(to_dev(more, dev)).cpu().numpy()
     assert cache[0].offset == n + 40
     assert rel_err(got2, want2[-1:]) <= 2 * TOL
+
+
+def test_device_loop_depth_five(dev):
+    """Depth 5: 40 expansion rows, so the draft attention uses both mask words."""
+    from mlx_eagle_spec_decoding_tree_amd import spec
+
+    (targs, tw, target), (dargs, dw, draft) = tiny_pair(dev, same=True, seed=21)
+    rng = np.random.default_rng(22)
+    prompt = rng.integers(0, targs.vocab_size, 50).astype(np.int32)
+    dec = spec.SpeculativeDecoder(target, draft, capacity=256, k=8, depth=5, verify_num_tokens=31)
+    first = dec.prefill(to_dev(prompt.astype(np.int64), dev))
+    dec.capture()
+    tokens = dec.generate(5)
+    (_, _, ref), _ = tiny_pair(dev, same=True, seed=21)
+    assert_greedy_stream(ref, prompt, [first] + tokens, dev)
+    assert len(tokens) >= 3 * 5                       # two drafted tokens and the bonus per step
