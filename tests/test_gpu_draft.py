@@ -367,3 +367,57 @@ def test_device_loop_depth_five(dev):
     (_, _, ref), _ = tiny_pair(dev, same=True, seed=21)
     assert_greedy_stream(ref, prompt, [first] + tokens, dev)
     assert len(tokens) >= 3 * 5                       # two drafted tokens and the bonus per step
+
+
+def test_draft_attention_random_shapes(dev):
+    """Seeded sweep over query counts, masked-row counts, prefix lengths and head layouts."""
+    rng = np.random.default_rng(2024)
+    for case in range(24):
+        hd = int(rng.choice([64, 128]))
+        G = int(rng.choice([1, 2, 4, 8]))
+        rep = int(rng.choice([1, 2, 4, 7, 8]))
+        H = G * rep
+        T = int(rng.integers(1, 33))
+        Tk = int(rng.integers(T, 65))
+        P = int(rng.choice([0, 1, 31, 32, 33, 63, 64, 65, 200, 517]))
+        cap = P + Tk + int(rng.integers(0, 40))
+        print(f"case {case}: H={H} G={G} hd={hd} T={T} Tk={Tk} P={P} cap={cap}", flush=True)
+        q = synth.make_x(rng, H, T, hd)
+        k = synth.make_x(rng, G, cap, hd)
+        v = synth.make_x(rng, G, cap, hd)
+        k[:, P + Tk:] = np.nan
+        v[:, P + Tk:] = np.nan
+        vis = rng.random((T, Tk)) < 0.5
+        vis[np.arange(T), Tk - T + np.arange(T)] = True
+        mask = np.concatenate([np.zeros((T, P), np.float16),
+                               np.where(vis, np.float16(0), np.float16(-np.inf))], axis=1)
+        want = oracle.tree_attention(q, k, v, mask, hd ** -0.5, S=P + Tk)
+        want_t = np.ascontiguousarray(want.transpose(1, 0, 2)).reshape(T, H * hd)
+        got = ops.draft_attention(to_dev(q, dev), to_dev(k, dev), to_dev(v, dev),
+                                  ops.mask_to_words(to_dev(vis, dev)),
+                                  torch.tensor([P], dtype=torch.int32, device=dev), Tk, hd ** -0.5,
+                                  max_len=cap).cpu().numpy()
+        assert np.isfinite(got.astype(np.float32)).all(), case
+        assert rel_err(got, want_t) <= TOL, case
+
+
+def test_causal_attention_pieces(dev):
+    """All 32-row pieces of a chunk in one launch pair against per-piece causal attention."""
+    rng = np.random.default_rng(77)
+    for (H, G, hd, P, R) in ((4, 2, 64, 0, 64), (14, 2, 64, 100, 96), (32, 8, 128, 37, 160), (8, 8, 128, 500, 32)):
+        print(f"chunk attention H={H} G={G} hd={hd} P={P} R={R}", flush=True)
+        cap = P + R + 5
+        q = synth.make_x(rng, H, R, hd)
+        k = synth.make_x(rng, G, cap, hd)
+        v = synth.make_x(rng, G, cap, hd)
+        k[:, P + R:] = np.nan
+        v[:, P + R:] = np.nan
+        mask = np.zeros((R, P + R), np.float16)
+        mask[:, P:] = np.where(np.tril(np.ones((R, R), bool)), np.float16(0), np.float16(-np.inf))
+        want = oracle.tree_attention(q, k, v, mask, hd ** -0.5, S=P + R)
+        want_t = np.ascontiguousarray(want.transpose(1, 0, 2)).reshape(R, H * hd)
+        piece_len = torch.tensor([P + 32 * j for j in range(R // 32)], dtype=torch.int32, device=dev)
+        got = ops.causal_attention(to_dev(q, dev), to_dev(k, dev), to_dev(v, dev), piece_len, hd ** -0.5,
+                                   max_len=cap).cpu().numpy()
+        assert np.isfinite(got.astype(np.float32)).all()
+        assert rel_err(got, want_t) <= TOL

@@ -51,3 +51,26 @@ def test_gemm_form_rejects_bad_shapes(dev):
     s = torch.zeros((64, 1), dtype=torch.float16, device=dev)
     with pytest.raises(ValueError):
         ops.quantized_matmul(x, w, s, s)
+
+
+def test_gemm_form_random_shapes(dev):
+    """Seeded sweep: ragged row counts, N down to one tile, K with and without the vector
+    scale loads (multiples of 512 or not), every block shape."""
+    rng = np.random.default_rng(99)
+    for case in range(14):
+        M = int(rng.integers(33, 700))
+        N = 8 * int(rng.integers(1, 700))
+        K = 64 * int(rng.integers(1, 40))
+        bias = bool(rng.integers(0, 2))
+        print(f"case {case}: M={M} N={N} K={K} bias={bias}", flush=True)
+        layer = synth.make_qlinear(rng, N, K, bias=bias)
+        x = synth.make_x(rng, M, K)
+        want = oracle.qmm(x, layer["weight"], layer["scales"], layer["biases"], layer.get("bias"))
+        d = layer_to_dev(layer, dev)
+        out = torch.full((M + 1, N), float("nan"), dtype=torch.float16, device=dev)
+        ops.quantized_matmul(to_dev(x, dev), d["weight"], d["scales"], d["biases"], bias=d.get("bias"),
+                             out=out[:M])
+        got = out.cpu().numpy()
+        assert np.isnan(got[M].astype(np.float32)).all(), case          # nothing written past the rows
+        assert np.isfinite(got[:M].astype(np.float32)).all(), case
+        assert rel_err(got[:M], want) <= TOL, case
