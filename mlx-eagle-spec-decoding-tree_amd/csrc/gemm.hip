@@ -63,11 +63,11 @@ struct StepIndex {
   static constexpr int value = E;
 };
 
-// SB8: K is a multiple of 512, so that scales and biases can be fetched eight groups (16 bytes)
-// at a time, one fetch per eight K steps, instead of one 2-byte load per row and step (the
-// loads of one instruction go to 32 or 64 different cache lines either way, and the rate of
-// such requests, not their bytes, is what the kernel runs up against).
-template <int NTW, int MT, bool SB8>
+// SBW = groups per fetch of scales and biases (1, 2, 4 or 8; K is a multiple of 64 * SBW): one
+// fetch per SBW K steps instead of one 2-byte load per row and step (the loads of one
+// instruction go to 32 or 64 different cache lines either way, and the rate of such requests,
+// not their bytes, is what the kernel runs up against).
+template <int NTW, int MT, int SBW>
 __global__ __launch_bounds__(256) void qmm_gemm_w4g64_kernel(
     const half_t* __restrict__ x, const uint32_t* __restrict__ w, const half_t* __restrict__ s,
     const half_t* __restrict__ b, const half_t* __restrict__ bias, half_t* __restrict__ out, int M,
@@ -106,8 +106,10 @@ __global__ __launch_bounds__(256) void qmm_gemm_w4g64_kernel(
 
   half8_t xreg[PP];                         // x of the next step
   uint4_t wreg[2][NTW];                     // packed weights, two steps in flight
-  half_t sreg[2][NTW], breg[2][NTW];        // !SB8: scale and bias of those steps
-  half8_t s8[2][NTW], b8[2][NTW];           // SB8: of this chunk of eight steps and of the next
+  constexpr bool SBV = SBW > 1;
+  typedef half_t sbvec_t __attribute__((ext_vector_type(SBV ? SBW : 2)));
+  half_t sreg[2][NTW], breg[2][NTW];        // SBW = 1: scale and bias of those steps
+  sbvec_t s8[2][NTW], b8[2][NTW];           // SBW > 1: of this chunk of SBW steps and of the next
   half8_t af[2][NTW][4];                    // expanded weights of this step and the next
   auto fetch_x = [&](int ks) {
 #pragma unroll
@@ -117,7 +119,7 @@ __global__ __launch_bounds__(256) void qmm_gemm_w4g64_kernel(
 #pragma unroll
     for (int nt = 0; nt < NTW; ++nt) {
       wreg[p][nt] = *reinterpret_cast<const uint4_t*>(w + (long)nrow[nt] * KW + ks * 8 + hb * 4);
-      if (!SB8) {
+      if (!SBV) {
         sreg[p][nt] = s[(long)nrow[nt] * KG + ks];
         breg[p][nt] = b[(long)nrow[nt] * KG + ks];
       }
@@ -126,8 +128,8 @@ __global__ __launch_bounds__(256) void qmm_gemm_w4g64_kernel(
   auto fetch_sb = [&](int chunk, int q) {
 #pragma unroll
     for (int nt = 0; nt < NTW; ++nt) {
-      s8[q][nt] = *reinterpret_cast<const half8_t*>(s + (long)nrow[nt] * KG + chunk * 8);
-      b8[q][nt] = *reinterpret_cast<const half8_t*>(b + (long)nrow[nt] * KG + chunk * 8);
+      s8[q][nt] = *reinterpret_cast<const sbvec_t*>(s + (long)nrow[nt] * KG + chunk * SBW);
+      b8[q][nt] = *reinterpret_cast<const sbvec_t*>(b + (long)nrow[nt] * KG + chunk * SBW);
     }
   };
   auto stash = [&](int buf) {
@@ -136,12 +138,12 @@ __global__ __launch_bounds__(256) void qmm_gemm_w4g64_kernel(
       *reinterpret_cast<half8_t*>(&xs[buf][xr * XS + xh * (BK / TPR) + g * 8]) = permute8(xreg[g]);
   };
   // word j of the weight tiles of register set p; e = index of their step within the chunk of
-  // eight (8 = first step of the next chunk)
+  // SBW (SBW = first step of the next chunk)
   auto expand = [&](int p, int j, int e) {
 #pragma unroll
     for (int nt = 0; nt < NTW; ++nt) {
-      const half_t sc = SB8 ? s8[e >> 3][nt][e & 7] : sreg[p][nt];
-      const half_t bi = SB8 ? b8[e >> 3][nt][e & 7] : breg[p][nt];
+      const half_t sc = SBV ? s8[e / SBW][nt][e % SBW] : sreg[p][nt];
+      const half_t bi = SBV ? b8[e / SBW][nt][e % SBW] : breg[p][nt];
       const half_t b16 = (half_t)((float)bi - 16.f * (float)sc);
       af[p][nt][j] = dequant_word(wreg[p][nt][j], half2_t{sc, sc}, half2_t{b16, b16});
     }
@@ -155,11 +157,11 @@ __global__ __launch_bounds__(256) void qmm_gemm_w4g64_kernel(
 #pragma unroll
       for (int i = 0; i < 16; ++i) acc[nt][mt][i] = 0.f;
 
-  const int chunks = steps >> 3;
+  const int chunks = steps / SBW;
   fetch_x(0);
   fetch_w(0, 0);
   fetch_w(steps > 1 ? 1 : 0, 1);
-  if (SB8) {
+  if (SBV) {
     fetch_sb(0, 0);
     fetch_sb(chunks > 1 ? 1 : 0, 1);
   }
@@ -175,7 +177,7 @@ __global__ __launch_bounds__(256) void qmm_gemm_w4g64_kernel(
   // wait for the load), and the loads are issued first (left alone, the scheduler sinks them
   // to the end of the step, where the in-order counter waits for them at once).
   auto body = [&](int ks, auto E) {
-    constexpr int e = decltype(E)::value;   // step within its chunk (SB8) / parity of the step
+    constexpr int e = decltype(E)::value;   // step within its chunk (SBW > 1) / parity of the step
     constexpr int p = e & 1;
     fetch_x(ks + 1 < steps ? ks + 1 : steps - 1);
     fetch_w(ks + 2 < steps ? ks + 2 : steps - 1, p);
@@ -195,19 +197,19 @@ __global__ __launch_bounds__(256) void qmm_gemm_w4g64_kernel(
     }
     __builtin_amdgcn_sched_barrier(0);
     stash(p ^ 1);
-    if (SB8 && e == 7) {
-      // the next chunk becomes the current one (its loads were issued eight steps ago)
+    if (SBV && e == SBW - 1) {
+      // the next chunk becomes the current one (its loads were issued SBW steps ago)
 #pragma unroll
       for (int nt = 0; nt < NTW; ++nt) {
         s8[0][nt] = s8[1][nt];
         b8[0][nt] = b8[1][nt];
       }
-      const int c = (ks >> 3) + 2;
+      const int c = ks / SBW + 2;
       fetch_sb(c < chunks ? c : chunks - 1, 1);
     }
     __syncthreads();
   };
-  if (SB8) {
+  if constexpr (SBW == 8) {
     for (int ks = 0; ks < steps; ks += 8) {
       body(ks, StepIndex<0>{});
       body(ks + 1, StepIndex<1>{});
@@ -217,6 +219,18 @@ __global__ __launch_bounds__(256) void qmm_gemm_w4g64_kernel(
       body(ks + 5, StepIndex<5>{});
       body(ks + 6, StepIndex<6>{});
       body(ks + 7, StepIndex<7>{});
+    }
+  } else if constexpr (SBW == 4) {
+    for (int ks = 0; ks < steps; ks += 4) {
+      body(ks, StepIndex<0>{});
+      body(ks + 1, StepIndex<1>{});
+      body(ks + 2, StepIndex<2>{});
+      body(ks + 3, StepIndex<3>{});
+    }
+  } else if constexpr (SBW == 2) {
+    for (int ks = 0; ks < steps; ks += 2) {
+      body(ks, StepIndex<0>{});
+      body(ks + 1, StepIndex<1>{});
     }
   } else {
     int ks = 0;
@@ -248,7 +262,7 @@ __global__ __launch_bounds__(256) void qmm_gemm_w4g64_kernel(
   }
 }
 
-template <int NTW, int MT, bool SB8>
+template <int NTW, int MT, int SBW>
 int launch_gemm(const half_t* x, const uint32_t* w, const half_t* s, const half_t* b, const half_t* bias,
                 half_t* out, int M, int N, int K, hipStream_t st) {
   constexpr int BMT = 32 * MT;
@@ -257,13 +271,13 @@ int launch_gemm(const half_t* x, const uint32_t* w, const half_t* s, const half_
   const size_t lds = 2 * (size_t)BMT * XS * sizeof(half_t);
   static bool configured = false;
   if (!configured) {
-    if (hipFuncSetAttribute(reinterpret_cast<const void*>(&qmm_gemm_w4g64_kernel<NTW, MT, SB8>),
+    if (hipFuncSetAttribute(reinterpret_cast<const void*>(&qmm_gemm_w4g64_kernel<NTW, MT, SBW>),
                             hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds) != hipSuccess)
       return EAGLE_ERR_HIP;
     configured = true;
   }
   const dim3 grid((N + BN - 1) / BN, (M + BMT - 1) / BMT);
-  hipLaunchKernelGGL((qmm_gemm_w4g64_kernel<NTW, MT, SB8>), grid, dim3(256), lds, st, x, w, s, b, bias, out, M, N, K);
+  hipLaunchKernelGGL((qmm_gemm_w4g64_kernel<NTW, MT, SBW>), grid, dim3(256), lds, st, x, w, s, b, bias, out, M, N, K);
   return eagle_launch_status();
 }
 
@@ -295,15 +309,22 @@ EAGLE_EXPORT int eagle_qmm_gemm_w4g64_f16(const void* x, const uint32_t* wq, con
   const double cost_big = 1.85 * most(((N + 255) / 256) * (long)((M + 127) / 128));
   const bool small = cost_small < cost_norm && cost_small <= cost_big;
   const bool big = !small && cost_big < cost_norm;
-  const bool sb8 = (K % 512) == 0 && eagle_aligned16(scales) && eagle_aligned16(biases);
-  if (small) {
-    if (sb8) return launch_gemm<1, 2, true>(xh, wq, sh, bh, bi, oh, M, N, K, st);
-    return launch_gemm<1, 2, false>(xh, wq, sh, bh, bi, oh, M, N, K, st);
+  // scales and biases per fetch: as many groups as divide a row and as the base addresses are
+  // aligned for
+  const uintptr_t sb_addr = reinterpret_cast<uintptr_t>(scales) | reinterpret_cast<uintptr_t>(biases);
+  const int sbw = (K % 512) == 0 && (sb_addr & 15u) == 0 ? 8
+                : (K % 256) == 0 && (sb_addr & 7u) == 0  ? 4
+                : (K % 128) == 0 && (sb_addr & 3u) == 0  ? 2
+                                                         : 1;
+#define EAGLE_GEMM_SHAPE(NTW, MT)                                                              \
+  switch (sbw) {                                                                               \
+    case 8: return launch_gemm<NTW, MT, 8>(xh, wq, sh, bh, bi, oh, M, N, K, st);               \
+    case 4: return launch_gemm<NTW, MT, 4>(xh, wq, sh, bh, bi, oh, M, N, K, st);               \
+    case 2: return launch_gemm<NTW, MT, 2>(xh, wq, sh, bh, bi, oh, M, N, K, st);               \
+    default: return launch_gemm<NTW, MT, 1>(xh, wq, sh, bh, bi, oh, M, N, K, st);              \
   }
-  if (big) {
-    if (sb8) return launch_gemm<2, 4, true>(xh, wq, sh, bh, bi, oh, M, N, K, st);
-    return launch_gemm<2, 4, false>(xh, wq, sh, bh, bi, oh, M, N, K, st);
-  }
-  if (sb8) return launch_gemm<1, 4, true>(xh, wq, sh, bh, bi, oh, M, N, K, st);
-  return launch_gemm<1, 4, false>(xh, wq, sh, bh, bi, oh, M, N, K, st);
+  if (small) { EAGLE_GEMM_SHAPE(1, 2) }
+  if (big) { EAGLE_GEMM_SHAPE(2, 4) }
+  EAGLE_GEMM_SHAPE(1, 4)
+#undef EAGLE_GEMM_SHAPE
 }
