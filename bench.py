@@ -86,6 +86,9 @@ def main():
     ap.add_argument("--warmup", type=int, default=5)
     ap.add_argument("--seed", type=int, default=1234)
     ap.add_argument("--no-cpu", action="store_true", help="skip the CPU baseline / full-size parity leg")
+    ap.add_argument("--slabs", default=None,
+                    help="force the slab form of the matmul: e.g. qkv=8,o=8,down=32 (K steps per slab; "
+                         "'' = streaming kernel everywhere; default: the library's choice)")
     ap.add_argument("--sweep", action="store_true", help="also print the per-shape QMM table to stderr")
     ap.add_argument("--calibrate-copy", action="store_true",
                     help="before anything else run one 1 GiB device copy (a kernel of known traffic: "
@@ -147,7 +150,10 @@ def main():
     depth, anc, bits = synth.tree_arrays(parents)
     tokens = rng.integers(0, args.vocab_size, NODES).astype(np.int32)
 
-    ver = eagle.TreeVerifier(model, cache, total_tokens=NODES - 1, max_len=cap)
+    slab_plan = None
+    if opt.slabs is not None:
+        slab_plan = {kv.split("=")[0]: int(kv.split("=")[1]) for kv in opt.slabs.split(",") if kv}
+    ver = eagle.TreeVerifier(model, cache, total_tokens=NODES - 1, max_len=cap, slab_plan=slab_plan)
     ver.set_tree(torch.from_numpy(tokens).to(dev), torch.from_numpy(depth.astype(np.int32)).to(dev),
                  torch.from_numpy(parents).to(dev),
                  torch.from_numpy(bits.view(np.int32)).to(dev))
@@ -182,9 +188,11 @@ def main():
     ver.act.normal_()
 
     def qmm_only():
-        for wq, sc, bi, bias, x, out, swiglu in launches:
-            if swiglu:
+        for wq, sc, bi, bias, x, out, form in launches:
+            if form is True:
                 ops.quantized_matmul_swiglu(x, wq, sc, bi, bias=bias, out=out)
+            elif form:
+                ops.quantized_matmul_slabs(x, wq, sc, bi, form, partial=ver.partial)
             else:
                 ops.quantized_matmul(x, wq, sc, bi, bias=bias, out=out)
 

@@ -99,6 +99,30 @@ int eagle_qmm_gemm_w4g64_f16(const void* x, const uint32_t* wq, const void* scal
                              const void* biases, const void* bias, void* out, int M, int N, int K,
                              int group_size, int bits, eagle_stream_t stream);
 
+/* The same product for 1..32 rows in the slab form, with the result left as fp32 partial sums:
+ * every workgroup owns 128 weight rows and one K slab of `steps_per_slab` quantisation groups
+ * (8, 16, 24 or 32), holds its x slab in LDS and expands the weights to fp16 in registers for
+ * v_mfma_f32_32x32x16_f16.  partial [slabs][32][N] fp32 (rows >= M are not written),
+ * slabs = eagle_qmm_slab_count(K, steps_per_slab) (0 for a shape the form does not take:
+ * K % 512 == 0 is required, scales and biases 16-byte aligned).  The product is
+ * fp16(sum over the slabs, in slab order) (+ fp16 bias): the kernel that consumes it adds the
+ * slabs while it loads (eagle_rmsnorm_slabs_f16, eagle_rope_kv_append_slabs_f16), or
+ * eagle_slab_sum_f16 writes it out.  No counters, no workspace.  For the small projections of
+ * a verification step this is about twice as fast as a kernel that reduces its own slabs.
+ * Replaces the same mx.quantized_matmul call sites (mlx_model_fwd_bench.py:65-73). */
+int eagle_qmm_slab_count(int K, int steps_per_slab);
+/* K steps per slab recommended for this product, 0 where eagle_qmm_w4g64_f16 is the faster form
+ * (few rows, very many weight rows, or K not a multiple of 512). */
+int eagle_qmm_slab_steps(int M, int N, int K);
+size_t eagle_qmm_slab_partial_bytes(int N, int K, int steps_per_slab);
+int eagle_qmm_slab_partial_w4g64(const void* x, const uint32_t* wq, const void* scales,
+                                 const void* biases, float* partial, size_t partial_bytes,
+                                 int M, int N, int K, int group_size, int bits,
+                                 int steps_per_slab, eagle_stream_t stream);
+/* out [M,N] fp16 = fp16(sum of the slabs) (+ bias [N] fp16, 16-byte aligned, may be NULL). */
+int eagle_slab_sum_f16(const float* partial, int slabs, const void* bias, void* out, int M, int N,
+                       eagle_stream_t stream);
+
 /* Quantised embedding gather: out[t,:] = fp16(scales*q + biases) of row ids[t].
  * ids [T] int32, out [T,D] fp16, D % 64 == 0.  Replaces the quantised
  * nn.Embedding lookup of mlx_llama.py:273. */
@@ -152,6 +176,10 @@ int eagle_tree_attention_f16(const void* q, const void* k_cache, const void* v_c
  * (the residual adds of mlx_llama.py:246,248 fused with the following norm). */
 int eagle_rmsnorm_f16(const void* x, const void* residual, const void* w, float eps,
                       void* h_out, void* out, int T, int D, eagle_stream_t stream);
+/* The same with x held as fp32 partial sums of K slabs (eagle_qmm_slab_partial_w4g64 with
+ * N = D): x = fp16(sum of the slabs).  T <= 32. */
+int eagle_rmsnorm_slabs_f16(const float* partial, int slabs, const void* residual, const void* w,
+                            float eps, void* h_out, void* out, int T, int D, eagle_stream_t stream);
 
 /* out = fp16( fp16(silu(g)) * u ); g, u are the two halves of gate_up [T,2*I]
  * when `up` is NULL (g = gate_up[:, :I], u = gate_up[:, I:]) or separate [T,I]
@@ -170,6 +198,14 @@ int eagle_rope_kv_append_table_f16(const void* q_lin, const void* k_lin, const v
                                    const float* rope_cs, void* q_out, void* k_cache, void* v_cache,
                                    const int32_t* cache_len_dev, int T, int H, int G, int hd,
                                    long capacity, long row_stride, eagle_stream_t stream);
+/* The same with the fused q|k|v projection held as fp32 partial sums of K slabs
+ * (eagle_qmm_slab_partial_w4g64 with N = (H + 2G) hd, rows [q heads | k heads | v heads]):
+ * every value is fp16(sum of the slabs) + bias (bias [N] fp16, 16-byte aligned, may be NULL)
+ * before the rotation.  T <= 32. */
+int eagle_rope_kv_append_slabs_f16(const float* partial, int slabs, const void* bias,
+                                   const float* rope_cs, void* q_out, void* k_cache, void* v_cache,
+                                   const int32_t* cache_len_dev, int T, int H, int G, int hd,
+                                   long capacity, eagle_stream_t stream);
 
 /* cos/sin table for eagle_rope_kv_append_table_f16 and eagle_tree_attention_rope_f16: out[t][i] = (cos, sin)(positions[t] *
  * scaling_factor * inv_freqs[i]), fp32 [T, half_dim, 2]; the same angles as

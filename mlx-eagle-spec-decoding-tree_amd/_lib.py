@@ -26,6 +26,15 @@ SIGNATURES = {
     "eagle_qmm_workspace_bytes_tuned": (c_size_t, [c_int] * 3),
     "eagle_qmm_w4g64_f16_tuned": (c_int, [c_void_p] * 6 + [c_int] * 8 + [c_void_p, c_size_t, c_void_p]),
     "eagle_qmm_gemm_w4g64_f16": (c_int, [c_void_p] * 6 + [c_int] * 5 + [c_void_p]),
+    "eagle_qmm_slab_count": (c_int, [c_int] * 2),
+    "eagle_qmm_slab_steps": (c_int, [c_int] * 3),
+    "eagle_qmm_slab_partial_bytes": (c_size_t, [c_int] * 3),
+    "eagle_qmm_slab_partial_w4g64": (c_int, [c_void_p] * 5 + [c_size_t] + [c_int] * 6 + [c_void_p]),
+    "eagle_slab_sum_f16": (c_int, [c_void_p, c_int, c_void_p, c_void_p, c_int, c_int, c_void_p]),
+    "eagle_rmsnorm_slabs_f16": (c_int, [c_void_p, c_int, c_void_p, c_void_p, c_float, c_void_p, c_void_p,
+                                        c_int, c_int, c_void_p]),
+    "eagle_rope_kv_append_slabs_f16": (c_int, [c_void_p, c_int] + [c_void_p] * 6 + [c_int] * 4
+                                       + [c_long, c_void_p]),
     "eagle_embed_w4g64_f16": (c_int, [c_void_p] * 5 + [c_int] * 3 + [c_void_p]),
     "eagle_rope_arrayed_f16": (c_int, [c_void_p] * 3 + [c_float, c_void_p] + [c_int] * 4 + [c_void_p]),
     "eagle_rope_kv_append_f16": (c_int, [c_void_p] * 5 + [c_float] + [c_void_p] * 4 + [c_int] * 4

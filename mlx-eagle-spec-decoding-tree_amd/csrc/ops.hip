@@ -136,6 +136,92 @@ __global__ void rope_kv_append_kernel(const half_t* __restrict__ q_lin,
   }
 }
 
+// The same with the fused q|k|v projection held as fp32 partial sums of nslab K slabs,
+// [slab][32][(H + 2G) hd] with a row = [q heads | k heads | v heads]: every value is
+// fp16(sum of the slabs) + bias before the rotation.  One thread per four column pairs
+// (half of the work of a thread above, twice the threads: all its slab loads are in flight
+// together and the launch is a few dozen workgroups either way).
+__global__ void rope_kv_append_slabs_kernel(const float* __restrict__ partial, int nslab,
+                                            const half_t* __restrict__ bias,
+                                            const float* __restrict__ rope_cs,
+                                            half_t* __restrict__ q_out, half_t* __restrict__ k_cache,
+                                            half_t* __restrict__ v_cache,
+                                            const int32_t* __restrict__ len_dev, int T, int H, int G,
+                                            int hd, long cap) {
+  const int half = hd >> 1;
+  const int per_row = half >> 2;
+  const int heads = H + 2 * G;
+  const long total = (long)T * heads * per_row;
+  const long idx = (long)blockIdx.x * blockDim.x + threadIdx.x;
+  if (idx >= total) return;
+  const int c = (int)(idx % per_row) * 4;
+  const int hh = (int)((idx / per_row) % heads);
+  const int t = (int)(idx / ((long)per_row * heads));
+  const size_t ld = (size_t)heads * hd;
+  const size_t stride = 32 * ld;
+  const float* p = partial + (size_t)t * ld + (size_t)hh * hd + c;
+  // cos / sin and the bias are requested with the slabs
+  float4_t cs0 = float4_t{0.f, 0.f, 0.f, 0.f}, cs1 = cs0;
+  if (hh < H + G) {
+    const float4_t* cs = reinterpret_cast<const float4_t*>(rope_cs + ((long)t * half + c) * 2);
+    cs0 = cs[0];
+    cs1 = cs[1];
+  }
+  half4_t blo = half4_t{0, 0, 0, 0}, bhi = blo;
+  if (bias) {
+    blo = *reinterpret_cast<const half4_t*>(bias + (size_t)hh * hd + c);
+    bhi = *reinterpret_cast<const half4_t*>(bias + (size_t)hh * hd + half + c);
+  }
+  float4_t lo = float4_t{0.f, 0.f, 0.f, 0.f}, hi = lo;
+  for (int z = 0; z < nslab; z += 8) {
+    float4_t a[8], b[8];
+#pragma unroll
+    for (int k = 0; k < 8; ++k) {
+      const int zz = z + k < nslab ? z + k : nslab - 1;
+      a[k] = *reinterpret_cast<const float4_t*>(p + (size_t)zz * stride);
+      b[k] = *reinterpret_cast<const float4_t*>(p + (size_t)zz * stride + half);
+    }
+#pragma unroll
+    for (int k = 0; k < 8; ++k)
+      if (z + k < nslab) {
+        lo += a[k];
+        hi += b[k];
+      }
+  }
+  half4_t xlo, xhi;
+#pragma unroll
+  for (int j = 0; j < 4; ++j) {
+    xlo[j] = (half_t)lo[j];
+    xhi[j] = (half_t)hi[j];
+  }
+  if (bias) {
+    xlo += blo;
+    xhi += bhi;
+  }
+  const long P = *len_dev;
+  if (P + t >= cap) return;   // host checks capacity; never write past the buffer
+  if (hh < H + G) {
+    const bool is_q = hh < H;
+    const int head = is_q ? hh : hh - H;
+    half_t* dst = is_q ? q_out + ((long)head * T + t) * hd : k_cache + ((long)head * cap + P + t) * hd;
+    half4_t olo, ohi;
+#pragma unroll
+    for (int j = 0; j < 4; ++j) {
+      const float co = j < 2 ? cs0[2 * j] : cs1[2 * (j - 2)];
+      const float sn = j < 2 ? cs0[2 * j + 1] : cs1[2 * (j - 2) + 1];
+      const float x1 = (float)xlo[j], x2 = (float)xhi[j];
+      olo[j] = (half_t)__builtin_fmaf(x1, co, -(x2 * sn));
+      ohi[j] = (half_t)__builtin_fmaf(x1, sn, x2 * co);
+    }
+    *reinterpret_cast<half4_t*>(dst + c) = olo;
+    *reinterpret_cast<half4_t*>(dst + half + c) = ohi;
+  } else {
+    half_t* dst = v_cache + ((long)(hh - H - G) * cap + P + t) * hd;
+    *reinterpret_cast<half4_t*>(dst + c) = xlo;
+    *reinterpret_cast<half4_t*>(dst + half + c) = xhi;
+  }
+}
+
 // ------------------------------------------------------------------------------------
 // RMSNorm with optional residual add; one 256-thread workgroup per row, the row stays
 // in registers between the two passes.  D % 8 == 0, D <= 256 * 8 * RMS_MAXV.
@@ -149,7 +235,9 @@ __global__ __launch_bounds__(BLOCK) void rmsnorm_kernel(const half_t* __restrict
                                                         const half_t* __restrict__ res,
                                                         const half_t* __restrict__ w, float eps,
                                                         half_t* __restrict__ h_out,
-                                                        half_t* __restrict__ out, int D) {
+                                                        half_t* __restrict__ out, int D,
+                                                        const float* __restrict__ partial, int nslab) {
+  // partial != nullptr: x is held as fp32 partial sums of nslab K slabs, [slab][32][D]
   constexpr int NV = 256 * RMS_MAXV / BLOCK;     // vectors per thread
   __shared__ float red[BLOCK / 64];
   const int t = blockIdx.x;
@@ -161,10 +249,15 @@ __global__ __launch_bounds__(BLOCK) void rmsnorm_kernel(const half_t* __restrict
   for (int i = 0; i < NV; ++i) {
     const int c = threadIdx.x + i * BLOCK;
     if (c < nvec) {
-      half8_t a = *reinterpret_cast<const half8_t*>(xr + c * 8);
       w8[i] = *reinterpret_cast<const half8_t*>(w + c * 8);
+      half8_t r8;
+      if (res) r8 = *reinterpret_cast<const half8_t*>(res + (long)t * D + c * 8);
+      half8_t a;
+      if (partial)
+        a = eagle_slab_sum8(partial, nslab, (size_t)32 * D, (size_t)t * D + c * 8, nullptr);
+      else
+        a = *reinterpret_cast<const half8_t*>(xr + c * 8);
       if (res) {
-        const half8_t r8 = *reinterpret_cast<const half8_t*>(res + (long)t * D + c * 8);
 #pragma unroll
         for (int j = 0; j < 8; ++j) a[j] = (half_t)((float)a[j] + (float)r8[j]);
         *reinterpret_cast<half8_t*>(h_out + (long)t * D + c * 8) = a;
@@ -390,6 +483,26 @@ EAGLE_EXPORT int eagle_rope_kv_append_table_f16(const void* q_lin, const void* k
   return eagle_launch_status();
 }
 
+EAGLE_EXPORT int eagle_rope_kv_append_slabs_f16(const float* partial, int slabs, const void* bias,
+                                                const float* rope_cs, void* q_out, void* k_cache,
+                                                void* v_cache, const int32_t* cache_len_dev, int T,
+                                                int H, int G, int hd, long capacity,
+                                                eagle_stream_t stream) {
+  if (!partial || !rope_cs || !q_out || !k_cache || !v_cache || !cache_len_dev) return EAGLE_ERR_NULL;
+  if (slabs < 1 || T < 1 || T > 32 || H < 1 || G < 1 || (H % G) != 0 || hd < 16 || (hd % 16) != 0 ||
+      capacity < T)
+    return EAGLE_ERR_SHAPE;
+  if (!eagle_aligned16(partial) || !eagle_aligned16(rope_cs) || !eagle_aligned16(q_out) ||
+      !eagle_aligned16(k_cache) || !eagle_aligned16(v_cache) || (bias && !eagle_aligned16(bias)))
+    return EAGLE_ERR_ALIGN;
+  const long total = (long)T * (H + 2 * G) * (hd / 8);
+  hipLaunchKernelGGL(rope_kv_append_slabs_kernel, dim3(blocks_for(total, 256)), dim3(256), 0,
+                     static_cast<hipStream_t>(stream), partial, slabs, (const half_t*)bias, rope_cs,
+                     (half_t*)q_out, (half_t*)k_cache, (half_t*)v_cache, cache_len_dev, T, H, G, hd,
+                     capacity);
+  return eagle_launch_status();
+}
+
 EAGLE_EXPORT int eagle_rmsnorm_f16(const void* x, const void* residual, const void* w, float eps,
                                    void* h_out, void* out, int T, int D, eagle_stream_t stream) {
   if (!x || !w || !out || (residual && !h_out)) return EAGLE_ERR_NULL;
@@ -400,11 +513,30 @@ EAGLE_EXPORT int eagle_rmsnorm_f16(const void* x, const void* residual, const vo
   if (D > 256 * 8)   // one vector per thread while the row is short enough
     hipLaunchKernelGGL(rmsnorm_kernel<512>, dim3(T), dim3(512), 0, static_cast<hipStream_t>(stream),
                        (const half_t*)x, (const half_t*)residual, (const half_t*)w, eps,
-                       (half_t*)h_out, (half_t*)out, D);
+                       (half_t*)h_out, (half_t*)out, D, (const float*)nullptr, 0);
   else
     hipLaunchKernelGGL(rmsnorm_kernel<256>, dim3(T), dim3(256), 0, static_cast<hipStream_t>(stream),
                        (const half_t*)x, (const half_t*)residual, (const half_t*)w, eps,
-                       (half_t*)h_out, (half_t*)out, D);
+                       (half_t*)h_out, (half_t*)out, D, (const float*)nullptr, 0);
+  return eagle_launch_status();
+}
+
+EAGLE_EXPORT int eagle_rmsnorm_slabs_f16(const float* partial, int slabs, const void* residual,
+                                         const void* w, float eps, void* h_out, void* out, int T, int D,
+                                         eagle_stream_t stream) {
+  if (!partial || !w || !out || (residual && !h_out)) return EAGLE_ERR_NULL;
+  if (slabs < 1 || T < 1 || T > 32 || D < 8 || (D % 8) != 0 || D > 256 * 8 * RMS_MAXV) return EAGLE_ERR_SHAPE;
+  if (!eagle_aligned16(partial) || !eagle_aligned16(w) || !eagle_aligned16(out) ||
+      (residual && (!eagle_aligned16(residual) || !eagle_aligned16(h_out))))
+    return EAGLE_ERR_ALIGN;
+  if (D > 256 * 8)
+    hipLaunchKernelGGL(rmsnorm_kernel<512>, dim3(T), dim3(512), 0, static_cast<hipStream_t>(stream),
+                       (const half_t*)nullptr, (const half_t*)residual, (const half_t*)w, eps,
+                       (half_t*)h_out, (half_t*)out, D, partial, slabs);
+  else
+    hipLaunchKernelGGL(rmsnorm_kernel<256>, dim3(T), dim3(256), 0, static_cast<hipStream_t>(stream),
+                       (const half_t*)nullptr, (const half_t*)residual, (const half_t*)w, eps,
+                       (half_t*)h_out, (half_t*)out, D, partial, slabs);
   return eagle_launch_status();
 }
 

@@ -389,7 +389,10 @@ class TreeVerifier:
     Same kernels and operator order as Model.__call__ + the host functions above."""
 
     def __init__(self, model, cache, total_tokens=31, max_len=None, compact=True, fuse=True,
-                 swiglu=True, one_launch_attention=False):
+                 swiglu=True, one_launch_attention=False, slab_plan=None):
+        """slab_plan: {"qkv": s, "o": s, "down": s}, K steps per slab for the projections that go
+        through the slab form of the matmul (their consumer adds the slabs), 0 for the
+        streaming kernel; None: the library's choice for this shape."""
         args = model.args
         self.model, self.cache, self.args = model, cache, args
         self.V = total_tokens
@@ -409,6 +412,7 @@ class TreeVerifier:
         self.one_launch_attention = bool(fuse and one_launch_attention)
         if fuse:
             self._fuse_projections()
+        self.slab = self._slab_plan(slab_plan)
         i32 = dict(dtype=torch.int32, device=dev)
         f16 = dict(dtype=torch.float16, device=dev)
         self.tokens = torch.zeros(T, **i32)
@@ -438,6 +442,10 @@ class TreeVerifier:
         self.act = torch.empty((T, I), **f16)
         self.down = torch.empty((T, D), **f16)
         self.logits = torch.empty((T, args.vocab_size), **f16)
+        need = max([1] + [ops.slab_count(k, self.slab[name]) * 32 * n
+                          for name, n, k in (("qkv", (H + 2 * G) * hd, D), ("o", D, H * hd), ("down", D, I))
+                          if self.slab[name]])
+        self.partial = torch.empty(need, dtype=torch.float32, device=dev)
         self.len_dev = cache[0].len_dev
         self.cache_ptrs = torch.tensor([c.keys.data_ptr() for c in cache]
                                        + [c.values.data_ptr() for c in cache],
@@ -457,20 +465,44 @@ class TreeVerifier:
     def _fuse_projections(self):
         self.qkv_w, self.gu_w = fuse_projections(self.model, self.swiglu)
 
+    def _slab_plan(self, forced):
+        """K steps per slab for q|k|v, o and down (0: streaming kernel).  The slab form needs
+        the fused step (its consumers are the table-driven rope kernel and the norm with the
+        residual), K % 512 == 0, and projections without a bias for o and down."""
+        args = self.args
+        D, I = args.hidden_size, args.intermediate_size
+        H, G, hd = args.num_attention_heads, args.num_key_value_heads, args.head_dim
+        layer = self.model.model.layers[0]
+        shapes = {"qkv": ((H + 2 * G) * hd, D), "o": (D, H * hd), "down": (D, I)}
+        plan = {}
+        for name, (n, k) in shapes.items():
+            s = ops.slab_steps(self.T, n, k) if forced is None else int(forced.get(name, 0))
+            ok = self.fuse and s > 0 and ops.slab_count(k, s) > 0
+            if name == "qkv":
+                ok = ok and not self.one_launch_attention
+            if name == "o":
+                ok = ok and layer.self_attn.o_proj.bias is None
+            if name == "down":
+                ok = ok and layer.mlp.down_proj.bias is None
+            plan[name] = s if ok else 0
+        return plan
+
     def qmm_launches(self):
-        """(weight, scales, biases, bias, x, out, swiglu) of every quantised matmul of one step,
-        in order; `swiglu` marks the launches that go through `quantized_matmul_swiglu`."""
+        """(weight, scales, biases, bias, x, out, form) of every quantised matmul of one step,
+        in order; `form` is True for the launches that go through `quantized_matmul_swiglu`,
+        the K steps per slab for those that go through `quantized_matmul_slabs` (into
+        `self.partial`), False for `quantized_matmul`."""
         m = self.model
         out = []
         for i, layer in enumerate(m.model.layers):
             at, mlp = layer.self_attn, layer.mlp
             if self.fuse:
-                out.append((*self.qkv_w[i], self.hn, self.qkv, False))
+                out.append((*self.qkv_w[i], self.hn, self.qkv, self.slab["qkv"] or False))
             else:
                 for lin, o in ((at.q_proj, self.q), (at.k_proj, self.k), (at.v_proj, self.v)):
                     out.append((lin.weight, lin.scales, lin.biases, lin.bias, self.hn, o, False))
             out.append((at.o_proj.weight, at.o_proj.scales, at.o_proj.biases, at.o_proj.bias,
-                        self.attn, self.o, False))
+                        self.attn, self.o, self.slab["o"] or False))
             if self.fuse:
                 out.append((*self.gu_w[i], self.hn, self.act if self.swiglu else self.gate_up,
                             self.swiglu))
@@ -478,7 +510,7 @@ class TreeVerifier:
                 for lin, o in ((mlp.gate_proj, self.gate), (mlp.up_proj, self.up)):
                     out.append((lin.weight, lin.scales, lin.biases, lin.bias, self.hn, o, False))
             out.append((mlp.down_proj.weight, mlp.down_proj.scales, mlp.down_proj.biases,
-                        mlp.down_proj.bias, self.act, self.down, False))
+                        mlp.down_proj.bias, self.act, self.down, self.slab["down"] or False))
         head = m.model.embed_tokens if self.args.tie_word_embeddings else m.lm_head
         out.append((head.weight, head.scales, head.biases, None, self.hn, self.logits, False))
         return out
@@ -513,14 +545,21 @@ class TreeVerifier:
             c = self.cache[i]
             if self.fuse:
                 w, sc, bi, b = self.qkv_w[i]
-                ops.quantized_matmul(self.hn, w, sc, bi, bias=b, out=self.qkv)
                 q_lin, k_lin, v_lin = self.qkv, self.qkv[:, H * hd:], self.qkv[:, (H + G) * hd:]
-                if self.one_launch_attention:
+                if self.slab["qkv"]:
+                    s = self.slab["qkv"]
+                    ops.quantized_matmul_slabs(self.hn, w, sc, bi, s, partial=self.partial)
+                    ops.rope_kv_append_slabs(self.partial, ops.slab_count(args.hidden_size, s), b,
+                                             self.rope_cs, self.q_rot, c.keys[0], c.values[0],
+                                             self.len_dev, T, H, G, hd)
+                elif self.one_launch_attention:
+                    ops.quantized_matmul(self.hn, w, sc, bi, bias=b, out=self.qkv)
                     ops.tree_attention_rope(q_lin, k_lin, v_lin, self.rope_cs, c.keys[0], c.values[0],
                                             self.mask_bits, self.len_dev, at.scale, H, G, hd,
                                             row_stride=(H + 2 * G) * hd, max_len=self.max_len,
                                             out=self.attn)
                 else:
+                    ops.quantized_matmul(self.hn, w, sc, bi, bias=b, out=self.qkv)
                     ops.rope_kv_append(q_lin, k_lin, v_lin, self.positions, at._inv_freqs,
                                        at._scaling_factor, self.q_rot, c.keys[0], c.values[0],
                                        self.len_dev, H, G, hd, row_stride=(H + 2 * G) * hd,
@@ -534,10 +573,18 @@ class TreeVerifier:
             if not self.one_launch_attention:
                 ops.tree_attention(self.q_rot, c.keys[0], c.values[0], self.mask_bits, self.len_dev,
                                    at.scale, max_len=self.max_len, out=self.attn)
-            ops.quantized_matmul(self.attn, at.o_proj.weight, at.o_proj.scales, at.o_proj.biases,
-                                 bias=at.o_proj.bias, out=self.o)
-            ops.rms_norm(self.o, layer.post_attention_layernorm.weight, args.rms_norm_eps,
-                         residual=self.h, out=self.hn, h_out=self.h)
+            if self.slab["o"]:
+                s = self.slab["o"]
+                ops.quantized_matmul_slabs(self.attn, at.o_proj.weight, at.o_proj.scales, at.o_proj.biases,
+                                           s, partial=self.partial)
+                ops.rms_norm_slabs(self.partial, ops.slab_count(H * hd, s),
+                                   layer.post_attention_layernorm.weight, args.rms_norm_eps, T,
+                                   residual=self.h, out=self.hn, h_out=self.h)
+            else:
+                ops.quantized_matmul(self.attn, at.o_proj.weight, at.o_proj.scales, at.o_proj.biases,
+                                     bias=at.o_proj.bias, out=self.o)
+                ops.rms_norm(self.o, layer.post_attention_layernorm.weight, args.rms_norm_eps,
+                             residual=self.h, out=self.hn, h_out=self.h)
             mlp = layer.mlp
             if self.fuse:
                 w, sc, bi, b = self.gu_w[i]
@@ -552,10 +599,17 @@ class TreeVerifier:
                 ops.quantized_matmul(self.hn, mlp.up_proj.weight, mlp.up_proj.scales,
                                      mlp.up_proj.biases, bias=mlp.up_proj.bias, out=self.up)
                 ops.silu_mul(self.gate, self.up, out=self.act)
-            ops.quantized_matmul(self.act, mlp.down_proj.weight, mlp.down_proj.scales,
-                                 mlp.down_proj.biases, bias=mlp.down_proj.bias, out=self.down)
             nxt = layers[i + 1].input_layernorm.weight if i + 1 < len(layers) else m.model.norm.weight
-            ops.rms_norm(self.down, nxt, args.rms_norm_eps, residual=self.h, out=self.hn, h_out=self.h)
+            if self.slab["down"]:
+                s = self.slab["down"]
+                ops.quantized_matmul_slabs(self.act, mlp.down_proj.weight, mlp.down_proj.scales,
+                                           mlp.down_proj.biases, s, partial=self.partial)
+                ops.rms_norm_slabs(self.partial, ops.slab_count(args.intermediate_size, s), nxt,
+                                   args.rms_norm_eps, T, residual=self.h, out=self.hn, h_out=self.h)
+            else:
+                ops.quantized_matmul(self.act, mlp.down_proj.weight, mlp.down_proj.scales,
+                                     mlp.down_proj.biases, bias=mlp.down_proj.bias, out=self.down)
+                ops.rms_norm(self.down, nxt, args.rms_norm_eps, residual=self.h, out=self.hn, h_out=self.h)
         head = m.model.embed_tokens if args.tie_word_embeddings else m.lm_head
         ops.quantized_matmul(self.hn, head.weight, head.scales, head.biases, out=self.logits)
         ops.argmax_rows(self.logits, out=self.node_argmax)

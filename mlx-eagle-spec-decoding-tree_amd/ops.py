@@ -67,7 +67,7 @@ def quantized_matmul(x, w_q, scales, biases, transpose=True, group_size=64, bits
     (any leading dims, flattened as qmm_kernel.py:99-100,136): the streaming kernel for 1..32
     rows of x, a tiled GEMM above that.
     `bias` ([N] fp16) is added after rounding, as the patched linear layer does
-    (mlx_model_fwd_bench.py:70-71)."""
+    (mlx_model_fwd_bench.py:70-71).  `tuned` forces a launch shape of the streaming kernel."""
     if not transpose:
         raise ValueError("only transpose=True (x @ dequant(w).T) is implemented")
     _need_cuda(x, w_q, scales, biases, bias)
@@ -112,6 +112,55 @@ def quantized_matmul(x, w_q, scales, biases, transpose=True, group_size=64, bits
                                          _ptr(bias), _ptr(out), M, N, K, nw, phases, splits, ranges,
                                          unit_cols, _ptr(ws), ws.numel(), _stream())
     _lib.check(rc, "quantized_matmul")
+    return out
+
+
+def slab_count(K, steps_per_slab):
+    """K slabs of the slab form of the matmul; 0 when it does not take this K."""
+    return _lib.lib().eagle_qmm_slab_count(int(K), int(steps_per_slab))
+
+
+def slab_steps(M, N, K):
+    """K steps per slab the library recommends for the slab form of this product, 0 where the
+    streaming kernel is the faster form."""
+    return _lib.lib().eagle_qmm_slab_steps(int(M), int(N), int(K))
+
+
+def quantized_matmul_slabs(x, w_q, scales, biases, steps_per_slab, partial=None):
+    """The product for 1..32 rows as fp32 partial sums of K slabs, [slabs, 32, N]: the result
+    is fp16(partial.sum(0)) (+ bias), formed by `slab_sum`, `rms_norm_slabs` or
+    `rope_kv_append_slabs`.  K % 512 == 0."""
+    _need_cuda(x, w_q, scales, biases)
+    x = _f16(x, "x")
+    w_q = as_packed_u32(w_q)
+    scales, biases = _f16(scales, "scales"), _f16(biases, "biases")
+    *lead, K = x.shape
+    M = reduce(lambda a, b: a * b, lead, 1)
+    N = w_q.shape[0]
+    if w_q.shape[1] * 8 != K or tuple(scales.shape) != (N, K // 64) or tuple(biases.shape) != (N, K // 64):
+        raise ValueError(f"shape mismatch: x {tuple(x.shape)}, w {tuple(w_q.shape)}, "
+                         f"scales {tuple(scales.shape)}, biases {tuple(biases.shape)}")
+    slabs = slab_count(K, steps_per_slab)
+    if slabs < 1:
+        raise ValueError(f"the slab form does not take K = {K} with {steps_per_slab} steps per slab")
+    if partial is None:
+        partial = torch.empty((slabs, 32, N), dtype=torch.float32, device=x.device)
+    elif partial.dtype != torch.float32 or partial.numel() < slabs * 32 * N or not partial.is_contiguous():
+        raise ValueError("partial must be a contiguous fp32 buffer of at least slabs * 32 * N elements")
+    rc = _lib.lib().eagle_qmm_slab_partial_w4g64(_ptr(x), _ptr(w_q), _ptr(scales), _ptr(biases),
+                                                 _ptr(partial), partial.numel() * 4, M, N, K, 64, 4,
+                                                 int(steps_per_slab), _stream())
+    _lib.check(rc, "quantized_matmul_slabs")
+    return partial
+
+
+def slab_sum(partial, slabs, M, N, bias=None, out=None):
+    """fp16(sum of the slabs, in slab order) (+ bias) -> [M, N]."""
+    _need_cuda(partial, bias)
+    if out is None:
+        out = torch.empty((M, N), dtype=torch.float16, device=partial.device)
+    rc = _lib.lib().eagle_slab_sum_f16(_ptr(partial), int(slabs), _ptr(bias), _ptr(out), M, N, _stream())
+    _lib.check(rc, "slab_sum")
     return out
 
 
@@ -227,6 +276,15 @@ def rope_kv_append(q_lin, k_lin, v_lin, positions, inv_freqs, scaling_factor, q_
         float(scaling_factor), _ptr(q_out), _ptr(k_cache), _ptr(v_cache), _ptr(cache_len_dev),
         T, H, G, hd, k_cache.shape[1], int(row_stride), _stream())
     _lib.check(rc, "rope_kv_append")
+
+
+def rope_kv_append_slabs(partial, slabs, bias, rope_cs, q_out, k_cache, v_cache, cache_len_dev, T, H, G, hd):
+    """`rope_kv_append` (table form) of the fused q|k|v projection held as [slabs, 32, (H+2G) hd]
+    fp32 partial sums; `bias` is the projection's fp16 bias or None."""
+    rc = _lib.lib().eagle_rope_kv_append_slabs_f16(
+        _ptr(partial), int(slabs), _ptr(bias), _ptr(rope_cs), _ptr(q_out), _ptr(k_cache), _ptr(v_cache),
+        _ptr(cache_len_dev), T, H, G, hd, k_cache.shape[1], _stream())
+    _lib.check(rc, "rope_kv_append_slabs")
 
 
 def mask_to_bits(tree_mask):
@@ -421,6 +479,22 @@ def rms_norm(x, weight, eps, residual=None, out=None, h_out=None):
     rc = _lib.lib().eagle_rmsnorm_f16(_ptr(x), _ptr(residual), _ptr(_f16(weight, "weight")),
                                       float(eps), _ptr(h), _ptr(out), T, D, _stream())
     _lib.check(rc, "rms_norm")
+    return out if residual is None else (h, out)
+
+
+def rms_norm_slabs(partial, slabs, weight, eps, T, residual=None, out=None, h_out=None):
+    """`rms_norm` of x = fp16(sum of the slabs) held as [slabs, 32, D] fp32 partial sums."""
+    _need_cuda(partial, weight, residual)
+    D = weight.shape[-1]
+    if out is None:
+        out = torch.empty((T, D), dtype=torch.float16, device=partial.device)
+    h = None
+    if residual is not None:
+        h = h_out if h_out is not None else torch.empty((T, D), dtype=torch.float16, device=partial.device)
+    rc = _lib.lib().eagle_rmsnorm_slabs_f16(_ptr(partial), int(slabs), _ptr(residual),
+                                            _ptr(_f16(weight, "weight")), float(eps), _ptr(h), _ptr(out),
+                                            T, D, _stream())
+    _lib.check(rc, "rms_norm_slabs")
     return out if residual is None else (h, out)
 
 
