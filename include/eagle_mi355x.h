@@ -101,8 +101,8 @@ int eagle_qmm_gemm_w4g64_f16(const void* x, const uint32_t* wq, const void* scal
 
 /* The same product for 1..32 rows in the slab form, with the result left as fp32 partial sums:
  * every workgroup owns 128 weight rows and one K slab of `steps_per_slab` quantisation groups
- * (8, 16, 24 or 32), holds its x slab in LDS and expands the weights to fp16 in registers for
- * v_mfma_f32_32x32x16_f16.  partial [slabs][32][N] fp32 (rows >= M are not written),
+ * (a multiple of 8), moves x through LDS eight groups at a time and expands the weights to fp16
+ * in registers for v_mfma_f32_32x32x16_f16.  partial [slabs][32][N] fp32 (rows >= M are not written),
  * slabs = eagle_qmm_slab_count(K, steps_per_slab) (0 for a shape the form does not take:
  * K % 512 == 0 is required, scales and biases 16-byte aligned).  The product is
  * fp16(sum over the slabs, in slab order) (+ fp16 bias): the kernel that consumes it adds the

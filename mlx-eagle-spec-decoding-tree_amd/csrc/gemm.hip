@@ -56,6 +56,28 @@ __device__ inline half8_t dequant_word(uint32_t w, half2_t s2, half2_t b16) {
   return o;
 }
 
+// The same with the offset taken off first: (16 + q) - 24 = q - 8 exactly, then one packed fma
+// with (s, b + 8 s).  For weights quantised the usual way b is close to -8 s, so b + 8 s is
+// small and its rounding no longer matters (with b - 16 s, about 24 s in size, that rounding is
+// 0.15 % of a weight, and it is the same for all 64 weights of a group).  One packed add more
+// per pair: for the kernel below, which is not bound by the expansion.
+__device__ inline half8_t dequant_word_centred(uint32_t w, half2_t s2, half2_t b8) {
+  union { uint32_t u; half2_t h; } c[4];
+  c[0].u = and_or(w << 6, 0x03c003c0u, 0x4c004c00u);
+  c[1].u = and_or(w << 2, 0x03c003c0u, 0x4c004c00u);
+  c[2].u = and_or(w >> 2, 0x03c003c0u, 0x4c004c00u);
+  c[3].u = and_or(w >> 6, 0x03c003c0u, 0x4c004c00u);
+  const half2_t off = half2_t{(half_t)24.f, (half_t)24.f};
+  half8_t o;
+#pragma unroll
+  for (int i = 0; i < 4; ++i) {
+    const half2_t v = __builtin_elementwise_fma(c[i].h - off, s2, b8);
+    o[2 * i] = v[0];
+    o[2 * i + 1] = v[1];
+  }
+  return o;
+}
+
 // MT = 32-row x tiles per wave: 2 (128-row blocks) or 4 (256-row blocks: twice the matrix work
 // per expanded weight and per byte read from LDS).
 template <int E>
@@ -283,15 +305,18 @@ int launch_gemm(const half_t* x, const uint32_t* w, const half_t* s, const half_
 
 
 // ------------------------------------------------------------------------------------------
-// Up to 32 rows: K slabs, the x slab resident in LDS, fp32 partial sums as the result
+// Up to 32 rows: K slabs, x through LDS a chunk of eight steps at a time, fp32 partial sums as
+// the result
 // ------------------------------------------------------------------------------------------
-// A workgroup of NWV (four or eight) waves owns 32 NWV weight rows (one 32-row tile per wave)
-// and one K slab of `spz` steps (a multiple of eight).  The x slab [32 x 64 spz] is loaded once into LDS (in the
-// operand order of the weights, as above); after the one barrier that follows, the waves run
-// on their own: eight weight loads in flight per lane (the register of a step is loaded again
-// for the step eight ahead as soon as it has been expanded), scales and biases eight groups
-// per fetch, four matrix instructions per step.  Several workgroups share a compute unit
-// (33 KB of LDS at spz = 8), so one workgroup's expansion overlaps another's loads.
+// A workgroup of four waves owns 128 weight rows (one 32-row tile per wave) and one K slab of
+// `spz` steps (a multiple of eight).  x travels through LDS in chunks of eight steps
+// [32 x 512], in the operand order of the weights as above, double buffered: the chunk after
+// next is in flight in registers while the waves work on the current one, and the one barrier
+// per chunk is all that ties the waves together.  Each lane keeps eight weight loads in flight
+// (the register of a step is loaded again for the step eight ahead as soon as it has been
+// expanded); scales and biases come eight groups per fetch; four matrix instructions per step.
+// Two to four workgroups share a compute unit (33 KB of LDS per x buffer), so one workgroup's
+// expansion overlaps another's loads.
 // The kernel ends with the fp32 partial tile of its slab, partial[slab][row][column]: adding
 // the slabs is left to the kernel that reads the result (normalisation, rotary embedding, or
 // slab_sum_kernel below).  A last-arriver reduction inside this kernel (partial store, wait,
@@ -299,14 +324,13 @@ int launch_gemm(const half_t* x, const uint32_t* w, const half_t* s, const half_
 // than the product itself: 14.1 us against 5.7 us for 32 x 4608 x 3584.
 constexpr int SLAB_RING = 8;
 constexpr int SLAB_ROWS = 32;               // rows of a partial tile (EAGLE_MAX_M)
+constexpr int SLAB_XR = SLAB_RING * 64 + 8; // LDS row stride of an x chunk in halves
+constexpr int SLAB_XBUF = SLAB_ROWS * SLAB_XR;
 
-template <int NWV>
-__global__ __launch_bounds__(64 * NWV) void qmm_slab_w4g64_kernel(
+__global__ __launch_bounds__(256) void qmm_slab_w4g64_kernel(
     const half_t* __restrict__ x, const uint32_t* __restrict__ w, const half_t* __restrict__ s,
     const half_t* __restrict__ b, float* __restrict__ partial, int M, int N, int K, int spz) {
-  constexpr int BN = 32 * NWV;               // weight rows per workgroup
-  constexpr int TPRW = 2 * NWV;              // threads per x row in the slab load (8 or 16)
-  extern __shared__ __attribute__((aligned(16))) half_t xslab[];
+  extern __shared__ __attribute__((aligned(16))) half_t xlds[];   // one or two x chunks
   const int tid = threadIdx.x;
   const int wave = tid >> 6, lane = tid & 63;
   const int ql = lane & 31, hb = lane >> 5;
@@ -316,14 +340,11 @@ __global__ __launch_bounds__(64 * NWV) void qmm_slab_w4g64_kernel(
   const int g0 = z * spz;
   const int steps = G - g0 < spz ? G - g0 : spz;   // a multiple of eight
   const int chunks = steps >> 3;
-  const int XR = spz * 64 + 8;               // LDS row stride in halves
 
-  // thread (xr, xc) moves the 16-byte pieces xc + i * TPRW of row xr, eight per round
-  const int xr = tid / TPRW, xc = tid % TPRW;
-  const int rounds = (steps * 8 / TPRW + SLAB_RING - 1) / SLAB_RING;
-  const int last_piece = steps * 8 - TPRW + xc;     // the last piece of this thread inside the slab
-  const half_t* xp = x + (long)(xr < M ? xr : M - 1) * K + g0 * 64;
-  int nrow = blockIdx.x * BN + wave * 32 + ql;
+  // thread (xr, xc) moves the 16 bytes at column 64 i + 8 xc of row xr for the steps i of a chunk
+  const int xr = tid >> 3, xc = tid & 7;
+  const half_t* xp = x + (long)(xr < M ? xr : M - 1) * K + g0 * 64 + xc * 8;
+  int nrow = blockIdx.x * 128 + wave * 32 + ql;
   if (nrow > N - 1) nrow = N - 1;
   const uint32_t* wp = w + (long)nrow * KW + g0 * 8 + hb * 4;
   const half_t* sp = s + (long)nrow * G + g0;
@@ -332,36 +353,33 @@ __global__ __launch_bounds__(64 * NWV) void qmm_slab_w4g64_kernel(
   half8_t xreg[SLAB_RING];
   uint4_t wreg[SLAB_RING];
   half8_t s8, b8, s8n, b8n;
-  auto piece = [&](int i) {
-    const int pc = xc + i * TPRW;
-    return pc < last_piece ? pc : last_piece;       // past the slab: the last piece again
-  };
+  auto fetch_x = [&](int c) {
 #pragma unroll
-  for (int i = 0; i < SLAB_RING; ++i) xreg[i] = *reinterpret_cast<const half8_t*>(xp + piece(i) * 8);
+    for (int i = 0; i < SLAB_RING; ++i) xreg[i] = *reinterpret_cast<const half8_t*>(xp + (c * 8 + i) * 64);
+  };
+  auto stash_x = [&](int buf) {
+#pragma unroll
+    for (int i = 0; i < SLAB_RING; ++i)
+      *reinterpret_cast<half8_t*>(&xlds[buf * SLAB_XBUF + xr * SLAB_XR + i * 64 + xc * 8]) = permute8(xreg[i]);
+  };
+  fetch_x(0);
   s8 = *reinterpret_cast<const half8_t*>(sp);
   b8 = *reinterpret_cast<const half8_t*>(bp);
 #pragma unroll
   for (int i = 0; i < SLAB_RING; ++i) wreg[i] = *reinterpret_cast<const uint4_t*>(wp + i * 8);
   __builtin_amdgcn_sched_barrier(0);
-  for (int r = 0; r < rounds; ++r) {
-#pragma unroll
-    for (int i = 0; i < SLAB_RING; ++i)
-      *reinterpret_cast<half8_t*>(&xslab[xr * XR + piece(r * 8 + i) * 8]) = permute8(xreg[i]);
-    if (r + 1 < rounds) {
-#pragma unroll
-      for (int i = 0; i < SLAB_RING; ++i)
-        xreg[i] = *reinterpret_cast<const half8_t*>(xp + piece((r + 1) * 8 + i) * 8);
-    }
-  }
+  stash_x(0);
+  if (chunks > 1) fetch_x(1);
   __syncthreads();
 
   float16_t acc;
 #pragma unroll
   for (int i = 0; i < 16; ++i) acc[i] = 0.f;
-  const half_t* xrow = xslab + ql * XR + hb * 32;
+  const half_t* xrow = xlds + ql * SLAB_XR + hb * 32;
 
-  // one chunk of eight steps; RELOAD: the registers are loaded again for the next chunk
-  auto chunk = [&](int c, auto RELOAD) {
+  // one chunk of eight steps on the x chunk in buffer `buf`; RELOAD: the weight registers are
+  // loaded again for the next chunk
+  auto chunk = [&](int c, int buf, auto RELOAD) {
     constexpr bool reload = decltype(RELOAD)::value != 0;
     if (reload) {
       s8n = *reinterpret_cast<const half8_t*>(sp + (c + 1) * 8);
@@ -370,14 +388,14 @@ __global__ __launch_bounds__(64 * NWV) void qmm_slab_w4g64_kernel(
 #pragma unroll
     for (int e = 0; e < 8; ++e) {
       const half_t sc = s8[e], bi = b8[e];
-      const half_t b16 = (half_t)((float)bi - 16.f * (float)sc);
+      const half_t bc = (half_t)((float)bi + 8.f * (float)sc);
       half8_t af[4];
 #pragma unroll
-      for (int j = 0; j < 4; ++j) af[j] = dequant_word(wreg[e][j], half2_t{sc, sc}, half2_t{b16, b16});
+      for (int j = 0; j < 4; ++j) af[j] = dequant_word_centred(wreg[e][j], half2_t{sc, sc}, half2_t{bc, bc});
       if (reload) wreg[e] = *reinterpret_cast<const uint4_t*>(wp + ((c + 1) * 8 + e) * 8);
 #pragma unroll
       for (int j = 0; j < 4; ++j) {
-        const half8_t bf = *reinterpret_cast<const half8_t*>(xrow + (c * 8 + e) * 64 + j * 8);
+        const half8_t bf = *reinterpret_cast<const half8_t*>(xrow + buf * SLAB_XBUF + e * 64 + j * 8);
         acc = __builtin_amdgcn_mfma_f32_32x32x16_f16(af[j], bf, acc, 0, 0, 0);
       }
     }
@@ -386,25 +404,33 @@ __global__ __launch_bounds__(64 * NWV) void qmm_slab_w4g64_kernel(
       b8 = b8n;
     }
   };
-  for (int c = 0; c + 1 < chunks; ++c) chunk(c, StepIndex<1>{});
-  chunk(chunks - 1, StepIndex<0>{});
+  for (int c = 0; c + 1 < chunks; ++c) {
+    chunk(c, c & 1, StepIndex<1>{});
+    // x of chunk c + 1 (requested before this chunk's weight reloads, so that waiting for it
+    // leaves those in flight) into the buffer that chunk c - 1 used: every wave left that one
+    // before the barrier that ended chunk c - 1
+    stash_x((c + 1) & 1);
+    if (c + 2 < chunks) fetch_x(c + 2);
+    __syncthreads();
+  }
+  chunk(chunks - 1, (chunks - 1) & 1, StepIndex<0>{});
 
   // accumulator register i of a lane: weight row 8*(i/4) + 4*hb + i%4 of the wave's tile, x
   // row ql.  Through LDS, so that the lanes of a wave store whole 512-byte row segments.
-  constexpr int OS = BN + 4;                 // floats per row of the tile in LDS
-  float* ot = reinterpret_cast<float*>(xslab);
-  __syncthreads();                           // every wave is done with the x slab
+  constexpr int OS = 128 + 4;                // floats per row of the tile in LDS
+  float* ot = reinterpret_cast<float*>(xlds);
+  __syncthreads();                           // every wave is done with the x chunks
 #pragma unroll
   for (int i4 = 0; i4 < 4; ++i4)
     *reinterpret_cast<float4_t*>(&ot[ql * OS + wave * 32 + 8 * i4 + 4 * hb]) =
         float4_t{acc[4 * i4], acc[4 * i4 + 1], acc[4 * i4 + 2], acc[4 * i4 + 3]};
   __syncthreads();
   float* dst = partial + (size_t)z * SLAB_ROWS * N;
-  const int c = (tid % (BN / 4)) * 4;        // BN / 4 threads per row, eight rows per pass
-  const int n = blockIdx.x * BN + c;
+  const int c = (tid & 31) * 4;
+  const int n = blockIdx.x * 128 + c;
 #pragma unroll
   for (int pass = 0; pass < 4; ++pass) {
-    const int m = pass * 8 + tid / (BN / 4);
+    const int m = pass * 8 + (tid >> 5);
     if (m < M && n < N)
       *reinterpret_cast<float4_t*>(dst + (size_t)m * N + n) = *reinterpret_cast<const float4_t*>(&ot[m * OS + c]);
   }
@@ -424,15 +450,22 @@ __global__ void slab_sum_kernel(const float* __restrict__ partial, int nslab, co
 }  // namespace
 
 EAGLE_EXPORT int eagle_qmm_slab_count(int K, int steps_per_slab) {
-  if (K < 512 || (K % 512) != 0 || steps_per_slab < 8 || (steps_per_slab % 8) != 0 || steps_per_slab > 32)
+  if (K < 512 || (K % 512) != 0 || steps_per_slab < 8 || (steps_per_slab % 8) != 0 || steps_per_slab > 4096)
     return 0;
   return (K / 64 + steps_per_slab - 1) / steps_per_slab;
 }
 
 EAGLE_EXPORT int eagle_qmm_slab_steps(int M, int N, int K) {
-  // placeholder until the step has been measured with each form: off
-  (void)M; (void)N; (void)K;
-  return 0;
+  // Measured at 8, 16 and 32 rows on the projections of the 7B and 8B models, alone and inside
+  // the verification step: the slab form wins for the projections with a few thousand weight
+  // rows (q|k|v, o, down: 5-8 us against 9-14 us, 14 us against 24 us); the streaming kernel
+  // keeps gate|up (its SwiGLU epilogue saves a launch) and the vocabulary projection.  Eight
+  // steps per slab while that gives at most eight slabs, otherwise longer slabs so that the
+  // reader of the result has about ten slabs to add.
+  if (M < 1 || M > SLAB_ROWS || N < 8 || (N % 8) != 0 || K < 512 || (K % 512) != 0) return 0;
+  if (N > 8192) return 0;
+  const int G = K / 64;
+  return G <= 64 ? 8 : G <= 128 ? 16 : 32;
 }
 
 EAGLE_EXPORT size_t eagle_qmm_slab_partial_bytes(int N, int K, int steps_per_slab) {
@@ -453,35 +486,20 @@ EAGLE_EXPORT int eagle_qmm_slab_partial_w4g64(const void* x, const uint32_t* wq,
       !eagle_aligned16(partial))
     return EAGLE_ERR_ALIGN;
   if (partial_bytes < eagle_qmm_slab_partial_bytes(N, K, steps_per_slab)) return EAGLE_ERR_WORKSPACE;
+  const int bufs = steps_per_slab > SLAB_RING ? 2 : 1;
+  const size_t lds = (size_t)bufs * SLAB_XBUF * sizeof(half_t);
   static bool configured = false;
   if (!configured) {
-    const int most = SLAB_ROWS * (32 * 64 + 8) * (int)sizeof(half_t);
-    if (hipFuncSetAttribute(reinterpret_cast<const void*>(&qmm_slab_w4g64_kernel<4>),
-                            hipFuncAttributeMaxDynamicSharedMemorySize, most) != hipSuccess ||
-        hipFuncSetAttribute(reinterpret_cast<const void*>(&qmm_slab_w4g64_kernel<8>),
-                            hipFuncAttributeMaxDynamicSharedMemorySize, most) != hipSuccess)
+    if (hipFuncSetAttribute(reinterpret_cast<const void*>(&qmm_slab_w4g64_kernel),
+                            hipFuncAttributeMaxDynamicSharedMemorySize,
+                            2 * SLAB_XBUF * (int)sizeof(half_t)) != hipSuccess)
       return EAGLE_ERR_HIP;
     configured = true;
   }
-  // Workgroups of eight waves (256 weight rows) where four-wave workgroups, one per compute
-  // unit for the size of their x slab, would not all fit on the device at once.
-  const long wg4 = (long)((N + 127) / 128) * slabs;
-  const size_t xbytes = SLAB_ROWS * (size_t)(steps_per_slab * 64 + 8) * sizeof(half_t);
-  const long per_cu = (long)(160 * 1024 / xbytes);
-  const bool wide = wg4 > NUM_CU * per_cu;
-  const int bn = wide ? 256 : 128;
-  const size_t tile = SLAB_ROWS * (size_t)(bn + 4) * sizeof(float);
-  const size_t lds = xbytes > tile ? xbytes : tile;
-  const dim3 grid((N + bn - 1) / bn, slabs);
-  hipStream_t st = static_cast<hipStream_t>(stream);
-  if (wide)
-    hipLaunchKernelGGL(qmm_slab_w4g64_kernel<8>, grid, dim3(512), lds, st, static_cast<const half_t*>(x), wq,
-                       static_cast<const half_t*>(scales), static_cast<const half_t*>(biases), partial, M, N,
-                       K, steps_per_slab);
-  else
-    hipLaunchKernelGGL(qmm_slab_w4g64_kernel<4>, grid, dim3(256), lds, st, static_cast<const half_t*>(x), wq,
-                       static_cast<const half_t*>(scales), static_cast<const half_t*>(biases), partial, M, N,
-                       K, steps_per_slab);
+  hipLaunchKernelGGL(qmm_slab_w4g64_kernel, dim3((N + 127) / 128, slabs), dim3(256), lds,
+                     static_cast<hipStream_t>(stream), static_cast<const half_t*>(x), wq,
+                     static_cast<const half_t*>(scales), static_cast<const half_t*>(biases), partial, M, N, K,
+                     steps_per_slab);
   return eagle_launch_status();
 }
 

@@ -217,9 +217,11 @@ def test_accepted_path_cache_equals_sequential_decode(dev):
     assert r[1] == 4 and list(r[4:8]) == [1, 3, 5, 7] and r[3] == toks[5]
     n = ver.sync_host_offsets()
     assert n == P + 5 == seq_cache[0].offset
+    # the two paths go through different forms of the matmul (the step's down projection is the
+    # slab form, which rounds the expanded weights to fp16): the stated tolerance, not equality
     for a, b in zip(s2["cache"], seq_cache):
-        assert rel_err(a.keys[0, :, :n].cpu().numpy(), b.keys[0, :, :n].cpu().numpy()) <= 5e-3
-        assert rel_err(a.values[0, :, :n].cpu().numpy(), b.values[0, :, :n].cpu().numpy()) <= 5e-3
+        assert rel_err(a.keys[0, :, :n].cpu().numpy(), b.keys[0, :, :n].cpu().numpy()) <= TOL
+        assert rel_err(a.values[0, :, :n].cpu().numpy(), b.values[0, :, :n].cpu().numpy()) <= TOL
 
 
 def test_patch_model_uses_the_supplied_kernel(dev):

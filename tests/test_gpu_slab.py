@@ -24,7 +24,9 @@ def ordered_sum_f16(partial, slabs, M):
 @pytest.mark.parametrize("M,N,K,steps,bias", [(32, 512, 512, 8, True), (32, 4608, 3584, 8, True),
                                               (31, 3584, 3584, 16, False), (17, 200, 1536, 8, True),
                                               (1, 128, 1024, 8, False), (8, 136, 2048, 24, False),
-                                              (32, 3584, 18944, 32, False), (24, 1000, 4096, 32, True)])
+                                              (32, 3584, 18944, 32, False), (24, 1000, 4096, 32, True),
+                                              (32, 3584, 18944, 48, False), (32, 256, 4096, 64, True),
+                                              (13, 136, 1536, 16, False)])
 def test_slab_partials_match_oracle(dev, M, N, K, steps, bias):
     print(f"slab M={M} N={N} K={K} steps={steps}", flush=True)
     rng = np.random.default_rng(M + N + K + steps)
@@ -70,7 +72,7 @@ def test_slab_form_rejects_bad_arguments(dev):
     x = torch.zeros((32, 896), dtype=torch.float16, device=dev)
     w = torch.zeros((64, 112), dtype=torch.int32, device=dev)
     s = torch.zeros((64, 14), dtype=torch.float16, device=dev)
-    assert ops.slab_count(896, 8) == 0 and ops.slab_count(1024, 12) == 0 and ops.slab_count(1024, 40) == 0
+    assert ops.slab_count(896, 8) == 0 and ops.slab_count(1024, 12) == 0 and ops.slab_count(1024, 4104) == 0
     with pytest.raises(ValueError):
         ops.quantized_matmul_slabs(x, w, s, s, 8)                      # K not a multiple of 512
     x = torch.zeros((33, 1024), dtype=torch.float16, device=dev)

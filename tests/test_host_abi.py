@@ -169,3 +169,36 @@ def test_draft_side_entry_points_reject_bad_arguments():
     assert L.eagle_qmm_gemm_w4g64_f16(p, p, p, p, None, p, 512, 128, 100, 64, 4, None) == 2
     assert L.eagle_qmm_gemm_w4g64_f16(p, p, p, p, None, p, 512, 128, 128, 32, 4, None) == 4
     assert L.eagle_qmm_gemm_w4g64_f16(p + 2, p, p, p, None, p, 512, 128, 128, 64, 4, None) == 3
+
+
+def test_slab_form_entry_points_reject_bad_arguments():
+    L = _lib.lib()
+    buf = (ctypes.c_char * 4096)()
+    p = (ctypes.addressof(buf) + 15) & ~15
+    big = 1 << 30
+    assert L.eagle_qmm_slab_count(3584, 8) == 7 and L.eagle_qmm_slab_count(18944, 32) == 10
+    assert L.eagle_qmm_slab_count(896, 8) == 0 and L.eagle_qmm_slab_count(1024, 12) == 0
+    assert L.eagle_qmm_slab_partial_bytes(4608, 3584, 8) == 7 * 32 * 4608 * 4
+    # the library's choice: the small projections of the 7B / 8B models, not gate|up or the head
+    assert L.eagle_qmm_slab_steps(32, 4608, 3584) == 8 and L.eagle_qmm_slab_steps(32, 3584, 18944) == 32
+    assert L.eagle_qmm_slab_steps(8, 4096, 4096) == 8 and L.eagle_qmm_slab_steps(32, 4096, 14336) == 32
+    assert L.eagle_qmm_slab_steps(32, 37888, 3584) == 0 and L.eagle_qmm_slab_steps(32, 152064, 3584) == 0
+    assert L.eagle_qmm_slab_steps(32, 1152, 896) == 0 and L.eagle_qmm_slab_steps(33, 4608, 3584) == 0
+    call = lambda **kw: L.eagle_qmm_slab_partial_w4g64(
+        kw.get("x", p), p, p, p, kw.get("partial", p), kw.get("bytes", big), kw.get("M", 32), kw.get("N", 128),
+        kw.get("K", 1024), kw.get("gs", 64), kw.get("bits", 4), kw.get("steps", 8), None)
+    assert call(x=None) == 1 and call(partial=None) == 1
+    assert call(M=33) == 2 and call(N=100) == 2 and call(K=896) == 2 and call(steps=12) == 2
+    assert call(x=p + 2) == 3
+    assert call(gs=32) == 4
+    assert call(bytes=1024) == 5
+    assert L.eagle_slab_sum_f16(p, 0, None, p, 8, 128, None) == 2
+    assert L.eagle_slab_sum_f16(p, 2, None, p, 33, 128, None) == 2
+    assert L.eagle_slab_sum_f16(p, 2, p + 2, p, 8, 128, None) == 3
+    assert L.eagle_rmsnorm_slabs_f16(p, 2, None, p, 1e-6, None, p, 33, 128, None) == 2
+    assert L.eagle_rmsnorm_slabs_f16(p, 0, None, p, 1e-6, None, p, 8, 128, None) == 2
+    assert L.eagle_rmsnorm_slabs_f16(p, 2, p, p, 1e-6, None, p, 8, 128, None) == 1     # residual needs h_out
+    assert L.eagle_rope_kv_append_slabs_f16(p, 2, None, p, p, p, p, p, 33, 4, 2, 64, 100, None) == 2
+    assert L.eagle_rope_kv_append_slabs_f16(p, 2, None, p, p, p, p, p, 8, 4, 3, 64, 100, None) == 2
+    assert L.eagle_rope_kv_append_slabs_f16(p, 2, p + 2, p, p, p, p, p, 8, 4, 2, 64, 100, None) == 3
+    assert L.eagle_rope_kv_append_slabs_f16(None, 2, None, p, p, p, p, p, 8, 4, 2, 64, 100, None) == 1
