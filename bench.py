@@ -32,7 +32,7 @@ sys.path.insert(0, ROOT)
 HBM_PEAK_GBS = 8000.0
 # HBM bytes per QMM launch of this workload (FETCH_SIZE + WRITE_SIZE from two rocprofv3 --pmc
 # runs of this script, scaled by a copy kernel of known size); None until measured.
-QMM_TRAFFIC_BYTES_PER_LAUNCH = 47795789
+QMM_TRAFFIC_BYTES_PER_LAUNCH = 46400799
 PREFIX = 2048
 NODES = 32
 
@@ -203,7 +203,7 @@ def main():
     kv_bytes = 2 * L * G * (PREFIX + NODES) * hd * 2
     achieved = alg / (qmm_ms * 1e-3) / 1e9
     traffic = QMM_TRAFFIC_BYTES_PER_LAUNCH
-    roofline = {"bound": "hbm", "kernel": "qmm_w4g64_kernel", "achieved": round(achieved, 1),
+    roofline = {"bound": "hbm", "kernel": "qmm_w4g64_kernel + qmm_slab_w4g64_kernel", "achieved": round(achieved, 1),
                 "peak": HBM_PEAK_GBS, "unit": "GB/s", "frac": round(achieved / HBM_PEAK_GBS, 4),
                 "traffic": traffic, "launches_per_step": n_launch,
                 "avg_launch_us": round(qmm_ms * 1e3 / n_launch, 3),
