@@ -379,6 +379,42 @@ def fuse_projections(model, swiglu):
     return qkv_w, gu_w
 
 
+def slab_plan(model, T, forced=None, fused=True, rope_launch=True):
+    """K steps per slab for the q|k|v, o and down projections of a pass of T rows (0: streaming
+    kernel): the library's choice per shape, or `forced` ({"qkv": s, "o": s, "down": s}).  The
+    slab form leaves the product as partial sums for its consumer to add, so it needs the fused
+    pass (table-driven rope launch after q|k|v, norm with the residual after o and down),
+    K % 512 == 0, and projections without a bias for o and down."""
+    args = model.args
+    D, I = args.hidden_size, args.intermediate_size
+    H, G, hd = args.num_attention_heads, args.num_key_value_heads, args.head_dim
+    layer = model.model.layers[0]
+    shapes = {"qkv": ((H + 2 * G) * hd, D), "o": (D, H * hd), "down": (D, I)}
+    plan = {}
+    for name, (n, k) in shapes.items():
+        s = ops.slab_steps(T, n, k) if forced is None else int(forced.get(name, 0))
+        ok = fused and s > 0 and ops.slab_count(k, s) > 0
+        if name == "qkv":
+            ok = ok and rope_launch
+        if name == "o":
+            ok = ok and layer.self_attn.o_proj.bias is None
+        if name == "down":
+            ok = ok and layer.mlp.down_proj.bias is None
+        plan[name] = s if ok else 0
+    return plan
+
+
+def slab_partial_buffer(model, plan):
+    """fp32 buffer large enough for the partial sums of any projection in `plan`."""
+    args = model.args
+    D, I = args.hidden_size, args.intermediate_size
+    H, G, hd = args.num_attention_heads, args.num_key_value_heads, args.head_dim
+    need = max([1] + [ops.slab_count(k, plan[name]) * 32 * n
+                      for name, n, k in (("qkv", (H + 2 * G) * hd, D), ("o", D, H * hd), ("down", D, I))
+                      if plan[name]])
+    return torch.empty(need, dtype=torch.float32, device=model.device)
+
+
 class TreeVerifier:
     """One target-model tree-verification step with static buffers, so that it can be
     captured once in a HIP graph and replayed: embedding, all decoder layers, final norm,
@@ -442,10 +478,7 @@ class TreeVerifier:
         self.act = torch.empty((T, I), **f16)
         self.down = torch.empty((T, D), **f16)
         self.logits = torch.empty((T, args.vocab_size), **f16)
-        need = max([1] + [ops.slab_count(k, self.slab[name]) * 32 * n
-                          for name, n, k in (("qkv", (H + 2 * G) * hd, D), ("o", D, H * hd), ("down", D, I))
-                          if self.slab[name]])
-        self.partial = torch.empty(need, dtype=torch.float32, device=dev)
+        self.partial = slab_partial_buffer(model, self.slab)
         self.len_dev = cache[0].len_dev
         self.cache_ptrs = torch.tensor([c.keys.data_ptr() for c in cache]
                                        + [c.values.data_ptr() for c in cache],
@@ -466,26 +499,8 @@ class TreeVerifier:
         self.qkv_w, self.gu_w = fuse_projections(self.model, self.swiglu)
 
     def _slab_plan(self, forced):
-        """K steps per slab for q|k|v, o and down (0: streaming kernel).  The slab form needs
-        the fused step (its consumers are the table-driven rope kernel and the norm with the
-        residual), K % 512 == 0, and projections without a bias for o and down."""
-        args = self.args
-        D, I = args.hidden_size, args.intermediate_size
-        H, G, hd = args.num_attention_heads, args.num_key_value_heads, args.head_dim
-        layer = self.model.model.layers[0]
-        shapes = {"qkv": ((H + 2 * G) * hd, D), "o": (D, H * hd), "down": (D, I)}
-        plan = {}
-        for name, (n, k) in shapes.items():
-            s = ops.slab_steps(self.T, n, k) if forced is None else int(forced.get(name, 0))
-            ok = self.fuse and s > 0 and ops.slab_count(k, s) > 0
-            if name == "qkv":
-                ok = ok and not self.one_launch_attention
-            if name == "o":
-                ok = ok and layer.self_attn.o_proj.bias is None
-            if name == "down":
-                ok = ok and layer.mlp.down_proj.bias is None
-            plan[name] = s if ok else 0
-        return plan
+        return slab_plan(self.model, self.T, forced, fused=self.fuse,
+                         rope_launch=not self.one_launch_attention)
 
     def qmm_launches(self):
         """(weight, scales, biases, bias, x, out, form) of every quantised matmul of one step,

@@ -14,7 +14,8 @@ import torch
 
 from . import _lib, ops
 from .eagle import (MAXT, TreeVerifier, _level_buffers, _ptr, _stream, draft_tree_init, draft_tree_level,
-                    fuse_projections, process_draft_tree_device)
+                    fuse_projections, process_draft_tree_device, slab_partial_buffer)
+from .eagle import slab_plan as eagle_slab_plan
 
 Y_LEN = 8
 
@@ -24,10 +25,12 @@ class DecoderPass:
     The rows are written to the cache at *write_len; query t sees the *attn_len rows before
     them and, of the Tk rows from there on, those its two mask words select."""
 
-    def __init__(self, model, cache, T, max_len=None, swiglu=True):
+    def __init__(self, model, cache, T, max_len=None, swiglu=True, slab_plan=None):
         args = model.args
         self.model, self.cache, self.args, self.T = model, cache, args, T
         dev = model.device
+        self.slab = eagle_slab_plan(model, T, slab_plan)
+        self.partial = slab_partial_buffer(model, self.slab)
         D, I = args.hidden_size, args.intermediate_size
         H, G, hd = args.num_attention_heads, args.num_key_value_heads, args.head_dim
         self.max_len = max_len or cache[0].capacity
@@ -67,26 +70,47 @@ class DecoderPass:
         for i, layer in enumerate(layers):
             at, mlp, c = layer.self_attn, layer.mlp, self.cache[i]
             w, sc, bi, b = self.qkv_w[i]
-            ops.quantized_matmul(self.hn, w, sc, bi, bias=b, out=self.qkv)
-            ops.rope_kv_append(self.qkv, self.qkv[:, H * hd:], self.qkv[:, (H + G) * hd:], positions,
-                               at._inv_freqs, at._scaling_factor, self.q_rot, c.keys[0], c.values[0],
-                               write_len, H, G, hd, row_stride=W, rope_cs=self.rope_cs)
+            if self.slab["qkv"]:
+                s = self.slab["qkv"]
+                ops.quantized_matmul_slabs(self.hn, w, sc, bi, s, partial=self.partial)
+                ops.rope_kv_append_slabs(self.partial, ops.slab_count(args.hidden_size, s), b, self.rope_cs,
+                                         self.q_rot, c.keys[0], c.values[0], write_len, self.T, H, G, hd)
+            else:
+                ops.quantized_matmul(self.hn, w, sc, bi, bias=b, out=self.qkv)
+                ops.rope_kv_append(self.qkv, self.qkv[:, H * hd:], self.qkv[:, (H + G) * hd:], positions,
+                                   at._inv_freqs, at._scaling_factor, self.q_rot, c.keys[0], c.values[0],
+                                   write_len, H, G, hd, row_stride=W, rope_cs=self.rope_cs)
             ops.draft_attention(self.q_rot, c.keys[0], c.values[0], mask_words, attn_len, Tk, at.scale,
                                 max_len=self.max_len, out=self.attn)
-            ops.quantized_matmul(self.attn, at.o_proj.weight, at.o_proj.scales, at.o_proj.biases,
-                                 bias=at.o_proj.bias, out=self.o)
-            ops.rms_norm(self.o, layer.post_attention_layernorm.weight, args.rms_norm_eps,
-                         residual=self.h, out=self.hn, h_out=self.h)
+            if self.slab["o"]:
+                s = self.slab["o"]
+                ops.quantized_matmul_slabs(self.attn, at.o_proj.weight, at.o_proj.scales, at.o_proj.biases,
+                                           s, partial=self.partial)
+                ops.rms_norm_slabs(self.partial, ops.slab_count(H * hd, s),
+                                   layer.post_attention_layernorm.weight, args.rms_norm_eps, self.T,
+                                   residual=self.h, out=self.hn, h_out=self.h)
+            else:
+                ops.quantized_matmul(self.attn, at.o_proj.weight, at.o_proj.scales, at.o_proj.biases,
+                                     bias=at.o_proj.bias, out=self.o)
+                ops.rms_norm(self.o, layer.post_attention_layernorm.weight, args.rms_norm_eps,
+                             residual=self.h, out=self.hn, h_out=self.h)
             w, sc, bi, b = self.gu_w[i]
             if self.swiglu:
                 ops.quantized_matmul_swiglu(self.hn, w, sc, bi, bias=b, out=self.act)
             else:
                 ops.quantized_matmul(self.hn, w, sc, bi, bias=b, out=self.gate_up)
                 ops.silu_mul(self.gate_up, None, out=self.act)
-            ops.quantized_matmul(self.act, mlp.down_proj.weight, mlp.down_proj.scales,
-                                 mlp.down_proj.biases, bias=mlp.down_proj.bias, out=self.down)
             nxt = layers[i + 1].input_layernorm.weight if i + 1 < len(layers) else m.model.norm.weight
-            ops.rms_norm(self.down, nxt, args.rms_norm_eps, residual=self.h, out=self.hn, h_out=self.h)
+            if self.slab["down"]:
+                s = self.slab["down"]
+                ops.quantized_matmul_slabs(self.act, mlp.down_proj.weight, mlp.down_proj.scales,
+                                           mlp.down_proj.biases, s, partial=self.partial)
+                ops.rms_norm_slabs(self.partial, ops.slab_count(args.intermediate_size, s), nxt,
+                                   args.rms_norm_eps, self.T, residual=self.h, out=self.hn, h_out=self.h)
+            else:
+                ops.quantized_matmul(self.act, mlp.down_proj.weight, mlp.down_proj.scales,
+                                     mlp.down_proj.biases, bias=mlp.down_proj.bias, out=self.down)
+                ops.rms_norm(self.down, nxt, args.rms_norm_eps, residual=self.h, out=self.hn, h_out=self.h)
         if not head:
             return None
         head = m.model.embed_tokens if args.tie_word_embeddings else m.lm_head
