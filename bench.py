@@ -89,6 +89,8 @@ def main():
     ap.add_argument("--slabs", default=None,
                     help="force the slab form of the matmul: e.g. qkv=8,o=8,down=32 (K steps per slab; "
                          "'' = streaming kernel everywhere; default: the library's choice)")
+    ap.add_argument("--draft-slabs", default=None,
+                    help="--loop: the same for the drafter's passes")
     ap.add_argument("--sweep", action="store_true", help="also print the per-shape QMM table to stderr")
     ap.add_argument("--calibrate-copy", action="store_true",
                     help="before anything else run one 1 GiB device copy (a kernel of known traffic: "
@@ -331,8 +333,11 @@ def loop_bench(opt):
     rng = np.random.default_rng(opt.seed + 2)
     prompt = torch.from_numpy(rng.integers(0, min(targs.vocab_size, dargs.vocab_size), prompt_len)).to(dev)
     capacity = prompt_len + (opt.warmup + steps) * (depth + 2) + k * depth + 64
+    plans = [None if s is None else {kv.split("=")[0]: int(kv.split("=")[1]) for kv in s.split(",") if kv}
+             for s in (opt.slabs, opt.draft_slabs)]
     dec = spec.SpeculativeDecoder(target, draft, capacity=capacity, k=k, depth=depth,
-                                  verify_num_tokens=nodes, max_out=(opt.warmup + steps) * (depth + 2) + 8)
+                                  verify_num_tokens=nodes, max_out=(opt.warmup + steps) * (depth + 2) + 8,
+                                  slab_plan=plans[0], draft_slab_plan=plans[1])
     dec.prepare(prompt_len)
     torch.cuda.synchronize()
     t0 = time.time()

@@ -104,7 +104,8 @@ int eagle_qmm_gemm_w4g64_f16(const void* x, const uint32_t* wq, const void* scal
  * (a multiple of 8), moves x through LDS eight groups at a time and expands the weights to fp16
  * in registers for v_mfma_f32_32x32x16_f16.  partial [slabs][32][N] fp32 (rows >= M are not written),
  * slabs = eagle_qmm_slab_count(K, steps_per_slab) (0 for a shape the form does not take:
- * K % 512 == 0 is required, scales and biases 16-byte aligned).  The product is
+ * K % 128 == 0 is required; scales and biases 16-byte aligned when K % 512 == 0, 4-byte aligned
+ * otherwise).  The product is
  * fp16(sum over the slabs, in slab order) (+ fp16 bias): the kernel that consumes it adds the
  * slabs while it loads (eagle_rmsnorm_slabs_f16, eagle_rope_kv_append_slabs_f16), or
  * eagle_slab_sum_f16 writes it out.  No counters, no workspace.  For the small projections of

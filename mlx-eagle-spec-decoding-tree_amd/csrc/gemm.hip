@@ -327,6 +327,10 @@ constexpr int SLAB_ROWS = 32;               // rows of a partial tile (EAGLE_MAX
 constexpr int SLAB_XR = SLAB_RING * 64 + 8; // LDS row stride of an x chunk in halves
 constexpr int SLAB_XBUF = SLAB_ROWS * SLAB_XR;
 
+// RAGGED: K is a multiple of 128 but not of 512.  A slab may then hold any number of steps:
+// the last chunk is partial (its loads are repeated from the slab's last step, its extra
+// steps are skipped) and scales / biases come two groups per fetch.
+template <bool RAGGED>
 __global__ __launch_bounds__(256) void qmm_slab_w4g64_kernel(
     const half_t* __restrict__ x, const uint32_t* __restrict__ w, const half_t* __restrict__ s,
     const half_t* __restrict__ b, float* __restrict__ partial, int M, int N, int K, int spz) {
@@ -338,8 +342,10 @@ __global__ __launch_bounds__(256) void qmm_slab_w4g64_kernel(
   const int G = K >> 6;                      // groups (K steps) per weight row
   const int KW = K >> 3;                     // packed words per weight row
   const int g0 = z * spz;
-  const int steps = G - g0 < spz ? G - g0 : spz;   // a multiple of eight
-  const int chunks = steps >> 3;
+  const int steps = G - g0 < spz ? G - g0 : spz;   // a multiple of eight unless RAGGED (then even)
+  const int chunks = (steps + 7) >> 3;
+  const int rem = steps - (chunks - 1) * 8;  // steps of the last chunk
+  auto step_of = [&](int i) { return RAGGED && i > steps - 1 ? steps - 1 : i; };
 
   // thread (xr, xc) moves the 16 bytes at column 64 i + 8 xc of row xr for the steps i of a chunk
   const int xr = tid >> 3, xc = tid & 7;
@@ -355,7 +361,25 @@ __global__ __launch_bounds__(256) void qmm_slab_w4g64_kernel(
   half8_t s8, b8, s8n, b8n;
   auto fetch_x = [&](int c) {
 #pragma unroll
-    for (int i = 0; i < SLAB_RING; ++i) xreg[i] = *reinterpret_cast<const half8_t*>(xp + (c * 8 + i) * 64);
+    for (int i = 0; i < SLAB_RING; ++i) xreg[i] = *reinterpret_cast<const half8_t*>(xp + step_of(c * 8 + i) * 64);
+  };
+  // scales and biases of chunk c: one 16-byte fetch, or four 4-byte fetches kept inside the slab
+  auto fetch_sb = [&](int c, half8_t& s_out, half8_t& b_out) {
+    if (!RAGGED) {
+      s_out = *reinterpret_cast<const half8_t*>(sp + c * 8);
+      b_out = *reinterpret_cast<const half8_t*>(bp + c * 8);
+    } else {
+#pragma unroll
+      for (int i = 0; i < 4; ++i) {
+        const int g = c * 8 + 2 * i < steps - 2 ? c * 8 + 2 * i : steps - 2;
+        const half2_t sv = *reinterpret_cast<const half2_t*>(sp + g);
+        const half2_t bv = *reinterpret_cast<const half2_t*>(bp + g);
+        s_out[2 * i] = sv[0];
+        s_out[2 * i + 1] = sv[1];
+        b_out[2 * i] = bv[0];
+        b_out[2 * i + 1] = bv[1];
+      }
+    }
   };
   auto stash_x = [&](int buf) {
 #pragma unroll
@@ -363,10 +387,9 @@ __global__ __launch_bounds__(256) void qmm_slab_w4g64_kernel(
       *reinterpret_cast<half8_t*>(&xlds[buf * SLAB_XBUF + xr * SLAB_XR + i * 64 + xc * 8]) = permute8(xreg[i]);
   };
   fetch_x(0);
-  s8 = *reinterpret_cast<const half8_t*>(sp);
-  b8 = *reinterpret_cast<const half8_t*>(bp);
+  fetch_sb(0, s8, b8);
 #pragma unroll
-  for (int i = 0; i < SLAB_RING; ++i) wreg[i] = *reinterpret_cast<const uint4_t*>(wp + i * 8);
+  for (int i = 0; i < SLAB_RING; ++i) wreg[i] = *reinterpret_cast<const uint4_t*>(wp + step_of(i) * 8);
   __builtin_amdgcn_sched_barrier(0);
   stash_x(0);
   if (chunks > 1) fetch_x(1);
@@ -381,18 +404,16 @@ __global__ __launch_bounds__(256) void qmm_slab_w4g64_kernel(
   // loaded again for the next chunk
   auto chunk = [&](int c, int buf, auto RELOAD) {
     constexpr bool reload = decltype(RELOAD)::value != 0;
-    if (reload) {
-      s8n = *reinterpret_cast<const half8_t*>(sp + (c + 1) * 8);
-      b8n = *reinterpret_cast<const half8_t*>(bp + (c + 1) * 8);
-    }
+    if (reload) fetch_sb(c + 1, s8n, b8n);
 #pragma unroll
     for (int e = 0; e < 8; ++e) {
+      if (RAGGED && !reload && e >= rem) break;            // the last chunk may be partial
       const half_t sc = s8[e], bi = b8[e];
       const half_t bc = (half_t)((float)bi + 8.f * (float)sc);
       half8_t af[4];
 #pragma unroll
       for (int j = 0; j < 4; ++j) af[j] = dequant_word_centred(wreg[e][j], half2_t{sc, sc}, half2_t{bc, bc});
-      if (reload) wreg[e] = *reinterpret_cast<const uint4_t*>(wp + ((c + 1) * 8 + e) * 8);
+      if (reload) wreg[e] = *reinterpret_cast<const uint4_t*>(wp + step_of((c + 1) * 8 + e) * 8);
 #pragma unroll
       for (int j = 0; j < 4; ++j) {
         const half8_t bf = *reinterpret_cast<const half8_t*>(xrow + buf * SLAB_XBUF + e * 64 + j * 8);
@@ -450,7 +471,7 @@ __global__ void slab_sum_kernel(const float* __restrict__ partial, int nslab, co
 }  // namespace
 
 EAGLE_EXPORT int eagle_qmm_slab_count(int K, int steps_per_slab) {
-  if (K < 512 || (K % 512) != 0 || steps_per_slab < 8 || (steps_per_slab % 8) != 0 || steps_per_slab > 4096)
+  if (K < 128 || (K % 128) != 0 || steps_per_slab < 8 || (steps_per_slab % 8) != 0 || steps_per_slab > 4096)
     return 0;
   return (K / 64 + steps_per_slab - 1) / steps_per_slab;
 }
@@ -479,27 +500,37 @@ EAGLE_EXPORT int eagle_qmm_slab_partial_w4g64(const void* x, const uint32_t* wq,
                                               int steps_per_slab, eagle_stream_t stream) {
   if (!x || !wq || !scales || !biases || !partial) return EAGLE_ERR_NULL;
   if (group_size != 64 || bits != 4) return EAGLE_ERR_UNSUPPORTED;
-  if (M < 1 || M > SLAB_ROWS || N < 8 || (N % 8) != 0 || K < 512 || (K % 512) != 0) return EAGLE_ERR_SHAPE;
+  if (M < 1 || M > SLAB_ROWS || N < 8 || (N % 8) != 0 || K < 128 || (K % 128) != 0) return EAGLE_ERR_SHAPE;
   const int slabs = eagle_qmm_slab_count(K, steps_per_slab);
   if (slabs < 1 || slabs > 65535) return EAGLE_ERR_SHAPE;
-  if (!eagle_aligned16(x) || !eagle_aligned16(wq) || !eagle_aligned16(scales) || !eagle_aligned16(biases) ||
-      !eagle_aligned16(partial))
+  const bool ragged = (K % 512) != 0;
+  const uintptr_t sb_mask = ragged ? 3u : 15u;
+  if (!eagle_aligned16(x) || !eagle_aligned16(wq) || !eagle_aligned16(partial) ||
+      (reinterpret_cast<uintptr_t>(scales) & sb_mask) || (reinterpret_cast<uintptr_t>(biases) & sb_mask))
     return EAGLE_ERR_ALIGN;
   if (partial_bytes < eagle_qmm_slab_partial_bytes(N, K, steps_per_slab)) return EAGLE_ERR_WORKSPACE;
   const int bufs = steps_per_slab > SLAB_RING ? 2 : 1;
   const size_t lds = (size_t)bufs * SLAB_XBUF * sizeof(half_t);
   static bool configured = false;
   if (!configured) {
-    if (hipFuncSetAttribute(reinterpret_cast<const void*>(&qmm_slab_w4g64_kernel),
-                            hipFuncAttributeMaxDynamicSharedMemorySize,
-                            2 * SLAB_XBUF * (int)sizeof(half_t)) != hipSuccess)
+    const int most = 2 * SLAB_XBUF * (int)sizeof(half_t);
+    if (hipFuncSetAttribute(reinterpret_cast<const void*>(&qmm_slab_w4g64_kernel<false>),
+                            hipFuncAttributeMaxDynamicSharedMemorySize, most) != hipSuccess ||
+        hipFuncSetAttribute(reinterpret_cast<const void*>(&qmm_slab_w4g64_kernel<true>),
+                            hipFuncAttributeMaxDynamicSharedMemorySize, most) != hipSuccess)
       return EAGLE_ERR_HIP;
     configured = true;
   }
-  hipLaunchKernelGGL(qmm_slab_w4g64_kernel, dim3((N + 127) / 128, slabs), dim3(256), lds,
-                     static_cast<hipStream_t>(stream), static_cast<const half_t*>(x), wq,
-                     static_cast<const half_t*>(scales), static_cast<const half_t*>(biases), partial, M, N, K,
-                     steps_per_slab);
+  const dim3 grid((N + 127) / 128, slabs);
+  hipStream_t st = static_cast<hipStream_t>(stream);
+  if (ragged)
+    hipLaunchKernelGGL(qmm_slab_w4g64_kernel<true>, grid, dim3(256), lds, st, static_cast<const half_t*>(x), wq,
+                       static_cast<const half_t*>(scales), static_cast<const half_t*>(biases), partial, M, N,
+                       K, steps_per_slab);
+  else
+    hipLaunchKernelGGL(qmm_slab_w4g64_kernel<false>, grid, dim3(256), lds, st, static_cast<const half_t*>(x), wq,
+                       static_cast<const half_t*>(scales), static_cast<const half_t*>(biases), partial, M, N,
+                       K, steps_per_slab);
   return eagle_launch_status();
 }
 

@@ -302,7 +302,7 @@ class SpeculativeDecoder:
     """
 
     def __init__(self, base_model, draft_model, capacity, k=8, depth=3, verify_num_tokens=31,
-                 max_out=8192):
+                 max_out=8192, slab_plan=None, draft_slab_plan=None):
         from .cache import make_prompt_cache
 
         if k != Y_LEN:
@@ -319,8 +319,8 @@ class SpeculativeDecoder:
         self.base_cache = make_prompt_cache(base_model, capacity=capacity)
         self.draft_cache = make_prompt_cache(draft_model, capacity=capacity)
         self.verifier = TreeVerifier(base_model, self.base_cache, total_tokens=verify_num_tokens,
-                                     max_len=capacity)
-        self.draft = DecoderPass(draft_model, self.draft_cache, k, max_len=capacity)
+                                     max_len=capacity, slab_plan=slab_plan)
+        self.draft = DecoderPass(draft_model, self.draft_cache, k, max_len=capacity, slab_plan=draft_slab_plan)
         i32 = dict(dtype=torch.int32, device=dev)
         self.y = torch.zeros(Y_LEN, **i32)
         self.root_token = torch.zeros(1, **i32)

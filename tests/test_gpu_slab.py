@@ -26,7 +26,10 @@ def ordered_sum_f16(partial, slabs, M):
                                               (1, 128, 1024, 8, False), (8, 136, 2048, 24, False),
                                               (32, 3584, 18944, 32, False), (24, 1000, 4096, 32, True),
                                               (32, 3584, 18944, 48, False), (32, 256, 4096, 64, True),
-                                              (13, 136, 1536, 16, False)])
+                                              (13, 136, 1536, 16, False),
+                                              # K a multiple of 128 only: partial last chunk, 4-byte scale fetches
+                                              (8, 1152, 896, 8, True), (8, 896, 4864, 8, False), (32, 896, 4864, 32, False),
+                                              (32, 200, 128, 8, True), (5, 128, 640, 8, False), (32, 264, 1920, 16, True)])
 def test_slab_partials_match_oracle(dev, M, N, K, steps, bias):
     print(f"slab M={M} N={N} K={K} steps={steps}", flush=True)
     rng = np.random.default_rng(M + N + K + steps)
@@ -72,9 +75,11 @@ def test_slab_form_rejects_bad_arguments(dev):
     x = torch.zeros((32, 896), dtype=torch.float16, device=dev)
     w = torch.zeros((64, 112), dtype=torch.int32, device=dev)
     s = torch.zeros((64, 14), dtype=torch.float16, device=dev)
-    assert ops.slab_count(896, 8) == 0 and ops.slab_count(1024, 12) == 0 and ops.slab_count(1024, 4104) == 0
+    assert ops.slab_count(832, 8) == 0 and ops.slab_count(1024, 12) == 0 and ops.slab_count(1024, 4104) == 0
+    assert ops.slab_count(896, 8) == 2
     with pytest.raises(ValueError):
-        ops.quantized_matmul_slabs(x, w, s, s, 8)                      # K not a multiple of 512
+        ops.quantized_matmul_slabs(x[:, :832].contiguous(), w[:, :104].contiguous(), s[:, :13].contiguous(),
+                                   s[:, :13].contiguous(), 8)          # K not a multiple of 128
     x = torch.zeros((33, 1024), dtype=torch.float16, device=dev)
     w = torch.zeros((64, 128), dtype=torch.int32, device=dev)
     s = torch.zeros((64, 16), dtype=torch.float16, device=dev)

@@ -177,7 +177,8 @@ def test_slab_form_entry_points_reject_bad_arguments():
     p = (ctypes.addressof(buf) + 15) & ~15
     big = 1 << 30
     assert L.eagle_qmm_slab_count(3584, 8) == 7 and L.eagle_qmm_slab_count(18944, 32) == 10
-    assert L.eagle_qmm_slab_count(896, 8) == 0 and L.eagle_qmm_slab_count(1024, 12) == 0
+    assert L.eagle_qmm_slab_count(896, 8) == 2 and L.eagle_qmm_slab_count(4864, 32) == 3
+    assert L.eagle_qmm_slab_count(832, 8) == 0 and L.eagle_qmm_slab_count(1024, 12) == 0
     assert L.eagle_qmm_slab_partial_bytes(4608, 3584, 8) == 7 * 32 * 4608 * 4
     # the library's choice: the small projections of the 7B / 8B models, not gate|up or the head
     assert L.eagle_qmm_slab_steps(32, 4608, 3584) == 8 and L.eagle_qmm_slab_steps(32, 3584, 18944) == 32
@@ -188,7 +189,7 @@ def test_slab_form_entry_points_reject_bad_arguments():
         kw.get("x", p), p, p, p, kw.get("partial", p), kw.get("bytes", big), kw.get("M", 32), kw.get("N", 128),
         kw.get("K", 1024), kw.get("gs", 64), kw.get("bits", 4), kw.get("steps", 8), None)
     assert call(x=None) == 1 and call(partial=None) == 1
-    assert call(M=33) == 2 and call(N=100) == 2 and call(K=896) == 2 and call(steps=12) == 2
+    assert call(M=33) == 2 and call(N=100) == 2 and call(K=832) == 2 and call(steps=12) == 2
     assert call(x=p + 2) == 3
     assert call(gs=32) == 4
     assert call(bytes=1024) == 5
