@@ -187,3 +187,64 @@ def test_step_with_slab_projections(dev, plan, monkeypatch):
         cap.step()
         torch.cuda.synchronize()
         assert torch.equal(cap.logits, ver.logits)
+
+
+def test_full_size_properties(dev):
+    """The down projection of the 7B shape (3584 x 18944, 32 rows), too large for the CPU checker
+    in a test: rows are independent (bit for bit), the slab length only changes the fp32
+    summation order, and the product is linear in x."""
+    g = torch.Generator(device="cpu").manual_seed(21)
+    N, K, M = 3584, 18944, 32
+    w = torch.randint(-2 ** 31, 2 ** 31 - 1, (N, K // 8), dtype=torch.int32, generator=g).to(dev)
+    s = (torch.rand(N, K // 64, generator=g) * 0.0015 + 0.0005).half().to(dev)
+    b = (-7.5 * s.float() + 1e-4 * torch.randn(N, K // 64, generator=g).to(dev)).half()
+    x = torch.randn(M, K, generator=g).half().to(dev)
+    slabs = ops.slab_count(K, 32)
+    full = ops.slab_sum(ops.quantized_matmul_slabs(x, w, s, b, 32), slabs, M, N)
+    assert torch.isfinite(full).all()
+    # row 5 alone, and rows 3..12 alone, give the same bits as inside the batch of 32
+    one = ops.slab_sum(ops.quantized_matmul_slabs(x[5:6].contiguous(), w, s, b, 32), slabs, 1, N)
+    assert torch.equal(one[0], full[5])
+    some = ops.slab_sum(ops.quantized_matmul_slabs(x[3:13].contiguous(), w, s, b, 32), slabs, 10, N)
+    assert torch.equal(some, full[3:13])
+    # another slab length: same products, another order of the fp32 sums
+    other = ops.slab_sum(ops.quantized_matmul_slabs(x, w, s, b, 16), ops.slab_count(K, 16), M, N)
+    rms = full.float().pow(2).mean().sqrt()
+    assert (other.float() - full.float()).abs().max() <= 2e-3 * rms
+    # the streaming kernel (exact weights, fp32 accumulation) within the stated tolerance
+    stream = ops.quantized_matmul(x, w, s, b)
+    assert (stream.float() - full.float()).abs().max() <= TOL * rms
+    # linear in x: f(x) + f(y) = f(x + y) up to the fp16 roundings of x + y and of the three results
+    y = torch.randn(M, K, generator=g).half().to(dev)
+    xy = (x.float() + y.float()).half()
+    f_y = ops.slab_sum(ops.quantized_matmul_slabs(y, w, s, b, 32), slabs, M, N)
+    f_xy = ops.slab_sum(ops.quantized_matmul_slabs(xy, w, s, b, 32), slabs, M, N)
+    assert (f_xy.float() - full.float() - f_y.float()).abs().max() <= TOL * f_xy.float().pow(2).mean().sqrt()
+
+
+@pytest.mark.parametrize("graph", [False, True])
+def test_device_loop_with_slab_projections(dev, graph):
+    """The device-resident loop with q|k|v, o and down of both models on the slab kernel emits
+    the target's greedy stream."""
+    from mlx_eagle_spec_decoding_tree_amd import llama, spec
+    from test_gpu_draft import assert_greedy_stream
+
+    targs = synth.tiny(layers=2, hidden=512, inter=1024, heads=4, kv_heads=2, head_dim=128, vocab=1024,
+                       attention_bias=True)
+    dargs = synth.tiny(layers=1, hidden=512, inter=512, heads=8, kv_heads=2, head_dim=64, vocab=1024)
+    tw = synth.make_model_weights(targs, seed=31)
+    dw = synth.make_model_weights(dargs, seed=32)
+    target, draft = llama.Model.from_numpy(targs, tw, dev), llama.Model.from_numpy(dargs, dw, dev)
+    rng = np.random.default_rng(33)
+    prompt = rng.integers(0, 1024, 45).astype(np.int32)
+    plan = dict(qkv=8, o=8, down=8)
+    dec = spec.SpeculativeDecoder(target, draft, capacity=256, k=8, depth=3, verify_num_tokens=31,
+                                  slab_plan=plan, draft_slab_plan=plan)
+    assert dec.verifier.slab == plan and dec.draft.slab == plan
+    first = dec.prefill(to_dev(prompt.astype(np.int64), dev))
+    if graph:
+        dec.capture()
+    tokens = dec.generate(5)
+    assert len(tokens) >= 5
+    reference = llama.Model.from_numpy(targs, tw, dev)
+    assert_greedy_stream(reference, prompt, [first] + tokens, dev)
