@@ -189,8 +189,8 @@ def main():
     ver.attn.normal_()
     ver.act.normal_()
 
-    def qmm_only():
-        for wq, sc, bi, bias, x, out, form in launches:
+    def qmm_only(subset=None):
+        for wq, sc, bi, bias, x, out, form in (launches if subset is None else subset):
             if form is True:
                 ops.quantized_matmul_swiglu(x, wq, sc, bi, bias=bias, out=out)
             elif form:
@@ -211,6 +211,21 @@ def main():
                 "avg_launch_us": round(qmm_ms * 1e3 / n_launch, 3),
                 "algorithmic_bytes_per_launch": round(alg / n_launch),
                 "step_frac": round((alg + kv_bytes) / (ms_per_step * 1e-3) / 1e9 / HBM_PEAK_GBS, 4)}
+
+    # the same for each of the two kernels on its own launches
+    per_kernel = {}
+    for kname, sub in (("qmm_w4g64_kernel", [l for l in launches if l[6] is True or not l[6]]),
+                       ("qmm_slab_w4g64_kernel", [l for l in launches if l[6] and l[6] is not True])):
+        if not sub:
+            continue
+        st, _ = graph_time_ms(torch, lambda: qmm_only(sub), reps=10)
+        sub_ms = float(np.median(st))
+        sub_alg = sum(qmm_bytes(NODES, l[0].shape[0], l[0].shape[1] * 8, l[5].shape[-1]) for l in sub)
+        per_kernel[kname] = {"launches_per_step": len(sub), "avg_launch_us": round(sub_ms * 1e3 / len(sub), 3),
+                             "algorithmic_bytes_per_launch": round(sub_alg / len(sub)),
+                             "achieved": round(sub_alg / (sub_ms * 1e-3) / 1e9, 1),
+                             "frac": round(sub_alg / (sub_ms * 1e-3) / 1e9 / HBM_PEAK_GBS, 4)}
+    roofline["per_kernel"] = per_kernel
 
     if opt.sweep:
         sweep(torch, ops, dev, args)
