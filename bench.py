@@ -413,7 +413,9 @@ def sweep(torch, ops, dev, args):
     """QMM microbenchmark over the projection shapes, weights rotated over > 1 GB of
     distinct copies so that no replay is served from cache."""
     per_layer, head = qmm_shapes(args)
-    shapes = [("cfg1", 8192, 2048)] + [s for s in per_layer if s[0] in ("q", "k", "gate", "down")] + [head]
+    D, Hq, Gk, hdim = args.hidden_size, args.num_attention_heads, args.num_key_value_heads, args.head_dim
+    shapes = ([("cfg1", 8192, 2048)] + [s for s in per_layer if s[0] in ("q", "k", "gate", "down")]
+              + [("q|k|v", (Hq + 2 * Gk) * hdim, D), head])
     print(f"{'shape':>8} {'N':>7} {'K':>6} {'M':>3} {'us':>9} {'GB/s':>8} {'frac':>6}", file=sys.stderr)
     for name, N, K in shapes:
         wbytes = 0.5625 * N * K
@@ -433,8 +435,22 @@ def sweep(torch, ops, dev, args):
             ts, _ = graph_time_ms(torch, fn, reps=5)
             us = float(np.median(ts)) * 1e3 / iters
             gbs = qmm_bytes(M, N, K) / us / 1e3
-            print(f"{name:>8} {N:>7} {K:>6} {M:>3} {us:>9.2f} {gbs:>8.0f} {gbs / HBM_PEAK_GBS:>6.3f}",
-                  file=sys.stderr, flush=True)
+            line = f"{name:>8} {N:>7} {K:>6} {M:>3} {us:>9.2f} {gbs:>8.0f} {gbs / HBM_PEAK_GBS:>6.3f}"
+            steps = ops.slab_steps(M, N, K)
+            if steps:
+                # the slab form at the library's slab length (partial sums only: their sum is
+                # taken by the kernel that reads them)
+                part = torch.empty(ops.slab_count(K, steps) * 32 * N, dtype=torch.float32, device=dev)
+
+                def fn_slab():
+                    for i in range(iters):
+                        ops.quantized_matmul_slabs(x, ws[i % ncopy], ss[i % ncopy], bs[i % ncopy], steps, partial=part)
+
+                ts, _ = graph_time_ms(torch, fn_slab, reps=5)
+                us_s = float(np.median(ts)) * 1e3 / iters
+                gbs_s = qmm_bytes(M, N, K) / us_s / 1e3
+                line += f"   slab form ({steps} steps per slab): {us_s:.2f} us {gbs_s:.0f} GB/s {gbs_s / HBM_PEAK_GBS:.3f}"
+            print(line, file=sys.stderr, flush=True)
         del ws, ss, bs
 
 
