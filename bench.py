@@ -450,6 +450,16 @@ def sweep(torch, ops, dev, args):
                 us_s = float(np.median(ts)) * 1e3 / iters
                 gbs_s = qmm_bytes(M, N, K) / us_s / 1e3
                 line += f"   slab form ({steps} steps per slab): {us_s:.2f} us {gbs_s:.0f} GB/s {gbs_s / HBM_PEAK_GBS:.3f}"
+
+                nsl = ops.slab_count(K, steps)
+
+                def fn_auto():            # the slab form and the sum of its slabs as a launch of its own
+                    for i in range(iters):
+                        ops.quantized_matmul_slabs(x, ws[i % ncopy], ss[i % ncopy], bs[i % ncopy], steps, partial=part)
+                        ops.slab_sum(part, nsl, M, N, out=o)
+
+                ts, _ = graph_time_ms(torch, fn_auto, reps=5)
+                line += f"   with the sum as a second launch: {float(np.median(ts)) * 1e3 / iters:.2f} us"
             print(line, file=sys.stderr, flush=True)
         del ws, ss, bs
 
