@@ -126,16 +126,19 @@ __global__ __launch_bounds__(256) void qmm_gemm_w4g64_kernel(
     if (nrow[nt] > N - 1) nrow[nt] = N - 1;
   }
 
-  half8_t xreg[PP];                         // x of the next step
+  // x is requested one step ahead, or two with the small blocks: their few matrix instructions
+  // per step do not cover the latency of that load, and a step cannot be shorter than the lead
+  constexpr int XD = MT <= 2 ? 2 : 1;
+  half8_t xreg[XD][PP];
   uint4_t wreg[2][NTW];                     // packed weights, two steps in flight
   constexpr bool SBV = SBW > 1;
   typedef half_t sbvec_t __attribute__((ext_vector_type(SBV ? SBW : 2)));
   half_t sreg[2][NTW], breg[2][NTW];        // SBW = 1: scale and bias of those steps
   sbvec_t s8[2][NTW], b8[2][NTW];           // SBW > 1: of this chunk of SBW steps and of the next
   half8_t af[2][NTW][4];                    // expanded weights of this step and the next
-  auto fetch_x = [&](int ks) {
+  auto fetch_x = [&](int ks, int set) {
 #pragma unroll
-    for (int g = 0; g < PP; ++g) xreg[g] = *reinterpret_cast<const half8_t*>(xp + (long)ks * BK + g * 8);
+    for (int g = 0; g < PP; ++g) xreg[set][g] = *reinterpret_cast<const half8_t*>(xp + (long)ks * BK + g * 8);
   };
   auto fetch_w = [&](int ks, int p) {
 #pragma unroll
@@ -154,10 +157,10 @@ __global__ __launch_bounds__(256) void qmm_gemm_w4g64_kernel(
       b8[q][nt] = *reinterpret_cast<const sbvec_t*>(b + (long)nrow[nt] * KG + chunk * SBW);
     }
   };
-  auto stash = [&](int buf) {
+  auto stash = [&](int buf) {                // x of a step travels in register set (step % XD)
 #pragma unroll
     for (int g = 0; g < PP; ++g)
-      *reinterpret_cast<half8_t*>(&xs[buf][xr * XS + xh * (BK / TPR) + g * 8]) = permute8(xreg[g]);
+      *reinterpret_cast<half8_t*>(&xs[buf][xr * XS + xh * (BK / TPR) + g * 8]) = permute8(xreg[buf % XD][g]);
   };
   // word j of the weight tiles of register set p; e = index of their step within the chunk of
   // SBW (SBW = first step of the next chunk)
@@ -180,7 +183,8 @@ __global__ __launch_bounds__(256) void qmm_gemm_w4g64_kernel(
       for (int i = 0; i < 16; ++i) acc[nt][mt][i] = 0.f;
 
   const int chunks = steps / SBW;
-  fetch_x(0);
+  fetch_x(0, 0);
+  if (XD == 2) fetch_x(steps > 1 ? 1 : 0, 1);
   fetch_w(0, 0);
   fetch_w(steps > 1 ? 1 : 0, 1);
   if (SBV) {
@@ -193,15 +197,16 @@ __global__ __launch_bounds__(256) void qmm_gemm_w4g64_kernel(
   __syncthreads();
 
   // One K step, p = ks & 1: LDS buffer p holds x of this step and af[p] its expanded weights;
-  // register set p ^ 1 holds the packed weights of the next step, which are expanded between
-  // this step's matrix instructions; set p is free for the loads of step ks + 2.  Loaded
+  // register set p ^ 1 holds the packed weights and the x of the next step (the weights are
+  // expanded between this step's matrix instructions, the x goes to LDS at its end); set p is
+  // free for the loads of step ks + 2.  Loaded
   // values are used where they were loaded (a copy of a register with a load in flight would
   // wait for the load), and the loads are issued first (left alone, the scheduler sinks them
   // to the end of the step, where the in-order counter waits for them at once).
   auto body = [&](int ks, auto E) {
     constexpr int e = decltype(E)::value;   // step within its chunk (SBW > 1) / parity of the step
     constexpr int p = e & 1;
-    fetch_x(ks + 1 < steps ? ks + 1 : steps - 1);
+    fetch_x(ks + XD < steps ? ks + XD : steps - 1, p % XD);   // that set's x is in LDS already
     fetch_w(ks + 2 < steps ? ks + 2 : steps - 1, p);
     __builtin_amdgcn_sched_barrier(0);
 #pragma unroll
