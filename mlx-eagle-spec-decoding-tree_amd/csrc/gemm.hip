@@ -130,7 +130,10 @@ __global__ __launch_bounds__(256) void qmm_gemm_w4g64_kernel(
   // per step do not cover the latency of that load, and a step cannot be shorter than the lead
   constexpr int XD = MT <= 2 ? 2 : 1;
   half8_t xreg[XD][PP];
-  uint4_t wreg[2][NTW];                     // packed weights, two steps in flight
+  // packed weights: two steps in flight, four with the small blocks (where the unrolled loop
+  // makes the register set of a step a constant), for the same reason
+  constexpr int WD = (MT <= 2 && SBW >= 4) ? 4 : 2;
+  uint4_t wreg[WD][NTW];
   constexpr bool SBV = SBW > 1;
   typedef half_t sbvec_t __attribute__((ext_vector_type(SBV ? SBW : 2)));
   half_t sreg[2][NTW], breg[2][NTW];        // SBW = 1: scale and bias of those steps
@@ -170,7 +173,7 @@ __global__ __launch_bounds__(256) void qmm_gemm_w4g64_kernel(
       const half_t sc = SBV ? s8[e / SBW][nt][e % SBW] : sreg[p][nt];
       const half_t bi = SBV ? b8[e / SBW][nt][e % SBW] : breg[p][nt];
       const half_t b16 = (half_t)((float)bi - 16.f * (float)sc);
-      af[p][nt][j] = dequant_word(wreg[p][nt][j], half2_t{sc, sc}, half2_t{b16, b16});
+      af[p][nt][j] = dequant_word(wreg[e % WD][nt][j], half2_t{sc, sc}, half2_t{b16, b16});
     }
   };
 
@@ -185,8 +188,8 @@ __global__ __launch_bounds__(256) void qmm_gemm_w4g64_kernel(
   const int chunks = steps / SBW;
   fetch_x(0, 0);
   if (XD == 2) fetch_x(steps > 1 ? 1 : 0, 1);
-  fetch_w(0, 0);
-  fetch_w(steps > 1 ? 1 : 0, 1);
+#pragma unroll
+  for (int i = 0; i < WD; ++i) fetch_w(i < steps ? i : steps - 1, i);
   if (SBV) {
     fetch_sb(0, 0);
     fetch_sb(chunks > 1 ? 1 : 0, 1);
@@ -207,7 +210,7 @@ __global__ __launch_bounds__(256) void qmm_gemm_w4g64_kernel(
     constexpr int e = decltype(E)::value;   // step within its chunk (SBW > 1) / parity of the step
     constexpr int p = e & 1;
     fetch_x(ks + XD < steps ? ks + XD : steps - 1, p % XD);   // that set's x is in LDS already
-    fetch_w(ks + 2 < steps ? ks + 2 : steps - 1, p);
+    fetch_w(ks + WD < steps ? ks + WD : steps - 1, e % WD);   // that set was expanded a step ago
     __builtin_amdgcn_sched_barrier(0);
 #pragma unroll
     for (int j = 0; j < 4; ++j) {
