@@ -61,7 +61,8 @@ def sanitize(weights):
 def load_weights(model_path, device="cpu"):
     """All tensors of every shard as a flat dict of torch tensors on `device`.  Packed uint32
     words are kept bit for bit (as int32 storage); floating-point tensors that are not fp16
-    (bf16 exports) are converted to fp16, the type the kernels compute in."""
+    (bf16 exports) are converted to fp16, the type the kernels compute in; a value that does not
+    fit fp16 raises ValueError."""
     from safetensors import safe_open
 
     out = {}
@@ -72,7 +73,12 @@ def load_weights(model_path, device="cpu"):
                 if t.dtype == torch.uint32:
                     t = t.view(torch.int32)
                 elif t.dtype.is_floating_point and t.dtype != torch.float16:
-                    t = t.to(torch.float16)
+                    wide = t
+                    t = wide.to(torch.float16)
+                    # bf16 / fp32 reach beyond fp16's range: refuse rather than carry inf
+                    if bool((torch.isinf(t) & ~torch.isinf(wide)).any()):
+                        raise ValueError(f"{key} ({wide.dtype}) holds values beyond the fp16 range; "
+                                         "the kernels compute in fp16")
                 out[key] = t.contiguous().to(device)
     return sanitize(out)
 

@@ -164,20 +164,48 @@ def make_model_weights(args: ModelArgs, seed=42, layers=None, gain=1.0):
     return out
 
 
-def inv_freqs(args: ModelArgs):
-    """fp32 inverse-frequency table and scaling factor for the default / linear
-    rope types: inv_freq[i] = 2 ** (-log2(theta) * 2i / head_dim)
-    (mlx_llama.py:105-113)."""
+def inv_freqs(args: ModelArgs, seq_len=None):
+    """fp32 inverse-frequency table and scaling factor of the rotary embedding
+    (mlx_llama.py:98-116).
+
+    default / linear: inv_freq[i] = 2 ** (-log2(theta) * 2i / head_dim), scaling factor
+    1 / factor for linear (:105-113).
+    llama3: the table of the Llama-3.1 rule, 1 / fast_rope._freqs in the reference (:114-116):
+    pairs whose wavelength exceeds original_max_position_embeddings / low_freq_factor are slowed
+    by `factor`, those below original_max_position_embeddings / high_freq_factor are kept, and
+    the band between is interpolated in the frequency.
+    dynamic: the NTK rule, theta * (factor * L / max_pos - (factor - 1)) ** (hd / (hd - 2)) with
+    L = max(seq_len, max_position_embeddings); up to max_position_embeddings tokens (seq_len None)
+    this is the default table."""
     rope_type = "default"
-    if args.rope_scaling is not None:
-        rope_type = args.rope_scaling.get("type") or args.rope_scaling.get("rope_type", "default")
-    if rope_type not in ("default", "linear"):
-        raise NotImplementedError("only default/linear rope tables are generated here")
+    rs = args.rope_scaling
+    if rs is not None:
+        rope_type = rs.get("type") or rs.get("rope_type", "default")
+    if rope_type not in ("default", "linear", "llama3", "dynamic"):
+        raise NotImplementedError(f"rope type {rope_type!r}")
     hd = args.head_dim
-    expo = (-np.log2(np.float32(args.rope_theta)) * np.arange(0, hd, 2, dtype=np.float32)
+    theta = float(args.rope_theta)
+    if rope_type == "dynamic":
+        max_pos = args.max_position_embeddings
+        if not max_pos:
+            raise ValueError("dynamic rope scaling needs max_position_embeddings")
+        L = max(int(seq_len or max_pos), int(max_pos))
+        theta = theta * ((rs["factor"] * L / max_pos) - (rs["factor"] - 1)) ** (hd / (hd - 2))
+    expo = (-np.log2(np.float32(theta)) * np.arange(0, hd, 2, dtype=np.float32)
             / np.float32(hd)).astype(np.float32)
     inv = np.exp2(expo).astype(np.float32)
-    scale = 1.0 / args.rope_scaling["factor"] if rope_type == "linear" else 1.0
+    if rope_type == "llama3":
+        factor = np.float32(rs["factor"])
+        low = np.float32(rs.get("low_freq_factor", 1.0))
+        high = np.float32(rs.get("high_freq_factor", 4.0))
+        old_len = np.float32(rs.get("original_max_position_embeddings", 8192))
+        wavelen = (np.float32(2 * np.pi) / inv).astype(np.float32)
+        slowed = np.where(wavelen > old_len / low, inv / factor, inv).astype(np.float32)
+        smooth = ((old_len / wavelen - low) / (high - low)).astype(np.float32)
+        mixed = ((1 - smooth) * slowed / factor + smooth * slowed).astype(np.float32)
+        medium = ~(wavelen < old_len / high) & ~(wavelen > old_len / low)
+        inv = np.where(medium, mixed, slowed).astype(np.float32)
+    scale = 1.0 / rs["factor"] if rope_type == "linear" else 1.0
     return inv, float(scale)
 
 

@@ -169,3 +169,54 @@ def test_loaded_model_matches_in_memory_model(tmp_path, tiny):
         outs.append(logits.float().cpu())
     assert torch.isfinite(outs[0]).all()
     assert torch.equal(outs[0], outs[1])
+
+
+def test_bf16_values_beyond_fp16_are_refused(tmp_path, tiny):
+    """bf16 exports are converted to fp16; a scale that fp16 cannot hold must not become inf
+    silently."""
+    from safetensors.torch import save_file as save_torch
+
+    args, weights = tiny
+    with open(os.path.join(tmp_path, "config.json"), "w") as f:
+        json.dump(config_of(args), f)
+    tw = {}
+    for k, v in weights.items():
+        t = torch.from_numpy(v.view(np.int32) if v.dtype == np.uint32 else v)
+        tw[k] = t.to(torch.bfloat16) if t.dtype == torch.float16 else t
+    save_torch(tw, os.path.join(tmp_path, "model.safetensors"))
+    got = checkpoint.load_weights(tmp_path)
+    assert got["model.norm.weight"].dtype == torch.float16
+    bad = dict(tw)
+    bad["model.norm.weight"] = tw["model.norm.weight"].clone()
+    bad["model.norm.weight"][3] = 1e5
+    save_torch(bad, os.path.join(tmp_path, "model.safetensors"))
+    with pytest.raises(ValueError, match="fp16 range"):
+        checkpoint.load_weights(tmp_path)
+
+
+LLAMA3_SCALING = {"factor": 32.0, "low_freq_factor": 1.0, "high_freq_factor": 4.0,
+                  "original_max_position_embeddings": 8192, "rope_type": "llama3"}
+
+
+def test_llama32_style_config_loads_with_the_llama3_table(tmp_path):
+    """The configuration of the model the reference's own test loads
+    (mlx_eagle_tests.py:19: Llama-3.2-1B): rope_scaling of type llama3, tied head, head_dim 64."""
+    args = synth.ModelArgs(model_type="llama", hidden_size=256, num_hidden_layers=1,
+                           intermediate_size=512, num_attention_heads=4, num_key_value_heads=2,
+                           head_dim=64, vocab_size=512, rms_norm_eps=1e-5, rope_theta=5e5,
+                           attention_bias=False, tie_word_embeddings=True,
+                           max_position_embeddings=131072, rope_scaling=dict(LLAMA3_SCALING))
+    weights = synth.make_model_weights(args, seed=3)
+    cfg = config_of(args, rope_scaling=dict(LLAMA3_SCALING), max_position_embeddings=131072,
+                    architectures=["LlamaForCausalLM"])
+    write_checkpoint(tmp_path, args, weights, shards=1, cfg=cfg)
+    got = checkpoint.model_args_from_config(checkpoint.load_config(tmp_path))
+    assert got.rope_scaling == LLAMA3_SCALING and got.max_position_embeddings == 131072
+    inv, scale = synth.inv_freqs(got)
+    plain, _ = synth.inv_freqs(synth.ModelArgs(model_type="llama", hidden_size=256, num_attention_heads=4,
+                                               head_dim=64, rope_theta=5e5))
+    assert scale == 1.0 and inv.shape == (32,) and inv.dtype == np.float32
+    assert np.array_equal(inv[:8], plain[:8])                    # short wavelengths untouched
+    assert np.allclose(inv[-4:], plain[-4:] / 32.0, rtol=1e-6)   # long ones slowed by `factor`
+    model, _ = checkpoint.load_model(tmp_path, "cpu")
+    assert np.array_equal(model.model.layers[0].self_attn._inv_freqs.numpy(), inv)

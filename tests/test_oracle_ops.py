@@ -195,3 +195,52 @@ def test_rmsnorm_silu_add_argmax():
     lg[2, [5, 700]] = lg[2].max()                                   # tie -> first index
     assert np.array_equal(oracle.argmax_rows(lg), np.argmax(lg.astype(np.float32), axis=-1))
     assert oracle.argmax_rows(lg)[2] == min(5, int(np.argmax(lg[2].astype(np.float32))))
+
+
+# ----------------------------------------------------------------------------- rope tables
+def _hf_inv_freq(rope_type, theta, hd, scaling, max_pos, seq_len=None):
+    from transformers import LlamaConfig
+    from transformers.modeling_rope_utils import ROPE_INIT_FUNCTIONS
+
+    params = dict(scaling, rope_type=rope_type, rope_theta=theta)
+    cfg = LlamaConfig(hidden_size=hd * 4, num_attention_heads=4, head_dim=hd,
+                      max_position_embeddings=max_pos, rope_parameters=params)
+    inv, att = ROPE_INIT_FUNCTIONS[rope_type](cfg, "cpu", seq_len=seq_len)
+    assert att == 1.0
+    return inv.numpy()
+
+
+@pytest.mark.parametrize("hd,theta,factor,old_len", [(64, 5e5, 32.0, 8192), (128, 5e5, 8.0, 8192),
+                                                      (128, 1e6, 4.0, 4096)])
+def test_llama3_inv_freq_table_against_transformers(hd, theta, factor, old_len):
+    """The table the reference takes from 1 / fast_rope._freqs (mlx_llama.py:114-116), pinned
+    against transformers' _compute_llama3_parameters to fp32 rounding; all three bands
+    (kept, interpolated, slowed) are populated."""
+    scaling = {"factor": factor, "low_freq_factor": 1.0, "high_freq_factor": 4.0,
+               "original_max_position_embeddings": old_len}
+    args = synth.ModelArgs(model_type="llama", hidden_size=hd * 4, num_attention_heads=4, head_dim=hd,
+                           rope_theta=theta, max_position_embeddings=131072,
+                           rope_scaling=dict(scaling, rope_type="llama3"))
+    inv, scale = synth.inv_freqs(args)
+    want = _hf_inv_freq("llama3", theta, hd, scaling, 131072)
+    assert scale == 1.0 and inv.dtype == np.float32
+    assert np.allclose(inv, want, rtol=4e-6, atol=0), np.max(np.abs(inv / want - 1))
+    plain, _ = synth.inv_freqs(synth.ModelArgs(hidden_size=hd * 4, num_attention_heads=4, head_dim=hd,
+                                               rope_theta=theta))
+    ratio = plain / inv
+    assert (np.isclose(ratio, 1.0, rtol=1e-5)).any() and (np.isclose(ratio, factor, rtol=1e-5)).any()
+    assert ((ratio > 1.001) & (ratio < factor * 0.999)).any()
+
+
+def test_dynamic_inv_freq_table_against_transformers():
+    scaling = {"factor": 2.0}
+    args = synth.ModelArgs(hidden_size=512, num_attention_heads=4, head_dim=128, rope_theta=1e4,
+                           max_position_embeddings=2048, rope_scaling={"factor": 2.0, "type": "dynamic"})
+    plain, _ = synth.inv_freqs(synth.ModelArgs(hidden_size=512, num_attention_heads=4, head_dim=128,
+                                               rope_theta=1e4))
+    inv, scale = synth.inv_freqs(args)
+    assert scale == 1.0 and np.allclose(inv, plain, rtol=2e-6)       # within max_position_embeddings
+    for L in (2048, 3000, 8192):
+        got, _ = synth.inv_freqs(args, seq_len=L)
+        want = _hf_inv_freq("dynamic", 1e4, 128, scaling, 2048, seq_len=L)
+        assert np.allclose(got, want, rtol=2e-5), (L, np.max(np.abs(got / want - 1)))
