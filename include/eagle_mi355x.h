@@ -99,6 +99,21 @@ int eagle_qmm_gemm_w4g64_f16(const void* x, const uint32_t* wq, const void* scal
                              const void* biases, const void* bias, void* out, int M, int N, int K,
                              int group_size, int bits, eagle_stream_t stream);
 
+/* The same product (and its SwiGLU form when `swiglu` != 0, weights interleaved as for
+ * eagle_qmm_swiglu_w4g64_f16, out [M, N/2]) for 1..32 rows with x resident in registers: one
+ * workgroup per compute unit, the K range split in units of 512 over its waves, whole K per
+ * workgroup, so no workspace and no counters.  K % 512 == 0 and K <= 3584
+ * (eagle_qmm_res_supported returns 1), N % 8 == 0 (N % 32 == 0 with swiglu); x, wq, scales and
+ * biases 16-byte aligned, out 8-byte aligned.  Every scale must be below 0.2499 (weights are
+ * expanded through fp16 subnormals, scale * 2^18 has to be finite in fp16); larger scales give
+ * inf / NaN, never a finite wrong value.
+ * Replaces the same call sites as eagle_qmm_w4g64_f16 (qmm_kernel.py:84-164,
+ * mlx_model_fwd_bench.py:65-73) and, with swiglu, mlx_llama.py:214-215. */
+int eagle_qmm_res_supported(int M, int N, int K);
+int eagle_qmm_res_w4g64_f16(const void* x, const uint32_t* wq, const void* scales,
+                            const void* biases, const void* bias, void* out, int M, int N, int K,
+                            int group_size, int bits, int swiglu, eagle_stream_t stream);
+
 /* The same product for 1..32 rows in the slab form, with the result left as fp32 partial sums:
  * every workgroup owns 128 weight rows and one K slab of `steps_per_slab` quantisation groups
  * (a multiple of 8), moves x through LDS eight groups at a time and expands the weights to fp16

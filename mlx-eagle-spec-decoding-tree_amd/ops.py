@@ -217,6 +217,37 @@ def quantized_matmul_swiglu(x, w_q, scales, biases, bias=None, out=None):
     return out
 
 
+def resident_supported(M, N, K):
+    """True when `quantized_matmul_resident` takes this shape (K a multiple of 512, <= 3584)."""
+    return bool(_lib.lib().eagle_qmm_res_supported(M, N, K))
+
+
+def quantized_matmul_resident(x, w_q, scales, biases, bias=None, out=None, swiglu=False):
+    """The same product as `quantized_matmul` (or `quantized_matmul_swiglu` with swiglu=True)
+    through the kernel that keeps x in registers and splits K over the waves of one workgroup
+    per compute unit (mlx_model_fwd_bench.py:65-73; mlx_llama.py:214-215)."""
+    _need_cuda(x, w_q, scales, biases, bias)
+    x = _f16(x, "x")
+    w_q = as_packed_u32(w_q)
+    scales, biases = _f16(scales, "scales"), _f16(biases, "biases")
+    *lead, K = x.shape
+    M = reduce(lambda a, b: a * b, lead, 1)
+    N = w_q.shape[0]
+    if w_q.shape[1] * 8 != K or tuple(scales.shape) != (N, K // 64) or tuple(biases.shape) != (N, K // 64):
+        raise ValueError(f"shape mismatch: x {tuple(x.shape)}, w {tuple(w_q.shape)}, "
+                         f"scales {tuple(scales.shape)}, biases {tuple(biases.shape)}")
+    if bias is not None:
+        bias = _f16(bias, "bias")
+        if tuple(bias.shape) != (N,):
+            raise ValueError("bias must have shape [N]")
+    if out is None:
+        out = torch.empty((*lead, N // 2 if swiglu else N), dtype=torch.float16, device=x.device)
+    rc = _lib.lib().eagle_qmm_res_w4g64_f16(_ptr(x), _ptr(w_q), _ptr(scales), _ptr(biases), _ptr(bias),
+                                            _ptr(out), M, N, K, 64, 4, int(bool(swiglu)), _stream())
+    _lib.check(rc, "quantized_matmul_resident")
+    return out
+
+
 def matmul(x, w, s, b, group_size, **_ignored):
     """Same contract as the reference's `qmm_kernel.matmul` (qmm_kernel.py:84-164):
     returns a one-element list.  The Metal tuning keywords are accepted and ignored."""

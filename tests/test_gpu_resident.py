@@ -1,0 +1,95 @@
+"""The matmul with x resident in registers (csrc/resident.hip) vs the CPU oracle, through the
+C ABI: plain and SwiGLU forms, ragged rows, edge shapes, and the cfg2 shapes it serves."""
+import numpy as np
+import pytest
+import torch
+
+from mlx_eagle_spec_decoding_tree_amd import _lib, ops, synth
+from oracle import oracle
+from util import TOL, layer_to_dev, rel_err, to_dev
+
+pytestmark = pytest.mark.gpu
+
+
+@pytest.mark.parametrize("N,K", [(8, 512), (40, 1024), (136, 1536), (512, 3584), (8192, 2048),
+                                 (3584, 3584), (4608, 3584)])
+@pytest.mark.parametrize("M", [1, 8, 17, 32])
+def test_plain_form(dev, M, N, K):
+    print(f"resident qmm M={M} N={N} K={K}", flush=True)
+    assert ops.resident_supported(M, N, K)
+    rng = np.random.default_rng(N + K + M)
+    bias = (N // 8) % 2 == 1
+    layer = synth.make_qlinear(rng, N, K, bias=bias)
+    x = synth.make_x(rng, M, K)
+    want = oracle.qmm(x, layer["weight"], layer["scales"], layer["biases"], layer.get("bias"))
+    d = layer_to_dev(layer, dev)
+    got = ops.quantized_matmul_resident(to_dev(x, dev), d["weight"], d["scales"], d["biases"],
+                                        bias=d.get("bias"))
+    torch.cuda.synchronize()
+    assert rel_err(got.cpu().numpy(), want) <= TOL
+
+
+def test_known_answers(dev):
+    """One-hot x rows give the dequantised weight column exactly (pins the nibble order and the
+    subnormal expansion: fp16(s q + b) with a single rounding); s = 1/8, b = 0 with integer x is
+    an exact integer matmul."""
+    rng = np.random.default_rng(3)
+    N, K = 96, 1024
+    layer = synth.make_qlinear(rng, N, K)
+    cols = rng.choice(K, size=32, replace=False)
+    x = np.zeros((32, K), np.float16)
+    x[np.arange(32), cols] = 1.0
+    d = layer_to_dev(layer, dev)
+    got = ops.quantized_matmul_resident(to_dev(x, dev), d["weight"], d["scales"], d["biases"]).cpu().numpy()
+    q = synth.unpack_nibbles(layer["weight"])[:, cols].astype(np.float32)
+    s = layer["scales"].astype(np.float32)[:, cols // 64]
+    b = layer["biases"].astype(np.float32)[:, cols // 64]
+    want = (s * q + b).astype(np.float16).T
+    assert np.array_equal(got, want)
+    layer["scales"][:] = np.float16(0.125)
+    layer["biases"][:] = np.float16(0)
+    xi = rng.integers(-3, 4, size=(8, K)).astype(np.float16)
+    d = layer_to_dev(layer, dev)
+    got = ops.quantized_matmul_resident(to_dev(xi, dev), d["weight"], d["scales"], d["biases"]).cpu().numpy()
+    want = xi.astype(np.float64) @ synth.unpack_nibbles(layer["weight"]).astype(np.float64).T / 8
+    assert np.array_equal(got.astype(np.float64), want.astype(np.float16).astype(np.float64))
+
+
+@pytest.mark.parametrize("I,K,bias", [(16, 512, False), (48, 1024, True), (272, 1536, True), (18944, 3584, True)])
+def test_swiglu_form(dev, I, K, bias):
+    for M in (1, 8, 17, 32):
+        print(f"resident swiglu I={I} K={K} M={M}", flush=True)
+        rng = np.random.default_rng(I + K + M)
+        g = synth.make_qlinear(rng, I, K, bias=bias, gain=1.0)
+        u = synth.make_qlinear(rng, I, K, bias=bias, gain=1.0)
+        x = synth.make_x(rng, M, K)
+        want = oracle.silu_mul(oracle.qmm(x, g["weight"], g["scales"], g["biases"], g.get("bias")),
+                               oracle.qmm(x, u["weight"], u["scales"], u["biases"], u.get("bias")))
+        gd, ud = layer_to_dev(g, dev), layer_to_dev(u, dev)
+        keys = ["weight", "scales", "biases"] + (["bias"] if bias else [])
+        inter = {k: ops.interleave_gate_up(gd[k], ud[k]) for k in keys}
+        got = ops.quantized_matmul_resident(to_dev(x, dev), inter["weight"], inter["scales"], inter["biases"],
+                                            bias=inter.get("bias"), swiglu=True)
+        torch.cuda.synchronize()
+        assert tuple(got.shape) == (M, I)
+        # The product of two rounded values: where |g| and |u| are several sigma, one fp16 ulp of
+        # g (the sum lands on the other side of a rounding boundary) moves the output by more
+        # than 2e-2 of the output RMS (seen: g 2.986 vs 2.984, u 3.33, output 9.48 vs 9.46 with an
+        # RMS of 0.6).  So the bound is the QMM one plus two fp16 ulps of the expected value, and
+        # the RMS error, which no single element dominates, has to stay 10 times below the bound.
+        g64, w64 = got.cpu().numpy().astype(np.float64), want.astype(np.float64)
+        rms = np.sqrt(np.mean(w64 * w64))
+        ulp = 2.0 ** (np.floor(np.log2(np.maximum(np.abs(w64), 2.0 ** -14))) - 10)
+        assert np.all(np.abs(g64 - w64) <= TOL * rms + 2 * ulp)
+        assert np.sqrt(np.mean((g64 - w64) ** 2)) <= 0.1 * TOL * rms
+
+
+def test_rejects_what_it_does_not_take(dev):
+    assert not ops.resident_supported(8, 64, 4096)
+    assert not ops.resident_supported(8, 64, 896)
+    assert not ops.resident_supported(33, 64, 512)
+    x = torch.zeros((8, 4096), dtype=torch.float16, device=dev)
+    w = torch.zeros((64, 512), dtype=torch.int32, device=dev)
+    s = torch.zeros((64, 64), dtype=torch.float16, device=dev)
+    with pytest.raises(ValueError):
+        ops.quantized_matmul_resident(x, w, s, s)
