@@ -536,8 +536,10 @@ class TreeVerifier:
         self.mask_index.copy_(mask_index.reshape(-1))
         self.mask_bits.copy_(mask_bits.reshape(-1))
 
-    def forward(self):
-        """Enqueue the whole step on the current stream (no synchronisation)."""
+    def forward(self, tap=None):
+        """Enqueue the whole step on the current stream (no synchronisation).  tap(i, h):
+        called after decoder layer i with the residual stream `self.h` (eager runs only: tests
+        that follow the error through the layers)."""
         L = _lib.lib()
         m = self.model
         args = self.args
@@ -625,6 +627,8 @@ class TreeVerifier:
                 ops.quantized_matmul(self.act, mlp.down_proj.weight, mlp.down_proj.scales,
                                      mlp.down_proj.biases, bias=mlp.down_proj.bias, out=self.down)
                 ops.rms_norm(self.down, nxt, args.rms_norm_eps, residual=self.h, out=self.hn, h_out=self.h)
+            if tap is not None:
+                tap(i, self.h)
         head = m.model.embed_tokens if args.tie_word_embeddings else m.lm_head
         ops.quantized_matmul(self.hn, head.weight, head.scales, head.biases, out=self.logits)
         ops.argmax_rows(self.logits, out=self.node_argmax)

@@ -52,6 +52,15 @@ ORC_API void orc_f2h(const float* in, uint16_t* out, long n) {
  * added to the rounded result in fp16, as the patched linear layer does after
  * the kernel returns (mlx_model_fwd_bench.py:69-71).
  */
+/* Weight rounding of orc_qmm_w4g64: 0 (default) keeps s*q + b in fp32; 1 rounds every
+ * dequantised weight to fp16 first, as the reference Metal kernel holds them (half2
+ * `w1 = w1 * s0 + b0`, kernels/progression/simd_no_swizzle_cast.metal:82-84).  Both are the
+ * reference's arithmetic (MLX CPU path and Metal path); tests use 1 to separate the rounding of
+ * the weights from other differences.  Pinned by the same float64 closed form with the
+ * weights rounded. */
+static int orc_round_weights = 0;
+ORC_API void orc_set_weight_rounding(int on) { orc_round_weights = on ? 1 : 0; }
+
 ORC_API int orc_qmm_w4g64(const uint16_t* x, const uint32_t* w, const uint16_t* s,
                           const uint16_t* b, const uint16_t* bias, uint16_t* out,
                           int M, int N, int K) {
@@ -75,6 +84,8 @@ ORC_API int orc_qmm_w4g64(const uint16_t* x, const uint32_t* w, const uint16_t* 
             wf[g * 64 + j * 8 + i] = sc * (float)((word >> (4 * i)) & 15u) + bi;
         }
       }
+      if (orc_round_weights)
+        for (int k = 0; k < K; ++k) wf[k] = h2f(f2h(wf[k]));
       for (int m = 0; m < M; ++m) {
         const float* xr = xf + (size_t)m * K;
         float acc = 0.f;

@@ -24,11 +24,12 @@ def new_cache(args, capacity, layers=None):
 
 
 def tree_forward(args, weights, inv_freq, rope_scale, token_ids, positions, mask, cache, offset,
-                 layers=None, return_hidden=False):
+                 layers=None, return_hidden=False, tap=None):
     """Logits [T, V] of T tree tokens appended at `offset`.
 
     token_ids [T] int, positions [T] int (absolute), mask [T, offset+T] additive fp16,
     cache: list of (keys, values) [G, capacity, hd] modified in place (rows offset..offset+T-1).
+    tap(i, h): called with the residual stream [T, D] after decoder layer i (tests).
     """
     T = len(token_ids)
     H, G, hd = args.num_attention_heads, args.num_key_value_heads, args.head_dim
@@ -55,6 +56,8 @@ def tree_forward(args, weights, inv_freq, rope_scale, token_ids, positions, mask
         act = oracle.silu_mul(_lin(weights, f"{p}.mlp.gate_proj", xn),
                               _lin(weights, f"{p}.mlp.up_proj", xn))
         h = oracle.add(h, _lin(weights, f"{p}.mlp.down_proj", act))
+        if tap is not None:
+            tap(i, h)
     hn = oracle.rmsnorm(h, weights["model.norm.weight"], args.rms_norm_eps)
     if return_hidden:
         return hn
@@ -64,14 +67,14 @@ def tree_forward(args, weights, inv_freq, rope_scale, token_ids, positions, mask
 
 
 def verify_step(args, weights, inv_freq, rope_scale, draft_tokens, tree_position_ids, mask_index,
-                anc, cache, offset, layers=None):
+                anc, cache, offset, layers=None, tap=None):
     """Full verification step: forward, per-node argmax, greedy acceptance, KV compaction.
     Returns dict(logits, node_argmax, retrieve_indices, best, accept_length, bonus_node,
     next_token, accept_indices, new_offset)."""
     T = len(draft_tokens)
     mask = np.concatenate([np.zeros((T, offset), np.float16), tree_oracle.additive_mask(anc)], axis=1)
     logits = tree_forward(args, weights, inv_freq, rope_scale, draft_tokens,
-                          np.asarray(tree_position_ids) + offset, mask, cache, offset, layers)
+                          np.asarray(tree_position_ids) + offset, mask, cache, offset, layers, tap=tap)
     node_argmax = oracle.argmax_rows(logits)
     ri = tree_oracle.post_process_draft_tree(tree_position_ids, T - 1, mask_index)
     best, al, bonus = tree_oracle.greedy_accept(node_argmax, draft_tokens, ri)

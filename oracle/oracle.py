@@ -43,6 +43,23 @@ def _h(a):
     return a
 
 
+class weight_rounding:
+    """Context manager: inside it `qmm` rounds every dequantised weight to fp16 before the
+    product, as the reference's Metal kernel holds them
+    (kernels/progression/simd_no_swizzle_cast.metal:82-84); outside it s*q + b stays in fp32."""
+
+    def __init__(self, on=True):
+        self.on = bool(on)
+
+    def __enter__(self):
+        lib().orc_set_weight_rounding(ctypes.c_int(int(self.on)))
+        return self
+
+    def __exit__(self, *exc):
+        lib().orc_set_weight_rounding(ctypes.c_int(0))
+        return False
+
+
 def qmm(x, w, scales, biases, bias=None):
     """out[..., N] = x[..., K] . dequant(w)[N, K]^T  (4 bit, group 64), fp16."""
     x = _h(x)

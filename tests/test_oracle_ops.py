@@ -77,6 +77,24 @@ def test_qmm_matches_torch_matmul_on_dequantised_weights():
     assert rel_err(oracle.qmm(x, layer["weight"], layer["scales"], layer["biases"]), want) <= 2e-3
 
 
+def test_qmm_with_rounded_weights_is_the_closed_form_on_fp16_weights():
+    """The oracle's second mode (weights rounded to fp16 before the product, as the reference's
+    Metal kernel holds them): float64 product over fp16(s q + b); off again after the block."""
+    rng = np.random.default_rng(4)
+    layer = synth.make_qlinear(rng, 64, 1024)
+    x = synth.make_x(rng, 8, 1024)
+    w16 = synth.dequantize(layer, np.float32).astype(np.float16).astype(np.float64)
+    want = x.astype(np.float64) @ w16.T
+    plain = oracle.qmm(x, layer["weight"], layer["scales"], layer["biases"])
+    with oracle.weight_rounding():
+        got = oracle.qmm(x, layer["weight"], layer["scales"], layer["biases"])
+    assert rel_err(got, want) <= 1.2e-3          # one fp16 rounding of the output
+    # the two modes differ by what the rounding of the weights is worth, and no more
+    assert 0 < rel_err(got, plain.astype(np.float64)) <= 5e-3
+    again = oracle.qmm(x, layer["weight"], layer["scales"], layer["biases"])
+    assert np.array_equal(again, plain)
+
+
 def test_embed_is_qmm_with_one_hot_rows():
     rng = np.random.default_rng(4)
     V, D = 64, 128
