@@ -317,7 +317,7 @@ int eagle_greedy_accept(const int32_t* node_argmax, const int32_t* draft_tokens,
 
 /* accept_candidate (mlx_eagle.py:349-376) for n_caches K or V buffers at once:
  * rows P + accept_indices[j] move to P + 1 + j for j < accept_length (gather
- * first, then scatter), then *cache_len_dev = P + accept_length + 1.
+ * first, then scatter), then *cache_len_dev = min(P + accept_length + 1, capacity).
  * caches: device array of n_caches pointers to [G,capacity,hd] fp16 buffers.
  * accept [4 + 32] int32 in the layout of eagle_greedy_accept's result. */
 int eagle_kv_compact_f16(void* const* caches_dev, int n_caches, const int32_t* accept,

@@ -92,10 +92,10 @@ __global__ __launch_bounds__(512) void tree_attn_split_kernel(
   // rows 32 * piece of q [H, q_rows, hd]); a single piece otherwise
   const int piece = blockIdx.z;
   int P = len_dev[piece];
-  if (ROPE || WIDE) {                   // never index past the cache, whatever the counter says
-    if (P > cap - Tk) P = (int)(cap - Tk);
-    if (P < 0) P = 0;
-  }
+  // never index past the cache, whatever the counter says (a graph replayed beyond the
+  // capacity would otherwise read beyond the last head's buffer)
+  if (P > cap - Tk) P = (int)(cap - Tk);
+  if (P < 0) P = 0;
   const int Ltot = P + Tk;                // Tk = T unless WIDE
   const int ntiles = (Ltot + KT - 1) / KT;
   // Splits in use for this length: every workgroup gets at most `tpw` key tiles, two at
@@ -325,7 +325,7 @@ template <int HD>
 __global__ void tree_attn_merge_kernel(const half_t* __restrict__ part_o,
                                        const float* __restrict__ part_ml,
                                        half_t* __restrict__ out, int T, int H, int nsplit,
-                                       const int32_t* __restrict__ len_dev, long cap, int clamp_len,
+                                       const int32_t* __restrict__ len_dev, long cap,
                                        int Tk) {
   const int piece = blockIdx.z;                     // as in the split kernel
   part_o += (long)piece * H * nsplit * 32 * HD;
@@ -361,10 +361,8 @@ __global__ void tree_attn_merge_kernel(const half_t* __restrict__ part_o,
     pre[k] = *reinterpret_cast<const half4_t*>(src + (long)(k < nsplit ? k : nsplit - 1) * 32 * HD);
 
   int P = len_dev[piece];
-  if (clamp_len) {
-    if (P > cap - Tk) P = (int)(cap - Tk);
-    if (P < 0) P = 0;
-  }
+  if (P > cap - Tk) P = (int)(cap - Tk);    // as in the split kernel
+  if (P < 0) P = 0;
   const int nact = active_splits((P + Tk + KT - 1) / KT, nsplit);   // as in the split kernel
 #pragma unroll
   for (int k = 0; k < TPW; ++k) {
@@ -433,7 +431,7 @@ int launch_attention(const half_t* q, half_t* kc, half_t* vc, const uint32_t* bi
                      q_rows);
   hipLaunchKernelGGL(tree_attn_merge_kernel<HD>, dim3(H, (T + MERGE_TOK - 1) / MERGE_TOK, pieces),
                      dim3(MERGE_TOK * HD / 4), 0, st, part_o, part_ml, (half_t*)out, T, H, nsplit,
-                     len, cap, (ROPE || WIDE) ? 1 : 0, Tk);
+                     len, cap, Tk);
   return eagle_launch_status();
 }
 

@@ -22,7 +22,12 @@ __global__ __launch_bounds__(256) void process_draft_tree_kernel(
   __shared__ int midx[MAXT];
   __shared__ uint32_t bits[MAXT];
   const int tid = threadIdx.x;
-  for (int i = tid; i < C; i += blockDim.x) sc[i] = (float)scores[i];
+  // a NaN score ranks as -inf: with the index tie rule the order below is then total, so
+  // exactly `total` candidates are picked whatever the scores hold
+  for (int i = tid; i < C; i += blockDim.x) {
+    const float v = (float)scores[i];
+    sc[i] = v != v ? -INFINITY : v;
+  }
   __syncthreads();
   // rank in the stable descending order: candidates ahead of i are those with a larger
   // score, or an equal score and a lower flat index
@@ -41,7 +46,7 @@ __global__ __launch_bounds__(256) void process_draft_tree_kernel(
     if (!picked[i]) continue;
     int before = 0;
     for (int j = 0; j < i; ++j) before += picked[j];
-    sel[before] = i;
+    if (before < total) sel[before] = i;
   }
   __syncthreads();
   if (tid < total) {
@@ -67,10 +72,13 @@ __global__ __launch_bounds__(256) void process_draft_tree_kernel(
   if (tid == 0) draft_tokens[0] = sampled[0];
   __syncthreads();
   if (tid == 0) {
-    bits[0] = 1u;
+    // identity rows first, then the sequential OR of mlx_eagle.py:239-243 (a parent slot ahead
+    // of its child, which only poisoned scores can produce, then reads an identity row, as the
+    // reference's loop over an identity matrix does)
+    for (int i = 0; i <= total; ++i) bits[i] = 1u << i;
     for (int i = 0; i < total; ++i) {
       const int par = midx[i] < 0 ? 0 : (midx[i] > total ? total : midx[i]);
-      bits[i + 1] = (1u << (i + 1)) | bits[par];
+      bits[i + 1] |= bits[par];
     }
   }
   __syncthreads();
@@ -197,10 +205,14 @@ __global__ __launch_bounds__(256) void kv_compact_kernel(half_t* const* __restri
   }
 }
 
-__global__ void set_len_after_accept(const int32_t* __restrict__ accept, int32_t* len_dev) {
+// the length saturates at the capacity: a caller that replays steps beyond it gets a full
+// cache (the append kernels skip rows at or beyond the capacity), never a length that points
+// outside the buffers
+__global__ void set_len_after_accept(const int32_t* __restrict__ accept, int32_t* len_dev, long cap) {
   if (threadIdx.x == 0 && blockIdx.x == 0) {
     const int al = accept[1] < 0 ? 0 : accept[1];
-    *len_dev = *len_dev + al + 1;
+    const long n = (long)*len_dev + al + 1;
+    *len_dev = (int32_t)(n < cap ? n : cap);
   }
 }
 
@@ -275,7 +287,7 @@ EAGLE_EXPORT int eagle_kv_compact_f16(void* const* caches_dev, int n_caches, con
   hipLaunchKernelGGL(kv_compact_kernel, dim3(G, n_caches), dim3(256), lds, st,
                      reinterpret_cast<half_t* const*>(caches_dev), accept, cache_len_dev, hd,
                      capacity);
-  hipLaunchKernelGGL(set_len_after_accept, dim3(1), dim3(64), 0, st, accept, cache_len_dev);
+  hipLaunchKernelGGL(set_len_after_accept, dim3(1), dim3(64), 0, st, accept, cache_len_dev, capacity);
   return eagle_launch_status();
 }
 

@@ -238,12 +238,24 @@ def accept_candidate(cache, accept_indices, accept_length, offset):
         c.offset = offset + accept_length + 1
 
 
+def _check_tree_size(verify_num_tokens):
+    """The tree kernels, the mask words of the verification attention and the matmul rows are
+    laid out for 32 tree tokens (root + 31 nodes); the reference's default of 39 nodes
+    (mlx_eagle.py:390,510) is kept in the signatures and refused here."""
+    if verify_num_tokens + 1 > MAXT:
+        raise NotImplementedError(
+            f"verify_num_tokens={verify_num_tokens}: this build verifies at most {MAXT - 1} draft nodes per "
+            f"step (a tree of {MAXT} tokens); pass verify_num_tokens={MAXT - 1} or less")
+
+
 def spec_step(y, base_model, draft_model, base_cache, draft_cache, offset=None, accept_length=0,
-              k=8, depth=5, verify_num_tokens=31, tokenizer=None):
-    """mlx_eagle.py:379-463 up to its first return: the draft forward of the tokens accepted
+              k=8, depth=5, verify_num_tokens=39, tokenizer=None):
+    """mlx_eagle.py:379-463 up to its first return (same defaults; this build lays a tree out in
+    32 slots, so verify_num_tokens above 31 raises NotImplementedError): the draft forward of the tokens accepted
     last step, the level-0 top-k, the expansion, the tree layout and the target forward.
     y [1, accept_length + 1] int.  Returns (tree_position_ids, mask_index, draft_tokens,
     base_logits, base_offset, draft_offset)."""
+    _check_tree_size(verify_num_tokens)
     base_offset = base_cache[0].offset
     draft_offset = draft_cache[0].offset + 1 + accept_length
     _y = y
@@ -269,15 +281,14 @@ def spec_step(y, base_model, draft_model, base_cache, draft_cache, offset=None, 
 
 
 def generate_step(prompt, base_model, draft_model, prefill_step_size=512, k=8, depth=5,
-                  verify_num_tokens=31, max_tokens=128, tokenizer=None, N=20, capacity=None):
+                  verify_num_tokens=39, max_tokens=128, tokenizer=None, N=20, capacity=None):
     """mlx_eagle.py:503-606, greedy.  prompt: 1-D int tensor on the models' device.  Instead of
     printing, returns dict(tokens: every generated token in order, first: the token sampled
     from the prompt, steps: per step (accept_length, best_candidate, accept_indices, y), n,
     mean_tokens_per_step)."""
     from .cache import make_prompt_cache
 
-    if verify_num_tokens + 1 > MAXT:
-        raise ValueError(f"at most {MAXT - 1} draft nodes per verification")
+    _check_tree_size(verify_num_tokens)
     y = prompt.reshape(-1).to(torch.int64)
     if capacity is None:
         capacity = y.numel() + max_tokens + N + k * depth + MAXT + 16
@@ -415,6 +426,27 @@ def slab_partial_buffer(model, plan):
     return torch.empty(need, dtype=torch.float32, device=model.device)
 
 
+class LengthBudget:
+    """Host-side upper bound of a cache length that lives on the device.  A step appends
+    `rows_per_step` rows and keeps at most that many; `reserve` is called before every step
+    and reads the true length back (`read_length()`, one device-to-host copy) only when the
+    bound has reached the capacity.  Raises ValueError when a step would not fit."""
+
+    def __init__(self, capacity, rows_per_step, length=0):
+        self.capacity, self.rows, self.bound = int(capacity), int(rows_per_step), int(length)
+
+    def reset(self, length):
+        self.bound = int(length)
+
+    def reserve(self, read_length):
+        if self.bound + self.rows > self.capacity:
+            self.bound = int(read_length())
+            if self.bound + self.rows > self.capacity:
+                raise ValueError(f"KV caches of {self.capacity} rows have no room for {self.rows} more rows "
+                                 f"at length {self.bound}")
+        self.bound += self.rows
+
+
 class TreeVerifier:
     """One target-model tree-verification step with static buffers, so that it can be
     captured once in a HIP graph and replayed: embedding, all decoder layers, final norm,
@@ -484,6 +516,11 @@ class TreeVerifier:
                                        + [c.values.data_ptr() for c in cache],
                                        dtype=torch.int64, device=dev)
         self.graph = None
+        # host-side upper bound of the device cache length (a step adds at most T rows); step()
+        # refreshes it from the device before it could pass the capacity
+        self._budget = LengthBudget(self.capacity, T, max(c.offset for c in cache))
+        # the captured graph holds raw addresses of these tensors: keep them alive with it
+        self._graph_keepalive = None
         # size every workspace before any capture
         L = _lib.lib()
         head = model.lm_head if not args.tie_word_embeddings else model.model.embed_tokens
@@ -657,10 +694,18 @@ class TreeVerifier:
             self.forward()
         self.len_dev.copy_(saved_len)
         torch.cuda.synchronize()
+        self._graph_keepalive = ([c.keys for c in self.cache], [c.values for c in self.cache],
+                                 self.qkv_w if self.fuse else None, self.gu_w if self.fuse else None,
+                                 self.model)
+        self._budget.reset(int(saved_len.item()))
         return self
 
     def step(self):
-        """Run one verification step (graph replay when captured)."""
+        """Run one verification step (graph replay when captured).  The cache length lives on
+        the device; the host keeps an upper bound (a step appends T rows and keeps at most T of
+        them) and reads the true length back only when that bound reaches the capacity.
+        Raises ValueError instead of running a step that the caches have no room for."""
+        self._budget.reserve(lambda: self.len_dev.item())
         if self.graph is not None:
             self.graph.replay()
         else:
@@ -671,4 +716,5 @@ class TreeVerifier:
         n = int(self.len_dev.item())
         for c in self.cache:
             c.offset = n
+        self._budget.reset(n)
         return n

@@ -20,9 +20,13 @@ def topk(x, k, stable=False):
     index first.  mlx_eagle.py:24-58.  The reference's non-stable branch leaves
     the order of equal values to argpartition; this build fixes "lowest index
     first" for both branches, so `stable` only documents the caller's intent.
+    A NaN score ranks as -inf (where MLX's argsort puts NaN is unpinned; an fp16 overflow
+    in a drafter can produce them, and the tree must stay well formed).
     Returns (indices int64, values)."""
     x = np.asarray(x)
-    order = np.argsort(-x.astype(np.float64), kind="stable")[:k]
+    key = x.astype(np.float64)
+    key = np.where(np.isnan(key), -np.inf, key)
+    order = np.argsort(-key, kind="stable")[:k]
     return order, x[order]
 
 

@@ -42,6 +42,26 @@ def test_process_and_post_process_bit_exact(dev, depth, V):
         assert ri.shape == ri_w.shape and np.array_equal(ri, ri_w)
 
 
+@pytest.mark.parametrize("n_nan", [1, 33, 150, 200])
+def test_nan_scores_leave_a_well_formed_tree(dev, n_nan):
+    """More NaN scores than tree slots: the device picks exactly V candidates (NaN ranks as
+    -inf, ties by index) and equals the oracle bit for bit; nothing outside the outputs is
+    written (the tokens after the tree and a second call on clean scores are intact)."""
+    rng = np.random.default_rng(n_nan)
+    V = 31
+    scores, tokens, parents_list, _ = simulate_draft(rng, 3)
+    clean = scores.copy()
+    bad = rng.choice(scores.size, size=min(n_nan, scores.size), replace=False)
+    scores[bad] = np.nan
+    for sc in (scores, clean):
+        pos_w, midx_w, toks_w, anc_w = to.process_draft_tree(sc, tokens, parents_list, np.array([[9]]), 8, V)
+        pos, midx, toks, bits = dev_process(dev, sc, tokens, parents_list, 9, 8, V)
+        assert np.array_equal(pos.cpu().numpy(), pos_w)
+        assert np.array_equal(midx.cpu().numpy(), midx_w)
+        assert np.array_equal(toks.cpu().numpy(), toks_w[0])
+        assert np.array_equal(bits.cpu().numpy().view(np.uint32), to.mask_bits(anc_w))
+
+
 def test_reference_signature_process_draft_tree(dev):
     """List-of-levels inputs and the (position_ids, mask_index, draft_tokens[1,T], bf16 mask) tuple."""
     rng = np.random.default_rng(5)

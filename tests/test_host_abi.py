@@ -203,3 +203,32 @@ def test_slab_form_entry_points_reject_bad_arguments():
     assert L.eagle_rope_kv_append_slabs_f16(p, 2, None, p, p, p, p, p, 8, 4, 3, 64, 100, None) == 2
     assert L.eagle_rope_kv_append_slabs_f16(p, 2, p + 2, p, p, p, p, p, 8, 4, 2, 64, 100, None) == 3
     assert L.eagle_rope_kv_append_slabs_f16(None, 2, None, p, p, p, p, p, 8, 4, 2, 64, 100, None) == 1
+
+
+def test_length_budget_bounds_the_device_length():
+    """The verifier's host-side bound of the device cache length: no read-back while the bound
+    is below the capacity, one read-back when it reaches it, ValueError when the true length
+    leaves no room for a step."""
+    from mlx_eagle_spec_decoding_tree_amd.eagle import LengthBudget
+    reads = []
+    true_len = [100]
+
+    def read():
+        reads.append(true_len[0])
+        return true_len[0]
+
+    b = LengthBudget(capacity=200, rows_per_step=32, length=100)
+    for _ in range(3):                       # bound 100 -> 196: fits without asking the device
+        b.reserve(read)
+        true_len[0] += 1                     # the device really keeps one row per step
+    assert reads == []
+    b.reserve(read)                          # bound 196 + 32 > 200: read back 103, fits again
+    assert reads == [103] and b.bound == 135
+    true_len[0] = 170
+    b.reset(170)
+    with pytest.raises(ValueError):
+        b.reserve(read)                      # 170 + 32 > 200
+    assert reads == [103, 170]
+    b.reset(168)
+    true_len[0] = 168
+    b.reserve(read)                          # 168 + 32 == 200 still fits

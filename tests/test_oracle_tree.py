@@ -120,6 +120,30 @@ def test_topk_ties_keep_lowest_index():
     assert idx.tolist() == [1, 2, 4] and vals.tolist() == [3.0, 3.0, 3.0]
 
 
+def test_nan_scores_rank_last_and_the_tree_stays_well_formed():
+    """NaN ranks as -inf, ties by index: exactly V nodes whatever the scores hold, the NaN
+    candidates after every real score, indices in range (a drafter that overflows fp16 hands
+    NaN scores to the tree builder)."""
+    x = np.array([np.nan, 1.0, -np.inf, np.nan, 2.0], np.float16)
+    idx, _ = to.topk(x, 5)
+    assert idx.tolist() == [4, 1, 0, 2, 3]
+    rng = np.random.default_rng(11)
+    for n_nan in (1, 33, 150, 200):
+        scores, tokens, parents_list, _ = simulate_draft(rng, 3)
+        bad = rng.choice(scores.size, size=min(n_nan, scores.size), replace=False)
+        scores = scores.copy()
+        scores[bad] = np.nan
+        V = 31
+        pos, midx, dtoks, anc = to.process_draft_tree(scores, tokens, parents_list, np.array([[5]]), 8, V)
+        assert dtoks.shape == (1, V + 1) and midx.shape == (V,) and anc.shape == (V + 1, V + 1)
+        assert midx.min() >= 0 and midx.max() <= V
+        good = np.flatnonzero(~np.isnan(scores.astype(np.float32)))
+        order = np.argsort(-scores[good].astype(np.float64), kind="stable")
+        n_good = min(V, good.size)
+        sel = np.sort(np.concatenate([good[order[:n_good]], np.sort(bad)[:V - n_good]]))
+        assert np.array_equal(dtoks[0, 1:], tokens[sel])
+
+
 def test_search_sorted_matches_numpy_on_found_targets():
     """ceil(log2(n)) steps resolve n+1 possible answers for the node counts the reference
     uses (7, 15, 23, 31); the step count is part of the restated behaviour."""
