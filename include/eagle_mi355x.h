@@ -65,6 +65,21 @@ int eagle_qmm_w4g64_f16(const void* x, const uint32_t* wq, const void* scales,
                         const void* biases, const void* bias, void* out,
                         int M, int N, int K, int group_size, int bits,
                         void* workspace, size_t workspace_bytes, eagle_stream_t stream);
+/* The same matmul for callers that cannot allocate or bring a workspace (code under HIP graph
+ * capture, tight serving loops, harnesses that forbid hipMalloc).  It has no counterpart in the
+ * reference.  The split-K partial sums and arrival counters live in a fixed array of
+ * EAGLE_QMM_NOALLOC_SCRATCH_BYTES in device memory that the library owns (one copy per GPU,
+ * held until the process ends); the call allocates and frees nothing.  A shape whose workspace
+ * (eagle_qmm_workspace_bytes) exceeds that size returns EAGLE_ERR_WORKSPACE.  Same kernels,
+ * launch shapes and results, bit for bit, as eagle_qmm_w4g64_f16.  Every call on one GPU
+ * shares the array: calls that overlap on one GPU (different streams) race; the counters are
+ * cleared at the start of every call. */
+#define EAGLE_QMM_NOALLOC_SCRATCH_BYTES (8u << 20)
+size_t eagle_qmm_noalloc_scratch_bytes(void);
+int eagle_qmm_w4g64_f16_noalloc(const void* x, const uint32_t* wq, const void* scales,
+                                const void* biases, const void* bias, void* out,
+                                int M, int N, int K, int group_size, int bits,
+                                eagle_stream_t stream);
 /* The launch shape the library would pick: plan5 = {streaming waves per workgroup,
  * phases (column units each streaming wave owns, one after the other), K slabs, tile
  * ranges (workgroups per slab), columns per unit (256 for M <= 16; 128 or 256 above)}. */

@@ -40,6 +40,8 @@
 //    write-back / invalidate fence, which costs microseconds on a multi-XCD part.
 #include "common.h"
 
+#include <mutex>
+
 namespace {
 
 constexpr int MAX_STREAM_WAVES = 14;   // + 2 reducing waves = 1024 threads
@@ -947,6 +949,75 @@ EAGLE_EXPORT int eagle_qmm_w4g64_f16(const void* x, const uint32_t* wq, const vo
   if (rc != EAGLE_OK) return rc;
   return run(x, wq, scales, biases, bias, out, M, N, K, L, 0, workspace, workspace_bytes,
              static_cast<hipStream_t>(stream));
+}
+
+// ------------------------------------------------------------------------------------------
+// The same matmul for callers that cannot allocate: the split-K workspace is a fixed array in
+// device memory that belongs to the library.
+// ------------------------------------------------------------------------------------------
+namespace {
+
+constexpr size_t NOALLOC_SCRATCH_BYTES = (size_t)EAGLE_QMM_NOALLOC_SCRATCH_BYTES;
+constexpr int NOALLOC_MAX_DEVICES = 64;
+
+// Every GPU the library runs on holds its own copy of this array, at its own address, until
+// the process ends.  In host code the name is only a handle for hipGetSymbolAddress.
+static __device__ __align__(256) unsigned char scratch[NOALLOC_SCRATCH_BYTES];
+
+__global__ void zero_u32_kernel(unsigned* p, int n) {
+  const int i = blockIdx.x * blockDim.x + threadIdx.x;
+  if (i < n) p[i] = 0u;
+}
+
+// device address of `scratch` on the current device, looked up once per device
+int noalloc_scratch(void** out) {
+  static void* ptrs[NOALLOC_MAX_DEVICES];
+  static bool known[NOALLOC_MAX_DEVICES];
+  static std::mutex lock;
+  int dev = -1;
+  if (hipGetDevice(&dev) != hipSuccess) return EAGLE_ERR_HIP;
+  if (dev < 0 || dev >= NOALLOC_MAX_DEVICES) return EAGLE_ERR_UNSUPPORTED;
+  std::lock_guard<std::mutex> guard(lock);
+  if (!known[dev]) {
+    void* p = nullptr;
+    if (hipGetSymbolAddress(&p, HIP_SYMBOL(scratch)) != hipSuccess || !p) return EAGLE_ERR_HIP;
+    ptrs[dev] = p;
+    known[dev] = true;
+  }
+  *out = ptrs[dev];
+  return EAGLE_OK;
+}
+
+}  // namespace
+
+EAGLE_EXPORT size_t eagle_qmm_noalloc_scratch_bytes(void) { return NOALLOC_SCRATCH_BYTES; }
+
+EAGLE_EXPORT int eagle_qmm_w4g64_f16_noalloc(const void* x, const uint32_t* wq, const void* scales,
+                                             const void* biases, const void* bias, void* out, int M,
+                                             int N, int K, int group_size, int bits,
+                                             eagle_stream_t stream) {
+  if (group_size != 64 || bits != 4) return EAGLE_ERR_UNSUPPORTED;
+  int rc = validate(x, wq, scales, biases, bias, out, M, N, K);
+  if (rc != EAGLE_OK) return rc;
+  Launch L;
+  choose(M, N, K, &L);
+  rc = validate_launch(M, N, K, L);
+  if (rc != EAGLE_OK) return rc;
+  hipStream_t st = static_cast<hipStream_t>(stream);
+  void* ws = nullptr;
+  size_t ws_bytes = 0;
+  if (L.splits > 1) {
+    ws_bytes = (size_t)EAGLE_QMM_COUNTER_BYTES + partial_bytes(M, N, L.splits);
+    if (ws_bytes > NOALLOC_SCRATCH_BYTES) return EAGLE_ERR_WORKSPACE;   // shape needs more than the fixed array
+    rc = noalloc_scratch(&ws);
+    if (rc != EAGLE_OK) return rc;
+    // The arrival counters have to start at zero.  Every call leaves them zero, but the array
+    // is shared by all calls on this GPU and outlives them, so they are cleared here as well:
+    // a call that was cut short cannot poison the next one.
+    const int n = L.ranges < MAX_RANGES ? L.ranges : MAX_RANGES;
+    hipLaunchKernelGGL(zero_u32_kernel, dim3((n + 255) / 256), dim3(256), 0, st, static_cast<unsigned*>(ws), n);
+  }
+  return run(x, wq, scales, biases, bias, out, M, N, K, L, 0, ws, ws_bytes, st);
 }
 
 EAGLE_EXPORT int eagle_qmm_swiglu_w4g64_f16(const void* x, const uint32_t* wq, const void* scales,
