@@ -174,6 +174,9 @@ def main():
                     help="measure the end-to-end tree loop (drafter + target) instead of the verify step")
     ap.add_argument("--gemm", action="store_true",
                     help="measure the many-row (prompt pass) form of the quantised matmul instead")
+    ap.add_argument("--small-m", action="store_true",
+                    help="one-row products of the 7B projection shapes: the vector-ALU kernel beside the "
+                         "matrix kernel (one JSON line; the A/B behind the dispatch rule for M = 1)")
     ap.add_argument("--self-draft", action="store_true",
                     help="with --loop: the target drafts for itself (high acceptance; exercises the "
                          "accept path at full size)")
@@ -190,6 +193,9 @@ def main():
         return
     if opt.gemm:
         print(json.dumps(gemm_bench(opt)), flush=True)
+        return
+    if opt.small_m:
+        print(json.dumps(small_m_bench(opt)), flush=True)
         return
 
     import torch
@@ -445,6 +451,55 @@ def gemm_bench(opt):
         "shapes": rows,
     }
     return line
+
+
+def small_m_bench(opt):
+    """M = 1 over the projection shapes of the Qwen2.5-7B-shaped model: eagle_qmv_w4g64_f16
+    (v_dot2_f32_f16 + DPP row sums) beside eagle_qmm_w4g64_f16 (16-row MFMA tiles, 15 rows idle),
+    each launch on its own copy of the weights (> 1 GB in rotation)."""
+    import torch
+    from mlx_eagle_spec_decoding_tree_amd import _lib, ops
+
+    dev = torch.device("cuda:0")
+    _lib.check(_lib.lib().eagle_check_device(), "device check")
+    L = _lib.lib()
+    shapes = [("q/o", 3584, 3584), ("k/v", 512, 3584), ("gate/up", 18944, 3584), ("down", 3584, 18944),
+              ("lm_head", 152064, 3584), ("cfg1", 8192, 2048)]
+    rows = []
+    st = lambda: torch.cuda.current_stream().cuda_stream
+    for name, N, K in shapes:
+        ncopy = max(2, min(16, (1 << 30) // (N * K // 2)))
+        ws = [torch.randint(-2 ** 31, 2 ** 31 - 1, (N, K // 8), dtype=torch.int32, device=dev) for _ in range(ncopy)]
+        ss = [(torch.rand(N, K // 64, device=dev) * 0.015 + 0.005).half() for _ in range(ncopy)]
+        bs = [(-8 * s.float()).half() for s in ss]
+        x = torch.randn(1, K, device=dev).half()
+        o = torch.empty(1, N, device=dev, dtype=torch.float16)
+        wsp = ops.workspace("qmm", L.eagle_qmm_workspace_bytes(1, N, K), dev)
+        iters = 24
+
+        def mfma():
+            for i in range(iters):
+                j = i % ncopy
+                _lib.check(L.eagle_qmm_w4g64_f16(x.data_ptr(), ws[j].data_ptr(), ss[j].data_ptr(), bs[j].data_ptr(),
+                                                 None, o.data_ptr(), 1, N, K, 64, 4, wsp.data_ptr(), wsp.numel(),
+                                                 st()), "qmm")
+
+        def valu():
+            for i in range(iters):
+                j = i % ncopy
+                _lib.check(L.eagle_qmv_w4g64_f16(x.data_ptr(), ws[j].data_ptr(), ss[j].data_ptr(), bs[j].data_ptr(),
+                                                 None, o.data_ptr(), N, K, 64, 4, st()), "qmv")
+
+        t_m = float(np.median(graph_time_ms(torch, mfma, reps=7)[0])) * 1e3 / iters
+        t_v = float(np.median(graph_time_ms(torch, valu, reps=7)[0])) * 1e3 / iters
+        byts = qmm_bytes(1, N, K)
+        rows.append({"name": name, "N": N, "K": K, "mfma_us": round(t_m, 2), "valu_us": round(t_v, 2),
+                     "mfma_frac": round(byts / t_m / 1e3 / HBM_PEAK_GBS, 4),
+                     "valu_frac": round(byts / t_v / 1e3 / HBM_PEAK_GBS, 4),
+                     "dispatched_to": "valu" if ops.qmv_preferred(N, K) else "mfma"})
+        del ws, ss, bs
+    return {"metric": "one-row quantised product, us per launch (vector ALU beside matrix tiles)", "unit": "us",
+            "dtype": "f16", "data": "synthetic", "rows": rows}
 
 
 def loop_bench(opt):

@@ -65,6 +65,16 @@ int eagle_qmm_w4g64_f16(const void* x, const uint32_t* wq, const void* scales,
                         const void* biases, const void* bias, void* out,
                         int M, int N, int K, int group_size, int bits,
                         void* workspace, size_t workspace_bytes, eagle_stream_t stream);
+/* The product for ONE row of x on the vector ALU (v_dot2_f32_f16 on magic-number fp16 nibbles,
+ * sum over the sixteen lanes of a row with DPP), no matrix instructions: the M = 1 case of
+ * mx.quantized_matmul (mlx_model_fwd_bench.py:65-73), factorised as in kernels/qmv/1b.metal:121-147.
+ * K % 512 == 0 and x plus its group sums must fit LDS (eagle_qmv_supported returns 1); x and wq
+ * 16-byte aligned.  out [N] fp16. */
+int eagle_qmv_supported(int N, int K);
+int eagle_qmv_w4g64_f16(const void* x, const uint32_t* wq, const void* scales, const void* biases,
+                        const void* bias, void* out, int N, int K, int group_size, int bits,
+                        eagle_stream_t stream);
+
 /* The same matmul for callers that cannot allocate or bring a workspace (code under HIP graph
  * capture, tight serving loops, harnesses that forbid hipMalloc).  It has no counterpart in the
  * reference.  The split-K partial sums and arrival counters live in a fixed array of

@@ -184,7 +184,12 @@ def test_swiglu_form_equals_separate_launches(dev, I, K, bias):
                                                 bias=cat.get("bias")))
         torch.cuda.synchronize()
         assert tuple(got.shape) == (M, I)
-        assert torch.equal(got, two), f"I={I} K={K} M={M}: swiglu form differs from matmul + silu_mul"
+        if M == 1 and ops.qmv_preferred(2 * I, K):
+            # one row of the concatenated launch goes to the vector-ALU kernel (another order
+            # of the fp32 sums): the tolerance applies, not bit equality
+            assert rel_err(got.cpu().numpy(), two.cpu().numpy().astype(np.float64)) <= TOL
+        else:
+            assert torch.equal(got, two), f"I={I} K={K} M={M}: swiglu form differs from matmul + silu_mul"
         assert rel_err(got.cpu().numpy(), want) <= TOL
 
 

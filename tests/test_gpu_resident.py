@@ -93,3 +93,18 @@ def test_rejects_what_it_does_not_take(dev):
     s = torch.zeros((64, 64), dtype=torch.float16, device=dev)
     with pytest.raises(ValueError):
         ops.quantized_matmul_resident(x, w, s, s)
+
+
+@pytest.mark.parametrize("N,K", [(8, 512), (40, 1024), (3584, 3584), (512, 3584), (3584, 18944), (8192, 2048)])
+def test_vector_alu_matvec(dev, N, K):
+    """The M = 1 product on the vector ALU (csrc/qmv.hip) against the oracle."""
+    print(f"qmv N={N} K={K}", flush=True)
+    rng = np.random.default_rng(N + K)
+    layer = synth.make_qlinear(rng, N, K, bias=(N % 16 == 8))
+    x = synth.make_x(rng, 1, K)
+    want = oracle.qmm(x, layer["weight"], layer["scales"], layer["biases"], layer.get("bias"))
+    d = layer_to_dev(layer, dev)
+    got = ops.quantized_matvec(to_dev(x, dev), d["weight"], d["scales"], d["biases"], bias=d.get("bias"))
+    torch.cuda.synchronize()
+    assert tuple(got.shape) == (1, N)
+    assert rel_err(got.cpu().numpy(), want) <= TOL
