@@ -166,6 +166,9 @@ def main():
                          "'' = streaming kernel everywhere; default: the library's choice)")
     ap.add_argument("--draft-slabs", default=None,
                     help="--loop: the same for the drafter's passes")
+    ap.add_argument("--chain", action="store_true",
+                    help="residual add + norm + gate|up + SwiGLU as one launch of a resident grid with a "
+                         "grid-wide barrier inside (off by default: slower than the two launches it replaces)")
     ap.add_argument("--sweep", action="store_true", help="also print the per-shape QMM table to stderr")
     ap.add_argument("--calibrate-copy", action="store_true",
                     help="before anything else run one 1 GiB device copy (a kernel of known traffic: "
@@ -242,7 +245,8 @@ def main():
     slab_plan = None
     if opt.slabs is not None:
         slab_plan = {kv.split("=")[0]: int(kv.split("=")[1]) for kv in opt.slabs.split(",") if kv}
-    ver = eagle.TreeVerifier(model, cache, total_tokens=NODES - 1, max_len=cap, slab_plan=slab_plan)
+    ver = eagle.TreeVerifier(model, cache, total_tokens=NODES - 1, max_len=cap, slab_plan=slab_plan,
+                             chain=opt.chain)
     ver.set_tree(torch.from_numpy(tokens).to(dev), torch.from_numpy(depth.astype(np.int32)).to(dev),
                  torch.from_numpy(parents).to(dev),
                  torch.from_numpy(bits.view(np.int32)).to(dev))
@@ -278,41 +282,56 @@ def main():
 
     def qmm_only(subset=None):
         for wq, sc, bi, bias, x, out, form in (launches if subset is None else subset):
-            if form is True:
+            if form == "chain":
+                (gw, gs, gb, gbias), nw, nslab = wq, sc, bi
+                ops.norm_mlp_in(x, nslab, ver.h, nw, args.rms_norm_eps, gw, gs, gb, gbias, out,
+                                ver.chain_scratch, ver.chain_err)
+            elif form is True:
                 ops.quantized_matmul_swiglu(x, wq, sc, bi, bias=bias, out=out)
             elif form:
                 ops.quantized_matmul_slabs(x, wq, sc, bi, form, partial=ver.partial)
             else:
                 ops.quantized_matmul(x, wq, sc, bi, bias=bias, out=out)
 
+    def alg_bytes(l):
+        if l[6] == "chain":               # the product inside the chained launch
+            gw = l[0][0]
+            return qmm_bytes(NODES, gw.shape[0], gw.shape[1] * 8, l[5].shape[-1])
+        return qmm_bytes(NODES, l[0].shape[0], l[0].shape[1] * 8, l[5].shape[-1])
+
     qt, _ = graph_time_ms(torch, qmm_only, reps=10)
     qmm_ms = float(np.median(qt))
     n_launch = len(launches)
-    alg = sum(qmm_bytes(NODES, l[0].shape[0], l[0].shape[1] * 8, l[5].shape[-1]) for l in launches)
+    alg = sum(alg_bytes(l) for l in launches)
     kv_bytes = 2 * L * G * (PREFIX + NODES) * hd * 2
     achieved = alg / (qmm_ms * 1e-3) / 1e9
     traffic, traffic_source = read_traffic_record()
-    roofline = {"bound": "hbm", "kernel": "qmm_w4g64_kernel + qmm_slab_w4g64_kernel", "achieved": round(achieved, 1),
+    kernels = "qmm_w4g64_kernel + qmm_slab_w4g64_kernel" + (" + norm_mlp_in_kernel" if ver.chain else "")
+    roofline = {"bound": "hbm", "kernel": kernels, "achieved": round(achieved, 1),
                 "peak": HBM_PEAK_GBS, "unit": "GB/s", "frac": round(achieved / HBM_PEAK_GBS, 4),
                 "traffic": traffic, "traffic_source": traffic_source, "launches_per_step": n_launch,
                 "avg_launch_us": round(qmm_ms * 1e3 / n_launch, 3),
                 "algorithmic_bytes_per_launch": round(alg / n_launch),
                 "step_frac": round((alg + kv_bytes) / (ms_per_step * 1e-3) / 1e9 / HBM_PEAK_GBS, 4)}
 
-    # the same for each of the two kernels on its own launches
+    # the same for each kernel on its own launches
     per_kernel = {}
     for kname, sub in (("qmm_w4g64_kernel", [l for l in launches if l[6] is True or not l[6]]),
-                       ("qmm_slab_w4g64_kernel", [l for l in launches if l[6] and l[6] is not True])):
+                       ("qmm_slab_w4g64_kernel", [l for l in launches if l[6] and l[6] is not True and l[6] != "chain"]),
+                       ("norm_mlp_in_kernel", [l for l in launches if l[6] == "chain"])):
         if not sub:
             continue
         st, _ = graph_time_ms(torch, lambda: qmm_only(sub), reps=10)
         sub_ms = float(np.median(st))
-        sub_alg = sum(qmm_bytes(NODES, l[0].shape[0], l[0].shape[1] * 8, l[5].shape[-1]) for l in sub)
+        sub_alg = sum(alg_bytes(l) for l in sub)
         per_kernel[kname] = {"launches_per_step": len(sub), "avg_launch_us": round(sub_ms * 1e3 / len(sub), 3),
                              "algorithmic_bytes_per_launch": round(sub_alg / len(sub)),
                              "achieved": round(sub_alg / (sub_ms * 1e-3) / 1e9, 1),
                              "frac": round(sub_alg / (sub_ms * 1e-3) / 1e9 / HBM_PEAK_GBS, 4)}
     roofline["per_kernel"] = per_kernel
+    if ver.chain and bool(ver.chain_err.item()):
+        print("bench.py: a grid barrier of the chained launch gave up", file=sys.stderr)
+        sys.exit(1)
 
     if opt.sweep:
         sweep(torch, ops, dev, args)

@@ -65,6 +65,36 @@ int eagle_qmm_w4g64_f16(const void* x, const uint32_t* wq, const void* scales,
                         const void* biases, const void* bias, void* out,
                         int M, int N, int K, int group_size, int bits,
                         void* workspace, size_t workspace_bytes, eagle_stream_t stream);
+/* Residual add, RMSNorm, gate|up and SwiGLU of a decoder layer in ONE launch of a resident grid
+ * (256 workgroups, one per compute unit): first h += fp16(sum of the K slabs of the product that
+ * precedes the norm) and the sums of squares of the new h, spread over the whole grid; then,
+ * across a grid-wide barrier, act = silu(g) * u with (g | u) = RMSNorm(h) . Wgu^T, the norm folded
+ * into the load of x (mlx_llama.py:240-243, 214-215, 225-228).  The weights of the product are
+ * requested at the start of the launch and stay in flight across the barrier, which a kernel
+ * boundary cannot do.  Replaces eagle_rmsnorm_slabs_f16 (residual form) followed by
+ * eagle_qmm_swiglu_w4g64_f16.
+ *   partial [slabs][32][D] fp32 from eagle_qmm_slab_partial_w4g64 (the o projection, no bias);
+ *   h [M, D] fp16, updated in place; norm_w [D] fp16; gu_* the gate and up projections [2 I, D]
+ *   interleaved in 16-row tiles as for eagle_qmm_swiglu_w4g64_f16, gu_bias [2 I] interleaved or
+ *   NULL; act [M, I] fp16.
+ * Constraints (eagle_norm_mlp_in_supported): D % 512 == 0, D <= 3584, I % 16 == 0, every scale
+ * below 0.2499 (as eagle_qmm_res_w4g64_f16), a device with at least 256 compute units; all
+ * pointers 16-byte aligned.
+ * `scratch` (eagle_norm_mlp_in_scratch_bytes) holds the sums of squares and the barrier counters;
+ * it must be ZERO before the first launch and belongs to this entry point from then on (the
+ * counters only grow; launches sharing it must be stream ordered and on one device).
+ * The wait at the barrier is bounded: after `spin_limit_ticks` (100 MHz ticks) a workgroup stores 1
+ * to *err_dev and the launch ends without the product; the caller then has to zero `scratch` and
+ * *err_dev before the next launch.  The grid needs every compute unit of the device to itself
+ * for the duration of the launch. */
+size_t eagle_norm_mlp_in_scratch_bytes(void);
+int eagle_norm_mlp_in_supported(int M, int D, int I);
+int eagle_norm_mlp_in_f16(const float* partial, int slabs, void* h, const void* norm_w, float eps,
+                          const uint32_t* gu_wq, const void* gu_scales, const void* gu_biases,
+                          const void* gu_bias, void* act, int M, int D, int I,
+                          void* scratch, size_t scratch_bytes, int* err_dev,
+                          long long spin_limit_ticks, eagle_stream_t stream);
+
 /* The product for ONE row of x on the vector ALU (v_dot2_f32_f16 on magic-number fp16 nibbles,
  * sum over the sixteen lanes of a row with DPP), no matrix instructions: the M = 1 case of
  * mx.quantized_matmul (mlx_model_fwd_bench.py:65-73), factorised as in kernels/qmv/1b.metal:121-147.

@@ -6,7 +6,7 @@ hard error (there is no CPU or eager fallback).  Build it with
 """
 import ctypes
 import os
-from ctypes import c_char_p, c_float, c_int, c_int32, c_long, c_size_t, c_void_p
+from ctypes import c_char_p, c_float, c_int, c_int32, c_long, c_longlong, c_size_t, c_void_p
 
 HERE = os.path.dirname(os.path.abspath(__file__))
 # EAGLE_MI355X_LIB selects another build of the same library (kernel experiments)
@@ -23,6 +23,10 @@ SIGNATURES = {
     "eagle_qmm_w4g64_f16": (c_int, [c_void_p] * 6 + [c_int] * 5 + [c_void_p, c_size_t, c_void_p]),
     "eagle_qmm_noalloc_scratch_bytes": (c_size_t, []),
     "eagle_qmm_w4g64_f16_noalloc": (c_int, [c_void_p] * 6 + [c_int] * 5 + [c_void_p]),
+    "eagle_norm_mlp_in_scratch_bytes": (c_size_t, []),
+    "eagle_norm_mlp_in_supported": (c_int, [c_int] * 3),
+    "eagle_norm_mlp_in_f16": (c_int, [c_void_p, c_int, c_void_p, c_void_p, c_float] + [c_void_p] * 5
+                              + [c_int] * 3 + [c_void_p, c_size_t, c_void_p, c_longlong, c_void_p]),
     "eagle_qmv_supported": (c_int, [c_int] * 2),
     "eagle_qmv_w4g64_f16": (c_int, [c_void_p] * 6 + [c_int] * 4 + [c_void_p]),
     "eagle_qmm_plan": (c_int, [c_int, c_int, c_int, c_void_p]),

@@ -457,10 +457,15 @@ class TreeVerifier:
     Same kernels and operator order as Model.__call__ + the host functions above."""
 
     def __init__(self, model, cache, total_tokens=31, max_len=None, compact=True, fuse=True,
-                 swiglu=True, one_launch_attention=False, slab_plan=None):
+                 swiglu=True, one_launch_attention=False, slab_plan=None, chain=None):
         """slab_plan: {"qkv": s, "o": s, "down": s}, K steps per slab for the projections that go
         through the slab form of the matmul (their consumer adds the slabs), 0 for the
-        streaming kernel; None: the library's choice for this shape."""
+        streaming kernel; None: the library's choice for this shape.
+        chain: the residual add after the o projection, the norm and gate|up + SwiGLU of a layer as
+        ONE launch of a resident grid with a grid-wide barrier inside (`ops.norm_mlp_in`; needs the
+        o projection in the slab form).  Off unless asked for: measured inside the 7B step it takes
+        43.7 us against 5.3 + 30.6 us for the two launches it replaces (step 2.99 against 2.70 ms).
+        `chain_error()` reports a barrier that gave up."""
         args = model.args
         self.model, self.cache, self.args = model, cache, args
         self.V = total_tokens
@@ -481,6 +486,13 @@ class TreeVerifier:
         if fuse:
             self._fuse_projections()
         self.slab = self._slab_plan(slab_plan)
+        can_chain = bool(self.swiglu and self.slab["o"] and ops.norm_mlp_in_supported(T, D, I)
+                         and torch.cuda.get_device_properties(dev).multi_processor_count >= 256)
+        if chain and not can_chain:
+            raise ValueError("the chained launch does not take this model shape")
+        self.chain = bool(chain)
+        if self.chain:
+            self.chain_scratch, self.chain_err = ops.norm_mlp_in_scratch(dev)
         i32 = dict(dtype=torch.int32, device=dev)
         f16 = dict(dtype=torch.float16, device=dev)
         self.tokens = torch.zeros(T, **i32)
@@ -543,7 +555,8 @@ class TreeVerifier:
         """(weight, scales, biases, bias, x, out, form) of every quantised matmul of one step,
         in order; `form` is True for the launches that go through `quantized_matmul_swiglu`,
         the K steps per slab for those that go through `quantized_matmul_slabs` (into
-        `self.partial`), False for `quantized_matmul`."""
+        `self.partial`), False for `quantized_matmul`; "chain" entries are (gate|up tuple, norm
+        weight, slabs, None, partial, out, "chain") for `norm_mlp_in`."""
         m = self.model
         out = []
         for i, layer in enumerate(m.model.layers):
@@ -553,6 +566,16 @@ class TreeVerifier:
             else:
                 for lin, o in ((at.q_proj, self.q), (at.k_proj, self.k), (at.v_proj, self.v)):
                     out.append((lin.weight, lin.scales, lin.biases, lin.bias, self.hn, o, False))
+            if self.chain:
+                # the o projection as slabs; gate|up + SwiGLU inside the chained launch that adds them
+                out.append((at.o_proj.weight, at.o_proj.scales, at.o_proj.biases, at.o_proj.bias,
+                            self.attn, self.o, self.slab["o"]))
+                out.append((self.gu_w[i], layer.post_attention_layernorm.weight,
+                            ops.slab_count(at.o_proj.weight.shape[1] * 8, self.slab["o"]), None, self.partial,
+                            self.act, "chain"))
+                out.append((mlp.down_proj.weight, mlp.down_proj.scales, mlp.down_proj.biases,
+                            mlp.down_proj.bias, self.act, self.down, self.slab["down"] or False))
+                continue
             out.append((at.o_proj.weight, at.o_proj.scales, at.o_proj.biases, at.o_proj.bias,
                         self.attn, self.o, self.slab["o"] or False))
             if self.fuse:
@@ -627,7 +650,16 @@ class TreeVerifier:
             if not self.one_launch_attention:
                 ops.tree_attention(self.q_rot, c.keys[0], c.values[0], self.mask_bits, self.len_dev,
                                    at.scale, max_len=self.max_len, out=self.attn)
-            if self.slab["o"]:
+            mlp = layer.mlp
+            if self.chain:
+                s = self.slab["o"]
+                ops.quantized_matmul_slabs(self.attn, at.o_proj.weight, at.o_proj.scales, at.o_proj.biases,
+                                           s, partial=self.partial)
+                w, sc, bi, b = self.gu_w[i]
+                ops.norm_mlp_in(self.partial, ops.slab_count(H * hd, s), self.h,
+                                layer.post_attention_layernorm.weight, args.rms_norm_eps, w, sc, bi, b,
+                                self.act, self.chain_scratch, self.chain_err)
+            elif self.slab["o"]:
                 s = self.slab["o"]
                 ops.quantized_matmul_slabs(self.attn, at.o_proj.weight, at.o_proj.scales, at.o_proj.biases,
                                            s, partial=self.partial)
@@ -639,8 +671,9 @@ class TreeVerifier:
                                      bias=at.o_proj.bias, out=self.o)
                 ops.rms_norm(self.o, layer.post_attention_layernorm.weight, args.rms_norm_eps,
                              residual=self.h, out=self.hn, h_out=self.h)
-            mlp = layer.mlp
-            if self.fuse:
+            if self.chain:
+                pass
+            elif self.fuse:
                 w, sc, bi, b = self.gu_w[i]
                 if self.swiglu:
                     ops.quantized_matmul_swiglu(self.hn, w, sc, bi, bias=b, out=self.act)
@@ -710,6 +743,17 @@ class TreeVerifier:
             self.graph.replay()
         else:
             self.forward()
+
+    def chain_error(self):
+        """True if a grid barrier of the chained launch gave up since the last call (one
+        device-to-host copy); the scratch is zeroed again so that later steps can run."""
+        if not self.chain:
+            return False
+        bad = bool(self.chain_err.item())
+        if bad:
+            self.chain_scratch.zero_()
+            self.chain_err.zero_()
+        return bad
 
     def sync_host_offsets(self):
         """Bring the host-side cache offsets in line with the device length (one D2H copy)."""

@@ -224,6 +224,38 @@ def quantized_matmul_swiglu(x, w_q, scales, biases, bias=None, out=None):
     return out
 
 
+CHAIN_SPIN_TICKS = 5_000_000     # 50 ms at 100 MHz: the bounded wait of the in-kernel grid barrier
+
+
+def norm_mlp_in_supported(M, D, I):
+    return bool(_lib.lib().eagle_norm_mlp_in_supported(M, D, I))
+
+
+def norm_mlp_in_scratch(device):
+    """Zeroed scratch (sums of squares + barrier counters) and error word for `norm_mlp_in`;
+    one pair per pass object, kept for its lifetime."""
+    n = _lib.lib().eagle_norm_mlp_in_scratch_bytes()
+    return (torch.zeros(n, dtype=torch.uint8, device=device), torch.zeros(1, dtype=torch.int32, device=device))
+
+
+def norm_mlp_in(partial, slabs, h, norm_weight, eps, gu_w, gu_scales, gu_biases, gu_bias, act, scratch, err,
+                spin_ticks=CHAIN_SPIN_TICKS):
+    """h += fp16(sum of the slabs); act = silu(g) * u with (g | u) = rms_norm(h) @ Wgu.T, in one
+    launch of a resident grid with a grid-wide barrier between the two parts
+    (mlx_llama.py:240-243, 214-215).  `partial` [slabs, 32, D] from `quantized_matmul_slabs`,
+    gate|up interleaved by `interleave_gate_up`.  `scratch`, `err` from `norm_mlp_in_scratch`;
+    err[0] != 0 afterwards means the barrier gave up."""
+    _need_cuda(partial, h, gu_w, act)
+    M, D = h.shape
+    I = act.shape[-1]
+    rc = _lib.lib().eagle_norm_mlp_in_f16(
+        _ptr(partial), int(slabs), _ptr(h), _ptr(norm_weight), float(eps), _ptr(as_packed_u32(gu_w)),
+        _ptr(gu_scales), _ptr(gu_biases), _ptr(gu_bias), _ptr(act), M, D, I, _ptr(scratch), scratch.numel(),
+        _ptr(err), int(spin_ticks), _stream())
+    _lib.check(rc, "norm_mlp_in")
+    return act
+
+
 def qmv_preferred(N, K):
     """True where the vector-ALU kernel is the faster form for one row of x: measured on the
     projection shapes of the 7B model (M = 1: 5.7 against 8.5 us for 3584 x 3584, 12.5 against

@@ -108,3 +108,109 @@ def test_vector_alu_matvec(dev, N, K):
     torch.cuda.synchronize()
     assert tuple(got.shape) == (1, N)
     assert rel_err(got.cpu().numpy(), want) <= TOL
+
+
+def chain_case(dev, M, D, I, seed, bias):
+    rng = np.random.default_rng(seed)
+    o = synth.make_qlinear(rng, D, D, gain=1.0)
+    g = synth.make_qlinear(rng, I, D, bias=bias, gain=1.0)
+    u = synth.make_qlinear(rng, I, D, bias=bias, gain=1.0)
+    attn = synth.make_x(rng, M, D)
+    h = synth.make_x(rng, M, D)
+    nw = (1.0 + rng.normal(0, 0.02, D)).astype(np.float16)
+    eps = 1e-6
+    od, gd, ud = layer_to_dev(o, dev), layer_to_dev(g, dev), layer_to_dev(u, dev)
+    # the product that precedes the norm, as K slabs (the o projection of the step)
+    partial = ops.quantized_matmul_slabs(to_dev(attn, dev), od["weight"], od["scales"], od["biases"], 8)
+    slabs = ops.slab_count(D, 8)
+    o16 = ops.slab_sum(partial, slabs, M, D).cpu().numpy()
+    h2 = oracle.add(h, o16)
+    xn = oracle.rmsnorm(h2, nw, eps)
+    want = oracle.silu_mul(oracle.qmm(xn, g["weight"], g["scales"], g["biases"], g.get("bias")),
+                           oracle.qmm(xn, u["weight"], u["scales"], u["biases"], u.get("bias")))
+    keys = ["weight", "scales", "biases"] + (["bias"] if bias else [])
+    inter = {k: ops.interleave_gate_up(gd[k], ud[k]) for k in keys}
+    return dict(partial=partial, slabs=slabs, h=to_dev(h, dev), nw=to_dev(nw, dev), eps=eps, inter=inter,
+                h2=h2, want=want, M=M, D=D, I=I)
+
+
+def run_chain(dev, c, scratch, err, spin=None):
+    h = c["h"].clone()
+    act = torch.full((c["M"], c["I"]), float("nan"), dtype=torch.float16, device=dev)
+    kw = {} if spin is None else {"spin_ticks": spin}
+    ops.norm_mlp_in(c["partial"], c["slabs"], h, c["nw"], c["eps"], c["inter"]["weight"], c["inter"]["scales"],
+                    c["inter"]["biases"], c["inter"].get("bias"), act, scratch, err, **kw)
+    torch.cuda.synchronize()
+    return h, act
+
+
+def check_swiglu(got, want):
+    g64, w64 = got.astype(np.float64), want.astype(np.float64)
+    rms = np.sqrt(np.mean(w64 * w64))
+    ulp = 2.0 ** (np.floor(np.log2(np.maximum(np.abs(w64), 2.0 ** -14))) - 10)
+    assert np.all(np.abs(g64 - w64) <= TOL * rms + 2 * ulp)
+    assert np.sqrt(np.mean((g64 - w64) ** 2)) <= 0.1 * TOL * rms
+
+
+@pytest.mark.parametrize("M,D,I,bias", [(32, 512, 256, False), (8, 1024, 1536, True), (17, 1536, 4864, True),
+                                        (32, 3584, 18944, False)])
+def test_norm_and_mlp_in_one_launch(dev, M, D, I, bias):
+    """Residual add + sums of squares, grid barrier, RMSNorm + gate|up + SwiGLU in one launch of
+    a resident grid, against the oracle's separate operators; three launches in a row on the same
+    scratch (the barrier counters only grow).  The new h is bit-identical to the separate
+    kernels' (same slab sums, same rounding)."""
+    print(f"chain M={M} D={D} I={I}", flush=True)
+    assert ops.norm_mlp_in_supported(M, D, I)
+    c = chain_case(dev, M, D, I, seed=M + D + I, bias=bias)
+    scratch, err = ops.norm_mlp_in_scratch(dev)
+    for rep in range(3):
+        h, act = run_chain(dev, c, scratch, err)
+        assert int(err.item()) == 0
+        assert np.array_equal(h.cpu().numpy(), c["h2"])
+        check_swiglu(act.cpu().numpy(), c["want"])
+
+
+def test_grid_barrier_gives_up_and_recovers(dev):
+    """The bounded wait of the in-kernel barrier, forced from the host: with a limit of one tick
+    (10 ns) workgroups give up, the error word is set, the launch still ends normally; after
+    the scratch and the error word are zeroed the next launch is correct."""
+    c = chain_case(dev, 32, 1024, 1536, seed=77, bias=False)
+    scratch, err = ops.norm_mlp_in_scratch(dev)
+    run_chain(dev, c, scratch, err, spin=1)
+    assert int(err.item()) == 1
+    scratch.zero_()
+    err.zero_()
+    h, act = run_chain(dev, c, scratch, err)
+    assert int(err.item()) == 0
+    assert np.array_equal(h.cpu().numpy(), c["h2"])
+    check_swiglu(act.cpu().numpy(), c["want"])
+
+
+def test_verifier_with_the_chained_launch(dev):
+    """TreeVerifier(chain=True): the whole step with norm + gate|up as one resident-grid launch
+    per layer against the oracle, replayed as a HIP graph (every replay equal to the first, the
+    barrier never gives up)."""
+    import test_gpu_model as tm
+    from mlx_eagle_spec_decoding_tree_amd import eagle
+    from oracle import model_oracle
+    P, T = 200, 32
+    s = tm.build(dev, "llama_like_tied", P, T, seed=9)
+    want = model_oracle.verify_step(s["args"], s["weights"], s["inv"], s["sc"], s["tokens"], s["depth"],
+                                    s["parents"], s["anc"], s["ocache"], P)
+    ver = tm.run_verifier(s, dev, graph=True, chain=True, compact=False)
+    assert ver.chain and ver.slab["o"]
+    outs = []
+    for rep in range(3):
+        ver.len_dev.fill_(P)
+        ver.step()
+        torch.cuda.synchronize()
+        outs.append(ver.logits.clone())
+        assert not ver.chain_error()
+    assert torch.equal(outs[0], outs[1]) and torch.equal(outs[0], outs[2])
+    assert rel_err(outs[0].cpu().numpy(), want["logits"]) <= TOL
+    r = ver.result.cpu().numpy()
+    am = ver.node_argmax.cpu().numpy()
+    assert np.array_equal(am, oracle.argmax_rows(outs[0].cpu().numpy()))
+    with pytest.raises(ValueError):
+        s2 = tm.build(dev, "qwen_like", 40, 8, seed=1)        # hidden 256: the chained launch does not take it
+        eagle.TreeVerifier(s2["model"], s2["cache"], total_tokens=7, chain=True)
