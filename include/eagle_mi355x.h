@@ -34,7 +34,9 @@ enum eagle_status {
   EAGLE_ERR_ARCH = 7         /* current device is not gfx950 */
 };
 
-#define EAGLE_MAX_TREE 32    /* tree tokens per verify step (root + 31 nodes) */
+#define EAGLE_MAX_TREE 32    /* tree tokens per fused verify step (root + 31 nodes): matmul rows, one mask word */
+#define EAGLE_MAX_TREE_SLOTS 64 /* tree tokens the tree-layout kernels take (root + 63 nodes; the reference's
+                                   default is 39 nodes, mlx_eagle.py:390,510) */
 #define EAGLE_MAX_CHUNK 1024 /* rows of one causal pass over a prompt chunk */
 #define EAGLE_MAX_M 32       /* rows of x accepted by the quantised matmul */
 
@@ -344,7 +346,8 @@ int eagle_argmax_rows_f16(const void* logits, int32_t* out, int R, long V,
  * best (descending score, ties to the lowest flat index), order them by flat
  * index and emit
  *   tree_position_ids [T] int32, mask_index [total] int32, draft_tokens [T] int32,
- *   tree_mask_bits [T] uint32 (ancestor-or-self rows), T = total + 1 <= 32.
+ *   tree_mask_bits (ancestor-or-self rows): [T] uint32 for T = total + 1 <= 32, [T][2] uint32
+ *   (low word, high word) for 32 < T <= EAGLE_MAX_TREE_SLOTS.
  * parents_list [C/k] uint32: 0 for the root's children, else parent flat id + 1.
  * sampled_token_dev: the root token. */
 int eagle_process_draft_tree(const void* scores, const int32_t* tokens,
@@ -354,7 +357,8 @@ int eagle_process_draft_tree(const void* scores, const int32_t* tokens,
                              uint32_t* tree_mask_bits, eagle_stream_t stream);
 
 /* post_process_draft_tree (mlx_eagle.py:254-295) without the host round trip:
- * retrieve_indices [32,32] int32 (row r = path of the r-th leaf, -1 padded),
+ * retrieve_indices [64,64] int32 (row r = path of the r-th leaf, -1 padded; EAGLE_MAX_TREE_SLOTS
+ * rows and columns whatever the tree size),
  * shape_out [2] int32 = {leaf_num, max_depth + 1}. */
 int eagle_post_process_draft_tree(const int32_t* tree_position_ids, const int32_t* mask_index,
                                   int total, int32_t* retrieve_indices, int32_t* shape_out,
@@ -362,10 +366,10 @@ int eagle_post_process_draft_tree(const int32_t* tree_position_ids, const int32_
 
 /* Greedy acceptance (evaluate_posterior_greedy, mlx_eagle.py:311-326, with the
  * gathers of :582-589).  node_argmax [T] is the argmax token of each tree node's
- * logits.  retrieve_indices [32,32] / shape as produced above; a -1 entry
- * selects node T-1, as the reference's negative gather index does.
- * result [4 + 32] int32 = {best, accept_length, bonus_node, next_token,
- * accept_indices[0..accept_length)}; accepted_tokens [32] int32. */
+ * logits, T <= EAGLE_MAX_TREE_SLOTS.  retrieve_indices [64,64] / shape as produced above; a -1
+ * entry selects node T-1, as the reference's negative gather index does.
+ * result [4 + 64] int32 = {best, accept_length, bonus_node, next_token,
+ * accept_indices[0..accept_length)}; accepted_tokens [64] int32. */
 int eagle_greedy_accept(const int32_t* node_argmax, const int32_t* draft_tokens,
                         const int32_t* retrieve_indices, const int32_t* shape, int T,
                         int32_t* result, int32_t* accepted_tokens, eagle_stream_t stream);
@@ -374,7 +378,7 @@ int eagle_greedy_accept(const int32_t* node_argmax, const int32_t* draft_tokens,
  * rows P + accept_indices[j] move to P + 1 + j for j < accept_length (gather
  * first, then scatter), then *cache_len_dev = min(P + accept_length + 1, capacity).
  * caches: device array of n_caches pointers to [G,capacity,hd] fp16 buffers.
- * accept [4 + 32] int32 in the layout of eagle_greedy_accept's result. */
+ * accept [4 + 64] int32 in the layout of eagle_greedy_accept's result. */
 int eagle_kv_compact_f16(void* const* caches_dev, int n_caches, const int32_t* accept,
                          int32_t* cache_len_dev, int G, int hd, long capacity,
                          eagle_stream_t stream);

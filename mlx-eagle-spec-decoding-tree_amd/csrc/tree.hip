@@ -7,7 +7,7 @@
 
 namespace {
 
-constexpr int MAXT = EAGLE_MAX_TREE;   // 32
+constexpr int MAXT = EAGLE_MAX_TREE_SLOTS;   // 64: tree tokens the kernels of this file lay out
 constexpr int MAXC = 1024;             // draft candidates (k + k*k*depth)
 
 // mlx_eagle.py:217-250 (with topk :24-58 and search_sorted :61-93).
@@ -20,7 +20,7 @@ __global__ __launch_bounds__(256) void process_draft_tree_kernel(
   __shared__ unsigned char picked[MAXC];
   __shared__ int sel[MAXT];
   __shared__ int midx[MAXT];
-  __shared__ uint32_t bits[MAXT];
+  __shared__ unsigned long long bits[MAXT];
   const int tid = threadIdx.x;
   // a NaN score ranks as -inf: with the index tie rule the order below is then total, so
   // exactly `total` candidates are picked whatever the scores hold
@@ -75,7 +75,7 @@ __global__ __launch_bounds__(256) void process_draft_tree_kernel(
     // identity rows first, then the sequential OR of mlx_eagle.py:239-243 (a parent slot ahead
     // of its child, which only poisoned scores can produce, then reads an identity row, as the
     // reference's loop over an identity matrix does)
-    for (int i = 0; i <= total; ++i) bits[i] = 1u << i;
+    for (int i = 0; i <= total; ++i) bits[i] = 1ull << i;
     for (int i = 0; i < total; ++i) {
       const int par = midx[i] < 0 ? 0 : (midx[i] > total ? total : midx[i]);
       bits[i + 1] |= bits[par];
@@ -83,13 +83,19 @@ __global__ __launch_bounds__(256) void process_draft_tree_kernel(
   }
   __syncthreads();
   if (tid <= total) {
-    bits_out[tid] = bits[tid];
-    pos_ids[tid] = __popc(bits[tid]) - 1;
+    // one mask word per row for trees of at most 32 tokens, two (low, high) above that
+    if (total + 1 <= 32) {
+      bits_out[tid] = (uint32_t)bits[tid];
+    } else {
+      bits_out[2 * tid] = (uint32_t)bits[tid];
+      bits_out[2 * tid + 1] = (uint32_t)(bits[tid] >> 32);
+    }
+    pos_ids[tid] = __popcll(bits[tid]) - 1;
   }
 }
 
-// mlx_eagle.py:254-295.  retrieve [32][32], shape {leaf_num, max_depth + 1}.
-__global__ __launch_bounds__(64) void post_process_kernel(const int32_t* __restrict__ pos_ids,
+// mlx_eagle.py:254-295.  retrieve [64][64], shape {leaf_num, max_depth + 1}.
+__global__ __launch_bounds__(128) void post_process_kernel(const int32_t* __restrict__ pos_ids,
                                                           const int32_t* __restrict__ mask_index,
                                                           int total, int32_t* __restrict__ retrieve,
                                                           int32_t* __restrict__ shape) {
@@ -128,7 +134,7 @@ __global__ __launch_bounds__(64) void post_process_kernel(const int32_t* __restr
 }
 
 // mlx_eagle.py:311-326 on per-node argmax tokens, with the gathers of :582-589.
-__global__ __launch_bounds__(64) void greedy_accept_kernel(
+__global__ __launch_bounds__(128) void greedy_accept_kernel(
     const int32_t* __restrict__ node_argmax, const int32_t* __restrict__ draft_tokens,
     const int32_t* __restrict__ retrieve, const int32_t* __restrict__ shape, int T,
     int32_t* __restrict__ result, int32_t* __restrict__ accepted_tokens) {
@@ -258,7 +264,7 @@ EAGLE_EXPORT int eagle_post_process_draft_tree(const int32_t* tree_position_ids,
                                                eagle_stream_t stream) {
   if (!tree_position_ids || !mask_index || !retrieve_indices || !shape_out) return EAGLE_ERR_NULL;
   if (total < 1 || total >= MAXT) return EAGLE_ERR_SHAPE;
-  hipLaunchKernelGGL(post_process_kernel, dim3(1), dim3(64), 0, static_cast<hipStream_t>(stream),
+  hipLaunchKernelGGL(post_process_kernel, dim3(1), dim3(128), 0, static_cast<hipStream_t>(stream),
                      tree_position_ids, mask_index, total, retrieve_indices, shape_out);
   return eagle_launch_status();
 }
@@ -270,7 +276,7 @@ EAGLE_EXPORT int eagle_greedy_accept(const int32_t* node_argmax, const int32_t* 
   if (!node_argmax || !draft_tokens || !retrieve_indices || !shape || !result || !accepted_tokens)
     return EAGLE_ERR_NULL;
   if (T < 1 || T > MAXT) return EAGLE_ERR_SHAPE;
-  hipLaunchKernelGGL(greedy_accept_kernel, dim3(1), dim3(64), 0, static_cast<hipStream_t>(stream),
+  hipLaunchKernelGGL(greedy_accept_kernel, dim3(1), dim3(128), 0, static_cast<hipStream_t>(stream),
                      node_argmax, draft_tokens, retrieve_indices, shape, T, result,
                      accepted_tokens);
   return eagle_launch_status();

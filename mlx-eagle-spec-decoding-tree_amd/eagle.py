@@ -11,7 +11,8 @@ import torch
 
 from . import _lib, ops
 
-MAXT = 32
+MAXT = 32            # tree tokens of the fused verification step (matmul rows, one mask word)
+TREE_SLOTS = 64      # tree tokens the tree-layout kernels and the module path take
 
 
 def _ptr(t):
@@ -55,9 +56,12 @@ def search_sorted(arr, target, left=True):
 
 
 def bits_to_mask(bits, dtype=torch.bfloat16):
-    """[T] int32 row bitmasks -> [T,T] additive mask (0 where visible, -inf elsewhere)."""
-    T = bits.numel()
+    """[T] int32 row bitmasks (or [T,2]: low and high word of trees above 32 tokens) -> [T,T]
+    additive mask (0 where visible, -inf elsewhere)."""
+    T = bits.shape[0]
     b = bits.to(torch.int64) & 0xFFFFFFFF
+    if bits.dim() == 2:
+        b = b[:, 0] | (b[:, 1] << 32)
     vis = ((b[:, None] >> torch.arange(T, device=bits.device)[None, :]) & 1).bool()
     zero = torch.zeros((), dtype=dtype, device=bits.device)
     return torch.where(vis, zero, torch.full((), -math.inf, dtype=dtype, device=bits.device))
@@ -152,7 +156,7 @@ def process_draft_tree_device(scores, tokens, parents_list, sampled_token_id, k,
         out = (torch.empty(T, dtype=torch.int32, device=dev),
                torch.empty(total_tokens, dtype=torch.int32, device=dev),
                torch.empty(T, dtype=torch.int32, device=dev),
-               torch.empty(T, dtype=torch.int32, device=dev))
+               torch.empty(T if T <= 32 else (T, 2), dtype=torch.int32, device=dev))
     pos, midx, toks, bits = out
     rc = _lib.lib().eagle_process_draft_tree(
         _ptr(scores), _ptr(tokens), _ptr(parents_list), _ptr(sampled_token_id), C, k,
@@ -175,10 +179,10 @@ def process_draft_tree(scores_list, ss_token, parents_list, sampled_token_id, k,
 
 
 def post_process_draft_tree_device(tree_position_ids, total_tokens, mask_index, out=None):
-    """retrieve_indices [32,32] (-1 padded) and shape [2] = {leaf_num, max_depth+1}, on device."""
+    """retrieve_indices [64,64] (-1 padded) and shape [2] = {leaf_num, max_depth+1}, on device."""
     dev = tree_position_ids.device
     if out is None:
-        out = (torch.empty((MAXT, MAXT), dtype=torch.int32, device=dev),
+        out = (torch.empty((TREE_SLOTS, TREE_SLOTS), dtype=torch.int32, device=dev),
                torch.empty(2, dtype=torch.int32, device=dev))
     rc = _lib.lib().eagle_post_process_draft_tree(_ptr(tree_position_ids), _ptr(mask_index),
                                                   total_tokens, _ptr(out[0]), _ptr(out[1]),
@@ -224,7 +228,7 @@ def accept_candidate(cache, accept_indices, accept_length, offset):
     accept_length = int(accept_length)
     if accept_length > 0:
         dev = cache[0].keys.device
-        acc = torch.zeros(4 + MAXT, dtype=torch.int32, device=dev)
+        acc = torch.zeros(4 + TREE_SLOTS, dtype=torch.int32, device=dev)
         acc[1] = accept_length
         acc[4:4 + accept_length] = accept_indices.to(torch.int32).reshape(-1)[:accept_length]
         len_dev = torch.tensor([offset], dtype=torch.int32, device=dev)
@@ -239,19 +243,19 @@ def accept_candidate(cache, accept_indices, accept_length, offset):
 
 
 def _check_tree_size(verify_num_tokens):
-    """The tree kernels, the mask words of the verification attention and the matmul rows are
-    laid out for 32 tree tokens (root + 31 nodes); the reference's default of 39 nodes
-    (mlx_eagle.py:390,510) is kept in the signatures and refused here."""
-    if verify_num_tokens + 1 > MAXT:
+    """The tree kernels lay a tree out in 64 slots (root + 63 nodes): the reference's default of
+    39 nodes (mlx_eagle.py:390,510) runs on the module path (matmuls of more than 32 rows as
+    tiled GEMMs, attention over two mask words per query in pieces of 32 queries); the fused
+    `TreeVerifier` / `SpeculativeDecoder` step takes 32 tree tokens."""
+    if verify_num_tokens + 1 > TREE_SLOTS:
         raise NotImplementedError(
-            f"verify_num_tokens={verify_num_tokens}: this build verifies at most {MAXT - 1} draft nodes per "
-            f"step (a tree of {MAXT} tokens); pass verify_num_tokens={MAXT - 1} or less")
+            f"verify_num_tokens={verify_num_tokens}: this build verifies at most {TREE_SLOTS - 1} draft nodes "
+            f"per step (a tree of {TREE_SLOTS} tokens)")
 
 
 def spec_step(y, base_model, draft_model, base_cache, draft_cache, offset=None, accept_length=0,
               k=8, depth=5, verify_num_tokens=39, tokenizer=None):
-    """mlx_eagle.py:379-463 up to its first return (same defaults; this build lays a tree out in
-    32 slots, so verify_num_tokens above 31 raises NotImplementedError): the draft forward of the tokens accepted
+    """mlx_eagle.py:379-463 up to its first return (same defaults; at most 63 draft nodes): the draft forward of the tokens accepted
     last step, the level-0 top-k, the expansion, the tree layout and the target forward.
     y [1, accept_length + 1] int.  Returns (tree_position_ids, mask_index, draft_tokens,
     base_logits, base_offset, draft_offset)."""
@@ -291,7 +295,7 @@ def generate_step(prompt, base_model, draft_model, prefill_step_size=512, k=8, d
     _check_tree_size(verify_num_tokens)
     y = prompt.reshape(-1).to(torch.int64)
     if capacity is None:
-        capacity = y.numel() + max_tokens + N + k * depth + MAXT + 16
+        capacity = y.numel() + max_tokens + N + k * depth + TREE_SLOTS + 16
     base_cache = make_prompt_cache(base_model, capacity=capacity)
     draft_cache = make_prompt_cache(draft_model, capacity=capacity)
     while y.numel() > prefill_step_size:
@@ -468,6 +472,10 @@ class TreeVerifier:
         `chain_error()` reports a barrier that gave up."""
         args = model.args
         self.model, self.cache, self.args = model, cache, args
+        if total_tokens + 1 > MAXT:
+            raise NotImplementedError(f"the fused verification step takes at most {MAXT} tree tokens "
+                                      f"(total_tokens <= {MAXT - 1}); larger trees run on the module path "
+                                      "(`tree_decoding`)")
         self.V = total_tokens
         self.T = T = total_tokens + 1
         dev = model.device
@@ -500,11 +508,11 @@ class TreeVerifier:
         self.mask_index = torch.zeros(total_tokens, **i32)
         self.mask_bits = torch.zeros(T, **i32)
         self.positions = torch.zeros(T, **i32)
-        self.retrieve = torch.zeros((MAXT, MAXT), **i32)
+        self.retrieve = torch.zeros((TREE_SLOTS, TREE_SLOTS), **i32)
         self.shape = torch.zeros(2, **i32)
         self.node_argmax = torch.zeros(T, **i32)
-        self.result = torch.zeros(4 + MAXT, **i32)
-        self.accepted_tokens = torch.zeros(MAXT, **i32)
+        self.result = torch.zeros(4 + TREE_SLOTS, **i32)
+        self.accepted_tokens = torch.zeros(TREE_SLOTS, **i32)
         self.h = torch.empty((T, D), **f16)
         self.hn = torch.empty((T, D), **f16)
         # q | k | v of a token side by side: one fused projection writes all three

@@ -499,7 +499,8 @@ def draft_attention(q, k_cache, v_cache, mask_words, cache_len_dev, Tk, scale, m
 
 def scaled_dot_product_attention(queries, keys, values, cache=None, scale=None, mask=None):
     """Drop-in for the call at mlx_llama.py:185-192 on the tree and draft paths:
-    queries [1,H,T,hd] with T <= 32, keys/values [1,G,S,hd], mask [1,1,T,S] additive.  Only
+    queries [1,H,T,hd] with T <= 64 (32 query rows per launch set), keys/values [1,G,S,hd],
+    mask [1,1,T,S] additive.  Only
     the last min(S, 64) columns of the mask are looked at: every earlier column has to be zero
     (a prefix that all queries see), which holds for the verification mask
     (mlx_eagle.py:337-338), the expansion masks up to depth 8 (mlx_eagle.py:143-171) and causal
@@ -521,7 +522,19 @@ def scaled_dot_product_attention(queries, keys, values, cache=None, scale=None, 
         k_buf, v_buf = cache.keys[0], cache.values[0]        # the fetched views alias the cache
     else:
         k_buf, v_buf = _f16(keys[0], "k"), _f16(values[0], "v")
-    out = draft_attention(_f16(queries[0], "q"), k_buf, v_buf, words, len_dev, Tk, scale, max_len=S)
+    q = _f16(queries[0], "q")
+    if T <= 32:
+        out = draft_attention(q, k_buf, v_buf, words, len_dev, Tk, scale, max_len=S)
+    else:
+        # more than 32 queries (a tree of up to 64 tokens): pieces of 32 query rows, each with
+        # its own mask rows over the same keys
+        if T > 64:
+            raise ValueError("at most 64 query rows")
+        out = torch.empty((T, H * hd), dtype=torch.float16, device=q.device)
+        for t0 in range(0, T, 32):
+            t1 = min(T, t0 + 32)
+            draft_attention(q[:, t0:t1].contiguous(), k_buf, v_buf, words[t0:t1].contiguous(), len_dev, Tk,
+                            scale, max_len=S, out=out[t0:t1])
     return out.reshape(T, H, hd).permute(1, 0, 2).unsqueeze(0).contiguous()
 
 

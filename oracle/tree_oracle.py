@@ -179,12 +179,11 @@ def tree_from_parents(parents):
 
 
 def mask_bits(anc):
-    """Row bitmasks (bit j of word i set iff node j is visible to node i)."""
+    """Row bitmasks (bit j of word i set iff node j is visible to node i): [T] uint32 for trees
+    of at most 32 tokens, [T, 2] (low word, high word) up to 64."""
     T = anc.shape[0]
-    assert T <= 32
-    out = np.zeros(T, np.uint32)
-    for i in range(T):
-        for j in range(T):
-            if anc[i, j]:
-                out[i] |= np.uint32(1 << j)
-    return out
+    assert T <= 64
+    rows = [sum(1 << j for j in range(T) if anc[i, j]) for i in range(T)]
+    if T <= 32:
+        return np.array(rows, np.uint64).astype(np.uint32)
+    return np.array([[r & 0xFFFFFFFF, r >> 32] for r in rows], np.uint64).astype(np.uint32)

@@ -251,6 +251,23 @@ def test_generate_step_stream_equals_target_greedy(dev, same):
         assert len(acc) == al and len(y) == al + 1
 
 
+def test_generate_step_with_the_reference_default_tree(dev):
+    """depth 5, 39 draft nodes (the reference's defaults, mlx_eagle.py:509-510): a tree of 40 tokens
+    runs on the module path (tiled GEMMs for 40 rows, attention in two pieces of query rows);
+    the emitted stream is the target's greedy stream."""
+    (targs, tw, target), (dargs, dw, draft) = tiny_pair(dev, same=True, seed=6)
+    rng = np.random.default_rng(9)
+    prompt = rng.integers(0, targs.vocab_size, 40).astype(np.int32)
+    res = eagle.generate_step(to_dev(prompt.astype(np.int64), dev), target, draft, max_tokens=48, N=5)
+    assert res["n"] == len(res["tokens"]) == sum(1 + s[0] for s in res["steps"])
+    assert_greedy_stream(target, prompt, [res["first"]] + res["tokens"], dev)
+    assert res["mean_tokens_per_step"] >= 3.0
+    with pytest.raises(NotImplementedError):
+        eagle.generate_step(to_dev(prompt.astype(np.int64), dev), target, draft, verify_num_tokens=64)
+    with pytest.raises(NotImplementedError):
+        eagle.TreeVerifier(target, make_prompt_cache(target, capacity=128), total_tokens=39)
+
+
 def test_generate_step_matches_oracle_loop(dev):
     (targs, tw, target), (dargs, dw, draft) = tiny_pair(dev, same=False, seed=11)
     rng = np.random.default_rng(12)

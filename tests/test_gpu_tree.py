@@ -62,6 +62,26 @@ def test_nan_scores_leave_a_well_formed_tree(dev, n_nan):
         assert np.array_equal(bits.cpu().numpy().view(np.uint32), to.mask_bits(anc_w))
 
 
+@pytest.mark.parametrize("depth,V", [(5, 39), (5, 63), (3, 32), (7, 47)])
+def test_trees_above_32_tokens_bit_exact(dev, depth, V):
+    """Up to 64 tree slots (the reference's default is 39 nodes at depth 5, mlx_eagle.py:390,510):
+    two mask words per row, 64 x 64 retrieve matrix."""
+    rng = np.random.default_rng(depth * 41 + V)
+    for trial in range(8):
+        scores, tokens, parents_list, _ = simulate_draft(rng, depth, tie_levels=(4 if trial % 2 else None))
+        pos_w, midx_w, toks_w, anc_w = to.process_draft_tree(scores, tokens, parents_list, np.array([[9]]), 8, V)
+        pos, midx, toks, bits = dev_process(dev, scores, tokens, parents_list, 9, 8, V)
+        assert tuple(bits.shape) == (V + 1, 2)
+        assert np.array_equal(pos.cpu().numpy(), pos_w)
+        assert np.array_equal(midx.cpu().numpy(), midx_w)
+        assert np.array_equal(toks.cpu().numpy(), toks_w[0])
+        assert np.array_equal(bits.cpu().numpy().view(np.uint32), to.mask_bits(anc_w))
+        assert np.array_equal(eagle.bits_to_mask(bits).float().cpu().numpy() == 0, anc_w)
+        ri_w = to.post_process_draft_tree(pos_w, V, midx_w)
+        ri = eagle.post_process_draft_tree(pos, V, midx).cpu().numpy()
+        assert ri.shape == ri_w.shape and np.array_equal(ri, ri_w)
+
+
 def test_reference_signature_process_draft_tree(dev):
     """List-of-levels inputs and the (position_ids, mask_index, draft_tokens[1,T], bf16 mask) tuple."""
     rng = np.random.default_rng(5)
@@ -101,16 +121,16 @@ def test_greedy_accept_kernel_bit_exact(dev):
     rng = np.random.default_rng(21)
     L = _lib.lib()
     for trial in range(150):
-        T = int(rng.integers(2, 33))
-        parents = synth.random_tree(rng, T)
+        T = int(rng.integers(2, 65))
+        parents = synth.random_tree(rng, T, max_depth=6 if T > 32 else 4, max_children=6 if T > 32 else 4)
         depth, anc = to.tree_from_parents(parents)
         ri_w = to.post_process_draft_tree(depth, T - 1, parents)
         tokens = rng.integers(0, 5, T).astype(np.int32)
         am = rng.integers(0, 5, T).astype(np.int32)
         best, al, bonus = to.greedy_accept(am, tokens, ri_w)
         full, shape = eagle.post_process_draft_tree_device(to_dev(depth, dev), T - 1, to_dev(parents, dev))
-        result = torch.zeros(36, dtype=torch.int32, device=dev)
-        acc_t = torch.zeros(32, dtype=torch.int32, device=dev)
+        result = torch.zeros(68, dtype=torch.int32, device=dev)
+        acc_t = torch.zeros(64, dtype=torch.int32, device=dev)
         am_d, tok_d = to_dev(am, dev), to_dev(tokens, dev)
         rc = L.eagle_greedy_accept(am_d.data_ptr(), tok_d.data_ptr(), full.data_ptr(),
                                    shape.data_ptr(), T, result.data_ptr(), acc_t.data_ptr(), None)
@@ -124,13 +144,13 @@ def test_greedy_accept_kernel_bit_exact(dev):
 
 def test_padding_quirk_on_device(dev):
     L = _lib.lib()
-    ri = np.full((32, 32), -1, np.int32)
+    ri = np.full((64, 64), -1, np.int32)
     ri[0, :5] = [0, 1, 2, 4, 6]
     ri[1, :6] = [0, 1, 2, 3, 5, 7]
     tokens = np.arange(8, dtype=np.int32)
     am = np.array([1, 2, 4, 9, 6, 9, 7, 9], np.int32)
-    result = torch.zeros(36, dtype=torch.int32, device=dev)
-    acc_t = torch.zeros(32, dtype=torch.int32, device=dev)
+    result = torch.zeros(68, dtype=torch.int32, device=dev)
+    acc_t = torch.zeros(64, dtype=torch.int32, device=dev)
     shape = torch.tensor([2, 6], dtype=torch.int32, device=dev)
     am_d, tok_d, ri_d = to_dev(am, dev), to_dev(tokens, dev), to_dev(ri, dev)
     rc = L.eagle_greedy_accept(am_d.data_ptr(), tok_d.data_ptr(), ri_d.data_ptr(),

@@ -74,10 +74,10 @@ def test_other_entry_points_reject_bad_arguments():
     assert L.eagle_add_f16(p, p, p + 2, 16, None) == 3
     assert L.eagle_embed_w4g64_f16(p, p, p, p, p, 4, 100, 10, None) == 2
     assert L.eagle_argmax_rows_f16(p, p, 4, 1000, None, 0, None) == 5
-    assert L.eagle_process_draft_tree(p, p, p, p, 200, 8, 32, p, p, p, p, None) == 2    # total must be < 32
+    assert L.eagle_process_draft_tree(p, p, p, p, 200, 8, 64, p, p, p, p, None) == 2    # total must be < 64
     assert L.eagle_process_draft_tree(p, p, p, p, 2000, 8, 31, p, p, p, p, None) == 2   # too many candidates
     assert L.eagle_post_process_draft_tree(p, p, 0, p, p, None) == 2
-    assert L.eagle_greedy_accept(p, p, p, p, 40, p, p, None) == 2
+    assert L.eagle_greedy_accept(p, p, p, p, 65, p, p, None) == 2
     assert L.eagle_kv_compact_f16(None, 4, p, p, 4, 128, 100, None) == 1
     assert L.eagle_tree_positions(p, p, p, 0, None) == 2
 
