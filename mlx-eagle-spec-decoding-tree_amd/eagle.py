@@ -10,6 +10,7 @@ import math
 import torch
 
 from . import _lib, ops
+from .layer import emit_layer
 
 MAXT = 32            # tree tokens of the fused verification step (matmul rows, one mask word)
 TREE_SLOTS = 64      # tree tokens the tree-layout kernels and the module path take
@@ -625,86 +626,22 @@ class TreeVerifier:
         if self.fuse:   # one cos/sin table per step: the positions are the same in every layer
             at0 = layers[0].self_attn
             ops.rope_table(self.positions, at0._inv_freqs, at0._scaling_factor, out=self.rope_cs)
+
+        def attend(at, c):
+            ops.tree_attention(self.q_rot, c.keys[0], c.values[0], self.mask_bits, self.len_dev, at.scale,
+                               max_len=self.max_len, out=self.attn)
+
+        def attend_with_rope(at, c, q_lin, k_lin, v_lin):
+            ops.tree_attention_rope(q_lin, k_lin, v_lin, self.rope_cs, c.keys[0], c.values[0], self.mask_bits,
+                                    self.len_dev, at.scale, H, G, hd, row_stride=(H + 2 * G) * hd,
+                                    max_len=self.max_len, out=self.attn)
+
         for i, layer in enumerate(layers):
-            at = layer.self_attn
-            c = self.cache[i]
             if self.fuse:
-                w, sc, bi, b = self.qkv_w[i]
-                q_lin, k_lin, v_lin = self.qkv, self.qkv[:, H * hd:], self.qkv[:, (H + G) * hd:]
-                if self.slab["qkv"]:
-                    s = self.slab["qkv"]
-                    ops.quantized_matmul_slabs(self.hn, w, sc, bi, s, partial=self.partial)
-                    ops.rope_kv_append_slabs(self.partial, ops.slab_count(args.hidden_size, s), b,
-                                             self.rope_cs, self.q_rot, c.keys[0], c.values[0],
-                                             self.len_dev, T, H, G, hd)
-                elif self.one_launch_attention:
-                    ops.quantized_matmul(self.hn, w, sc, bi, bias=b, out=self.qkv)
-                    ops.tree_attention_rope(q_lin, k_lin, v_lin, self.rope_cs, c.keys[0], c.values[0],
-                                            self.mask_bits, self.len_dev, at.scale, H, G, hd,
-                                            row_stride=(H + 2 * G) * hd, max_len=self.max_len,
-                                            out=self.attn)
-                else:
-                    ops.quantized_matmul(self.hn, w, sc, bi, bias=b, out=self.qkv)
-                    ops.rope_kv_append(q_lin, k_lin, v_lin, self.positions, at._inv_freqs,
-                                       at._scaling_factor, self.q_rot, c.keys[0], c.values[0],
-                                       self.len_dev, H, G, hd, row_stride=(H + 2 * G) * hd,
-                                       rope_cs=self.rope_cs)
+                emit_layer(self, i, self.len_dev, attend, positions=self.positions,
+                           attend_with_rope=attend_with_rope if self.one_launch_attention else None)
             else:
-                for lin, out in ((at.q_proj, self.q), (at.k_proj, self.k), (at.v_proj, self.v)):
-                    ops.quantized_matmul(self.hn, lin.weight, lin.scales, lin.biases, bias=lin.bias, out=out)
-                ops.rope_kv_append(self.q, self.k, self.v, self.positions, at._inv_freqs,
-                                   at._scaling_factor, self.q_rot, c.keys[0], c.values[0],
-                                   self.len_dev, H, G, hd)
-            if not self.one_launch_attention:
-                ops.tree_attention(self.q_rot, c.keys[0], c.values[0], self.mask_bits, self.len_dev,
-                                   at.scale, max_len=self.max_len, out=self.attn)
-            mlp = layer.mlp
-            if self.chain:
-                s = self.slab["o"]
-                ops.quantized_matmul_slabs(self.attn, at.o_proj.weight, at.o_proj.scales, at.o_proj.biases,
-                                           s, partial=self.partial)
-                w, sc, bi, b = self.gu_w[i]
-                ops.norm_mlp_in(self.partial, ops.slab_count(H * hd, s), self.h,
-                                layer.post_attention_layernorm.weight, args.rms_norm_eps, w, sc, bi, b,
-                                self.act, self.chain_scratch, self.chain_err)
-            elif self.slab["o"]:
-                s = self.slab["o"]
-                ops.quantized_matmul_slabs(self.attn, at.o_proj.weight, at.o_proj.scales, at.o_proj.biases,
-                                           s, partial=self.partial)
-                ops.rms_norm_slabs(self.partial, ops.slab_count(H * hd, s),
-                                   layer.post_attention_layernorm.weight, args.rms_norm_eps, T,
-                                   residual=self.h, out=self.hn, h_out=self.h)
-            else:
-                ops.quantized_matmul(self.attn, at.o_proj.weight, at.o_proj.scales, at.o_proj.biases,
-                                     bias=at.o_proj.bias, out=self.o)
-                ops.rms_norm(self.o, layer.post_attention_layernorm.weight, args.rms_norm_eps,
-                             residual=self.h, out=self.hn, h_out=self.h)
-            if self.chain:
-                pass
-            elif self.fuse:
-                w, sc, bi, b = self.gu_w[i]
-                if self.swiglu:
-                    ops.quantized_matmul_swiglu(self.hn, w, sc, bi, bias=b, out=self.act)
-                else:
-                    ops.quantized_matmul(self.hn, w, sc, bi, bias=b, out=self.gate_up)
-                    ops.silu_mul(self.gate_up, None, out=self.act)
-            else:
-                ops.quantized_matmul(self.hn, mlp.gate_proj.weight, mlp.gate_proj.scales,
-                                     mlp.gate_proj.biases, bias=mlp.gate_proj.bias, out=self.gate)
-                ops.quantized_matmul(self.hn, mlp.up_proj.weight, mlp.up_proj.scales,
-                                     mlp.up_proj.biases, bias=mlp.up_proj.bias, out=self.up)
-                ops.silu_mul(self.gate, self.up, out=self.act)
-            nxt = layers[i + 1].input_layernorm.weight if i + 1 < len(layers) else m.model.norm.weight
-            if self.slab["down"]:
-                s = self.slab["down"]
-                ops.quantized_matmul_slabs(self.act, mlp.down_proj.weight, mlp.down_proj.scales,
-                                           mlp.down_proj.biases, s, partial=self.partial)
-                ops.rms_norm_slabs(self.partial, ops.slab_count(args.intermediate_size, s), nxt,
-                                   args.rms_norm_eps, T, residual=self.h, out=self.hn, h_out=self.h)
-            else:
-                ops.quantized_matmul(self.act, mlp.down_proj.weight, mlp.down_proj.scales,
-                                     mlp.down_proj.biases, bias=mlp.down_proj.bias, out=self.down)
-                ops.rms_norm(self.down, nxt, args.rms_norm_eps, residual=self.h, out=self.hn, h_out=self.h)
+                self._layer_one_launch_per_projection(i, layer)
             if tap is not None:
                 tap(i, self.h)
         head = m.model.embed_tokens if args.tie_word_embeddings else m.lm_head
@@ -719,6 +656,33 @@ class TreeVerifier:
             _lib.check(L.eagle_kv_compact_f16(_ptr(self.cache_ptrs), self.cache_ptrs.numel(),
                                               _ptr(self.result), _ptr(self.len_dev), G, hd,
                                               c0.capacity, st), "kv_compact")
+
+    def _layer_one_launch_per_projection(self, i, layer):
+        """fuse=False: the kernels and launch shapes of the module path (one launch per
+        projection), on the static buffers."""
+        m, args, T = self.model, self.args, self.T
+        H, G, hd = args.num_attention_heads, args.num_key_value_heads, args.head_dim
+        layers = m.model.layers
+        at, mlp, c = layer.self_attn, layer.mlp, self.cache[i]
+        for lin, out in ((at.q_proj, self.q), (at.k_proj, self.k), (at.v_proj, self.v)):
+            ops.quantized_matmul(self.hn, lin.weight, lin.scales, lin.biases, bias=lin.bias, out=out)
+        ops.rope_kv_append(self.q, self.k, self.v, self.positions, at._inv_freqs, at._scaling_factor,
+                           self.q_rot, c.keys[0], c.values[0], self.len_dev, H, G, hd)
+        ops.tree_attention(self.q_rot, c.keys[0], c.values[0], self.mask_bits, self.len_dev, at.scale,
+                           max_len=self.max_len, out=self.attn)
+        ops.quantized_matmul(self.attn, at.o_proj.weight, at.o_proj.scales, at.o_proj.biases,
+                             bias=at.o_proj.bias, out=self.o)
+        ops.rms_norm(self.o, layer.post_attention_layernorm.weight, args.rms_norm_eps, residual=self.h,
+                     out=self.hn, h_out=self.h)
+        ops.quantized_matmul(self.hn, mlp.gate_proj.weight, mlp.gate_proj.scales, mlp.gate_proj.biases,
+                             bias=mlp.gate_proj.bias, out=self.gate)
+        ops.quantized_matmul(self.hn, mlp.up_proj.weight, mlp.up_proj.scales, mlp.up_proj.biases,
+                             bias=mlp.up_proj.bias, out=self.up)
+        ops.silu_mul(self.gate, self.up, out=self.act)
+        nxt = layers[i + 1].input_layernorm.weight if i + 1 < len(layers) else m.model.norm.weight
+        ops.quantized_matmul(self.act, mlp.down_proj.weight, mlp.down_proj.scales, mlp.down_proj.biases,
+                             bias=mlp.down_proj.bias, out=self.down)
+        ops.rms_norm(self.down, nxt, args.rms_norm_eps, residual=self.h, out=self.hn, h_out=self.h)
 
     def capture(self):
         """Record forward() into a HIP graph (after one eager warm-up on a side stream)."""

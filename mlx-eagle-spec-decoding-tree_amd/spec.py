@@ -13,6 +13,7 @@ depend on the rows after it), and the expansion masks travel as two 32-bit words
 import torch
 
 from . import _lib, ops
+from .layer import emit_layer
 from .eagle import (MAXT, TreeVerifier, _level_buffers, _ptr, _stream, draft_tree_init, draft_tree_level,
                     fuse_projections, process_draft_tree_device, slab_partial_buffer)
 from .eagle import slab_plan as eagle_slab_plan
@@ -67,50 +68,12 @@ class DecoderPass:
         ops.rms_norm(self.h, layers[0].input_layernorm.weight, args.rms_norm_eps, out=self.hn)
         at0 = layers[0].self_attn
         ops.rope_table(positions, at0._inv_freqs, at0._scaling_factor, out=self.rope_cs)
-        for i, layer in enumerate(layers):
-            at, mlp, c = layer.self_attn, layer.mlp, self.cache[i]
-            w, sc, bi, b = self.qkv_w[i]
-            if self.slab["qkv"]:
-                s = self.slab["qkv"]
-                ops.quantized_matmul_slabs(self.hn, w, sc, bi, s, partial=self.partial)
-                ops.rope_kv_append_slabs(self.partial, ops.slab_count(args.hidden_size, s), b, self.rope_cs,
-                                         self.q_rot, c.keys[0], c.values[0], write_len, self.T, H, G, hd)
-            else:
-                ops.quantized_matmul(self.hn, w, sc, bi, bias=b, out=self.qkv)
-                ops.rope_kv_append(self.qkv, self.qkv[:, H * hd:], self.qkv[:, (H + G) * hd:], positions,
-                                   at._inv_freqs, at._scaling_factor, self.q_rot, c.keys[0], c.values[0],
-                                   write_len, H, G, hd, row_stride=W, rope_cs=self.rope_cs)
+        def attend(at, c):
             ops.draft_attention(self.q_rot, c.keys[0], c.values[0], mask_words, attn_len, Tk, at.scale,
                                 max_len=self.max_len, out=self.attn)
-            if self.slab["o"]:
-                s = self.slab["o"]
-                ops.quantized_matmul_slabs(self.attn, at.o_proj.weight, at.o_proj.scales, at.o_proj.biases,
-                                           s, partial=self.partial)
-                ops.rms_norm_slabs(self.partial, ops.slab_count(H * hd, s),
-                                   layer.post_attention_layernorm.weight, args.rms_norm_eps, self.T,
-                                   residual=self.h, out=self.hn, h_out=self.h)
-            else:
-                ops.quantized_matmul(self.attn, at.o_proj.weight, at.o_proj.scales, at.o_proj.biases,
-                                     bias=at.o_proj.bias, out=self.o)
-                ops.rms_norm(self.o, layer.post_attention_layernorm.weight, args.rms_norm_eps,
-                             residual=self.h, out=self.hn, h_out=self.h)
-            w, sc, bi, b = self.gu_w[i]
-            if self.swiglu:
-                ops.quantized_matmul_swiglu(self.hn, w, sc, bi, bias=b, out=self.act)
-            else:
-                ops.quantized_matmul(self.hn, w, sc, bi, bias=b, out=self.gate_up)
-                ops.silu_mul(self.gate_up, None, out=self.act)
-            nxt = layers[i + 1].input_layernorm.weight if i + 1 < len(layers) else m.model.norm.weight
-            if self.slab["down"]:
-                s = self.slab["down"]
-                ops.quantized_matmul_slabs(self.act, mlp.down_proj.weight, mlp.down_proj.scales,
-                                           mlp.down_proj.biases, s, partial=self.partial)
-                ops.rms_norm_slabs(self.partial, ops.slab_count(args.intermediate_size, s), nxt,
-                                   args.rms_norm_eps, self.T, residual=self.h, out=self.hn, h_out=self.h)
-            else:
-                ops.quantized_matmul(self.act, mlp.down_proj.weight, mlp.down_proj.scales,
-                                     mlp.down_proj.biases, bias=mlp.down_proj.bias, out=self.down)
-                ops.rms_norm(self.down, nxt, args.rms_norm_eps, residual=self.h, out=self.hn, h_out=self.h)
+
+        for i in range(len(layers)):
+            emit_layer(self, i, write_len, attend, positions=positions)
         if not head:
             return None
         head = m.model.embed_tokens if args.tie_word_embeddings else m.lm_head
@@ -138,6 +101,9 @@ class ChunkPass:
         H, G, hd = args.num_attention_heads, args.num_key_value_heads, args.head_dim
         self.max_len = max_len or cache[0].capacity
         self.qkv_w, self.gu_w = fuse_projections(model, False)
+        self.T = R
+        self.swiglu = False                                   # above 32 rows: the tiled GEMM form everywhere
+        self.slab = {"qkv": 0, "o": 0, "down": 0}
         f16 = dict(dtype=torch.float16, device=dev)
         i32 = dict(dtype=torch.int32, device=dev)
         self.tokens = torch.zeros(R, **i32)
@@ -182,28 +148,14 @@ class ChunkPass:
         emb = m.model.embed_tokens
         ops.embed(self.tokens, emb.weight, emb.scales, emb.biases, out=self.h)
         ops.rms_norm(self.h, layers[0].input_layernorm.weight, args.rms_norm_eps, out=self.hn)
-        for i, layer in enumerate(layers):
-            at, mlp, c = layer.self_attn, layer.mlp, self.cache[i]
-            w, sc, bi, b = self.qkv_w[i]
-            ops.quantized_matmul(self.hn, w, sc, bi, bias=b, out=self.qkv)
-            # all rows at once: rotate and append, then attention with one 32-row piece per
-            # workgroup column
-            ops.rope_kv_append(self.qkv, self.qkv[:, H * hd:], self.qkv[:, (H + G) * hd:], None,
-                               at._inv_freqs, at._scaling_factor, self.q_rot, c.keys[0], c.values[0],
-                               self.len_dev, H, G, hd, row_stride=W, rope_cs=self.rope_cs)
+        # all rows at once through the linear layers, the rotation and the cache append; then
+        # attention with one 32-row piece per workgroup column
+        def attend(at, c):
             ops.causal_attention(self.q_rot, c.keys[0], c.values[0], self.piece_len, at.scale,
                                  max_len=self.max_len, out=self.attn)
-            ops.quantized_matmul(self.attn, at.o_proj.weight, at.o_proj.scales, at.o_proj.biases,
-                                 bias=at.o_proj.bias, out=self.o)
-            ops.rms_norm(self.o, layer.post_attention_layernorm.weight, args.rms_norm_eps,
-                         residual=self.h, out=self.hn, h_out=self.h)
-            w, sc, bi, b = self.gu_w[i]
-            ops.quantized_matmul(self.hn, w, sc, bi, bias=b, out=self.gate_up)
-            ops.silu_mul(self.gate_up, None, out=self.act)
-            ops.quantized_matmul(self.act, mlp.down_proj.weight, mlp.down_proj.scales,
-                                 mlp.down_proj.biases, bias=mlp.down_proj.bias, out=self.down)
-            nxt = layers[i + 1].input_layernorm.weight if i + 1 < len(layers) else m.model.norm.weight
-            ops.rms_norm(self.down, nxt, args.rms_norm_eps, residual=self.h, out=self.hn, h_out=self.h)
+
+        for i in range(len(layers)):
+            emit_layer(self, i, self.len_dev, attend)
         if self.head:
             hw = m.model.embed_tokens if args.tie_word_embeddings else m.lm_head
             ops.quantized_matmul(self.hn[self.R - P:], hw.weight, hw.scales, hw.biases, out=self.logits)
