@@ -3,6 +3,12 @@ import numpy as np
 import torch
 
 TOL = 2e-2   # max |err| <= TOL * RMS(reference output): the bound stated for fp16 QMM / RoPE / attention
+# Outputs of a whole multi-layer pass (cache rows of the second layer, logits): every operator
+# meets TOL on its own output, but the inputs of the later operators already differ by the
+# earlier ones' rounding, so the errors of the 7 matmuls per layer add up.  Measured on the
+# two-layer test models: up to 0.024; at 7B width 0.005 after one layer and 0.034 after 28
+# (tests/test_gpu_fullsize.py follows the growth).
+MODEL_TOL = 2 * TOL
 
 
 def to_dev(a, dev):
