@@ -180,6 +180,12 @@ def main():
     ap.add_argument("--small-m", action="store_true",
                     help="one-row products of the 7B projection shapes: the vector-ALU kernel beside the "
                          "matrix kernel (one JSON line; the A/B behind the dispatch rule for M = 1)")
+    ap.add_argument("--attention", action="store_true",
+                    help="tree-position rope + tree-masked attention alone (28 / 4 heads of 128, 32 tree tokens) "
+                         "over 1024- and 2048-token prefixes, one JSON line")
+    ap.add_argument("--cpu-qmm", action="store_true",
+                    help="time the CPU restatement of single quantised matmuls on the host cores (cfg1 and the "
+                         "7B projection shapes; one JSON line); no GPU work")
     ap.add_argument("--self-draft", action="store_true",
                     help="with --loop: the target drafts for itself (high acceptance; exercises the "
                          "accept path at full size)")
@@ -199,6 +205,12 @@ def main():
         return
     if opt.small_m:
         print(json.dumps(small_m_bench(opt)), flush=True)
+        return
+    if opt.cpu_qmm:
+        print(json.dumps(cpu_qmm_bench(opt)), flush=True)
+        return
+    if opt.attention:
+        print(json.dumps(attention_bench(opt)), flush=True)
         return
 
     import torch
@@ -470,6 +482,99 @@ def gemm_bench(opt):
         "shapes": rows,
     }
     return line
+
+
+def attention_bench(opt):
+    """Tree-position RoPE with the cache append, then tree-masked GQA attention, as the step
+    launches them per layer: 32 tree tokens (seeded random tree, depth <= 4), 28 query / 4 KV
+    heads of 128, fp16 KV prefix of P tokens.  28 caches in rotation (one per layer of the 7B
+    shape), graph-timed; bytes = the K and V rows read (2 * 4 * (P + 32) * 128 * 2)."""
+    import torch
+    from mlx_eagle_spec_decoding_tree_amd import _lib, ops, synth
+
+    dev = torch.device("cuda:0")
+    _lib.check(_lib.lib().eagle_check_device(), "device check")
+    H, G, hd, T, layers = 28, 4, 128, 32, 28
+    rng = np.random.default_rng(opt.seed)
+    parents = synth.random_tree(rng, T)
+    depth, anc, bits = synth.tree_arrays(parents)
+    bits_d = torch.from_numpy(bits.view(np.int32)).to(dev)
+    inv = ops.default_inv_freqs(hd, 1e6, dev)
+    rows = []
+    for P in (1024, 2048):
+        cap = P + 64
+        K = [torch.randn(G, cap, hd, device=dev).half() for _ in range(layers)]
+        V = [torch.randn(G, cap, hd, device=dev).half() for _ in range(layers)]
+        qkv = torch.randn(T, (H + 2 * G) * hd, device=dev).half()
+        pos = (torch.from_numpy(depth.astype(np.int32)).to(dev) + P).contiguous()
+        len_dev = torch.tensor([P], dtype=torch.int32, device=dev)
+        cs = ops.rope_table(pos, inv, 1.0)
+        q_rot = torch.empty(H, T, hd, device=dev, dtype=torch.float16)
+        out = torch.empty(T, H * hd, device=dev, dtype=torch.float16)
+        ops.workspace("attn", _lib.lib().eagle_tree_attention_workspace_bytes(H, hd, cap), dev)
+
+        def rope():
+            for i in range(layers):
+                ops.rope_kv_append(qkv, qkv[:, H * hd:], qkv[:, (H + G) * hd:], pos, inv, 1.0, q_rot, K[i], V[i],
+                                   len_dev, H, G, hd, row_stride=(H + 2 * G) * hd, rope_cs=cs)
+
+        def attn():
+            for i in range(layers):
+                ops.tree_attention(q_rot, K[i], V[i], bits_d, len_dev, hd ** -0.5, max_len=cap, out=out)
+
+        def both():
+            for i in range(layers):
+                ops.rope_kv_append(qkv, qkv[:, H * hd:], qkv[:, (H + G) * hd:], pos, inv, 1.0, q_rot, K[i], V[i],
+                                   len_dev, H, G, hd, row_stride=(H + 2 * G) * hd, rope_cs=cs)
+                ops.tree_attention(q_rot, K[i], V[i], bits_d, len_dev, hd ** -0.5, max_len=cap, out=out)
+
+        t = {n: float(np.median(graph_time_ms(torch, f, reps=7)[0])) * 1e3 / layers
+             for n, f in (("rope_append_us", rope), ("attention_us", attn), ("both_us", both))}
+        kv = 2 * G * (P + T) * hd * 2
+        rows.append({"prefix": P, **{k: round(v, 2) for k, v in t.items()}, "kv_bytes": kv,
+                     "attention_frac_of_hbm_peak": round(kv / t["attention_us"] / 1e3 / HBM_PEAK_GBS, 4)})
+    return {"metric": "tree-position rope + tree-masked attention, us per layer", "unit": "us", "dtype": "f16",
+            "data": "synthetic", "config": {"workload": "32 tree tokens, 28 q / 4 kv heads, head_dim 128, theta 1e6"},
+            "rows": rows}
+
+
+def cpu_qmm_bench(opt):
+    """The CPU restatement of one quantised matmul (oracle/eagle_oracle.c, OpenMP) on the host
+    cores: median of the timed calls after the warm-up calls (10 + 20 for the small shapes, as the
+    reference's own timing loop drops 10 of 30, utils.py:59-72; 3 + 7 for the 300 MB vocabulary
+    projection), with all threads and with one."""
+    from mlx_eagle_spec_decoding_tree_amd import synth
+    from oracle import oracle
+    oracle.build()
+    have = os.cpu_count() or 1
+    cores = int(os.environ.get("OMP_NUM_THREADS", 0)) or min(16, have)
+    shapes = [("cfg1", 8192, 2048), ("q/o", 3584, 3584), ("k/v", 512, 3584), ("gate/up", 18944, 3584),
+              ("down", 3584, 18944), ("lm_head", 152064, 3584)]
+    rng = np.random.default_rng(42)
+    rows = []
+    for name, N, K in shapes:
+        layer = synth.make_qlinear(rng, N, K)
+        big = N * K > 2e8
+        for M in (1, 8, 16, 24, 32):
+            x = synth.make_x(rng, M, K)
+            rec = {"name": name, "N": N, "K": K, "M": M}
+            for label, threads in (("all_threads_us", cores), ("one_thread_us", 1)):
+                if label == "one_thread_us" and (big or M not in (8, 32)):
+                    continue
+                set_omp_threads(threads)
+                warm, timed = (3, 7) if big else ((10, 20) if threads > 1 else (3, 7))
+                ts = []
+                for it in range(warm + timed):
+                    t0 = time.perf_counter()
+                    oracle.qmm(x, layer["weight"], layer["scales"], layer["biases"])
+                    if it >= warm:
+                        ts.append((time.perf_counter() - t0) * 1e6)
+                rec[label] = round(float(np.median(ts)), 1)
+            rows.append(rec)
+            print(f"[cpu-qmm] {rec}", file=sys.stderr, flush=True)
+    set_omp_threads(cores)
+    return {"metric": "CPU restatement of one quantised matmul, us per call (median)", "unit": "us",
+            "cores": cores, "cores_available": have, "cpu_model": cpu_model(), "kind": "port", "rows": rows}
 
 
 def small_m_bench(opt):
