@@ -166,6 +166,9 @@ def main():
                          "'' = streaming kernel everywhere; default: the library's choice)")
     ap.add_argument("--draft-slabs", default=None,
                     help="--loop: the same for the drafter's passes")
+    ap.add_argument("--no-draft-folded", action="store_true",
+                    help="--loop: the drafter's passes with one launch per operator instead of the small-row "
+                         "products with norm / residual / SwiGLU folded in")
     ap.add_argument("--chain", action="store_true",
                     help="residual add + norm + gate|up + SwiGLU as one launch of a resident grid with a "
                          "grid-wide barrier inside (off by default: slower than the two launches it replaces)")
@@ -655,7 +658,8 @@ def loop_bench(opt):
              for s in (opt.slabs, opt.draft_slabs)]
     dec = spec.SpeculativeDecoder(target, draft, capacity=capacity, k=k, depth=depth,
                                   verify_num_tokens=nodes, max_out=(opt.warmup + steps) * (depth + 2) + 8,
-                                  slab_plan=plans[0], draft_slab_plan=plans[1])
+                                  slab_plan=plans[0], draft_slab_plan=plans[1],
+                                  draft_folded=False if opt.no_draft_folded else None)
     dec.prepare(prompt_len)
     torch.cuda.synchronize()
     t0 = time.time()

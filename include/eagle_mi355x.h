@@ -97,6 +97,28 @@ int eagle_norm_mlp_in_f16(const float* partial, int slabs, void* h, const void* 
                           void* scratch, size_t scratch_bytes, int* err_dev,
                           long long spin_limit_ticks, eagle_stream_t stream);
 
+/* The product for a pass of at most 16 rows through a small model (the drafter's passes of the
+ * tree loop), with the operators around it folded in, so that a decoder layer needs four of
+ * these launches and no norm / add launch (mlx_llama.py:195-196, 214-215, 225-249):
+ *   norm_w != NULL: the rows of x are RMS-normalised with norm_w [K] (and eps) before the
+ *     product, as eagle_rmsnorm_f16 would (the input / post-attention norm of the layer);
+ *   residual != NULL: out = residual + fp16(x . W^T) (the o and down projections; residual may be
+ *     `out` itself: h is updated in place);
+ *   swiglu != 0: W holds gate and up interleaved in 16-row tiles as for
+ *     eagle_qmm_swiglu_w4g64_f16, N = 2 I rows, out [T, I] = silu(g) * u.
+ * Otherwise as eagle_qmm_w4g64_f16 (bias [N] or NULL added in fp16 after rounding).  Replaces the
+ * launches of eagle_qmm_w4g64_f16 / eagle_qmm_slab_partial_w4g64 and eagle_rmsnorm_f16 /
+ * eagle_rmsnorm_slabs_f16 of such a pass.
+ * Constraints (eagle_qmm_small_supported): T <= 16; K a multiple of 128, up to 5120 (the waves of
+ * a workgroup hold all of x between them); N a multiple of 16 (32 with SwiGLU); every scale
+ * below 0.2499 in magnitude (the nibbles are expanded through fp16 subnormals times
+ * scale * 2^18); x must not alias out; x, norm_w, wq, residual, out 16-byte aligned. */
+int eagle_qmm_small_supported(int T, int N, int K, int norm, int swiglu);
+int eagle_qmm_small_w4g64_f16(const void* x, const void* norm_w, float eps, const uint32_t* wq,
+                              const void* scales, const void* biases, const void* bias,
+                              const void* residual, void* out, int T, int N, int K,
+                              int group_size, int bits, int swiglu, eagle_stream_t stream);
+
 /* The product for ONE row of x on the vector ALU (v_dot2_f32_f16 on magic-number fp16 nibbles,
  * sum over the sixteen lanes of a row with DPP), no matrix instructions: the M = 1 case of
  * mx.quantized_matmul (mlx_model_fwd_bench.py:65-73), factorised as in kernels/qmv/1b.metal:121-147.

@@ -256,6 +256,46 @@ def norm_mlp_in(partial, slabs, h, norm_weight, eps, gu_w, gu_scales, gu_biases,
     return act
 
 
+SMALL_SCALE_LIMIT = 0.2499       # |scale| * 2^18 has to stay a finite fp16
+
+
+def small_supported(T, N, K, norm=False, swiglu=False):
+    """True when `quantized_matmul_small` takes this shape."""
+    return bool(_lib.lib().eagle_qmm_small_supported(T, N, K, int(bool(norm)), int(bool(swiglu))))
+
+
+def quantized_matmul_small(x, w_q, scales, biases, bias=None, out=None, norm_weight=None, eps=1e-6,
+                           residual=None, swiglu=False):
+    """The product for at most 16 rows with its neighbours folded in (mlx_llama.py:195-196,
+    214-215, 225-249): RMSNorm of x before it (norm_weight), the residual added to it (residual;
+    may be `out`), or SwiGLU over gate|up interleaved by `interleave_gate_up` (swiglu).  Every
+    scale must be below SMALL_SCALE_LIMIT in magnitude; the caller checks that once per matrix."""
+    _need_cuda(x, w_q, scales, biases, bias, norm_weight, residual)
+    x = _f16(x, "x")
+    w_q = as_packed_u32(w_q)
+    scales, biases = _f16(scales, "scales"), _f16(biases, "biases")
+    *lead, K = x.shape
+    T = reduce(lambda a, b: a * b, lead, 1)
+    N = w_q.shape[0]
+    if w_q.shape[1] * 8 != K or tuple(scales.shape) != (N, K // 64) or tuple(biases.shape) != (N, K // 64):
+        raise ValueError(f"shape mismatch: x {tuple(x.shape)}, w {tuple(w_q.shape)}, "
+                         f"scales {tuple(scales.shape)}, biases {tuple(biases.shape)}")
+    n_out = N // 2 if swiglu else N
+    if bias is not None and tuple(_f16(bias, "bias").shape) != (N,):
+        raise ValueError("bias must have shape [N]")
+    if norm_weight is not None and tuple(_f16(norm_weight, "norm_weight").shape) != (K,):
+        raise ValueError("norm_weight must have shape [K]")
+    if out is None:
+        out = torch.empty((*lead, n_out), dtype=torch.float16, device=x.device)
+    if residual is not None and (tuple(residual.shape) != tuple(out.shape) or not residual.is_contiguous()):
+        raise ValueError("residual must be contiguous with the shape of the result")
+    rc = _lib.lib().eagle_qmm_small_w4g64_f16(
+        _ptr(x), _ptr(norm_weight), float(eps), _ptr(w_q), _ptr(scales), _ptr(biases), _ptr(bias),
+        _ptr(residual), _ptr(out), T, N, K, 64, 4, int(bool(swiglu)), _stream())
+    _lib.check(rc, "quantized_matmul_small")
+    return out
+
+
 def qmv_preferred(N, K):
     """True where the vector-ALU kernel is the faster form for one row of x: measured on the
     projection shapes of the 7B model (M = 1: 5.7 against 8.5 us for 3584 x 3584, 12.5 against

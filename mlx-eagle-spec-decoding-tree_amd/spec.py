@@ -26,7 +26,10 @@ class DecoderPass:
     The rows are written to the cache at *write_len; query t sees the *attn_len rows before
     them and, of the Tk rows from there on, those its two mask words select."""
 
-    def __init__(self, model, cache, T, max_len=None, swiglu=True, slab_plan=None):
+    def __init__(self, model, cache, T, max_len=None, swiglu=True, slab_plan=None, folded=None):
+        """folded: the small-row form of the products with norm, residual add and SwiGLU folded in
+        (`ops.quantized_matmul_small`: four launches per layer besides rope and attention);
+        None = wherever the library takes the shapes and the weights."""
         args = model.args
         self.model, self.cache, self.args, self.T = model, cache, args, T
         dev = model.device
@@ -49,6 +52,13 @@ class DecoderPass:
         self.act = torch.empty((T, I), **f16)
         self.down = torch.empty((T, D), **f16)
         self.logits = torch.empty((T, args.vocab_size), **f16)
+        W = (H + 2 * G) * hd
+        can_fold = self.swiglu and ops.small_supported(T, W, D, norm=True) \
+            and ops.small_supported(T, D, H * hd) and ops.small_supported(T, 2 * I, D, norm=True, swiglu=True) \
+            and ops.small_supported(T, D, I) and self._scales_within(ops.SMALL_SCALE_LIMIT)
+        if folded and not can_fold:
+            raise ValueError("the small-row form does not take these shapes or weights")
+        self.folded = can_fold if folded is None else bool(folded)
         L = _lib.lib()
         head = model.lm_head if not args.tie_word_embeddings else model.model.embed_tokens
         need = max(L.eagle_qmm_workspace_bytes(T, n, k) for n, k in
@@ -56,6 +66,14 @@ class DecoderPass:
         ops.workspace("qmm", need, dev)
         ops.workspace("attn", L.eagle_tree_attention_workspace_bytes(H, hd, self.max_len), dev)
         ops.workspace("topk", L.eagle_logsoftmax_topk_workspace_bytes(T, args.vocab_size), dev)
+
+    def _scales_within(self, limit):
+        """Every quantisation scale of the layers' matrices is below `limit` in magnitude."""
+        worst = 0.0
+        for i, layer in enumerate(self.model.model.layers):
+            for sc in (self.qkv_w[i][1], layer.self_attn.o_proj.scales, self.gu_w[i][1], layer.mlp.down_proj.scales):
+                worst = max(worst, float(sc.abs().max()))
+        return worst < limit
 
     def forward(self, tokens, positions, write_len, attn_len, mask_words, Tk, head=True):
         """head=False: stop after the last layer (a pass that is only run for its KV rows)."""
@@ -65,15 +83,40 @@ class DecoderPass:
         emb = m.model.embed_tokens
         ops.embed(tokens, emb.weight, emb.scales, emb.biases, out=self.h)
         layers = m.model.layers
-        ops.rms_norm(self.h, layers[0].input_layernorm.weight, args.rms_norm_eps, out=self.hn)
         at0 = layers[0].self_attn
         ops.rope_table(positions, at0._inv_freqs, at0._scaling_factor, out=self.rope_cs)
         def attend(at, c):
             ops.draft_attention(self.q_rot, c.keys[0], c.values[0], mask_words, attn_len, Tk, at.scale,
                                 max_len=self.max_len, out=self.attn)
 
-        for i in range(len(layers)):
-            emit_layer(self, i, write_len, attend, positions=positions)
+        if self.folded:
+            # per layer: q|k|v with the input norm folded in, rope + cache append, attention, o with
+            # the residual, gate|up with the post-attention norm and SwiGLU, down with the residual
+            q_lin, k_lin, v_lin = self.qkv, self.qkv[:, H * hd:], self.qkv[:, (H + G) * hd:]
+            eps = args.rms_norm_eps
+            for i, layer in enumerate(layers):
+                at, mlp, c = layer.self_attn, layer.mlp, self.cache[i]
+                w, sc, bi, b = self.qkv_w[i]
+                ops.quantized_matmul_small(self.h, w, sc, bi, bias=b, out=self.qkv,
+                                           norm_weight=layer.input_layernorm.weight, eps=eps)
+                ops.rope_kv_append(q_lin, k_lin, v_lin, positions, at._inv_freqs, at._scaling_factor,
+                                   self.q_rot, c.keys[0], c.values[0], write_len, H, G, hd, row_stride=W,
+                                   rope_cs=self.rope_cs)
+                attend(at, c)
+                o = at.o_proj
+                ops.quantized_matmul_small(self.attn, o.weight, o.scales, o.biases, bias=o.bias, out=self.h,
+                                           residual=self.h)
+                w, sc, bi, b = self.gu_w[i]
+                ops.quantized_matmul_small(self.h, w, sc, bi, bias=b, out=self.act,
+                                           norm_weight=layer.post_attention_layernorm.weight, eps=eps, swiglu=True)
+                d = mlp.down_proj
+                ops.quantized_matmul_small(self.act, d.weight, d.scales, d.biases, bias=d.bias, out=self.h,
+                                           residual=self.h)
+            ops.rms_norm(self.h, m.model.norm.weight, eps, out=self.hn)
+        else:
+            ops.rms_norm(self.h, layers[0].input_layernorm.weight, args.rms_norm_eps, out=self.hn)
+            for i in range(len(layers)):
+                emit_layer(self, i, write_len, attend, positions=positions)
         if not head:
             return None
         head = m.model.embed_tokens if args.tie_word_embeddings else m.lm_head
@@ -254,7 +297,7 @@ class SpeculativeDecoder:
     """
 
     def __init__(self, base_model, draft_model, capacity, k=8, depth=3, verify_num_tokens=31,
-                 max_out=8192, slab_plan=None, draft_slab_plan=None):
+                 max_out=8192, slab_plan=None, draft_slab_plan=None, draft_folded=None):
         from .cache import make_prompt_cache
 
         if k != Y_LEN:
@@ -272,7 +315,8 @@ class SpeculativeDecoder:
         self.draft_cache = make_prompt_cache(draft_model, capacity=capacity)
         self.verifier = TreeVerifier(base_model, self.base_cache, total_tokens=verify_num_tokens,
                                      max_len=capacity, slab_plan=slab_plan)
-        self.draft = DecoderPass(draft_model, self.draft_cache, k, max_len=capacity, slab_plan=draft_slab_plan)
+        self.draft = DecoderPass(draft_model, self.draft_cache, k, max_len=capacity, slab_plan=draft_slab_plan,
+                                 folded=draft_folded)
         i32 = dict(dtype=torch.int32, device=dev)
         self.y = torch.zeros(Y_LEN, **i32)
         self.root_token = torch.zeros(1, **i32)
