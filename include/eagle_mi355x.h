@@ -109,7 +109,7 @@ int eagle_norm_mlp_in_f16(const float* partial, int slabs, void* h, const void* 
  * Otherwise as eagle_qmm_w4g64_f16 (bias [N] or NULL added in fp16 after rounding).  Replaces the
  * launches of eagle_qmm_w4g64_f16 / eagle_qmm_slab_partial_w4g64 and eagle_rmsnorm_f16 /
  * eagle_rmsnorm_slabs_f16 of such a pass.
- * Constraints (eagle_qmm_small_supported): T <= 16; K a multiple of 128, up to 5120 (the waves of
+ * Constraints (eagle_qmm_small_supported): T <= 16; K a multiple of 128, up to 6144 (the waves of
  * a workgroup hold all of x between them); N a multiple of 16 (32 with SwiGLU); every scale
  * below 0.2499 in magnitude (the nibbles are expanded through fp16 subnormals times
  * scale * 2^18); x must not alias out; x, norm_w, wq, residual, out 16-byte aligned. */
@@ -118,6 +118,23 @@ int eagle_qmm_small_w4g64_f16(const void* x, const void* norm_w, float eps, cons
                               const void* scales, const void* biases, const void* bias,
                               const void* residual, void* out, int T, int N, int K,
                               int group_size, int bits, int swiglu, eagle_stream_t stream);
+
+/* q|k|v of a small pass with everything around it in one launch: RMSNorm of x (norm_w, or NULL for
+ * none), the product with the fused q|k|v matrix [(H + 2 G) hd, D] (+ bias), the rotation of q and
+ * k with the per-token (cos, sin) table of eagle_rope_table_f32, and the append of the new K / V
+ * rows to the caches at row *cache_len_dev (mlx_llama.py:136-183, 231-233).  Replaces
+ * eagle_rmsnorm_f16 + eagle_qmm_w4g64_f16 + eagle_rope_kv_append_table_f16 of such a pass (same
+ * formula and roundings as the last of them).
+ *   x [T, D] fp16; rope_cs [T, hd / 2, 2] fp32; q_out [H, T, hd] fp16; k_cache, v_cache
+ *   [G, capacity, hd] fp16 (rows *cache_len_dev + t are written; rows at or past capacity are not).
+ * Constraints (eagle_qkv_rope_small_supported): T <= 16, D a multiple of 128 up to 6144, hd a
+ * multiple of 32, scales below 0.2499 in magnitude. */
+int eagle_qkv_rope_small_supported(int T, int D, int H, int G, int hd);
+int eagle_qkv_rope_small_w4g64_f16(const void* x, const void* norm_w, float eps, const uint32_t* wq,
+                                   const void* scales, const void* biases, const void* bias,
+                                   const float* rope_cs, void* q_out, void* k_cache, void* v_cache,
+                                   const int32_t* cache_len_dev, int T, int D, int H, int G, int hd,
+                                   long capacity, int group_size, int bits, eagle_stream_t stream);
 
 /* The product for ONE row of x on the vector ALU (v_dot2_f32_f16 on magic-number fp16 nibbles,
  * sum over the sixteen lanes of a row with DPP), no matrix instructions: the M = 1 case of

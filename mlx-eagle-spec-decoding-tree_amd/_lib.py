@@ -29,6 +29,9 @@ SIGNATURES = {
                               + [c_int] * 3 + [c_void_p, c_size_t, c_void_p, c_longlong, c_void_p]),
     "eagle_qmm_small_supported": (c_int, [c_int] * 5),
     "eagle_qmm_small_w4g64_f16": (c_int, [c_void_p, c_void_p, c_float] + [c_void_p] * 6 + [c_int] * 6 + [c_void_p]),
+    "eagle_qkv_rope_small_supported": (c_int, [c_int] * 5),
+    "eagle_qkv_rope_small_w4g64_f16": (c_int, [c_void_p, c_void_p, c_float] + [c_void_p] * 9 + [c_int] * 5
+                                       + [c_long, c_int, c_int, c_void_p]),
     "eagle_qmv_supported": (c_int, [c_int] * 2),
     "eagle_qmv_w4g64_f16": (c_int, [c_void_p] * 6 + [c_int] * 4 + [c_void_p]),
     "eagle_qmm_plan": (c_int, [c_int, c_int, c_int, c_void_p]),

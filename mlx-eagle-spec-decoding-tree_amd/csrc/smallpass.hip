@@ -6,23 +6,33 @@
 //   out = (RMSNorm(x, norm_w) or x) . W^T  (+ bias)              q|k|v
 //   out = residual + fp16(x . W^T)                               o and down projections, in place on h
 //   out = silu(g) * u,  (g | u) = (RMSNorm(x) or x) . Wgu^T      gate|up, interleaved 16-row tiles
+//   q [H,T,hd], cache rows = rope(RMSNorm(x) . Wqkv^T + bias)    q|k|v with rotation and cache append
 //
 // (mlx_llama.py:195-196, 214-215, 225-249).
 //
-//   * A workgroup owns one 16-row weight tile (a (gate, up) pair for SwiGLU); its four or eight
-//     waves deal the 128-column chunks of K among themselves (one to five each) and add their
-//     tiles in LDS.  Every request of a wave (weights, scales, its columns of x as the B operand
-//     of v_mfma_f32_16x16x32_f16) is in flight together; there is no loop over K, and the chain
-//     of dependent instructions per wave is a few hundred long.  (One wave per tile over the whole
-//     K was measured first: 2500 dependent instructions on one wave per SIMD, 15 us per launch.)
+//   * A workgroup owns one 16-row weight tile (a (gate, up) pair for SwiGLU, the two halves of a
+//     head that a rotation pairs for rope); its four, eight or sixteen waves deal the 128-column
+//     chunks of K among themselves (at most three each) and add their tiles in LDS.  Every request
+//     of a wave (weights, scales, its columns of x as the B operand of v_mfma_f32_16x16x32_f16) is
+//     in flight together; there is no loop over K.
 //   * The norm is folded into the load of x: each wave sums the squares of its columns, the row
 //     sums are added across the waves in LDS; no launch and no pass over memory for it.
 //   * Expansion of the nibbles through fp16 subnormals as in csrc/resident.hip: fp16(s q + b),
 //     single rounding; scales below 0.2499.
 //
-// A form of this file that ran a whole layer as ONE resident grid with grid-wide barriers between
-// the products was measured and dropped: a barrier plus the first load behind it costs what a
-// launch costs (56 us per layer against 33 us for the launches it replaced).
+// Measured on the way (8 rows, the 0.5B drafter's shapes, launches back to back in a graph):
+//   - one wave per tile over the whole K: 2500 instructions on one wave per SIMD, 15 us per launch;
+//   - K over the waves, loads under conditions (zero for what a wave does not own): the requests
+//     of a wave wait for one another where the branches join; time grows by 1.1 us per chunk;
+//   - unconditional loads, 16 bytes per lane straight into the operand layout: the time follows
+//     the number of cache lines the load instructions of a compute unit touch (x: 64 per chunk,
+//     scales 16 per 2-byte load), 7.8 us for the down projection; shaped as below: 5.7 us;
+//   - a whole layer as ONE resident grid with grid-wide barriers between the products: a barrier
+//     plus the first load behind it costs what a launch costs (56 us per layer against 33 us for
+//     the launches it replaced);
+//   - attention of such a pass in one launch (a workgroup per query head, keys over its sixteen
+//     waves, merge through LDS): 14.7 to 30.8 us against 9.9 to 13.4 us for the split and merge
+//     launches over 64 to 2048 keys.
 #include "common.h"
 
 namespace {
@@ -61,16 +71,41 @@ struct SmallArgs {
   half_t* out;              // [T, N] ([T, N / 2] for SwiGLU)
   float eps;
   int T, N, K;
+  // rope form: (cos, sin) table [T, hd / 2, 2], rotated q [H, T, hd], caches [G, cap, hd], *len_dev = row of
+  // the first new K / V row
+  const float* rope_cs;
+  half_t* q_out;
+  half_t* k_cache;
+  half_t* v_cache;
+  const int32_t* len_dev;
+  int H, G, hd;
+  long cap;
 };
 
-// NW waves per workgroup, at most MAXC chunks of 128 columns per wave, NT tiles per workgroup
-// (2: a (gate, up) pair with the SwiGLU epilogue).  Lane (r = lane % 16, kq = lane / 16) of a
-// wave holds, per chunk, weight row r columns 32 kq .. + 32 (one 16-byte load, four packed words,
-// one per matrix instruction) and x row r at the same columns; the accumulator of lane (m, q4)
-// is weight rows 4 q4 .. + 4 of x row m.
-template <int NW, int MAXC, int NT>
+enum { SMALL_PLAIN = 0, SMALL_SWIGLU = 1, SMALL_ROPE = 2 };
+
+// NW waves per workgroup, at most SMALL_MAXC chunks of 128 columns per wave, RP passes of four x rows
+// (2: T <= 8, 4: T <= 16).  MODE: one tile per workgroup (plain / residual), a (gate, up) tile pair
+// 16 rows apart with the SwiGLU epilogue, or two tiles of one head half a head apart (the two
+// halves a rotation pairs) with the rope epilogue.  Lane (r = lane % 16, kq = lane / 16) of a wave
+// holds, per chunk, weight row r columns 32 kq .. + 32 (one 16-byte load, four packed words, one
+// per matrix instruction) and x row r at the same columns; the accumulator of lane (m, q4) is
+// weight rows 4 q4 .. + 4 of x row m.
+//
+// What bounds this kernel is the number of cache lines its load instructions touch per compute
+// unit, so every request is shaped for few lines: x is read with whole rows of a chunk per
+// instruction (four rows x 256 bytes) and brought into the operand layout through a per-wave LDS
+// buffer; the two scales (biases) of a chunk come as one 4-byte load for the three chunks of a
+// wave at once and are handed to the lanes that need them with a lane shuffle.
+constexpr int SMALL_MAXC = 3;
+constexpr int SMALL_XROW = 256 + 16;       // bytes per staged x row: 128 columns, padded against bank conflicts
+
+template <int NW, int RP, int MODE>
 __global__ __launch_bounds__(NW * 64) void qmm_small_kernel(SmallArgs a) {
+  constexpr int NT = MODE == SMALL_PLAIN ? 1 : 2;
+  constexpr int MAXC = SMALL_MAXC;
   __shared__ __attribute__((aligned(16))) float4_t red[NW][NT][64];
+  __shared__ __attribute__((aligned(16))) unsigned char xstage[NW][RP * 4 * SMALL_XROW];
   __shared__ float ssq[NW][16];
   const int wave = threadIdx.x >> 6, lane = threadIdx.x & 63;
   const int r = lane & 15, kq = lane >> 4;
@@ -80,52 +115,86 @@ __global__ __launch_bounds__(NW * 64) void qmm_small_kernel(SmallArgs a) {
   const int per = chunks / NW, rem = chunks % NW;
   const int nch = per + (wave < rem ? 1 : 0);
   const int k0 = (wave * per + (wave < rem ? wave : rem)) * 128;
-  const int row0 = blockIdx.x * (16 * NT);
+  int row0, second;                       // first row of tile 0, distance of tile 1
+  if (MODE == SMALL_ROPE) {
+    const int per_head = a.hd >> 5;
+    row0 = (blockIdx.x / per_head) * a.hd + (blockIdx.x % per_head) * 16;
+    second = a.hd >> 1;
+  } else {
+    row0 = blockIdx.x * (16 * NT);
+    second = 16;
+  }
 
   // ---- every request of the wave at once ----
+  // All loads are unconditional (a load under a condition has to be waited for where the branches
+  // join, which puts the requests of a wave one behind the other): chunks the wave does not own
+  // and rows past T read a valid address again and their values are never used.
+  const int kb = nch > 0 ? k0 : 0;
   uint4_t wv[NT][MAXC];
-  half_t sv[NT][MAXC], bv[NT][MAXC];
+  uint32_t spair[NT], bpair[NT];          // lane (r, c): the two scales (biases) of row r in chunk c
 #pragma unroll
   for (int t = 0; t < NT; ++t) {
-    const long row = row0 + 16 * t + r;
-    const uint32_t* wp = a.w + row * KW + (k0 >> 3) + kq * 4;
-    const half_t* sp = a.s + row * G + (k0 >> 6) + (kq >> 1);
-    const half_t* bp = a.b + row * G + (k0 >> 6) + (kq >> 1);
+    const long row = row0 + second * t + r;
+    const uint32_t* wp = a.w + row * KW + (kb >> 3) + kq * 4;
 #pragma unroll
-    for (int c = 0; c < MAXC; ++c) {
-      if (c < nch) {
-        wv[t][c] = *reinterpret_cast<const uint4_t*>(wp + c * 16);
-        sv[t][c] = sp[c * 2];
-        bv[t][c] = bp[c * 2];
-      }
+    for (int c = 0; c < MAXC; ++c) wv[t][c] = *reinterpret_cast<const uint4_t*>(wp + (c < nch ? c : 0) * 16);
+    const int cpair = kq < nch ? kq : 0;
+    spair[t] = *reinterpret_cast<const uint32_t*>(a.s + row * G + (kb >> 6) + cpair * 2);
+    bpair[t] = *reinterpret_cast<const uint32_t*>(a.b + row * G + (kb >> 6) + cpair * 2);
+  }
+  // x: lane l reads 16 bytes of row 4 p + l / 16 at byte 16 (l % 16) of the chunk's 256
+  uint4_t xg[MAXC][RP];
+  {
+    const int xr = lane >> 4, xc = lane & 15;
+#pragma unroll
+    for (int p = 0; p < RP; ++p) {
+      int row = 4 * p + xr;
+      row = row < a.T ? row : a.T - 1;
+      const half_t* xp = a.x + (long)row * K + kb + xc * 8;
+#pragma unroll
+      for (int c = 0; c < MAXC; ++c) xg[c][p] = *reinterpret_cast<const uint4_t*>(xp + (c < nch ? c : 0) * 128);
     }
   }
+  half8_t nw[MAXC][4];
+  if (a.norm_w) {
+    const half_t* np = a.norm_w + kb + kq * 32;
+#pragma unroll
+    for (int c = 0; c < MAXC; ++c)
+#pragma unroll
+      for (int i = 0; i < 4; ++i) nw[c][i] = *reinterpret_cast<const half8_t*>(np + (c < nch ? c : 0) * 128 + i * 8);
+  }
+  // x through the wave's LDS buffer into the operand layout, a chunk at a time (rows past 4 RP,
+  // which are rows past T, read what is there: their columns of the result are not stored)
   half8_t xb[MAXC][4];
-  const bool live = r < a.T;
-  const half_t* xp = a.x + (long)(live ? r : 0) * K + k0 + kq * 32;
+  {
+    unsigned char* xs = xstage[wave];
+    const int xr = lane >> 4, xc = lane & 15;
 #pragma unroll
-  for (int c = 0; c < MAXC; ++c)
+    for (int c = 0; c < MAXC; ++c) {
 #pragma unroll
-    for (int i = 0; i < 4; ++i)
-      xb[c][i] = (c < nch && live) ? *reinterpret_cast<const half8_t*>(xp + c * 128 + i * 8)
-                                   : half8_t{0, 0, 0, 0, 0, 0, 0, 0};
+      for (int p = 0; p < RP; ++p)
+        *reinterpret_cast<uint4_t*>(xs + (4 * p + xr) * SMALL_XROW + xc * 16) = xg[c][p];
+      __builtin_amdgcn_wave_barrier();
+      const int mr = r < 4 * RP ? r : 0;
+#pragma unroll
+      for (int i = 0; i < 4; ++i)
+        xb[c][i] = *reinterpret_cast<const half8_t*>(xs + mr * SMALL_XROW + (4 * kq + i) * 16);
+      __builtin_amdgcn_wave_barrier();
+    }
+  }
 
   // ---- RMSNorm folded into x ----
   if (a.norm_w) {
-    half8_t nw[MAXC][4];
-    const half_t* np = a.norm_w + k0 + kq * 32;
-#pragma unroll
-    for (int c = 0; c < MAXC; ++c)
-#pragma unroll
-      for (int i = 0; i < 4; ++i)
-        if (c < nch) nw[c][i] = *reinterpret_cast<const half8_t*>(np + c * 128 + i * 8);
     float ss = 0.f;
 #pragma unroll
-    for (int c = 0; c < MAXC; ++c)
+    for (int c = 0; c < MAXC; ++c) {
+      if (c < nch) {
 #pragma unroll
-      for (int i = 0; i < 4; ++i)
+        for (int i = 0; i < 4; ++i)
 #pragma unroll
-        for (int e = 0; e < 8; ++e) ss += (float)xb[c][i][e] * (float)xb[c][i][e];
+          for (int e = 0; e < 8; ++e) ss += (float)xb[c][i][e] * (float)xb[c][i][e];
+      }
+    }
     ss += __shfl_xor(ss, 16, 64);
     ss += __shfl_xor(ss, 32, 64);
     if (kq == 0) ssq[wave][r] = ss;
@@ -156,8 +225,11 @@ __global__ __launch_bounds__(NW * 64) void qmm_small_kernel(SmallArgs a) {
 #pragma unroll
     for (int c = 0; c < MAXC; ++c) {
       if (c < nch) {
-        const half_t sc = (half_t)((float)sv[t][c] * 262144.f);
-        const half_t bi = bv[t][c];
+        // the pair of chunk c sits in lane (r, c); this lane's columns are in its half kq / 2
+        const uint32_t s2 = __shfl(spair[t], r + 16 * c, 64), b2 = __shfl(bpair[t], r + 16 * c, 64);
+        const half_t sraw = __builtin_bit_cast(half_t, (unsigned short)(kq & 2 ? s2 >> 16 : s2 & 0xffffu));
+        const half_t bi = __builtin_bit_cast(half_t, (unsigned short)(kq & 2 ? b2 >> 16 : b2 & 0xffffu));
+        const half_t sc = (half_t)((float)sraw * 262144.f);
 #pragma unroll
         for (int i = 0; i < 4; ++i) {
           const half8_t av = sp_dequant(wv[t][c][i], half2_t{sc, sc}, half2_t{bi, bi});
@@ -180,7 +252,52 @@ __global__ __launch_bounds__(NW * 64) void qmm_small_kernel(SmallArgs a) {
   // ---- epilogue: lane (m, q4) holds weight rows row0 (+ 16) + 4 q4 .. + 4 of x row m ----
   const int m = r, q4 = kq;
   if (m >= a.T) return;
-  if (NT == 2) {
+  if (MODE == SMALL_ROPE) {
+    // the linear output rounded to fp16 (bias added in fp16), rotated with the table's (cos, sin)
+    // exactly as the separate rope launch does; v rows pass through
+    const int half = a.hd >> 1;
+    const int hb = row0 / a.hd;
+    const int d = row0 - hb * a.hd + 4 * q4;            // < hd / 2
+    half4_t lo, hi;
+#pragma unroll
+    for (int i = 0; i < 4; ++i) {
+      lo[i] = (half_t)acc[0][i];
+      hi[i] = (half_t)acc[NT - 1][i];
+      if (a.bias) {
+        lo[i] = lo[i] + a.bias[row0 + 4 * q4 + i];
+        hi[i] = hi[i] + a.bias[row0 + half + 4 * q4 + i];
+      }
+    }
+    const long P = *a.len_dev;
+    if (P + m >= a.cap) return;                         // the host checks capacity; never write past the buffer
+    half_t* dst;
+    if (hb < a.H) {
+      dst = a.q_out + ((long)hb * a.T + m) * a.hd;
+    } else {
+      const int g = hb < a.H + a.G ? hb - a.H : hb - a.H - a.G;
+      dst = (hb < a.H + a.G ? a.k_cache : a.v_cache) + ((long)g * a.cap + P + m) * a.hd;
+    }
+    if (hb < a.H + a.G) {
+      const float4_t* cs = reinterpret_cast<const float4_t*>(a.rope_cs + ((long)m * half + d) * 2);
+      half4_t olo, ohi;
+#pragma unroll
+      for (int j2 = 0; j2 < 2; ++j2) {
+        const float4_t v = cs[j2];
+#pragma unroll
+        for (int e = 0; e < 2; ++e) {
+          const int j = 2 * j2 + e;
+          const float co = v[2 * e], sn = v[2 * e + 1];
+          const float x1 = (float)lo[j], x2 = (float)hi[j];
+          olo[j] = (half_t)__builtin_fmaf(x1, co, -(x2 * sn));
+          ohi[j] = (half_t)__builtin_fmaf(x1, sn, x2 * co);
+        }
+      }
+      lo = olo;
+      hi = ohi;
+    }
+    *reinterpret_cast<half4_t*>(dst + d) = lo;
+    *reinterpret_cast<half4_t*>(dst + half + d) = hi;
+  } else if (MODE == SMALL_SWIGLU) {
     const int n_g = row0 + 4 * q4;                      // gate rows; the matching up rows are 16 further
     half4_t o;
 #pragma unroll
@@ -212,15 +329,35 @@ __global__ __launch_bounds__(NW * 64) void qmm_small_kernel(SmallArgs a) {
   }
 }
 
-constexpr int SMALL_K4 = 4 * 3 * 128;      // four waves, three chunks each
-constexpr int SMALL_K8 = 8 * 5 * 128;      // eight waves, five chunks each
+constexpr int SMALL_K4 = 4 * SMALL_MAXC * 128;       // four waves, three chunks each
+constexpr int SMALL_K8 = 8 * SMALL_MAXC * 128;
+constexpr int SMALL_K16 = 16 * SMALL_MAXC * 128;
+
+template <int MODE>
+void small_launch(const SmallArgs& a, int grid, hipStream_t st) {
+  const bool tall = a.T > 8;
+#define SMALL_GO(NW)                                                                                   \
+  do {                                                                                                 \
+    if (tall)                                                                                          \
+      hipLaunchKernelGGL((qmm_small_kernel<NW, 4, MODE>), dim3(grid), dim3(NW * 64), 0, st, a);        \
+    else                                                                                               \
+      hipLaunchKernelGGL((qmm_small_kernel<NW, 2, MODE>), dim3(grid), dim3(NW * 64), 0, st, a);        \
+  } while (0)
+  if (a.K <= SMALL_K4)
+    SMALL_GO(4);
+  else if (a.K <= SMALL_K8)
+    SMALL_GO(8);
+  else
+    SMALL_GO(16);
+#undef SMALL_GO
+}
 
 }  // namespace
 
 EAGLE_EXPORT int eagle_qmm_small_supported(int T, int N, int K, int norm, int swiglu) {
   (void)norm;
   return T >= 1 && T <= 16 && N >= 16 && (N % (swiglu ? 32 : 16)) == 0 && K >= 128 && (K % 128) == 0 &&
-         K <= SMALL_K8;
+         K <= SMALL_K16;
 }
 
 EAGLE_EXPORT int eagle_qmm_small_w4g64_f16(const void* x, const void* norm_w, float eps, const uint32_t* wq,
@@ -248,18 +385,60 @@ EAGLE_EXPORT int eagle_qmm_small_w4g64_f16(const void* x, const void* norm_w, fl
   a.T = T;
   a.N = N;
   a.K = K;
+  a.rope_cs = nullptr;
+  a.q_out = a.k_cache = a.v_cache = nullptr;
+  a.len_dev = nullptr;
+  a.H = a.G = a.hd = 0;
+  a.cap = 0;
   hipStream_t st = static_cast<hipStream_t>(stream);
-  const bool wide = K > SMALL_K4;
-  if (swiglu) {
-    if (wide)
-      hipLaunchKernelGGL((qmm_small_kernel<8, 5, 2>), dim3(N / 32), dim3(512), 0, st, a);
-    else
-      hipLaunchKernelGGL((qmm_small_kernel<4, 3, 2>), dim3(N / 32), dim3(256), 0, st, a);
-  } else {
-    if (wide)
-      hipLaunchKernelGGL((qmm_small_kernel<8, 5, 1>), dim3(N / 16), dim3(512), 0, st, a);
-    else
-      hipLaunchKernelGGL((qmm_small_kernel<4, 3, 1>), dim3(N / 16), dim3(256), 0, st, a);
-  }
+  if (swiglu)
+    small_launch<SMALL_SWIGLU>(a, N / 32, st);
+  else
+    small_launch<SMALL_PLAIN>(a, N / 16, st);
+  return eagle_launch_status();
+}
+
+EAGLE_EXPORT int eagle_qkv_rope_small_supported(int T, int D, int H, int G, int hd) {
+  return T >= 1 && T <= 16 && H >= 1 && G >= 1 && (H % G) == 0 && hd >= 32 && (hd % 32) == 0 &&
+         D >= 128 && (D % 128) == 0 && D <= SMALL_K16;
+}
+
+EAGLE_EXPORT int eagle_qkv_rope_small_w4g64_f16(const void* x, const void* norm_w, float eps,
+                                                const uint32_t* wq, const void* scales, const void* biases,
+                                                const void* bias, const float* rope_cs, void* q_out,
+                                                void* k_cache, void* v_cache, const int32_t* cache_len_dev,
+                                                int T, int D, int H, int G, int hd, long capacity,
+                                                int group_size, int bits, eagle_stream_t stream) {
+  if (!x || !wq || !scales || !biases || !rope_cs || !q_out || !k_cache || !v_cache || !cache_len_dev)
+    return EAGLE_ERR_NULL;
+  if (group_size != 64 || bits != 4) return EAGLE_ERR_UNSUPPORTED;
+  if (!eagle_qkv_rope_small_supported(T, D, H, G, hd) || capacity < T) return EAGLE_ERR_SHAPE;
+  const void* aligned[] = {x, norm_w, wq, rope_cs, q_out, k_cache, v_cache};
+  for (const void* p : aligned)
+    if (p && !eagle_aligned16(p)) return EAGLE_ERR_ALIGN;
+  SmallArgs a;
+  a.x = static_cast<const half_t*>(x);
+  a.norm_w = static_cast<const half_t*>(norm_w);
+  a.w = wq;
+  a.s = static_cast<const half_t*>(scales);
+  a.b = static_cast<const half_t*>(biases);
+  a.bias = static_cast<const half_t*>(bias);
+  a.residual = nullptr;
+  a.out = nullptr;
+  a.eps = eps;
+  a.T = T;
+  a.N = (H + 2 * G) * hd;
+  a.K = D;
+  a.rope_cs = rope_cs;
+  a.q_out = static_cast<half_t*>(q_out);
+  a.k_cache = static_cast<half_t*>(k_cache);
+  a.v_cache = static_cast<half_t*>(v_cache);
+  a.len_dev = cache_len_dev;
+  a.H = H;
+  a.G = G;
+  a.hd = hd;
+  a.cap = capacity;
+  hipStream_t st = static_cast<hipStream_t>(stream);
+  small_launch<SMALL_ROPE>(a, (H + 2 * G) * (hd / 32), st);
   return eagle_launch_status();
 }

@@ -296,6 +296,33 @@ def quantized_matmul_small(x, w_q, scales, biases, bias=None, out=None, norm_wei
     return out
 
 
+def qkv_rope_small_supported(T, D, H, G, hd):
+    return bool(_lib.lib().eagle_qkv_rope_small_supported(T, D, H, G, hd))
+
+
+def qkv_rope_small(x, w_q, scales, biases, bias, rope_cs, q_rot, k_cache, v_cache, cache_len_dev, H, G, hd,
+                   norm_weight=None, eps=1e-6):
+    """RMSNorm, fused q|k|v product, rotation of q and k with the (cos, sin) table and append of the
+    new K / V rows at *cache_len_dev, in one launch (mlx_llama.py:136-183, 231-233).  x [T, D];
+    q_rot [H, T, hd] is written; k_cache, v_cache [G, capacity, hd]."""
+    _need_cuda(x, w_q, scales, biases, bias, rope_cs, q_rot, k_cache, v_cache, cache_len_dev, norm_weight)
+    x = _f16(x, "x")
+    T, D = x.shape
+    w_q = as_packed_u32(w_q)
+    if w_q.shape != ((H + 2 * G) * hd, D // 8) or tuple(q_rot.shape) != (H, T, hd) \
+            or tuple(k_cache.shape[-3:]) != (G, k_cache.shape[-2], hd) or tuple(rope_cs.shape) != (T, hd // 2, 2):
+        raise ValueError("shape mismatch")
+    for t in (q_rot, k_cache, v_cache, rope_cs):
+        if not t.is_contiguous():
+            raise ValueError("non-contiguous buffer")
+    rc = _lib.lib().eagle_qkv_rope_small_w4g64_f16(
+        _ptr(x), _ptr(norm_weight), float(eps), _ptr(w_q), _ptr(_f16(scales, "scales")), _ptr(_f16(biases, "biases")),
+        _ptr(bias), _ptr(rope_cs), _ptr(q_rot), _ptr(k_cache), _ptr(v_cache), _ptr(cache_len_dev), T, D, H, G, hd,
+        k_cache.shape[-2], 64, 4, _stream())
+    _lib.check(rc, "qkv_rope_small")
+    return q_rot
+
+
 def qmv_preferred(N, K):
     """True where the vector-ALU kernel is the faster form for one row of x: measured on the
     projection shapes of the 7B model (M = 1: 5.7 against 8.5 us for 3584 x 3584, 12.5 against

@@ -59,6 +59,8 @@ class DecoderPass:
         if folded and not can_fold:
             raise ValueError("the small-row form does not take these shapes or weights")
         self.folded = can_fold if folded is None else bool(folded)
+        # within the folded form: rotation and cache append in the q|k|v launch
+        self.rope_folded = self.folded and ops.qkv_rope_small_supported(T, D, H, G, hd)
         L = _lib.lib()
         head = model.lm_head if not args.tie_word_embeddings else model.model.embed_tokens
         need = max(L.eagle_qmm_workspace_bytes(T, n, k) for n, k in
@@ -97,11 +99,15 @@ class DecoderPass:
             for i, layer in enumerate(layers):
                 at, mlp, c = layer.self_attn, layer.mlp, self.cache[i]
                 w, sc, bi, b = self.qkv_w[i]
-                ops.quantized_matmul_small(self.h, w, sc, bi, bias=b, out=self.qkv,
-                                           norm_weight=layer.input_layernorm.weight, eps=eps)
-                ops.rope_kv_append(q_lin, k_lin, v_lin, positions, at._inv_freqs, at._scaling_factor,
-                                   self.q_rot, c.keys[0], c.values[0], write_len, H, G, hd, row_stride=W,
-                                   rope_cs=self.rope_cs)
+                if self.rope_folded:
+                    ops.qkv_rope_small(self.h, w, sc, bi, b, self.rope_cs, self.q_rot, c.keys[0], c.values[0],
+                                       write_len, H, G, hd, norm_weight=layer.input_layernorm.weight, eps=eps)
+                else:
+                    ops.quantized_matmul_small(self.h, w, sc, bi, bias=b, out=self.qkv,
+                                               norm_weight=layer.input_layernorm.weight, eps=eps)
+                    ops.rope_kv_append(q_lin, k_lin, v_lin, positions, at._inv_freqs, at._scaling_factor,
+                                       self.q_rot, c.keys[0], c.values[0], write_len, H, G, hd, row_stride=W,
+                                       rope_cs=self.rope_cs)
                 attend(at, c)
                 o = at.o_proj
                 ops.quantized_matmul_small(self.attn, o.weight, o.scales, o.biases, bias=o.bias, out=self.h,

@@ -35,9 +35,9 @@ def dev_args(layer, dev):
     return (d["weight"], d["scales"], d["biases"]), d.get("bias")
 
 
-# K: one chunk, the drafter's hidden size, the limit of the four-wave form; then eight waves
+# K: one chunk, the drafter's hidden size, the limit of the four-wave form; then eight and sixteen waves
 @pytest.mark.parametrize("N,K", [(16, 128), (1152, 896), (896, 896), (272, 1280), (896, 4864), (48, 1408),
-                                 (2048, 5120), (32, 2560)])
+                                 (2048, 5120), (32, 2560), (16, 3072), (48, 6144)])
 @pytest.mark.parametrize("T", [1, 8, 13, 16])
 def test_plain_and_residual_forms(dev, T, N, K):
     print(f"small rows T={T} N={N} K={K}", flush=True)
@@ -123,7 +123,7 @@ def test_swiglu_with_norm(dev, T, I, K, bias):
 def test_refusals(dev):
     assert not ops.small_supported(17, 896, 896)                       # rows
     assert not ops.small_supported(8, 896, 900)
-    assert not ops.small_supported(8, 896, 5248)                       # x does not fit the waves of a workgroup
+    assert not ops.small_supported(8, 896, 6272)                       # x does not fit the waves of a workgroup
     assert not ops.small_supported(8, 896, 18944)
     assert not ops.small_supported(8, 48, 896, swiglu=True)            # whole (gate, up) tile pairs
     rng = np.random.default_rng(1)
@@ -207,3 +207,47 @@ def test_pass_object_falls_back(dev):
     sc = model.model.layers[0].mlp.down_proj.scales
     sc[0, 0] = 0.25                                                    # scale * 2^18 no longer a finite fp16
     assert not spec.DecoderPass(model, cache, 8).folded
+
+
+@pytest.mark.parametrize("T,D,H,G,hd,bias", [(8, 896, 14, 2, 64, True), (8, 128, 2, 1, 64, False),
+                                             (3, 256, 4, 2, 64, True), (16, 1024, 8, 2, 128, True),
+                                             (8, 2048, 32, 8, 64, False), (5, 384, 3, 3, 32, True)])
+def test_qkv_with_rotation_and_append(dev, T, D, H, G, hd, bias):
+    """Norm + q|k|v + rope + cache append in one launch against the same small-row product followed
+    by the separate rope / append launch: the same q and new K rows (to the last bit but for rounding
+    ties of the rotation), identical V rows, and nothing else in the caches touched; rows past the capacity are dropped (their q rows too, as there)."""
+    rng = np.random.default_rng(T + D + H)
+    W = (H + 2 * G) * hd
+    layer = synth.make_qlinear(rng, W, D, bias=bias, gain=1.0)
+    (w, sc, bi), b = dev_args(layer, dev)
+    x = to_dev(synth.make_x(rng, T, D), dev)
+    nw = to_dev((1.0 + rng.normal(0, 0.1, D)).astype(np.float16), dev)
+    args = synth.ModelArgs(head_dim=hd, hidden_size=hd * H, num_attention_heads=H, rope_theta=1e4)
+    inv, scaling = synth.inv_freqs(args)
+    pos = to_dev(rng.integers(0, 500, T).astype(np.int32), dev)
+    cs = ops.rope_table(pos, to_dev(inv, dev), scaling)
+    for cap, P in ((64, 11), (40, 40 - T + 2)):
+        wl = torch.tensor([P], dtype=torch.int32, device=dev)
+        f16 = dict(dtype=torch.float16, device=dev)
+        outs = []
+        for fused in (False, True):
+            q_rot = torch.full((H, T, hd), 5.0, **f16)
+            kc = torch.full((G, cap, hd), 7.0, **f16)
+            vc = torch.full((G, cap, hd), 7.0, **f16)
+            if fused:
+                ops.qkv_rope_small(x, w, sc, bi, b, cs, q_rot, kc, vc, wl, H, G, hd, norm_weight=nw, eps=EPS)
+            else:
+                qkv = ops.quantized_matmul_small(x, w, sc, bi, bias=b, norm_weight=nw, eps=EPS)
+                ops.rope_kv_append(qkv, qkv[:, H * hd:], qkv[:, (H + G) * hd:], pos, to_dev(inv, dev), scaling,
+                                   q_rot, kc, vc, wl, H, G, hd, row_stride=W, rope_cs=cs)
+            torch.cuda.synchronize()
+            outs.append((q_rot, kc, vc))
+        for a, bb in zip(*outs):
+            # the two kernels contract the rotation's multiply-adds differently: a last-bit fp32
+            # difference can land on an fp16 rounding tie (seen: one element in 16 K)
+            a32, b32 = a.float(), bb.float()
+            ulp = torch.exp2(torch.floor(torch.log2(a32.abs().clamp_min(2.0 ** -14))) - 10)
+            assert bool(((a32 - b32).abs() <= ulp).all())
+            assert int((a != bb).sum()) <= max(1, a.numel() // 2000)
+        assert torch.equal(outs[0][2], outs[1][2])                   # v rows are not rotated
+        assert (outs[1][1][:, :P] == 7.0).all() and (outs[1][1][:, P + T:] == 7.0).all()
