@@ -2,20 +2,31 @@
 // the QuantizedLinear layers of mlx_llama.py): out[M,N] = fp16( x[M,K] . (s*q + b)[N,K]^T ).
 //
 // With hundreds of rows the product is bound by the matrix cores, not by the weight stream, so
-// this is a tiled GEMM: a workgroup of four waves owns a 128 x 128 output block, each wave a
-// 64 x 64 quarter as 2 x 2 v_mfma_f32_32x32x16_f16 tiles (weights are the A operand: an
-// accumulator lane then holds one output row and four consecutive columns per register
-// group).  Per 64-wide K step (one quantisation group):
-//   * the x block [128 x 64] goes through LDS (double buffered, one barrier per step), loaded
-//     two steps ahead into registers;
+// this is a tiled GEMM: a workgroup of four waves side by side along the weight rows owns a
+// 64 x 128, 128 x 128 or 128 x 256 output block (x rows x weight rows), each wave all x rows of
+// the block as v_mfma_f32_32x32x16_f16 tiles (weights are the A operand: an accumulator lane
+// then holds one output row and four consecutive columns per register group).  Per 64-wide K
+// step (one quantisation group):
+//   * the x block goes through LDS (double buffered, one barrier per step), loaded one or two
+//     steps ahead into registers, a whole 128-byte row of the step per eight lanes;
 //   * every lane loads the 16 bytes (four packed words = 32 weights) of its weight row that its
 //     half of the MFMA K range needs, two steps ahead, and expands them in registers:
 //     a shift and v_and_or_b32 make the fp16 pair (16 + q_i, 16 + q_{i+4}); one packed fp16
-//     fma with (s, b - 16 s) gives the weights in fp16, as the reference kernels hold them (the
-//     expansion is what bounds this kernel, so it is four packed instructions per word, not
-//     eight).  That yields the eight weights of a word in the order
-//     q0 q4 q1 q5 q2 q6 q3 q7; x is stored to LDS in the same order within every group of
-//     eight, so both MFMA operands agree on which K index sits where.
+//     fma with (s, b - 16 s) gives the weights in fp16, as the reference kernels hold them.
+//     That yields the eight weights of a word in the order q0 q4 q1 q5 q2 q6 q3 q7; x is stored
+//     to LDS in the same order within every group of eight, so both MFMA operands agree on
+//     which K index sits where.  The expanded word j of a step is replaced by the next step's
+//     as soon as this step's matrix instructions have read it (one register set, which lets
+//     two workgroups share a compute unit with the 128 x 256 block);
+//   * the output tile of a wave leaves through LDS as whole rows.
+// Measured for 512 x 28672 x 4096 (s_memtime / s_memrealtime inside the kernel): the core clock
+// is 1.55 - 1.85 GHz while this kernel runs (a loop of matrix instructions alone sustains 2.1 - 2.4
+// PFLOP/s on the same box), a workgroup alone on a compute unit needs 1900 clocks per step for
+// 1024 clocks of matrix instructions, two together 1330 each; 448 workgroups on 512 places leave
+// a quarter of the compute units with one workgroup, which ends 25 % before the others.  Blocks
+// of 128 x 512 and 256 x 256 (half the LDS reads, or half the expansions, per matrix instruction;
+// 512 registers, one workgroup per compute unit) were 3 - 5 % faster on that shape and half as
+// fast on the narrow ones, and are not built.
 // fp32 accumulation, one fp16 rounding, optional fp16 bias added after the rounding.
 #include "common.h"
 
@@ -90,7 +101,7 @@ struct StepIndex {
 // instruction go to 32 or 64 different cache lines either way, and the rate of such requests,
 // not their bytes, is what the kernel runs up against).
 template <int NTW, int MT, int SBW>
-__global__ __launch_bounds__(256) void qmm_gemm_w4g64_kernel(
+__global__ __launch_bounds__(256, 2) void qmm_gemm_w4g64_kernel(
     const half_t* __restrict__ x, const uint32_t* __restrict__ w, const half_t* __restrict__ s,
     const half_t* __restrict__ b, const half_t* __restrict__ bias, half_t* __restrict__ out, int M,
     int N, int K) {
@@ -115,10 +126,17 @@ __global__ __launch_bounds__(256) void qmm_gemm_w4g64_kernel(
   const int KG = K >> 6;                    // groups per weight row
   const int steps = K / BK;
 
-  const int xr = tid / TPR, xh = tid % TPR;
-  int xrow = m0 + xr;
-  if (xrow > M - 1) xrow = M - 1;           // rows past the end are never stored
-  const half_t* xp = x + (long)xrow * K + xh * (BK / TPR);
+  // thread (xr, xc) moves the 16 bytes at column 8 xc of rows xr + 32 g: a load instruction of a
+  // wave covers eight whole 128-byte rows of the step (the rate of cache lines touched, not
+  // bytes, bounds the loads of this kernel)
+  const int xr = tid >> 3, xc = tid & 7;
+  const half_t* xp[PP];
+#pragma unroll
+  for (int g = 0; g < PP; ++g) {
+    int xrow = m0 + xr + 32 * g;
+    if (xrow > M - 1) xrow = M - 1;         // rows past the end are never stored
+    xp[g] = x + (long)xrow * K + xc * 8;
+  }
   int nrow[NTW];
 #pragma unroll
   for (int nt = 0; nt < NTW; ++nt) {
@@ -138,10 +156,11 @@ __global__ __launch_bounds__(256) void qmm_gemm_w4g64_kernel(
   typedef half_t sbvec_t __attribute__((ext_vector_type(SBV ? SBW : 2)));
   half_t sreg[2][NTW], breg[2][NTW];        // SBW = 1: scale and bias of those steps
   sbvec_t s8[2][NTW], b8[2][NTW];           // SBW > 1: of this chunk of SBW steps and of the next
-  half8_t af[2][NTW][4];                    // expanded weights of this step and the next
+  half8_t af[NTW][4];                       // expanded weights of this step; word j is replaced by the next
+                                            // step's as soon as this step's matrix instructions have read it
   auto fetch_x = [&](int ks, int set) {
 #pragma unroll
-    for (int g = 0; g < PP; ++g) xreg[set][g] = *reinterpret_cast<const half8_t*>(xp + (long)ks * BK + g * 8);
+    for (int g = 0; g < PP; ++g) xreg[set][g] = *reinterpret_cast<const half8_t*>(xp[g] + (long)ks * BK);
   };
   auto fetch_w = [&](int ks, int p) {
 #pragma unroll
@@ -163,17 +182,17 @@ __global__ __launch_bounds__(256) void qmm_gemm_w4g64_kernel(
   auto stash = [&](int buf) {                // x of a step travels in register set (step % XD)
 #pragma unroll
     for (int g = 0; g < PP; ++g)
-      *reinterpret_cast<half8_t*>(&xs[buf][xr * XS + xh * (BK / TPR) + g * 8]) = permute8(xreg[buf % XD][g]);
+      *reinterpret_cast<half8_t*>(&xs[buf][(xr + 32 * g) * XS + xc * 8]) = permute8(xreg[buf % XD][g]);
   };
   // word j of the weight tiles of register set p; e = index of their step within the chunk of
   // SBW (SBW = first step of the next chunk)
-  auto expand = [&](int p, int j, int e) {
+  auto expand = [&](int j, int e) {
 #pragma unroll
     for (int nt = 0; nt < NTW; ++nt) {
-      const half_t sc = SBV ? s8[e / SBW][nt][e % SBW] : sreg[p][nt];
-      const half_t bi = SBV ? b8[e / SBW][nt][e % SBW] : breg[p][nt];
+      const half_t sc = SBV ? s8[e / SBW][nt][e % SBW] : sreg[e & 1][nt];
+      const half_t bi = SBV ? b8[e / SBW][nt][e % SBW] : breg[e & 1][nt];
       const half_t b16 = (half_t)((float)bi - 16.f * (float)sc);
-      af[p][nt][j] = dequant_word(wreg[e % WD][nt][j], half2_t{sc, sc}, half2_t{b16, b16});
+      af[nt][j] = dequant_word(wreg[e % WD][nt][j], half2_t{sc, sc}, half2_t{b16, b16});
     }
   };
 
@@ -196,13 +215,13 @@ __global__ __launch_bounds__(256) void qmm_gemm_w4g64_kernel(
   }
   stash(0);
 #pragma unroll
-  for (int j = 0; j < 4; ++j) expand(0, j, 0);
+  for (int j = 0; j < 4; ++j) expand(j, 0);
   __syncthreads();
 
-  // One K step, p = ks & 1: LDS buffer p holds x of this step and af[p] its expanded weights;
+  // One K step, p = ks & 1: LDS buffer p holds x of this step and af its expanded weights;
   // register set p ^ 1 holds the packed weights and the x of the next step (the weights are
-  // expanded between this step's matrix instructions, the x goes to LDS at its end); set p is
-  // free for the loads of step ks + 2.  Loaded
+  // expanded into af word by word behind this step's matrix instructions, the x goes to LDS at
+  // its end); set p is free for the loads of step ks + 2.  Loaded
   // values are used where they were loaded (a copy of a register with a load in flight would
   // wait for the load), and the loads are issued first (left alone, the scheduler sinks them
   // to the end of the step, where the in-order counter waits for them at once).
@@ -218,12 +237,12 @@ __global__ __launch_bounds__(256) void qmm_gemm_w4g64_kernel(
 #pragma unroll
       for (int mt = 0; mt < MT; ++mt)
         bf[mt] = *reinterpret_cast<const half8_t*>(&xs[p][(wm * 32 * MT + mt * 32 + ql) * XS + hb * 32 + j * 8]);
-      expand(p ^ 1, j, e + 1);
 #pragma unroll
       for (int nt = 0; nt < NTW; ++nt)
 #pragma unroll
         for (int mt = 0; mt < MT; ++mt)
-          acc[nt][mt] = __builtin_amdgcn_mfma_f32_32x32x16_f16(af[p][nt][j], bf[mt], acc[nt][mt], 0, 0, 0);
+          acc[nt][mt] = __builtin_amdgcn_mfma_f32_32x32x16_f16(af[nt][j], bf[mt], acc[nt][mt], 0, 0, 0);
+      expand(j, e + 1);
     }
     __builtin_amdgcn_sched_barrier(0);
     stash(p ^ 1);
@@ -271,23 +290,39 @@ __global__ __launch_bounds__(256) void qmm_gemm_w4g64_kernel(
     if (ks < steps) body(ks, StepIndex<0>{});
   }
 
-  // accumulator register i of a lane: weight row (output column) 8*(i/4) + 4*hb + i%4 of the
-  // tile, x row (output row) ql
+  // Accumulator register i of a lane: weight row (output column) 8*(i/4) + 4*hb + i%4 of the
+  // tile, x row (output row) ql: four columns (8 bytes) of a row per lane and store, so stores
+  // straight from the registers touch 32 output lines 16 bytes at a time, eight times over.  The
+  // wave's tile goes through LDS instead (its own region, over the x buffers, which every wave
+  // has finished reading) and leaves as whole rows: 16 bytes per lane, a row of the tile per
+  // 4 * NTW lanes.
+  __syncthreads();
+  {
+    constexpr int ROWB = 64 * NTW + 16;                  // bytes per staged row (padded)
+    unsigned char* stage = reinterpret_cast<unsigned char*>(xs_all) + wave * (32 * MT * ROWB);
 #pragma unroll
-  for (int mt = 0; mt < MT; ++mt) {
-    const int m = m0 + wm * 32 * MT + mt * 32 + ql;
-    if (m >= M) continue;
+    for (int mt = 0; mt < MT; ++mt)
 #pragma unroll
-    for (int nt = 0; nt < NTW; ++nt) {
+      for (int nt = 0; nt < NTW; ++nt)
 #pragma unroll
-      for (int i4 = 0; i4 < 4; ++i4) {
-        const int n = n0 + nt * 32 + 8 * i4 + 4 * hb;
-        if (n >= N) continue;                // N is a multiple of 4 columns (checked by the host)
-        half4_t v = half4_t{(half_t)acc[nt][mt][4 * i4 + 0], (half_t)acc[nt][mt][4 * i4 + 1],
-                            (half_t)acc[nt][mt][4 * i4 + 2], (half_t)acc[nt][mt][4 * i4 + 3]};
-        if (bias) v += *reinterpret_cast<const half4_t*>(bias + n);
-        *reinterpret_cast<half4_t*>(out + (long)m * N + n) = v;
-      }
+        for (int i4 = 0; i4 < 4; ++i4) {
+          half4_t v = half4_t{(half_t)acc[nt][mt][4 * i4 + 0], (half_t)acc[nt][mt][4 * i4 + 1],
+                              (half_t)acc[nt][mt][4 * i4 + 2], (half_t)acc[nt][mt][4 * i4 + 3]};
+          const int n = n0 + nt * 32 + 8 * i4 + 4 * hb;
+          if (bias && n < N) v += *reinterpret_cast<const half4_t*>(bias + n);
+          *reinterpret_cast<half4_t*>(stage + (mt * 32 + ql) * ROWB + nt * 64 + i4 * 16 + hb * 8) = v;
+        }
+    __builtin_amdgcn_wave_barrier();
+    constexpr int LPR = 4 * NTW;                         // lanes per row (16 bytes each)
+    constexpr int RPI = 64 / LPR;                        // rows per store instruction
+    const int pr = lane / LPR, pc = lane % LPR;
+#pragma unroll
+    for (int r0 = 0; r0 < 32 * MT; r0 += RPI) {
+      const int row = r0 + pr;
+      const int m = m0 + wm * 32 * MT + row;
+      const int n = n0 + pc * 8;
+      const half8_t v = *reinterpret_cast<const half8_t*>(stage + row * ROWB + pc * 16);
+      if (m < M && n < N) *reinterpret_cast<half8_t*>(out + (long)m * N + n) = v;
     }
   }
 }
@@ -298,7 +333,9 @@ int launch_gemm(const half_t* x, const uint32_t* w, const half_t* s, const half_
   constexpr int BMT = 32 * MT;
   constexpr int BN = 128 * NTW;
   static_assert(256 % BMT == 0 && BMT >= 32, "block load mapping");
-  const size_t lds = 2 * (size_t)BMT * XS * sizeof(half_t);
+  const size_t lds_x = 2 * (size_t)BMT * XS * sizeof(half_t);
+  const size_t lds_out = 4 * (size_t)BMT * (64 * NTW + 16);         // the output tiles of the four waves
+  const size_t lds = lds_x > lds_out ? lds_x : lds_out;
   static bool configured = false;
   if (!configured) {
     if (hipFuncSetAttribute(reinterpret_cast<const void*>(&qmm_gemm_w4g64_kernel<NTW, MT, SBW>),
