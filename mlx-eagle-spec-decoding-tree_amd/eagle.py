@@ -462,7 +462,7 @@ class TreeVerifier:
     Same kernels and operator order as Model.__call__ + the host functions above."""
 
     def __init__(self, model, cache, total_tokens=31, max_len=None, compact=True, fuse=True,
-                 swiglu=True, one_launch_attention=False, slab_plan=None, chain=None):
+                 swiglu=True, one_launch_attention=False, slab_plan=None, chain=None, resident_gate_up=None):
         """slab_plan: {"qkv": s, "o": s, "down": s}, K steps per slab for the projections that go
         through the slab form of the matmul (their consumer adds the slabs), 0 for the
         streaming kernel; None: the library's choice for this shape.
@@ -470,7 +470,13 @@ class TreeVerifier:
         ONE launch of a resident grid with a grid-wide barrier inside (`ops.norm_mlp_in`; needs the
         o projection in the slab form).  Off unless asked for: measured inside the 7B step it takes
         43.7 us against 5.3 + 30.6 us for the two launches it replaces (step 2.99 against 2.70 ms).
-        `chain_error()` reports a barrier that gave up."""
+        `chain_error()` reports a barrier that gave up.
+        resident_gate_up: gate|up + SwiGLU through the kernel that keeps x in registers and brings
+        the weights in by whole cache lines through LDS (`ops.quantized_matmul_resident`) instead of
+        the streaming kernel.  Off unless asked for; takes K a multiple of 512 up to 3584 and scales
+        below 0.2499 in magnitude.  Inside the 7B step it is 1.4 us per layer faster (2.661 against
+        2.699 ms per step, A/B on one box); the measurement and profile records of `bench.py` are
+        those of the default form."""
         args = model.args
         self.model, self.cache, self.args = model, cache, args
         if total_tokens + 1 > MAXT:
@@ -495,6 +501,11 @@ class TreeVerifier:
         if fuse:
             self._fuse_projections()
         self.slab = self._slab_plan(slab_plan)
+        can_res = bool(self.swiglu and ops.resident_supported(T, 2 * I, D)
+                       and all(float(g[1].abs().max()) < ops.SMALL_SCALE_LIMIT for g in self.gu_w))
+        if resident_gate_up and not can_res:
+            raise ValueError("the resident form of gate|up does not take this model")
+        self.resident_gate_up = bool(resident_gate_up)
         can_chain = bool(self.swiglu and self.slab["o"] and ops.norm_mlp_in_supported(T, D, I)
                          and torch.cuda.get_device_properties(dev).multi_processor_count >= 256)
         if chain and not can_chain:

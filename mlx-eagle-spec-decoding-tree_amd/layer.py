@@ -70,7 +70,9 @@ def emit_layer(p, i, write_len, attend, positions=None, attend_with_rope=None):
             ops.rms_norm(p.o, layer.post_attention_layernorm.weight, args.rms_norm_eps, residual=p.h,
                          out=p.hn, h_out=p.h)
         w, sc, bi, b = p.gu_w[i]
-        if p.swiglu:
+        if p.swiglu and getattr(p, "resident_gate_up", False):
+            ops.quantized_matmul_resident(p.hn, w, sc, bi, bias=b, out=p.act, swiglu=True)
+        elif p.swiglu:
             ops.quantized_matmul_swiglu(p.hn, w, sc, bi, bias=b, out=p.act)
         else:
             ops.quantized_matmul(p.hn, w, sc, bi, bias=b, out=p.gate_up)

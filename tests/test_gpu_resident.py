@@ -214,3 +214,33 @@ def test_verifier_with_the_chained_launch(dev):
     with pytest.raises(ValueError):
         s2 = tm.build(dev, "qwen_like", 40, 8, seed=1)        # hidden 256: the chained launch does not take it
         eagle.TreeVerifier(s2["model"], s2["cache"], total_tokens=7, chain=True)
+
+
+def test_verifier_with_resident_gate_up(dev):
+    """TreeVerifier(resident_gate_up=True): gate|up + SwiGLU of every layer through the kernel with
+    x resident in registers, the whole step against the oracle and against the default form; a
+    model whose hidden size the kernel does not take is refused."""
+    import test_gpu_model as tm
+    from mlx_eagle_spec_decoding_tree_amd import eagle
+    from oracle import model_oracle
+    P, T = 200, 32
+    s = tm.build(dev, "llama_like_tied", P, T, seed=9)          # hidden 512
+    want = model_oracle.verify_step(s["args"], s["weights"], s["inv"], s["sc"], s["tokens"], s["depth"],
+                                    s["parents"], s["anc"], s["ocache"], P)
+    ver = tm.run_verifier(s, dev, graph=True, resident_gate_up=True, compact=False)
+    assert ver.resident_gate_up
+    ver.len_dev.fill_(P)
+    ver.step()
+    torch.cuda.synchronize()
+    got = ver.logits.cpu().numpy()
+    assert rel_err(got, want["logits"]) <= TOL
+    assert np.array_equal(ver.node_argmax.cpu().numpy(), oracle.argmax_rows(got))
+    s1 = tm.build(dev, "llama_like_tied", P, T, seed=9)
+    plain = tm.run_verifier(s1, dev, graph=False, compact=False)
+    assert not plain.resident_gate_up
+    plain.step()
+    torch.cuda.synchronize()
+    assert rel_err(got, plain.logits.cpu().numpy()) <= TOL
+    with pytest.raises(ValueError):
+        s2 = tm.build(dev, "qwen_like", 40, 8, seed=1)          # hidden 256
+        eagle.TreeVerifier(s2["model"], s2["cache"], total_tokens=7, resident_gate_up=True)
