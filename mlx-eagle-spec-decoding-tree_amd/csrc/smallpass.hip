@@ -16,7 +16,10 @@
 //     of a wave (weights, scales, its columns of x as the B operand of v_mfma_f32_16x16x32_f16) is
 //     in flight together; there is no loop over K.
 //   * The norm is folded into the load of x: each wave sums the squares of its columns, the row
-//     sums are added across the waves in LDS; no launch and no pass over memory for it.
+//     sums are added across the waves in LDS; no launch and no pass over memory for it.  Every
+//     workgroup repeats it, so it is kept short: v_dot2 for the sums, x / rms rounded to fp16 and
+//     then multiplied by the norm weight in packed fp16 (two roundings where the norm launch has
+//     one).
 //   * Expansion of the nibbles through fp16 subnormals as in csrc/resident.hip: fp16(s q + b),
 //     single rounding; scales below 0.2499.
 //
@@ -163,6 +166,32 @@ __global__ __launch_bounds__(NW * 64) void qmm_small_kernel(SmallArgs a) {
 #pragma unroll
       for (int i = 0; i < 4; ++i) nw[c][i] = *reinterpret_cast<const half8_t*>(np + (c < nch ? c : 0) * 128 + i * 8);
   }
+  // what the epilogue of wave 0 adds (bias, residual, the rotation's cos / sin, the cache length)
+  // is requested here with everything else, not after the product: a load behind the product is
+  // a microsecond of latency on the critical path of a kernel that takes four.  The values are
+  // only read under the conditions they were loaded under.
+  half4_t e_bias0, e_bias1, e_res;
+  float4_t e_cs[2];
+  long e_len = 0;
+  const int e_rope_head = MODE == SMALL_ROPE ? row0 / a.hd : 0;
+  if (wave == 0) {
+    const int bn = row0 + 4 * kq;
+    if (a.bias) {
+      e_bias0 = *reinterpret_cast<const half4_t*>(a.bias + bn);
+      if (NT == 2) e_bias1 = *reinterpret_cast<const half4_t*>(a.bias + bn + second);
+    }
+    if (MODE == SMALL_PLAIN && a.residual && r < a.T)
+      e_res = *reinterpret_cast<const half4_t*>(a.residual + (long)r * a.N + bn);
+    if (MODE == SMALL_ROPE) {
+      e_len = *a.len_dev;
+      if (r < a.T && e_rope_head < a.H + a.G) {
+        const int d = row0 - e_rope_head * a.hd + 4 * kq;
+        const float4_t* cs = reinterpret_cast<const float4_t*>(a.rope_cs + ((long)r * (a.hd >> 1) + d) * 2);
+        e_cs[0] = cs[0];
+        e_cs[1] = cs[1];
+      }
+    }
+  }
   // x through the wave's LDS buffer into the operand layout, a chunk at a time (rows past 4 RP,
   // which are rows past T, read what is there: their columns of the result are not stored)
   half8_t xb[MAXC][4];
@@ -192,7 +221,10 @@ __global__ __launch_bounds__(NW * 64) void qmm_small_kernel(SmallArgs a) {
 #pragma unroll
         for (int i = 0; i < 4; ++i)
 #pragma unroll
-          for (int e = 0; e < 8; ++e) ss += (float)xb[c][i][e] * (float)xb[c][i][e];
+          for (int e = 0; e < 8; e += 2) {
+            const half2_t p2 = half2_t{xb[c][i][e], xb[c][i][e + 1]};
+            ss = __builtin_amdgcn_fdot2(p2, p2, ss, false);      // exact products, fp32 sum
+          }
       }
     }
     ss += __shfl_xor(ss, 16, 64);
@@ -210,8 +242,8 @@ __global__ __launch_bounds__(NW * 64) void qmm_small_kernel(SmallArgs a) {
         for (int i = 0; i < 4; ++i) {
           half8_t o;
 #pragma unroll
-          for (int e = 0; e < 8; ++e) o[e] = (half_t)((float)nw[c][i][e] * ((float)xb[c][i][e] * rinv));
-          xb[c][i] = o;
+          for (int e = 0; e < 8; ++e) o[e] = (half_t)((float)xb[c][i][e] * rinv);   // fp32 product, one rounding
+          xb[c][i] = o * nw[c][i];                                                      // packed fp16 products
         }
       }
     }
@@ -256,7 +288,7 @@ __global__ __launch_bounds__(NW * 64) void qmm_small_kernel(SmallArgs a) {
     // the linear output rounded to fp16 (bias added in fp16), rotated with the table's (cos, sin)
     // exactly as the separate rope launch does; v rows pass through
     const int half = a.hd >> 1;
-    const int hb = row0 / a.hd;
+    const int hb = e_rope_head;
     const int d = row0 - hb * a.hd + 4 * q4;            // < hd / 2
     half4_t lo, hi;
 #pragma unroll
@@ -264,11 +296,11 @@ __global__ __launch_bounds__(NW * 64) void qmm_small_kernel(SmallArgs a) {
       lo[i] = (half_t)acc[0][i];
       hi[i] = (half_t)acc[NT - 1][i];
       if (a.bias) {
-        lo[i] = lo[i] + a.bias[row0 + 4 * q4 + i];
-        hi[i] = hi[i] + a.bias[row0 + half + 4 * q4 + i];
+        lo[i] = lo[i] + e_bias0[i];
+        hi[i] = hi[i] + e_bias1[i];
       }
     }
-    const long P = *a.len_dev;
+    const long P = e_len;
     if (P + m >= a.cap) return;                         // the host checks capacity; never write past the buffer
     half_t* dst;
     if (hb < a.H) {
@@ -278,11 +310,10 @@ __global__ __launch_bounds__(NW * 64) void qmm_small_kernel(SmallArgs a) {
       dst = (hb < a.H + a.G ? a.k_cache : a.v_cache) + ((long)g * a.cap + P + m) * a.hd;
     }
     if (hb < a.H + a.G) {
-      const float4_t* cs = reinterpret_cast<const float4_t*>(a.rope_cs + ((long)m * half + d) * 2);
       half4_t olo, ohi;
 #pragma unroll
       for (int j2 = 0; j2 < 2; ++j2) {
-        const float4_t v = cs[j2];
+        const float4_t v = e_cs[j2];
 #pragma unroll
         for (int e = 0; e < 2; ++e) {
           const int j = 2 * j2 + e;
@@ -304,8 +335,8 @@ __global__ __launch_bounds__(NW * 64) void qmm_small_kernel(SmallArgs a) {
     for (int i = 0; i < 4; ++i) {
       half_t g = (half_t)acc[0][i], u = (half_t)acc[NT - 1][i];
       if (a.bias) {
-        g = g + a.bias[n_g + i];
-        u = u + a.bias[n_g + 16 + i];
+        g = g + e_bias0[i];
+        u = u + e_bias1[i];
       }
       const float gf = (float)g;
       const half_t act = (half_t)(gf / (1.0f + expf(-gf)));
@@ -318,12 +349,11 @@ __global__ __launch_bounds__(NW * 64) void qmm_small_kernel(SmallArgs a) {
 #pragma unroll
     for (int i = 0; i < 4; ++i) {
       o[i] = (half_t)acc[0][i];
-      if (a.bias) o[i] = o[i] + a.bias[n + i];
+      if (a.bias) o[i] = o[i] + e_bias0[i];
     }
     if (a.residual) {
-      const half4_t res = *reinterpret_cast<const half4_t*>(a.residual + (long)m * a.N + n);
 #pragma unroll
-      for (int i = 0; i < 4; ++i) o[i] = (half_t)((float)o[i] + (float)res[i]);
+      for (int i = 0; i < 4; ++i) o[i] = (half_t)((float)o[i] + (float)e_res[i]);
     }
     *reinterpret_cast<half4_t*>(a.out + (long)m * a.N + n) = o;
   }
