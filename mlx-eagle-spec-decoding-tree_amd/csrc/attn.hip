@@ -333,7 +333,7 @@ __global__ void tree_attn_merge_kernel(const half_t* __restrict__ part_o,
   out += (long)piece * 32 * H * HD;
   constexpr int QW = HD / 4;                       // threads per token
   constexpr int TPW = 256 / HD;                    // tokens per wave: MERGE_TOK tokens on HD / 64 waves
-  constexpr int PRE = 8;
+  constexpr int PRE = 32;                          // partial outputs requested before anything is waited for
   __shared__ float wts[MERGE_TOK][64];
   const int head = blockIdx.x;
   const int tid = threadIdx.x;
@@ -358,7 +358,7 @@ __global__ void tree_attn_merge_kernel(const half_t* __restrict__ part_o,
   half4_t pre[PRE];
 #pragma unroll
   for (int k = 0; k < PRE; ++k)
-    pre[k] = *reinterpret_cast<const half4_t*>(src + (long)(k < nsplit ? k : nsplit - 1) * 32 * HD);
+    if (k < nsplit) pre[k] = *reinterpret_cast<const half4_t*>(src + (long)k * 32 * HD);
 
   int P = len_dev[piece];
   if (P > cap - Tk) P = (int)(cap - Tk);    // as in the split kernel
