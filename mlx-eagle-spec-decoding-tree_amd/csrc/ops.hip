@@ -160,7 +160,8 @@ __global__ void rope_kv_append_slabs_kernel(const float* __restrict__ partial, i
   const size_t ld = (size_t)heads * hd;
   const size_t stride = 32 * ld;
   const float* p = partial + (size_t)t * ld + (size_t)hh * hd + c;
-  // cos / sin and the bias are requested with the slabs
+  // the cache length, cos / sin and the bias are requested with the slabs
+  const long P = *len_dev;
   float4_t cs0 = float4_t{0.f, 0.f, 0.f, 0.f}, cs1 = cs0;
   if (hh < H + G) {
     const float4_t* cs = reinterpret_cast<const float4_t*>(rope_cs + ((long)t * half + c) * 2);
@@ -198,7 +199,6 @@ __global__ void rope_kv_append_slabs_kernel(const float* __restrict__ partial, i
     xlo += blo;
     xhi += bhi;
   }
-  const long P = *len_dev;
   if (P + t >= cap) return;   // host checks capacity; never write past the buffer
   if (hh < H + G) {
     const bool is_q = hh < H;
