@@ -26,13 +26,16 @@
 // a quarter of the compute units with one workgroup, which ends 25 % before the others.  Blocks
 // of 128 x 512 and 256 x 256 (half the LDS reads, or half the expansions, per matrix instruction;
 // 512 registers, one workgroup per compute unit) were 3 - 5 % faster on that shape and half as
-// fast on the narrow ones, and are not built.
+// fast on the narrow ones, and are not built.  The narrow shapes (N = 4096: one 64 x 128 block per
+// compute unit) run two groups of four waves per workgroup, each over half of K (+5 %); loading
+// the packed weights by whole 128-byte lines (timing only, results wrong) is worth 0 - 7 %.
 // fp32 accumulation, one fp16 rounding, optional fp16 bias added after the rounding.
 #include "common.h"
 
 namespace {
 
 constexpr int BK = 64;
+constexpr long GEMM_SPLIT_WGS = 384;        // two K groups per workgroup up to this many workgroups
 constexpr long NUM_CU = 256;
 constexpr int XS = BK + 8;                  // LDS row stride in halves (144 bytes: conflict-free 16-byte reads)
 
@@ -100,8 +103,12 @@ struct StepIndex {
 // fetch per SBW K steps instead of one 2-byte load per row and step (the loads of one
 // instruction go to 32 or 64 different cache lines either way, and the rate of such requests,
 // not their bytes, is what the kernel runs up against).
-template <int NTW, int MT, int SBW>
-__global__ __launch_bounds__(256, 2) void qmm_gemm_w4g64_kernel(
+// KGRP = groups of four waves per workgroup (1 or 2).  With two, each group works through its
+// own half of K with its own x buffers (one barrier serves both) and the halves are added
+// through LDS at the end: for shapes that give a compute unit a single workgroup, whose four
+// waves would otherwise have nothing to overlap their waits with.
+template <int NTW, int MT, int SBW, int KGRP = 1>
+__global__ __launch_bounds__(256 * KGRP, (KGRP == 1 ? 2 : 1)) void qmm_gemm_w4g64_kernel(
     const half_t* __restrict__ x, const uint32_t* __restrict__ w, const half_t* __restrict__ s,
     const half_t* __restrict__ b, const half_t* __restrict__ bias, half_t* __restrict__ out, int M,
     int N, int K) {
@@ -115,8 +122,9 @@ __global__ __launch_bounds__(256, 2) void qmm_gemm_w4g64_kernel(
   constexpr int TPR = 256 / BMT;             // threads per x row in the block load (2 or 1)
   constexpr int PP = 8 / TPR;                // 16-byte pieces per thread
   extern __shared__ __attribute__((aligned(16))) half_t xs_all[];
-  half_t* xs[2] = {xs_all, xs_all + BMT * XS};
-  const int tid = threadIdx.x;
+  const int grp = KGRP == 1 ? 0 : (int)(threadIdx.x >> 8);    // which part of K this group of waves takes
+  half_t* xs[2] = {xs_all + grp * (2 * BMT * XS), xs_all + grp * (2 * BMT * XS) + BMT * XS};
+  const int tid = threadIdx.x & 255;
   const int wave = tid >> 6, lane = tid & 63;
   const int ql = lane & 31, hb = lane >> 5;
   const int wn = wave % WN, wm = wave / WN;
@@ -124,7 +132,12 @@ __global__ __launch_bounds__(256, 2) void qmm_gemm_w4g64_kernel(
   const int m0 = blockIdx.y * BMT;
   const int KW = K >> 3;                    // packed words per weight row
   const int KG = K >> 6;                    // groups per weight row
-  const int steps = K / BK;
+  const int steps = K / BK / KGRP;          // of this group
+  const int kbase = grp * steps * BK;       // its first column
+  x += kbase;
+  w += kbase >> 3;
+  s += kbase >> 6;
+  b += kbase >> 6;
 
   // thread (xr, xc) moves the 16 bytes at column 8 xc of rows xr + 32 g: a load instruction of a
   // wave covers eight whole 128-byte rows of the step (the rate of cache lines touched, not
@@ -297,6 +310,35 @@ __global__ __launch_bounds__(256, 2) void qmm_gemm_w4g64_kernel(
   // has finished reading) and leaves as whole rows: 16 bytes per lane, a row of the tile per
   // 4 * NTW lanes.
   __syncthreads();
+  if (KGRP > 1) {
+    // the second group's accumulators through LDS (over the x buffers), lane-contiguous
+    float4_t* red = reinterpret_cast<float4_t*>(xs_all) + (wave * (NTW * MT * 4)) * 64 + lane;
+    if (grp == 1) {
+#pragma unroll
+      for (int nt = 0; nt < NTW; ++nt)
+#pragma unroll
+        for (int mt = 0; mt < MT; ++mt)
+#pragma unroll
+          for (int i4 = 0; i4 < 4; ++i4)
+            red[((nt * MT + mt) * 4 + i4) * 64] = float4_t{acc[nt][mt][4 * i4], acc[nt][mt][4 * i4 + 1],
+                                                           acc[nt][mt][4 * i4 + 2], acc[nt][mt][4 * i4 + 3]};
+    }
+    __syncthreads();
+    if (grp == 0) {
+#pragma unroll
+      for (int nt = 0; nt < NTW; ++nt)
+#pragma unroll
+        for (int mt = 0; mt < MT; ++mt)
+#pragma unroll
+          for (int i4 = 0; i4 < 4; ++i4) {
+            const float4_t v = red[((nt * MT + mt) * 4 + i4) * 64];
+#pragma unroll
+            for (int e = 0; e < 4; ++e) acc[nt][mt][4 * i4 + e] += v[e];
+          }
+    }
+    __syncthreads();                                     // the sums are in registers: LDS is free again
+    if (grp != 0) return;
+  }
   {
     constexpr int ROWB = 64 * NTW + 16;                  // bytes per staged row (padded)
     unsigned char* stage = reinterpret_cast<unsigned char*>(xs_all) + wave * (32 * MT * ROWB);
@@ -327,24 +369,27 @@ __global__ __launch_bounds__(256, 2) void qmm_gemm_w4g64_kernel(
   }
 }
 
-template <int NTW, int MT, int SBW>
+template <int NTW, int MT, int SBW, int KGRP = 1>
 int launch_gemm(const half_t* x, const uint32_t* w, const half_t* s, const half_t* b, const half_t* bias,
                 half_t* out, int M, int N, int K, hipStream_t st) {
   constexpr int BMT = 32 * MT;
   constexpr int BN = 128 * NTW;
   static_assert(256 % BMT == 0 && BMT >= 32, "block load mapping");
-  const size_t lds_x = 2 * (size_t)BMT * XS * sizeof(half_t);
+  const size_t lds_x = KGRP * 2 * (size_t)BMT * XS * sizeof(half_t);
   const size_t lds_out = 4 * (size_t)BMT * (64 * NTW + 16);         // the output tiles of the four waves
-  const size_t lds = lds_x > lds_out ? lds_x : lds_out;
+  const size_t lds_red = KGRP > 1 ? 4 * (size_t)NTW * MT * 4 * 64 * sizeof(float4_t) : 0;
+  size_t lds = lds_x > lds_out ? lds_x : lds_out;
+  lds = lds > lds_red ? lds : lds_red;
   static bool configured = false;
   if (!configured) {
-    if (hipFuncSetAttribute(reinterpret_cast<const void*>(&qmm_gemm_w4g64_kernel<NTW, MT, SBW>),
+    if (hipFuncSetAttribute(reinterpret_cast<const void*>(&qmm_gemm_w4g64_kernel<NTW, MT, SBW, KGRP>),
                             hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds) != hipSuccess)
       return EAGLE_ERR_HIP;
     configured = true;
   }
   const dim3 grid((N + BN - 1) / BN, (M + BMT - 1) / BMT);
-  hipLaunchKernelGGL((qmm_gemm_w4g64_kernel<NTW, MT, SBW>), grid, dim3(256), lds, st, x, w, s, b, bias, out, M, N, K);
+  hipLaunchKernelGGL((qmm_gemm_w4g64_kernel<NTW, MT, SBW, KGRP>), grid, dim3(256 * KGRP), lds, st, x, w, s, b, bias,
+                     out, M, N, K);
   return eagle_launch_status();
 }
 
@@ -630,6 +675,13 @@ EAGLE_EXPORT int eagle_qmm_gemm_w4g64_f16(const void* x, const uint32_t* wq, con
     case 4: return launch_gemm<NTW, MT, 4>(xh, wq, sh, bh, bi, oh, M, N, K, st);               \
     case 2: return launch_gemm<NTW, MT, 2>(xh, wq, sh, bh, bi, oh, M, N, K, st);               \
     default: return launch_gemm<NTW, MT, 1>(xh, wq, sh, bh, bi, oh, M, N, K, st);              \
+  }
+  // two K groups per workgroup where the grid would leave a compute unit with one workgroup
+  const long wgs = small ? nb * ((M + 63) / 64) : big ? ((N + 255) / 256) * (long)((M + 127) / 128) : nb * ((M + 127) / 128);
+  const bool split_k = sbw == 8 && (K % 1024) == 0 && wgs <= GEMM_SPLIT_WGS;
+  if (split_k) {
+    if (small) return launch_gemm<1, 2, 8, 2>(xh, wq, sh, bh, bi, oh, M, N, K, st);
+    if (!big) return launch_gemm<1, 4, 8, 2>(xh, wq, sh, bh, bi, oh, M, N, K, st);
   }
   if (small) { EAGLE_GEMM_SHAPE(1, 2) }
   if (big) { EAGLE_GEMM_SHAPE(2, 4) }
