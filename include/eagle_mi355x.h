@@ -194,6 +194,13 @@ int eagle_qmm_swiglu_w4g64_f16(const void* x, const uint32_t* wq, const void* sc
 int eagle_qmm_gemm_w4g64_f16(const void* x, const uint32_t* wq, const void* scales,
                              const void* biases, const void* bias, void* out, int M, int N, int K,
                              int group_size, int bits, eagle_stream_t stream);
+/* The same with the SwiGLU epilogue of eagle_qmm_swiglu_w4g64_f16 (gate and up rows interleaved
+ * in 16-row tiles, N = 2 * intermediate size, N % 32 == 0, out [M, N / 2]): the gate|up projection
+ * of a prompt chunk without the intermediate [M, N] tensor and the eagle_silu_mul_f16 launch
+ * (mlx_llama.py:214-215). */
+int eagle_qmm_gemm_swiglu_w4g64_f16(const void* x, const uint32_t* wq, const void* scales,
+                                    const void* biases, const void* bias, void* out, int M, int N,
+                                    int K, int group_size, int bits, eagle_stream_t stream);
 
 /* The same product (and its SwiGLU form when `swiglu` != 0, weights interleaved as for
  * eagle_qmm_swiglu_w4g64_f16, out [M, N/2]) for 1..32 rows with x resident in registers: one

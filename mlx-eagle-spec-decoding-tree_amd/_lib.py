@@ -39,6 +39,7 @@ SIGNATURES = {
     "eagle_qmm_workspace_bytes_tuned": (c_size_t, [c_int] * 3),
     "eagle_qmm_w4g64_f16_tuned": (c_int, [c_void_p] * 6 + [c_int] * 8 + [c_void_p, c_size_t, c_void_p]),
     "eagle_qmm_gemm_w4g64_f16": (c_int, [c_void_p] * 6 + [c_int] * 5 + [c_void_p]),
+    "eagle_qmm_gemm_swiglu_w4g64_f16": (c_int, [c_void_p] * 6 + [c_int] * 5 + [c_void_p]),
     "eagle_qmm_res_supported": (c_int, [c_int] * 3),
     "eagle_qmm_res_w4g64_f16": (c_int, [c_void_p] * 6 + [c_int] * 6 + [c_void_p]),
     "eagle_qmm_slab_count": (c_int, [c_int] * 2),

@@ -107,7 +107,10 @@ struct StepIndex {
 // own half of K with its own x buffers (one barrier serves both) and the halves are added
 // through LDS at the end: for shapes that give a compute unit a single workgroup, whose four
 // waves would otherwise have nothing to overlap their waits with.
-template <int NTW, int MT, int SBW, int KGRP = 1>
+// SWI: the weight rows are gate and up rows interleaved in 16-row tiles (rows 0..15 of a 32-row
+// matrix tile gate, 16..31 the matching up rows: the same accumulator lane holds both); the
+// result is silu(g) * u, [M, N / 2].
+template <int NTW, int MT, int SBW, int KGRP = 1, bool SWI = false>
 __global__ __launch_bounds__(256 * KGRP, (KGRP == 1 ? 2 : 1)) void qmm_gemm_w4g64_kernel(
     const half_t* __restrict__ x, const uint32_t* __restrict__ w, const half_t* __restrict__ s,
     const half_t* __restrict__ b, const half_t* __restrict__ bias, half_t* __restrict__ out, int M,
@@ -339,7 +342,46 @@ __global__ __launch_bounds__(256 * KGRP, (KGRP == 1 ? 2 : 1)) void qmm_gemm_w4g6
     __syncthreads();                                     // the sums are in registers: LDS is free again
     if (grp != 0) return;
   }
-  {
+  if (SWI) {
+    // 16 output columns per 32-row tile: accumulator registers 0..7 are gate rows 8 (i / 4) + 4 hb +
+    // i % 4, registers 8..15 the up rows 16 further on
+    constexpr int ROWB = 32 * NTW + 16;
+    unsigned char* stage = reinterpret_cast<unsigned char*>(xs_all) + wave * (32 * MT * ROWB);
+    const int NO = N >> 1;
+#pragma unroll
+    for (int mt = 0; mt < MT; ++mt)
+#pragma unroll
+      for (int nt = 0; nt < NTW; ++nt)
+#pragma unroll
+        for (int i4 = 0; i4 < 2; ++i4) {
+          const int n = n0 + nt * 32 + 8 * i4 + 4 * hb;            // gate row; the up row is n + 16
+          half4_t o;
+#pragma unroll
+          for (int e = 0; e < 4; ++e) {
+            half_t g = (half_t)acc[nt][mt][4 * i4 + e], u = (half_t)acc[nt][mt][8 + 4 * i4 + e];
+            if (bias && n + 16 < N) {
+              g = g + bias[n + e];
+              u = u + bias[n + 16 + e];
+            }
+            const float gf = (float)g;
+            const half_t a = (half_t)(gf / (1.0f + expf(-gf)));
+            o[e] = (half_t)((float)a * (float)u);
+          }
+          *reinterpret_cast<half4_t*>(stage + (mt * 32 + ql) * ROWB + nt * 32 + i4 * 16 + hb * 8) = o;
+        }
+    __builtin_amdgcn_wave_barrier();
+    constexpr int LPR = 2 * NTW;                         // lanes per row (16 bytes each)
+    constexpr int RPI = 64 / LPR;
+    const int pr = lane / LPR, pc = lane % LPR;
+#pragma unroll
+    for (int r0 = 0; r0 < 32 * MT; r0 += RPI) {
+      const int row = r0 + pr;
+      const int m = m0 + wm * 32 * MT + row;
+      const int n = (n0 >> 1) + pc * 8;
+      const half8_t v = *reinterpret_cast<const half8_t*>(stage + row * ROWB + pc * 16);
+      if (m < M && n < NO) *reinterpret_cast<half8_t*>(out + (long)m * NO + n) = v;
+    }
+  } else {
     constexpr int ROWB = 64 * NTW + 16;                  // bytes per staged row (padded)
     unsigned char* stage = reinterpret_cast<unsigned char*>(xs_all) + wave * (32 * MT * ROWB);
 #pragma unroll
@@ -369,7 +411,7 @@ __global__ __launch_bounds__(256 * KGRP, (KGRP == 1 ? 2 : 1)) void qmm_gemm_w4g6
   }
 }
 
-template <int NTW, int MT, int SBW, int KGRP = 1>
+template <int NTW, int MT, int SBW, int KGRP = 1, bool SWI = false>
 int launch_gemm(const half_t* x, const uint32_t* w, const half_t* s, const half_t* b, const half_t* bias,
                 half_t* out, int M, int N, int K, hipStream_t st) {
   constexpr int BMT = 32 * MT;
@@ -382,14 +424,14 @@ int launch_gemm(const half_t* x, const uint32_t* w, const half_t* s, const half_
   lds = lds > lds_red ? lds : lds_red;
   static bool configured = false;
   if (!configured) {
-    if (hipFuncSetAttribute(reinterpret_cast<const void*>(&qmm_gemm_w4g64_kernel<NTW, MT, SBW, KGRP>),
+    if (hipFuncSetAttribute(reinterpret_cast<const void*>(&qmm_gemm_w4g64_kernel<NTW, MT, SBW, KGRP, SWI>),
                             hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds) != hipSuccess)
       return EAGLE_ERR_HIP;
     configured = true;
   }
   const dim3 grid((N + BN - 1) / BN, (M + BMT - 1) / BMT);
-  hipLaunchKernelGGL((qmm_gemm_w4g64_kernel<NTW, MT, SBW, KGRP>), grid, dim3(256 * KGRP), lds, st, x, w, s, b, bias,
-                     out, M, N, K);
+  hipLaunchKernelGGL((qmm_gemm_w4g64_kernel<NTW, MT, SBW, KGRP, SWI>), grid, dim3(256 * KGRP), lds, st, x, w, s, b,
+                     bias, out, M, N, K);
   return eagle_launch_status();
 }
 
@@ -636,12 +678,13 @@ EAGLE_EXPORT int eagle_slab_sum_f16(const float* partial, int slabs, const void*
   return eagle_launch_status();
 }
 
-EAGLE_EXPORT int eagle_qmm_gemm_w4g64_f16(const void* x, const uint32_t* wq, const void* scales,
-                                          const void* biases, const void* bias, void* out, int M, int N,
-                                          int K, int group_size, int bits, eagle_stream_t stream) {
+static int gemm_dispatch(const void* x, const uint32_t* wq, const void* scales, const void* biases,
+                         const void* bias, void* out, int M, int N, int K, int group_size, int bits,
+                         bool swiglu, eagle_stream_t stream) {
   if (!x || !wq || !scales || !biases || !out) return EAGLE_ERR_NULL;
   if (group_size != 64 || bits != 4) return EAGLE_ERR_UNSUPPORTED;
   if (M < 1 || N < 8 || (N % 8) != 0 || K < 64 || (K % 64) != 0) return EAGLE_ERR_SHAPE;
+  if (swiglu && (N % 32) != 0) return EAGLE_ERR_SHAPE;
   if (!eagle_aligned16(x) || !eagle_aligned16(wq) || !eagle_aligned16(out) ||
       (bias && (reinterpret_cast<uintptr_t>(bias) & 7u)))
     return EAGLE_ERR_ALIGN;
@@ -678,6 +721,16 @@ EAGLE_EXPORT int eagle_qmm_gemm_w4g64_f16(const void* x, const uint32_t* wq, con
   }
   // two K groups per workgroup where the grid would leave a compute unit with one workgroup
   const long wgs = small ? nb * ((M + 63) / 64) : big ? ((N + 255) / 256) * (long)((M + 127) / 128) : nb * ((M + 127) / 128);
+  if (swiglu) {
+    // the wide gate|up matrix: the 128 x 256 block where it pays, else 128 x 128
+    switch (sbw) {
+      case 8: return big ? launch_gemm<2, 4, 8, 1, true>(xh, wq, sh, bh, bi, oh, M, N, K, st)
+                         : launch_gemm<1, 4, 8, 1, true>(xh, wq, sh, bh, bi, oh, M, N, K, st);
+      case 4: return launch_gemm<1, 4, 4, 1, true>(xh, wq, sh, bh, bi, oh, M, N, K, st);
+      case 2: return launch_gemm<1, 4, 2, 1, true>(xh, wq, sh, bh, bi, oh, M, N, K, st);
+      default: return launch_gemm<1, 4, 1, 1, true>(xh, wq, sh, bh, bi, oh, M, N, K, st);
+    }
+  }
   const bool split_k = sbw == 8 && (K % 1024) == 0 && wgs <= GEMM_SPLIT_WGS;
   if (split_k) {
     if (small) return launch_gemm<1, 2, 8, 2>(xh, wq, sh, bh, bi, oh, M, N, K, st);
@@ -687,4 +740,17 @@ EAGLE_EXPORT int eagle_qmm_gemm_w4g64_f16(const void* x, const uint32_t* wq, con
   if (big) { EAGLE_GEMM_SHAPE(2, 4) }
   EAGLE_GEMM_SHAPE(1, 4)
 #undef EAGLE_GEMM_SHAPE
+}
+
+EAGLE_EXPORT int eagle_qmm_gemm_w4g64_f16(const void* x, const uint32_t* wq, const void* scales,
+                                          const void* biases, const void* bias, void* out, int M, int N,
+                                          int K, int group_size, int bits, eagle_stream_t stream) {
+  return gemm_dispatch(x, wq, scales, biases, bias, out, M, N, K, group_size, bits, false, stream);
+}
+
+EAGLE_EXPORT int eagle_qmm_gemm_swiglu_w4g64_f16(const void* x, const uint32_t* wq, const void* scales,
+                                                 const void* biases, const void* bias, void* out, int M,
+                                                 int N, int K, int group_size, int bits,
+                                                 eagle_stream_t stream) {
+  return gemm_dispatch(x, wq, scales, biases, bias, out, M, N, K, group_size, bits, true, stream);
 }

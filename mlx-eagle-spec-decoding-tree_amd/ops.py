@@ -193,13 +193,14 @@ def interleave_gate_up(gate, up):
 
 def swiglu_supported(M, I, K):
     """True when the SwiGLU matmul covers this shape (whole (gate, up) tile pairs)."""
-    return I % 16 == 0 and 1 <= M <= 32 and K % 64 == 0
+    return I % 16 == 0 and M >= 1 and K % 64 == 0
 
 
 def quantized_matmul_swiglu(x, w_q, scales, biases, bias=None, out=None):
     """silu(x @ Wg.T) * (x @ Wu.T) (mlx_llama.py:214-215) in one launch: w_q / scales / biases
     / bias hold the gate and up projections interleaved by `interleave_gate_up`.  The result
-    equals `silu_mul(quantized_matmul(x, gate...), quantized_matmul(x, up...))` bit for bit."""
+    equals `silu_mul(quantized_matmul(x, gate...), quantized_matmul(x, up...))` bit for bit.
+    Above 32 rows the tiled GEMM form runs with the same epilogue."""
     _need_cuda(x, w_q, scales, biases, bias)
     x = _f16(x, "x")
     w_q = as_packed_u32(w_q)
@@ -217,6 +218,12 @@ def quantized_matmul_swiglu(x, w_q, scales, biases, bias=None, out=None):
     if out is None:
         out = torch.empty((*lead, N // 2), dtype=torch.float16, device=x.device)
     L = _lib.lib()
+    if M > 32:
+        # many rows (a prompt chunk): the tiled GEMM with the same epilogue
+        rc = L.eagle_qmm_gemm_swiglu_w4g64_f16(_ptr(x), _ptr(w_q), _ptr(scales), _ptr(biases), _ptr(bias),
+                                               _ptr(out), M, N, K, 64, 4, _stream())
+        _lib.check(rc, "quantized_matmul_swiglu")
+        return out
     ws = workspace("qmm", L.eagle_qmm_workspace_bytes(M, N, K), x.device)
     rc = L.eagle_qmm_swiglu_w4g64_f16(_ptr(x), _ptr(w_q), _ptr(scales), _ptr(biases), _ptr(bias),
                                       _ptr(out), M, N, K, 64, 4, _ptr(ws), ws.numel(), _stream())

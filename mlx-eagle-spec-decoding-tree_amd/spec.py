@@ -149,9 +149,10 @@ class ChunkPass:
         D, I = args.hidden_size, args.intermediate_size
         H, G, hd = args.num_attention_heads, args.num_key_value_heads, args.head_dim
         self.max_len = max_len or cache[0].capacity
-        self.qkv_w, self.gu_w = fuse_projections(model, False)
         self.T = R
-        self.swiglu = False                                   # above 32 rows: the tiled GEMM form everywhere
+        # above 32 rows: the tiled GEMM form everywhere, gate|up with the SwiGLU epilogue
+        self.swiglu = bool(ops.swiglu_supported(R, args.intermediate_size, args.hidden_size))
+        self.qkv_w, self.gu_w = fuse_projections(model, self.swiglu)
         self.slab = {"qkv": 0, "o": 0, "down": 0}
         f16 = dict(dtype=torch.float16, device=dev)
         i32 = dict(dtype=torch.int32, device=dev)

@@ -5,7 +5,7 @@ import torch
 
 from mlx_eagle_spec_decoding_tree_amd import ops, synth
 from oracle import oracle
-from util import TOL, layer_to_dev, rel_err, to_dev
+from util import TOL, close_fp16, layer_to_dev, rel_err, to_dev
 
 pytestmark = pytest.mark.gpu
 
@@ -74,3 +74,43 @@ def test_gemm_form_random_shapes(dev):
         assert np.isnan(got[M].astype(np.float32)).all(), case          # nothing written past the rows
         assert np.isfinite(got[:M].astype(np.float32)).all(), case
         assert rel_err(got[:M], want) <= TOL, case
+
+
+@pytest.mark.parametrize("M,I,K,bias", [(33, 16, 64, True), (64, 48, 128, False), (100, 272, 256, True),
+                                        (512, 2432, 896, False), (300, 1024, 1024, True), (129, 14336, 4096, False)])
+def test_gemm_form_with_swiglu(dev, M, I, K, bias):
+    """gate|up of a prompt chunk with the activation in the GEMM's epilogue (tile-interleaved rows):
+    equal, bit for bit, to the GEMM over the concatenated rows followed by silu_mul wherever both
+    pick the same block shape, within tolerance of the oracle's qmm -> silu_mul always."""
+    print(f"gemm swiglu M={M} I={I} K={K}", flush=True)
+    rng = np.random.default_rng(M + I + K)
+    g = synth.make_qlinear(rng, I, K, bias=bias, gain=1.0)
+    u = synth.make_qlinear(rng, I, K, bias=bias, gain=1.0)
+    x = synth.make_x(rng, M, K)
+    rows = rng.choice(M, size=min(M, 40), replace=False)             # the oracle on a sample of the rows
+    og = oracle.qmm(x[rows], g["weight"], g["scales"], g["biases"], g.get("bias"))
+    ou = oracle.qmm(x[rows], u["weight"], u["scales"], u["biases"], u.get("bias"))
+    want = oracle.silu_mul(og, ou)
+    gd, ud = layer_to_dev(g, dev), layer_to_dev(u, dev)
+    keys = ["weight", "scales", "biases"] + (["bias"] if bias else [])
+    inter = {k: ops.interleave_gate_up(gd[k], ud[k]) for k in keys}
+    cat = {k: torch.cat([gd[k], ud[k]]).contiguous() for k in keys}
+    xd = to_dev(x, dev)
+    got = ops.quantized_matmul_swiglu(xd, inter["weight"], inter["scales"], inter["biases"], bias=inter.get("bias"))
+    two = ops.silu_mul(ops.quantized_matmul(xd, cat["weight"], cat["scales"], cat["biases"], bias=cat.get("bias")))
+    torch.cuda.synchronize()
+    assert tuple(got.shape) == (M, I)
+    # Against the oracle: each projection is within TOL of its own RMS (the bound of the plain form);
+    # through silu(g) * u an error dg moves the result by u silu'(g) dg (|silu'| <= 1.1) and du by
+    # silu(g) du, plus the two fp16 roundings of the epilogue.  The RMS error stays a fraction of TOL.
+    g64, u64 = og.astype(np.float64), ou.astype(np.float64)
+    rms_g, rms_u = np.sqrt(np.mean(g64 * g64)), np.sqrt(np.mean(u64 * u64))
+    w64, got64 = want.astype(np.float64), got.cpu().numpy()[rows].astype(np.float64)
+    ulp = 2.0 ** (np.floor(np.log2(np.maximum(np.abs(w64), 2.0 ** -14))) - 10)
+    bound = TOL * (1.1 * np.abs(u64) * rms_g + np.abs(g64 / (1 + np.exp(-g64))) * rms_u) + 2 * ulp
+    assert np.all(np.abs(got64 - w64) <= bound)
+    assert np.sqrt(np.mean((got64 - w64) ** 2)) <= 0.25 * TOL * np.sqrt(np.mean(w64 * w64))
+    # against the plain form followed by silu_mul (same roundings, possibly another block shape)
+    close_fp16(got.cpu().numpy(), two.cpu().numpy(), "two launches")
+    with pytest.raises(Exception):
+        ops.quantized_matmul_swiglu(xd, inter["weight"][:24], inter["scales"][:24], inter["biases"][:24])

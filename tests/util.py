@@ -28,3 +28,15 @@ def rel_err(got, want):
 
 def layer_to_dev(layer, dev):
     return {k: to_dev(v, dev) for k, v in layer.items()}
+
+
+def close_fp16(got, want, what="", rms_frac=0.1):
+    """Bound for fp16 results that are themselves products of rounded fp16 values (SwiGLU): every
+    element within TOL * RMS + 2 ulp of its own size (a rounding flip of an intermediate moves a
+    large element by an ulp or two), and the RMS error within rms_frac * TOL * RMS."""
+    g64, w64 = np.asarray(got, np.float64), np.asarray(want, np.float64)
+    assert np.isfinite(g64).all(), what
+    rms = np.sqrt(np.mean(w64 * w64))
+    ulp = 2.0 ** (np.floor(np.log2(np.maximum(np.abs(w64), 2.0 ** -14))) - 10)
+    assert np.all(np.abs(g64 - w64) <= TOL * rms + 2 * ulp), what
+    assert np.sqrt(np.mean((g64 - w64) ** 2)) <= rms_frac * TOL * rms, what
