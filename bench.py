@@ -150,6 +150,7 @@ def graph_time_ms(torch, fn, reps, warm=2):
 
 
 def main():
+    global NODES
     ap = argparse.ArgumentParser()
     ap.add_argument("--gpus", type=int, default=1)
     ap.add_argument("--steps", type=int, default=50)
@@ -189,6 +190,12 @@ def main():
     ap.add_argument("--cpu-qmm", action="store_true",
                     help="time the CPU restatement of single quantised matmuls on the host cores (cfg1 and the "
                          "7B projection shapes; one JSON line); no GPU work")
+    ap.add_argument("--tree-tokens", type=int, default=NODES,
+                    help="tree tokens of the verification step (root included; the headline is quoted on 32, "
+                         "the reference's default tree has 40)")
+    ap.add_argument("--depth", type=int, default=3, help="--loop: levels of the draft tree")
+    ap.add_argument("--draft-nodes", type=int, default=31,
+                    help="--loop: draft nodes verified per step (the reference's default is 39 at depth 5)")
     ap.add_argument("--self-draft", action="store_true",
                     help="with --loop: the target drafts for itself (high acceptance; exercises the "
                          "accept path at full size)")
@@ -198,6 +205,7 @@ def main():
         sys.exit(2)
     if opt.traffic_from:
         return write_traffic_record(*opt.traffic_from)
+    NODES = opt.tree_tokens
     if opt.loop:
         if opt.steps == 50:
             opt.steps = 300
@@ -321,7 +329,9 @@ def main():
     kv_bytes = 2 * L * G * (PREFIX + NODES) * hd * 2
     achieved = alg / (qmm_ms * 1e-3) / 1e9
     traffic, traffic_source = read_traffic_record()
-    kernels = "qmm_w4g64_kernel + qmm_slab_w4g64_kernel" + (" + norm_mlp_in_kernel" if ver.chain else "")
+    stream_kernel = "qmm_w4g64_kernel"          # (above 32 tree tokens: two launches of it per product)
+    kernels = (stream_kernel if ver.wide else stream_kernel + " + qmm_slab_w4g64_kernel") \
+        + (" + norm_mlp_in_kernel" if ver.chain else "")
     roofline = {"bound": "hbm", "kernel": kernels, "achieved": round(achieved, 1),
                 "peak": HBM_PEAK_GBS, "unit": "GB/s", "frac": round(achieved / HBM_PEAK_GBS, 4),
                 "traffic": traffic, "traffic_source": traffic_source, "launches_per_step": n_launch,
@@ -331,7 +341,7 @@ def main():
 
     # the same for each kernel on its own launches
     per_kernel = {}
-    for kname, sub in (("qmm_w4g64_kernel", [l for l in launches if l[6] is True or not l[6]]),
+    for kname, sub in ((stream_kernel, [l for l in launches if l[6] is True or not l[6]]),
                        ("qmm_slab_w4g64_kernel", [l for l in launches if l[6] and l[6] is not True and l[6] != "chain"]),
                        ("norm_mlp_in_kernel", [l for l in launches if l[6] == "chain"])):
         if not sub:
@@ -414,7 +424,7 @@ def main():
             "steps": opt.steps, "warmup": opt.warmup, "ms_per_step": round(ms_per_step, 4),
             "higher_is_better": False, "scaling": "weak", "vs_baseline": None, "dtype": "f16",
             "data": "synthetic",
-            "config": {"workload": "qwen2.5-7b-shape 4-bit g64 target, 28 layers, 32 tree nodes, "
+            "config": {"workload": f"qwen2.5-7b-shape 4-bit g64 target, 28 layers, {NODES} tree nodes, "
                                    "2048-token fp16 KV prefix, greedy accept + KV compaction, HIP-graph replay",
                        "nodes": NODES, "prefix": PREFIX, "wall_ms_per_step": round(wall_ms, 4),
                        "accept_length": int(result[1]),
@@ -429,6 +439,7 @@ def main():
         torch.cuda.empty_cache()
         extra = argparse.Namespace(**vars(opt))
         extra.steps, extra.warmup, extra.self_draft = 50, 3, False
+        extra.depth, extra.draft_nodes = 3, 31
         lp = loop_bench(extra)
         line["loop"] = {k: lp[k] for k in ("metric", "value", "unit", "steps", "ms_per_step", "tokens_per_step",
                                            "prefill_ms", "parity")}
@@ -640,7 +651,7 @@ def loop_bench(opt):
     dev = torch.device("cuda:0")
     _lib.check(_lib.lib().eagle_check_device(), "device check")
     steps = opt.steps
-    k, depth, nodes, prompt_len = 8, 3, 31, 512
+    k, depth, nodes, prompt_len = 8, opt.depth, opt.draft_nodes, 512
     targs = synth.llama3_8b()
     t0 = time.time()
     target = llama.Model.from_numpy(targs, synth.make_model_weights(targs, seed=opt.seed), dev)
@@ -704,8 +715,8 @@ def loop_bench(opt):
         "scaling": "weak", "vs_baseline": None, "dtype": "f16", "data": "synthetic",
         "config": {"workload": ("tree loop: " + ("target drafts for itself" if opt.self_draft else
                                                  "Qwen2.5-0.5B-shaped 4-bit drafter")
-                                + ", Llama-3-8B-shaped 4-bit target, 512-token prompt, k 8, depth 3, "
-                                  "31 draft nodes"),
+                                + f", Llama-3-8B-shaped 4-bit target, 512-token prompt, k 8, depth {depth}, "
+                                  f"{nodes} draft nodes"),
                    "prompt_len": prompt_len, "k": k, "depth": depth, "verify_num_tokens": nodes},
         "tokens": n, "tokens_per_step": round(n / steps, 4), "prefill_ms": round(prefill_ms, 1),
         "gpu_ms_total": round(gpu_ms, 2), "wall_ms_total": round(wall_ms, 2),

@@ -366,6 +366,19 @@ int eagle_draft_attention_f16(const void* q, const void* k_cache, const void* v_
                               float scale, void* workspace, size_t workspace_bytes,
                               eagle_stream_t stream);
 
+/* eagle_draft_attention_f16 for up to EAGLE_MAX_TREE_SLOTS query tokens, as the verification
+ * forward (mlx_eagle.py:329-346 through mlx_llama.py:185-192) of a tree above 32 tokens needs
+ * (the reference's default is 39 draft nodes, mlx_eagle.py:390,510; there Tk = T): T queries
+ * against the P = *cache_len_dev prefix rows and the Tk <= 64 rows P .. P+Tk-1, of which query t
+ * sees row j iff bit (j % 32) of mask_words[2*t + j/32] is set.  One launch pair: the queries go
+ * in pieces of 32 rows over the same keys.  q [H,T,hd], out [T, H*hd]. */
+size_t eagle_tree_attention_wide_workspace_bytes(int T, int H, int hd, int max_len);
+int eagle_tree_attention_wide_f16(const void* q, const void* k_cache, const void* v_cache,
+                                  const uint32_t* mask_words, const int32_t* cache_len_dev, void* out,
+                                  int T, int Tk, int H, int G, int hd, long capacity, int max_len,
+                                  float scale, void* workspace, size_t workspace_bytes,
+                                  eagle_stream_t stream);
+
 /* Causal attention of a prompt chunk (mlx_llama.py:185-192 with the causal mask of
  * mlx_llama.py:275-276; mlx_eagle.py:522-533): R query rows (a multiple of 32, at most
  * EAGLE_MAX_CHUNK) in pieces of 32.  Piece j has its rows at cache rows piece_len_dev[j] ..

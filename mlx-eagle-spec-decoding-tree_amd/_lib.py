@@ -61,6 +61,9 @@ SIGNATURES = {
                                                                        c_void_p, c_size_t, c_void_p]),
     "eagle_draft_attention_f16": (c_int, [c_void_p] * 6 + [c_int] * 5 + [c_long, c_int, c_float,
                                                                         c_void_p, c_size_t, c_void_p]),
+    "eagle_tree_attention_wide_workspace_bytes": (c_size_t, [c_int] * 4),
+    "eagle_tree_attention_wide_f16": (c_int, [c_void_p] * 6 + [c_int] * 5 + [c_long, c_int, c_float,
+                                                                            c_void_p, c_size_t, c_void_p]),
     "eagle_logsoftmax_topk_workspace_bytes": (c_size_t, [c_int, c_long]),
     "eagle_logsoftmax_topk_f16": (c_int, [c_void_p] * 2 + [c_int, c_long, c_int, c_int]
                                   + [c_void_p] * 3 + [c_size_t, c_void_p]),

@@ -65,7 +65,8 @@ __global__ __launch_bounds__(512) void tree_attn_split_kernel(
     const uint32_t* __restrict__ mask_bits, const int32_t* __restrict__ len_dev,
     half_t* __restrict__ part_o, float* __restrict__ part_ml, int T, int H, int G, long cap,
     int tiles_per_split, float scale_log2e, const half_t* __restrict__ k_lin,
-    const half_t* __restrict__ v_lin, long ld, const float* __restrict__ rope_cs, int Tk, int q_rows) {
+    const half_t* __restrict__ v_lin, long ld, const float* __restrict__ rope_cs, int Tk, int q_rows,
+    int len_stride) {
   constexpr int KSTEPS = HD / 16;       // MFMA steps over the head dimension for S
   constexpr int DB = HD / 32;           // 32-wide blocks of the head dimension for O
   constexpr int STR = HD * 2 + 16;      // LDS row stride in bytes (pad: conflict-free reads)
@@ -88,10 +89,14 @@ __global__ __launch_bounds__(512) void tree_attn_split_kernel(
   const int hb = lane >> 5;             // which half of the k / key index this lane holds
   const int head = g * rep + wave;
 
-  // blockIdx.z: piece of a causal pass (32 query rows each, its own cache length, queries at
-  // rows 32 * piece of q [H, q_rows, hd]); a single piece otherwise
+  // blockIdx.z: piece of 32 query rows, queries at rows 32 * piece of q [H, q_rows, hd] (the last
+  // piece may hold fewer).  The pieces of a causal pass have a cache length each (len_stride 1),
+  // those of a tree of more than 32 tokens share one length and the masked rows (len_stride 0,
+  // mask words of query row 32 * piece + ql); a single piece otherwise.
   const int piece = blockIdx.z;
-  int P = len_dev[piece];
+  const int qrow = piece * 32 + (lane & 31);
+  if (!ROPE && T > q_rows - piece * 32) T = q_rows - piece * 32;
+  int P = len_dev[piece * len_stride];
   // never index past the cache, whatever the counter says (a graph replayed beyond the
   // capacity would otherwise read beyond the last head's buffer)
   if (P > cap - Tk) P = (int)(cap - Tk);
@@ -110,14 +115,14 @@ __global__ __launch_bounds__(512) void tree_attn_split_kernel(
     qreg[kk] = half8_t{0, 0, 0, 0, 0, 0, 0, 0};
     if (ql < T) {
       const half_t* qp = ROPE ? q + (long)ql * ld + (long)head * HD
-                              : q + ((long)head * q_rows + piece * 32 + ql) * HD;
+                              : q + ((long)head * q_rows + qrow) * HD;
       qreg[kk] = *reinterpret_cast<const half8_t*>(qp + kk * 16 + hb * 8);
     }
   }
   // WIDE: two mask words per query (masked key rows 0..31 and 32..63)
   // no mask array: causal among the T rows
-  const uint32_t mybits = ql < T ? (mask_bits ? mask_bits[WIDE ? 2 * ql : ql] : (2u << ql) - 1u) : 0u;
-  const uint32_t mybits_hi = (WIDE && ql < T && mask_bits) ? mask_bits[2 * ql + 1] : 0u;
+  const uint32_t mybits = ql < T ? (mask_bits ? mask_bits[WIDE ? 2 * qrow : ql] : (2u << ql) - 1u) : 0u;
+  const uint32_t mybits_hi = (WIDE && ql < T && mask_bits) ? mask_bits[2 * qrow + 1] : 0u;
 
   float m_run = -INFINITY, l_run = 0.f;
   float16_t o_acc[DB];
@@ -326,8 +331,9 @@ __global__ void tree_attn_merge_kernel(const half_t* __restrict__ part_o,
                                        const float* __restrict__ part_ml,
                                        half_t* __restrict__ out, int T, int H, int nsplit,
                                        const int32_t* __restrict__ len_dev, long cap,
-                                       int Tk) {
+                                       int Tk, int q_rows, int len_stride) {
   const int piece = blockIdx.z;                     // as in the split kernel
+  if (T > q_rows - piece * 32) T = q_rows - piece * 32;
   part_o += (long)piece * H * nsplit * 32 * HD;
   part_ml += (long)piece * H * nsplit * 32 * 2;
   out += (long)piece * 32 * H * HD;
@@ -360,7 +366,7 @@ __global__ void tree_attn_merge_kernel(const half_t* __restrict__ part_o,
   for (int k = 0; k < PRE; ++k)
     if (k < nsplit) pre[k] = *reinterpret_cast<const half4_t*>(src + (long)k * 32 * HD);
 
-  int P = len_dev[piece];
+  int P = len_dev[piece * len_stride];
   if (P > cap - Tk) P = (int)(cap - Tk);    // as in the split kernel
   if (P < 0) P = 0;
   const int nact = active_splits((P + Tk + KT - 1) / KT, nsplit);   // as in the split kernel
@@ -417,9 +423,9 @@ template <int HD, bool ROPE, bool WIDE = false>
 int launch_attention(const half_t* q, half_t* kc, half_t* vc, const uint32_t* bits, const int32_t* len,
                      void* out, int T, int H, int G, long cap, int max_len, float scale, void* workspace,
                      const half_t* k_lin, const half_t* v_lin, long ld, const float* cs, hipStream_t st,
-                     int Tk = 0, int pieces = 1) {
+                     int Tk = 0, int pieces = 1, int q_rows = 0, int len_stride = 1) {
   if (!WIDE) Tk = T;
-  const int q_rows = pieces * T;
+  if (q_rows == 0) q_rows = pieces * T;
   const int nsplit = splits_for(max_len, G);
   float* part_ml = static_cast<float*>(workspace);
   half_t* part_o = reinterpret_cast<half_t*>(part_ml + (size_t)pieces * H * nsplit * 32 * 2);
@@ -428,10 +434,10 @@ int launch_attention(const half_t* q, half_t* kc, half_t* vc, const uint32_t* bi
   const size_t lds = 2 * KT * (HD * 2 + 16) + (ROPE ? (size_t)EAGLE_MAX_TREE * HD * 4 : 0);
   hipLaunchKernelGGL((tree_attn_split_kernel<HD, ROPE, WIDE>), dim3(G, nsplit, pieces), dim3(rep * 64), lds,
                      st, q, kc, vc, bits, len, part_o, part_ml, T, H, G, cap, 0, sl2, k_lin, v_lin, ld, cs, Tk,
-                     q_rows);
+                     q_rows, len_stride);
   hipLaunchKernelGGL(tree_attn_merge_kernel<HD>, dim3(H, (T + MERGE_TOK - 1) / MERGE_TOK, pieces),
                      dim3(MERGE_TOK * HD / 4), 0, st, part_o, part_ml, (half_t*)out, T, H, nsplit,
-                     len, cap, Tk);
+                     len, cap, Tk, q_rows, len_stride);
   return eagle_launch_status();
 }
 
@@ -509,6 +515,41 @@ EAGLE_EXPORT int eagle_draft_attention_f16(const void* q, const void* k_cache, c
   return launch_attention<64, false, true>((const half_t*)q, kc, vc, mask_words, cache_len_dev, out, T, H,
                                            G, capacity, max_len, scale, workspace, nullptr, nullptr, 0,
                                            nullptr, st, Tk);
+}
+
+EAGLE_EXPORT size_t eagle_tree_attention_wide_workspace_bytes(int T, int H, int hd, int max_len) {
+  if (T < 1 || T > EAGLE_MAX_TREE_SLOTS) return 0;
+  return (size_t)((T + 31) / 32) * eagle_tree_attention_workspace_bytes(H, hd, max_len);
+}
+
+EAGLE_EXPORT int eagle_tree_attention_wide_f16(const void* q, const void* k_cache, const void* v_cache,
+                                               const uint32_t* mask_words, const int32_t* cache_len_dev,
+                                               void* out, int T, int Tk, int H, int G, int hd,
+                                               long capacity, int max_len, float scale, void* workspace,
+                                               size_t workspace_bytes, eagle_stream_t stream) {
+  if (!q || !k_cache || !v_cache || !mask_words || !cache_len_dev || !out) return EAGLE_ERR_NULL;
+  if (T < 1 || T > EAGLE_MAX_TREE_SLOTS || Tk < 1 || Tk > EAGLE_MAX_TREE_SLOTS || H < 1 || G < 1 ||
+      (H % G) != 0 || (H / G) > 8 || (hd != 64 && hd != 128) || max_len < Tk || max_len > capacity)
+    return EAGLE_ERR_SHAPE;
+  if (!eagle_aligned16(q) || !eagle_aligned16(k_cache) || !eagle_aligned16(v_cache) ||
+      !eagle_aligned16(out))
+    return EAGLE_ERR_ALIGN;
+  if (!workspace || !eagle_aligned16(workspace) ||
+      workspace_bytes < eagle_tree_attention_wide_workspace_bytes(T, H, hd, max_len))
+    return EAGLE_ERR_WORKSPACE;
+  hipStream_t st = static_cast<hipStream_t>(stream);
+  half_t* kc = const_cast<half_t*>(static_cast<const half_t*>(k_cache));
+  half_t* vc = const_cast<half_t*>(static_cast<const half_t*>(v_cache));
+  // pieces of 32 query rows over the same Tk masked rows and one cache length
+  const int pieces = (T + 31) / 32;
+  const int rows = T < 32 ? T : 32;
+  if (hd == 128)
+    return launch_attention<128, false, true>((const half_t*)q, kc, vc, mask_words, cache_len_dev, out, rows,
+                                              H, G, capacity, max_len, scale, workspace, nullptr, nullptr,
+                                              0, nullptr, st, Tk, pieces, T, 0);
+  return launch_attention<64, false, true>((const half_t*)q, kc, vc, mask_words, cache_len_dev, out, rows, H,
+                                           G, capacity, max_len, scale, workspace, nullptr, nullptr, 0,
+                                           nullptr, st, Tk, pieces, T, 0);
 }
 
 EAGLE_EXPORT size_t eagle_causal_attention_workspace_bytes(int R, int H, int hd, int max_len) {

@@ -406,6 +406,8 @@ def slab_plan(model, T, forced=None, fused=True, rope_launch=True):
     H, G, hd = args.num_attention_heads, args.num_key_value_heads, args.head_dim
     layer = model.model.layers[0]
     shapes = {"qkv": ((H + 2 * G) * hd, D), "o": (D, H * hd), "down": (D, I)}
+    if T > MAXT:      # the slab kernel holds 32 rows
+        return {name: 0 for name in shapes}
     plan = {}
     for name, (n, k) in shapes.items():
         s = ops.slab_steps(T, n, k) if forced is None else int(forced.get(name, 0))
@@ -479,12 +481,18 @@ class TreeVerifier:
         those of the default form."""
         args = model.args
         self.model, self.cache, self.args = model, cache, args
-        if total_tokens + 1 > MAXT:
-            raise NotImplementedError(f"the fused verification step takes at most {MAXT} tree tokens "
-                                      f"(total_tokens <= {MAXT - 1}); larger trees run on the module path "
-                                      "(`tree_decoding`)")
+        if total_tokens + 1 > TREE_SLOTS:
+            raise NotImplementedError(f"the verification step takes at most {TREE_SLOTS} tree tokens "
+                                      f"(total_tokens <= {TREE_SLOTS - 1})")
         self.V = total_tokens
         self.T = T = total_tokens + 1
+        # above 32 tree tokens: the matmuls in two passes of the 32-row streaming kernel, two mask
+        # words per token and attention in pieces of 32 query rows (one launch pair); the slab,
+        # resident and chained forms hold 32 rows and do not apply
+        self.wide = T > MAXT
+        if self.wide and (not fuse or one_launch_attention or chain or resident_gate_up):
+            raise ValueError(f"a tree of more than {MAXT} tokens runs with the fused projections and "
+                             "none of the 32-row options")
         dev = model.device
         self.dev = dev
         D, I = args.hidden_size, args.intermediate_size
@@ -518,7 +526,7 @@ class TreeVerifier:
         self.tokens = torch.zeros(T, **i32)
         self.tree_position_ids = torch.zeros(T, **i32)
         self.mask_index = torch.zeros(total_tokens, **i32)
-        self.mask_bits = torch.zeros(T, **i32)
+        self.mask_bits = torch.zeros((T, 2) if self.wide else T, **i32)
         self.positions = torch.zeros(T, **i32)
         self.retrieve = torch.zeros((TREE_SLOTS, TREE_SLOTS), **i32)
         self.shape = torch.zeros(2, **i32)
@@ -556,11 +564,13 @@ class TreeVerifier:
         # size every workspace before any capture
         L = _lib.lib()
         head = model.lm_head if not args.tie_word_embeddings else model.model.embed_tokens
-        need = max(L.eagle_qmm_workspace_bytes(T, n, k) for n, k in
+        # (a tree above 32 tokens goes through the 32-row matmul kernel in two passes)
+        need = max(L.eagle_qmm_workspace_bytes(rows, n, k) for n, k in
                    ((H * hd, D), (G * hd, D), ((H + 2 * G) * hd, D), (D, H * hd), (I, D), (2 * I, D),
-                    (D, I), (head.weight.shape[0], D)))
+                    (D, I), (head.weight.shape[0], D))
+                   for rows in ((T,) if not self.wide else (MAXT, T - MAXT)))
         ops.workspace("qmm", need, dev)
-        ops.workspace("attn", L.eagle_tree_attention_workspace_bytes(H, hd, self.max_len), dev)
+        ops.workspace("attn", L.eagle_tree_attention_wide_workspace_bytes(T, H, hd, self.max_len), dev)
         ops.workspace("attn_rope", L.eagle_tree_attention_rope_workspace_bytes(H, hd, self.max_len), dev)
         ops.workspace("argmax", L.eagle_argmax_workspace_bytes(T, args.vocab_size), dev)
 
@@ -614,7 +624,7 @@ class TreeVerifier:
         self.tokens.copy_(tokens.reshape(-1))
         self.tree_position_ids.copy_(tree_position_ids.reshape(-1))
         self.mask_index.copy_(mask_index.reshape(-1))
-        self.mask_bits.copy_(mask_bits.reshape(-1))
+        self.mask_bits.copy_(mask_bits.reshape(self.mask_bits.shape))
 
     def forward(self, tap=None):
         """Enqueue the whole step on the current stream (no synchronisation).  tap(i, h):

@@ -53,6 +53,9 @@ def workspace(tag, nbytes, device):
     return buf
 
 
+ROW_PASS = 32        # rows of x the streaming kernel takes per launch
+
+
 def as_packed_u32(w_q):
     """MLX packs into uint32; torch has weak uint32 support, so int32 storage of
     the same bits is accepted too."""
@@ -62,12 +65,15 @@ def as_packed_u32(w_q):
 
 
 def quantized_matmul(x, w_q, scales, biases, transpose=True, group_size=64, bits=4, bias=None,
-                     out=None, tuned=None):
+                     out=None, tuned=None, gemm=None):
     """`mx.quantized_matmul(x, w, scales, biases, transpose=True, group_size=64, bits=4)`
     (any leading dims, flattened as qmm_kernel.py:99-100,136): the streaming kernel for 1..32
-    rows of x, a tiled GEMM above that.
+    rows of x, two passes of it for 33..64 rows (a tree above 32 tokens; faster there than the
+    GEMM's few long-running workgroups: 21 against 31 us for 40 x 4608 x 3584, 44 against 185 us
+    for 40 x 3584 x 18944), a tiled GEMM above that.
     `bias` ([N] fp16) is added after rounding, as the patched linear layer does
-    (mlx_model_fwd_bench.py:70-71).  `tuned` forces a launch shape of the streaming kernel."""
+    (mlx_model_fwd_bench.py:70-71).  `tuned` forces a launch shape of the streaming kernel,
+    `gemm=True` the tiled GEMM whatever the row count."""
     if not transpose:
         raise ValueError("only transpose=True (x @ dequant(w).T) is implemented")
     _need_cuda(x, w_q, scales, biases, bias)
@@ -87,10 +93,16 @@ def quantized_matmul(x, w_q, scales, biases, transpose=True, group_size=64, bits
     if out is None:
         out = torch.empty((*lead, N), dtype=torch.float16, device=x.device)
     L = _lib.lib()
-    if M > 32:
+    if M > 32 and tuned is not None:
+        raise ValueError("launch shapes can be forced for at most 32 rows")
+    if ROW_PASS < M <= 2 * ROW_PASS and not gemm:
+        x2, out2 = x.reshape(M, K), out.view(M, N)
+        for r0 in range(0, M, ROW_PASS):
+            quantized_matmul(x2[r0:r0 + ROW_PASS], w_q, scales, biases, group_size=group_size, bits=bits,
+                             bias=bias, out=out2[r0:r0 + ROW_PASS])
+        return out
+    if M > 32 or gemm:
         # many rows (the prompt pass): the tiled GEMM form
-        if tuned is not None:
-            raise ValueError("launch shapes can be forced for at most 32 rows")
         rc = L.eagle_qmm_gemm_w4g64_f16(_ptr(x), _ptr(w_q), _ptr(scales), _ptr(biases), _ptr(bias),
                                         _ptr(out), M, N, K, group_size, bits, _stream())
         _lib.check(rc, "quantized_matmul")
@@ -196,11 +208,12 @@ def swiglu_supported(M, I, K):
     return I % 16 == 0 and M >= 1 and K % 64 == 0
 
 
-def quantized_matmul_swiglu(x, w_q, scales, biases, bias=None, out=None):
+def quantized_matmul_swiglu(x, w_q, scales, biases, bias=None, out=None, gemm=None):
     """silu(x @ Wg.T) * (x @ Wu.T) (mlx_llama.py:214-215) in one launch: w_q / scales / biases
     / bias hold the gate and up projections interleaved by `interleave_gate_up`.  The result
     equals `silu_mul(quantized_matmul(x, gate...), quantized_matmul(x, up...))` bit for bit.
-    Above 32 rows the tiled GEMM form runs with the same epilogue."""
+    33..64 rows run as two passes of the 32-row kernel, more rows as the tiled GEMM form with the
+    same epilogue (`gemm=True`: that form whatever the row count)."""
     _need_cuda(x, w_q, scales, biases, bias)
     x = _f16(x, "x")
     w_q = as_packed_u32(w_q)
@@ -218,7 +231,13 @@ def quantized_matmul_swiglu(x, w_q, scales, biases, bias=None, out=None):
     if out is None:
         out = torch.empty((*lead, N // 2), dtype=torch.float16, device=x.device)
     L = _lib.lib()
-    if M > 32:
+    if ROW_PASS < M <= 2 * ROW_PASS and not gemm:
+        x2, out2 = x.reshape(M, K), out.view(M, N // 2)
+        for r0 in range(0, M, ROW_PASS):
+            quantized_matmul_swiglu(x2[r0:r0 + ROW_PASS], w_q, scales, biases, bias=bias,
+                                    out=out2[r0:r0 + ROW_PASS])
+        return out
+    if M > 32 or gemm:
         # many rows (a prompt chunk): the tiled GEMM with the same epilogue
         rc = L.eagle_qmm_gemm_swiglu_w4g64_f16(_ptr(x), _ptr(w_q), _ptr(scales), _ptr(biases), _ptr(bias),
                                                _ptr(out), M, N, K, 64, 4, _stream())
@@ -478,7 +497,8 @@ def mask_to_bits(tree_mask):
 def tree_attention(q, k_cache, v_cache, tree_mask_bits, cache_len_dev, scale, max_len=None,
                    out=None):
     """q [H,T,hd]; k_cache, v_cache [G,capacity,hd] holding *cache_len_dev prefix rows
-    followed by the T tree rows; tree_mask_bits [T] int32.  Returns [T, H*hd]."""
+    followed by the T tree rows; tree_mask_bits [T] int32, or [T,2] (`mask_to_words`) for
+    trees of up to 64 tokens.  Returns [T, H*hd]."""
     _need_cuda(q, k_cache, v_cache, tree_mask_bits, cache_len_dev)
     H, T, hd = q.shape
     G, cap, _ = k_cache.shape
@@ -487,6 +507,15 @@ def tree_attention(q, k_cache, v_cache, tree_mask_bits, cache_len_dev, scale, ma
     if out is None:
         out = torch.empty((T, H * hd), dtype=torch.float16, device=q.device)
     L = _lib.lib()
+    if tree_mask_bits.dim() == 2:
+        if tree_mask_bits.shape != (T, 2):
+            raise ValueError("two mask words per tree token")
+        ws = workspace("attn", L.eagle_tree_attention_wide_workspace_bytes(T, H, hd, max_len), q.device)
+        rc = L.eagle_tree_attention_wide_f16(_ptr(q), _ptr(k_cache), _ptr(v_cache), _ptr(tree_mask_bits),
+                                             _ptr(cache_len_dev), _ptr(out), T, T, H, G, hd, cap, max_len,
+                                             float(scale), _ptr(ws), ws.numel(), _stream())
+        _lib.check(rc, "tree_attention")
+        return out
     need = L.eagle_tree_attention_workspace_bytes(H, hd, max_len)
     ws = workspace("attn", need, q.device)
     rc = L.eagle_tree_attention_f16(_ptr(q), _ptr(k_cache), _ptr(v_cache), _ptr(tree_mask_bits),
@@ -553,7 +582,8 @@ def mask_to_words(mask):
 
 def draft_attention(q, k_cache, v_cache, mask_words, cache_len_dev, Tk, scale, max_len=None, out=None):
     """q [H,T,hd]; k_cache, v_cache [G,capacity,hd] holding *cache_len_dev prefix rows followed
-    by Tk <= 64 rows that query t sees according to mask_words [T,2].  Returns [T, H*hd]."""
+    by Tk <= 64 rows that query t sees according to mask_words [T,2].  Returns [T, H*hd].
+    More than 32 (up to 64) queries go in pieces of 32 rows through one launch pair."""
     _need_cuda(q, k_cache, v_cache, mask_words, cache_len_dev)
     H, T, hd = q.shape
     G, cap, _ = k_cache.shape
@@ -562,6 +592,13 @@ def draft_attention(q, k_cache, v_cache, mask_words, cache_len_dev, Tk, scale, m
     if out is None:
         out = torch.empty((T, H * hd), dtype=torch.float16, device=q.device)
     L = _lib.lib()
+    if T > 32:
+        ws = workspace("attn", L.eagle_tree_attention_wide_workspace_bytes(T, H, hd, max_len), q.device)
+        rc = L.eagle_tree_attention_wide_f16(_ptr(q), _ptr(k_cache), _ptr(v_cache), _ptr(mask_words),
+                                             _ptr(cache_len_dev), _ptr(out), T, int(Tk), H, G, hd, cap,
+                                             max_len, float(scale), _ptr(ws), ws.numel(), _stream())
+        _lib.check(rc, "draft_attention")
+        return out
     need = L.eagle_tree_attention_workspace_bytes(H, hd, max_len)
     ws = workspace("attn", need, q.device)
     rc = L.eagle_draft_attention_f16(_ptr(q), _ptr(k_cache), _ptr(v_cache), _ptr(mask_words),
@@ -597,18 +634,11 @@ def scaled_dot_product_attention(queries, keys, values, cache=None, scale=None, 
     else:
         k_buf, v_buf = _f16(keys[0], "k"), _f16(values[0], "v")
     q = _f16(queries[0], "q")
-    if T <= 32:
-        out = draft_attention(q, k_buf, v_buf, words, len_dev, Tk, scale, max_len=S)
-    else:
-        # more than 32 queries (a tree of up to 64 tokens): pieces of 32 query rows, each with
-        # its own mask rows over the same keys
-        if T > 64:
-            raise ValueError("at most 64 query rows")
-        out = torch.empty((T, H * hd), dtype=torch.float16, device=q.device)
-        for t0 in range(0, T, 32):
-            t1 = min(T, t0 + 32)
-            draft_attention(q[:, t0:t1].contiguous(), k_buf, v_buf, words[t0:t1].contiguous(), len_dev, Tk,
-                            scale, max_len=S, out=out[t0:t1])
+    if T > 64:
+        raise ValueError("at most 64 query rows")
+    # more than 32 queries (a tree of up to 64 tokens) go in pieces of 32 query rows, each with
+    # its own mask rows over the same keys, inside the one launch pair
+    out = draft_attention(q, k_buf, v_buf, words, len_dev, Tk, scale, max_len=S)
     return out.reshape(T, H, hd).permute(1, 0, 2).unsqueeze(0).contiguous()
 
 

@@ -14,7 +14,7 @@ import torch
 
 from . import _lib, ops
 from .layer import emit_layer
-from .eagle import (MAXT, TreeVerifier, _level_buffers, _ptr, _stream, draft_tree_init, draft_tree_level,
+from .eagle import (TREE_SLOTS, TreeVerifier, _level_buffers, _ptr, _stream, draft_tree_init, draft_tree_level,
                     fuse_projections, process_draft_tree_device, slab_partial_buffer)
 from .eagle import slab_plan as eagle_slab_plan
 
@@ -309,8 +309,9 @@ class SpeculativeDecoder:
 
         if k != Y_LEN:
             raise ValueError("the step is laid out for k = 8 candidates per node")
-        if verify_num_tokens + 1 > MAXT or k * depth > 64 or depth + 2 > Y_LEN:
-            raise ValueError("tree does not fit: at most 31 draft nodes, k * depth <= 64, depth <= 6")
+        if verify_num_tokens + 1 > TREE_SLOTS or k * depth > 64 or depth + 2 > Y_LEN:
+            raise ValueError(f"tree does not fit: at most {TREE_SLOTS - 1} draft nodes, k * depth <= 64, "
+                             "depth <= 6")
         if k + k * k * depth < verify_num_tokens:
             raise ValueError("fewer candidates than draft nodes")
         self.base_model, self.draft_model = base_model, draft_model
@@ -443,12 +444,13 @@ class SpeculativeDecoder:
 
     def generate(self, n_steps):
         """Run n_steps speculative steps; returns the emitted tokens (without the first one).
-        The caches must have room for n_steps * (depth + 2) + 8 * depth + 40 more rows."""
+        The caches must have room for n_steps * (depth + 2) + max(8 * (depth + 1), tree tokens)
+        more rows."""
         # upper bound of the rows either cache can hold after these steps (the lengths live on
-        # the device; a step adds at most depth + 2 tokens and writes up to 8 * depth + 32 rows
-        # beyond the length)
+        # the device; a step adds at most depth + 2 tokens and writes up to 8 * (depth + 1) draft
+        # rows or the tree's rows beyond the length)
         self._bound += n_steps * (self.depth + 2)
-        if self._bound + max(Y_LEN * (self.depth + 1), MAXT) > self.capacity:
+        if self._bound + max(Y_LEN * (self.depth + 1), self.verifier.T) > self.capacity:
             self._bound -= n_steps * (self.depth + 2)
             raise ValueError(f"KV caches of {self.capacity} rows are too small for {n_steps} more steps")
         for _ in range(n_steps):

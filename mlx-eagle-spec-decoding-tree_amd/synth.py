@@ -226,8 +226,9 @@ def random_tree(rng, n_nodes=32, max_depth=4, max_children=4):
 
 
 def tree_arrays(parents):
-    """(depth [T] int32, ancestor-or-self visibility [T,T] bool, row bitmasks [T] uint32)
-    of the tree given by `parents` (as returned by random_tree)."""
+    """(depth [T] int32, ancestor-or-self visibility [T,T] bool, row bitmasks [T] uint32, or
+    [T,2] (low word, high word) above 32 tokens) of the tree given by `parents` (as returned by
+    random_tree)."""
     T = len(parents) + 1
     depth = np.zeros(T, np.int32)
     vis = np.eye(T, dtype=bool)
@@ -235,5 +236,8 @@ def tree_arrays(parents):
         p = int(parents[node - 1])
         depth[node] = depth[p] + 1
         vis[node] |= vis[p]
-    bits = (vis.astype(np.uint64) << np.arange(T, dtype=np.uint64)[None, :]).sum(1).astype(np.uint32)
+    rows = (vis.astype(np.uint64) << np.arange(T, dtype=np.uint64)[None, :]).sum(1)
+    if T <= 32:
+        return depth, vis, rows.astype(np.uint32)
+    bits = np.stack([rows & np.uint64(0xFFFFFFFF), rows >> np.uint64(32)], axis=1).astype(np.uint32)
     return depth, vis, bits

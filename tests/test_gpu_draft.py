@@ -253,8 +253,8 @@ def test_generate_step_stream_equals_target_greedy(dev, same):
 
 def test_generate_step_with_the_reference_default_tree(dev):
     """depth 5, 39 draft nodes (the reference's defaults, mlx_eagle.py:509-510): a tree of 40 tokens
-    runs on the module path (tiled GEMMs for 40 rows, attention in two pieces of query rows);
-    the emitted stream is the target's greedy stream."""
+    on the module path (tiled GEMMs for 40 rows, attention in two pieces of query rows inside one
+    launch pair); the emitted stream is the target's greedy stream."""
     (targs, tw, target), (dargs, dw, draft) = tiny_pair(dev, same=True, seed=6)
     rng = np.random.default_rng(9)
     prompt = rng.integers(0, targs.vocab_size, 40).astype(np.int32)
@@ -265,7 +265,7 @@ def test_generate_step_with_the_reference_default_tree(dev):
     with pytest.raises(NotImplementedError):
         eagle.generate_step(to_dev(prompt.astype(np.int64), dev), target, draft, verify_num_tokens=64)
     with pytest.raises(NotImplementedError):
-        eagle.TreeVerifier(target, make_prompt_cache(target, capacity=128), total_tokens=39)
+        eagle.TreeVerifier(target, make_prompt_cache(target, capacity=128), total_tokens=64)
 
 
 def test_generate_step_matches_oracle_loop(dev):
@@ -337,7 +337,7 @@ def test_device_loop_refuses_to_overrun_the_caches(dev):
     with pytest.raises(ValueError):
         spec.SpeculativeDecoder(target, draft, capacity=128, k=8, depth=9)
     with pytest.raises(ValueError):
-        spec.SpeculativeDecoder(target, draft, capacity=128, k=8, depth=3, verify_num_tokens=32)
+        spec.SpeculativeDecoder(target, draft, capacity=128, k=8, depth=3, verify_num_tokens=64)
 
 
 @pytest.mark.parametrize("n,chunk,graphs", [(75, 512, True), (200, 64, False), (32, 512, True)])

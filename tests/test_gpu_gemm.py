@@ -20,7 +20,8 @@ def test_gemm_form_matches_oracle(dev, M, N, K, bias):
     x = synth.make_x(rng, M, K)
     want = oracle.qmm(x, layer["weight"], layer["scales"], layer["biases"], layer.get("bias"))
     d = layer_to_dev(layer, dev)
-    got = ops.quantized_matmul(to_dev(x, dev), d["weight"], d["scales"], d["biases"], bias=d.get("bias"))
+    got = ops.quantized_matmul(to_dev(x, dev), d["weight"], d["scales"], d["biases"], bias=d.get("bias"),
+                               gemm=True)
     got = got.cpu().numpy()
     assert got.shape == (M, N) and np.isfinite(got.astype(np.float32)).all()
     assert rel_err(got, want) <= TOL
@@ -58,7 +59,7 @@ def test_gemm_form_random_shapes(dev):
     scale loads (multiples of 512 or not), every block shape."""
     rng = np.random.default_rng(99)
     for case in range(14):
-        M = int(rng.integers(33, 700))
+        M = int(rng.integers(1, 700))
         N = 8 * int(rng.integers(1, 700))
         K = 64 * int(rng.integers(1, 40))
         bias = bool(rng.integers(0, 2))
@@ -69,7 +70,7 @@ def test_gemm_form_random_shapes(dev):
         d = layer_to_dev(layer, dev)
         out = torch.full((M + 1, N), float("nan"), dtype=torch.float16, device=dev)
         ops.quantized_matmul(to_dev(x, dev), d["weight"], d["scales"], d["biases"], bias=d.get("bias"),
-                             out=out[:M])
+                             out=out[:M], gemm=True)
         got = out.cpu().numpy()
         assert np.isnan(got[M].astype(np.float32)).all(), case          # nothing written past the rows
         assert np.isfinite(got[:M].astype(np.float32)).all(), case
@@ -96,8 +97,10 @@ def test_gemm_form_with_swiglu(dev, M, I, K, bias):
     inter = {k: ops.interleave_gate_up(gd[k], ud[k]) for k in keys}
     cat = {k: torch.cat([gd[k], ud[k]]).contiguous() for k in keys}
     xd = to_dev(x, dev)
-    got = ops.quantized_matmul_swiglu(xd, inter["weight"], inter["scales"], inter["biases"], bias=inter.get("bias"))
-    two = ops.silu_mul(ops.quantized_matmul(xd, cat["weight"], cat["scales"], cat["biases"], bias=cat.get("bias")))
+    got = ops.quantized_matmul_swiglu(xd, inter["weight"], inter["scales"], inter["biases"], bias=inter.get("bias"),
+                                      gemm=True)
+    two = ops.silu_mul(ops.quantized_matmul(xd, cat["weight"], cat["scales"], cat["biases"], bias=cat.get("bias"),
+                                            gemm=True))
     torch.cuda.synchronize()
     assert tuple(got.shape) == (M, I)
     # Against the oracle: each projection is within TOL of its own RMS (the bound of the plain form);
