@@ -217,10 +217,12 @@ int eagle_qmm_res_w4g64_f16(const void* x, const uint32_t* wq, const void* scale
                             const void* biases, const void* bias, void* out, int M, int N, int K,
                             int group_size, int bits, int swiglu, eagle_stream_t stream);
 
-/* The same product for 1..32 rows in the slab form, with the result left as fp32 partial sums:
+/* The same product for 1..64 rows in the slab form, with the result left as fp32 partial sums:
  * every workgroup owns 128 weight rows and one K slab of `steps_per_slab` quantisation groups
  * (a multiple of 8), moves x through LDS eight groups at a time and expands the weights to fp16
- * in registers for v_mfma_f32_32x32x16_f16.  partial [slabs][32][N] fp32 (rows >= M are not written),
+ * in registers for v_mfma_f32_32x32x16_f16.  partial [slabs][R][N] fp32, R = 32 for M <= 32 and 64
+ * for 33..64 rows (a tree above 32 tokens; every expanded weight then feeds two matrix
+ * instructions) (rows >= M are not written),
  * slabs = eagle_qmm_slab_count(K, steps_per_slab) (0 for a shape the form does not take:
  * K % 128 == 0 is required; scales and biases 16-byte aligned when K % 512 == 0, 4-byte aligned
  * otherwise).  The product is
@@ -233,7 +235,8 @@ int eagle_qmm_slab_count(int K, int steps_per_slab);
 /* K steps per slab recommended for this product, 0 where eagle_qmm_w4g64_f16 is the faster form
  * (few rows, very many weight rows, or K not a multiple of 512). */
 int eagle_qmm_slab_steps(int M, int N, int K);
-size_t eagle_qmm_slab_partial_bytes(int N, int K, int steps_per_slab);
+size_t eagle_qmm_slab_partial_bytes(int N, int K, int steps_per_slab);             /* M <= 32 */
+size_t eagle_qmm_slab_partial_bytes_rows(int M, int N, int K, int steps_per_slab); /* M <= 64 */
 int eagle_qmm_slab_partial_w4g64(const void* x, const uint32_t* wq, const void* scales,
                                  const void* biases, float* partial, size_t partial_bytes,
                                  int M, int N, int K, int group_size, int bits,
@@ -296,7 +299,8 @@ int eagle_tree_attention_f16(const void* q, const void* k_cache, const void* v_c
 int eagle_rmsnorm_f16(const void* x, const void* residual, const void* w, float eps,
                       void* h_out, void* out, int T, int D, eagle_stream_t stream);
 /* The same with x held as fp32 partial sums of K slabs (eagle_qmm_slab_partial_w4g64 with
- * N = D): x = fp16(sum of the slabs).  T <= 32. */
+ * N = D): x = fp16(sum of the slabs).  T <= 64 (partial rows as that entry point lays them out
+ * for M = T). */
 int eagle_rmsnorm_slabs_f16(const float* partial, int slabs, const void* residual, const void* w,
                             float eps, void* h_out, void* out, int T, int D, eagle_stream_t stream);
 
@@ -320,7 +324,7 @@ int eagle_rope_kv_append_table_f16(const void* q_lin, const void* k_lin, const v
 /* The same with the fused q|k|v projection held as fp32 partial sums of K slabs
  * (eagle_qmm_slab_partial_w4g64 with N = (H + 2G) hd, rows [q heads | k heads | v heads]):
  * every value is fp16(sum of the slabs) + bias (bias [N] fp16, 16-byte aligned, may be NULL)
- * before the rotation.  T <= 32. */
+ * before the rotation.  T <= 64 (partial rows as that entry point lays them out for M = T). */
 int eagle_rope_kv_append_slabs_f16(const float* partial, int slabs, const void* bias,
                                    const float* rope_cs, void* q_out, void* k_cache, void* v_cache,
                                    const int32_t* cache_len_dev, int T, int H, int G, int hd,

@@ -35,6 +35,9 @@ __device__ inline float wave_max(float v) {
   return v;
 }
 
+// Rows of a partial tile of the slab form: 32 for up to 32 rows of x, 64 for 33..64.
+__host__ __device__ inline int eagle_slab_rows(int M) { return M > 32 ? 64 : 32; }
+
 // Eight consecutive values of a matmul result that is held as fp32 partial sums of K slabs
 // (eagle_qmm_slab_partial_w4g64): fp16 of the sum in slab order, then the fp16 bias.  `at` is
 // the element offset inside a slab, `stride` the elements per slab.  All loads are issued

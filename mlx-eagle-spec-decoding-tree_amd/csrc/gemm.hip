@@ -455,18 +455,22 @@ int launch_gemm(const half_t* x, const uint32_t* w, const half_t* s, const half_
 // counter, loads of all slabs, store) is a chain of device-scope round trips that took longer
 // than the product itself: 14.1 us against 5.7 us for 32 x 4608 x 3584.
 constexpr int SLAB_RING = 8;
-constexpr int SLAB_ROWS = 32;               // rows of a partial tile (EAGLE_MAX_M)
+constexpr int SLAB_ROWS = 32;               // rows of x per accumulator tile
 constexpr int SLAB_XR = SLAB_RING * 64 + 8; // LDS row stride of an x chunk in halves
 constexpr int SLAB_XBUF = SLAB_ROWS * SLAB_XR;
 
 // RAGGED: K is a multiple of 128 but not of 512.  A slab may then hold any number of steps:
 // the last chunk is partial (its loads are repeated from the slab's last step, its extra
 // steps are skipped) and scales / biases come two groups per fetch.
-template <bool RAGGED>
+// MR: 32-row tiles of x (1: up to 32 rows, 2: 33..64 rows of a tree above 32 tokens).  With two,
+// every expanded weight operand feeds two matrix instructions, the x chunk in LDS has 64 rows
+// (66 KB per buffer) and the partial tile is [64][N].
+template <bool RAGGED, int MR = 1>
 __global__ __launch_bounds__(256) void qmm_slab_w4g64_kernel(
     const half_t* __restrict__ x, const uint32_t* __restrict__ w, const half_t* __restrict__ s,
     const half_t* __restrict__ b, float* __restrict__ partial, int M, int N, int K, int spz) {
   extern __shared__ __attribute__((aligned(16))) half_t xlds[];   // one or two x chunks
+  constexpr int XBUF = MR * SLAB_XBUF;
   const int tid = threadIdx.x;
   const int wave = tid >> 6, lane = tid & 63;
   const int ql = lane & 31, hb = lane >> 5;
@@ -479,21 +483,30 @@ __global__ __launch_bounds__(256) void qmm_slab_w4g64_kernel(
   const int rem = steps - (chunks - 1) * 8;  // steps of the last chunk
   auto step_of = [&](int i) { return RAGGED && i > steps - 1 ? steps - 1 : i; };
 
-  // thread (xr, xc) moves the 16 bytes at column 64 i + 8 xc of row xr for the steps i of a chunk
+  // thread (xr, xc) moves the 16 bytes at column 64 i + 8 xc of rows xr (and xr + 32) for the
+  // steps i of a chunk
   const int xr = tid >> 3, xc = tid & 7;
-  const half_t* xp = x + (long)(xr < M ? xr : M - 1) * K + g0 * 64 + xc * 8;
+  const half_t* xp[MR];
+#pragma unroll
+  for (int r = 0; r < MR; ++r) {
+    const int row = xr + 32 * r;
+    xp[r] = x + (long)(row < M ? row : M - 1) * K + g0 * 64 + xc * 8;
+  }
   int nrow = blockIdx.x * 128 + wave * 32 + ql;
   if (nrow > N - 1) nrow = N - 1;
   const uint32_t* wp = w + (long)nrow * KW + g0 * 8 + hb * 4;
   const half_t* sp = s + (long)nrow * G + g0;
   const half_t* bp = b + (long)nrow * G + g0;
 
-  half8_t xreg[SLAB_RING];
+  half8_t xreg[MR][SLAB_RING];
   uint4_t wreg[SLAB_RING];
   half8_t s8, b8, s8n, b8n;
   auto fetch_x = [&](int c) {
 #pragma unroll
-    for (int i = 0; i < SLAB_RING; ++i) xreg[i] = *reinterpret_cast<const half8_t*>(xp + step_of(c * 8 + i) * 64);
+    for (int r = 0; r < MR; ++r)
+#pragma unroll
+      for (int i = 0; i < SLAB_RING; ++i)
+        xreg[r][i] = *reinterpret_cast<const half8_t*>(xp[r] + step_of(c * 8 + i) * 64);
   };
   // scales and biases of chunk c: one 16-byte fetch, or four 4-byte fetches kept inside the slab
   auto fetch_sb = [&](int c, half8_t& s_out, half8_t& b_out) {
@@ -515,8 +528,11 @@ __global__ __launch_bounds__(256) void qmm_slab_w4g64_kernel(
   };
   auto stash_x = [&](int buf) {
 #pragma unroll
-    for (int i = 0; i < SLAB_RING; ++i)
-      *reinterpret_cast<half8_t*>(&xlds[buf * SLAB_XBUF + xr * SLAB_XR + i * 64 + xc * 8]) = permute8(xreg[i]);
+    for (int r = 0; r < MR; ++r)
+#pragma unroll
+      for (int i = 0; i < SLAB_RING; ++i)
+        *reinterpret_cast<half8_t*>(&xlds[buf * XBUF + (xr + 32 * r) * SLAB_XR + i * 64 + xc * 8]) =
+            permute8(xreg[r][i]);
   };
   fetch_x(0);
   fetch_sb(0, s8, b8);
@@ -527,9 +543,11 @@ __global__ __launch_bounds__(256) void qmm_slab_w4g64_kernel(
   if (chunks > 1) fetch_x(1);
   __syncthreads();
 
-  float16_t acc;
+  float16_t acc[MR];
 #pragma unroll
-  for (int i = 0; i < 16; ++i) acc[i] = 0.f;
+  for (int r = 0; r < MR; ++r)
+#pragma unroll
+    for (int i = 0; i < 16; ++i) acc[r][i] = 0.f;
   const half_t* xrow = xlds + ql * SLAB_XR + hb * 32;
 
   // one chunk of eight steps on the x chunk in buffer `buf`; RELOAD: the weight registers are
@@ -547,10 +565,13 @@ __global__ __launch_bounds__(256) void qmm_slab_w4g64_kernel(
       for (int j = 0; j < 4; ++j) af[j] = dequant_word_centred(wreg[e][j], half2_t{sc, sc}, half2_t{bc, bc});
       if (reload) wreg[e] = *reinterpret_cast<const uint4_t*>(wp + step_of((c + 1) * 8 + e) * 8);
 #pragma unroll
-      for (int j = 0; j < 4; ++j) {
-        const half8_t bf = *reinterpret_cast<const half8_t*>(xrow + buf * SLAB_XBUF + e * 64 + j * 8);
-        acc = __builtin_amdgcn_mfma_f32_32x32x16_f16(af[j], bf, acc, 0, 0, 0);
-      }
+      for (int j = 0; j < 4; ++j)
+#pragma unroll
+        for (int r = 0; r < MR; ++r) {
+          const half8_t bf =
+              *reinterpret_cast<const half8_t*>(xrow + buf * XBUF + r * SLAB_XBUF + e * 64 + j * 8);
+          acc[r] = __builtin_amdgcn_mfma_f32_32x32x16_f16(af[j], bf, acc[r], 0, 0, 0);
+        }
     }
     if (reload) {
       s8 = s8n;
@@ -569,20 +590,23 @@ __global__ __launch_bounds__(256) void qmm_slab_w4g64_kernel(
   chunk(chunks - 1, (chunks - 1) & 1, StepIndex<0>{});
 
   // accumulator register i of a lane: weight row 8*(i/4) + 4*hb + i%4 of the wave's tile, x
-  // row ql.  Through LDS, so that the lanes of a wave store whole 512-byte row segments.
+  // row ql (+ 32 for the second tile).  Through LDS, so that the lanes of a wave store whole
+  // 512-byte row segments.
   constexpr int OS = 128 + 4;                // floats per row of the tile in LDS
   float* ot = reinterpret_cast<float*>(xlds);
   __syncthreads();                           // every wave is done with the x chunks
 #pragma unroll
-  for (int i4 = 0; i4 < 4; ++i4)
-    *reinterpret_cast<float4_t*>(&ot[ql * OS + wave * 32 + 8 * i4 + 4 * hb]) =
-        float4_t{acc[4 * i4], acc[4 * i4 + 1], acc[4 * i4 + 2], acc[4 * i4 + 3]};
+  for (int r = 0; r < MR; ++r)
+#pragma unroll
+    for (int i4 = 0; i4 < 4; ++i4)
+      *reinterpret_cast<float4_t*>(&ot[(ql + 32 * r) * OS + wave * 32 + 8 * i4 + 4 * hb]) =
+          float4_t{acc[r][4 * i4], acc[r][4 * i4 + 1], acc[r][4 * i4 + 2], acc[r][4 * i4 + 3]};
   __syncthreads();
-  float* dst = partial + (size_t)z * SLAB_ROWS * N;
+  float* dst = partial + (size_t)z * (MR * SLAB_ROWS) * N;
   const int c = (tid & 31) * 4;
   const int n = blockIdx.x * 128 + c;
 #pragma unroll
-  for (int pass = 0; pass < 4; ++pass) {
+  for (int pass = 0; pass < 4 * MR; ++pass) {
     const int m = pass * 8 + (tid >> 5);
     if (m < M && n < N)
       *reinterpret_cast<float4_t*>(dst + (size_t)m * N + n) = *reinterpret_cast<const float4_t*>(&ot[m * OS + c]);
@@ -596,7 +620,7 @@ __global__ void slab_sum_kernel(const float* __restrict__ partial, int nslab, co
   const int per_row = N >> 3;
   if (idx >= (long)M * per_row) return;
   const int m = (int)(idx / per_row), n = (int)(idx % per_row) * 8;
-  const half8_t v = eagle_slab_sum8(partial, nslab, (size_t)SLAB_ROWS * N, (size_t)m * N + n, bias ? bias + n : nullptr);
+  const half8_t v = eagle_slab_sum8(partial, nslab, (size_t)eagle_slab_rows(M) * N, (size_t)m * N + n, bias ? bias + n : nullptr);
   *reinterpret_cast<half8_t*>(out + (size_t)m * N + n) = v;
 }
 
@@ -615,7 +639,7 @@ EAGLE_EXPORT int eagle_qmm_slab_steps(int M, int N, int K) {
   // keeps gate|up (its SwiGLU epilogue saves a launch) and the vocabulary projection.  Eight
   // steps per slab while that gives at most eight slabs, otherwise longer slabs so that the
   // reader of the result has about ten slabs to add.
-  if (M < 1 || M > SLAB_ROWS || N < 8 || (N % 8) != 0 || K < 512 || (K % 512) != 0) return 0;
+  if (M < 1 || M > 2 * SLAB_ROWS || N < 8 || (N % 8) != 0 || K < 512 || (K % 512) != 0) return 0;
   if (N > 8192) return 0;
   const int G = K / 64;
   return G <= 64 ? 8 : G <= 128 ? 16 : 32;
@@ -626,13 +650,18 @@ EAGLE_EXPORT size_t eagle_qmm_slab_partial_bytes(int N, int K, int steps_per_sla
   return (size_t)eagle_qmm_slab_count(K, steps_per_slab) * SLAB_ROWS * N * sizeof(float);
 }
 
+EAGLE_EXPORT size_t eagle_qmm_slab_partial_bytes_rows(int M, int N, int K, int steps_per_slab) {
+  if (N < 1 || M < 1 || M > 2 * SLAB_ROWS) return 0;
+  return (size_t)eagle_qmm_slab_count(K, steps_per_slab) * eagle_slab_rows(M) * N * sizeof(float);
+}
+
 EAGLE_EXPORT int eagle_qmm_slab_partial_w4g64(const void* x, const uint32_t* wq, const void* scales,
                                               const void* biases, float* partial, size_t partial_bytes,
                                               int M, int N, int K, int group_size, int bits,
                                               int steps_per_slab, eagle_stream_t stream) {
   if (!x || !wq || !scales || !biases || !partial) return EAGLE_ERR_NULL;
   if (group_size != 64 || bits != 4) return EAGLE_ERR_UNSUPPORTED;
-  if (M < 1 || M > SLAB_ROWS || N < 8 || (N % 8) != 0 || K < 128 || (K % 128) != 0) return EAGLE_ERR_SHAPE;
+  if (M < 1 || M > 2 * SLAB_ROWS || N < 8 || (N % 8) != 0 || K < 128 || (K % 128) != 0) return EAGLE_ERR_SHAPE;
   const int slabs = eagle_qmm_slab_count(K, steps_per_slab);
   if (slabs < 1 || slabs > 65535) return EAGLE_ERR_SHAPE;
   const bool ragged = (K % 512) != 0;
@@ -640,36 +669,43 @@ EAGLE_EXPORT int eagle_qmm_slab_partial_w4g64(const void* x, const uint32_t* wq,
   if (!eagle_aligned16(x) || !eagle_aligned16(wq) || !eagle_aligned16(partial) ||
       (reinterpret_cast<uintptr_t>(scales) & sb_mask) || (reinterpret_cast<uintptr_t>(biases) & sb_mask))
     return EAGLE_ERR_ALIGN;
-  if (partial_bytes < eagle_qmm_slab_partial_bytes(N, K, steps_per_slab)) return EAGLE_ERR_WORKSPACE;
+  if (partial_bytes < eagle_qmm_slab_partial_bytes_rows(M, N, K, steps_per_slab)) return EAGLE_ERR_WORKSPACE;
+  const int mr = M > SLAB_ROWS ? 2 : 1;
   const int bufs = steps_per_slab > SLAB_RING ? 2 : 1;
-  const size_t lds = (size_t)bufs * SLAB_XBUF * sizeof(half_t);
+  const size_t lds = (size_t)bufs * mr * SLAB_XBUF * sizeof(half_t);
   static bool configured = false;
   if (!configured) {
     const int most = 2 * SLAB_XBUF * (int)sizeof(half_t);
-    if (hipFuncSetAttribute(reinterpret_cast<const void*>(&qmm_slab_w4g64_kernel<false>),
+    if (hipFuncSetAttribute(reinterpret_cast<const void*>(&qmm_slab_w4g64_kernel<false, 1>),
                             hipFuncAttributeMaxDynamicSharedMemorySize, most) != hipSuccess ||
-        hipFuncSetAttribute(reinterpret_cast<const void*>(&qmm_slab_w4g64_kernel<true>),
-                            hipFuncAttributeMaxDynamicSharedMemorySize, most) != hipSuccess)
+        hipFuncSetAttribute(reinterpret_cast<const void*>(&qmm_slab_w4g64_kernel<true, 1>),
+                            hipFuncAttributeMaxDynamicSharedMemorySize, most) != hipSuccess ||
+        hipFuncSetAttribute(reinterpret_cast<const void*>(&qmm_slab_w4g64_kernel<false, 2>),
+                            hipFuncAttributeMaxDynamicSharedMemorySize, 2 * most) != hipSuccess ||
+        hipFuncSetAttribute(reinterpret_cast<const void*>(&qmm_slab_w4g64_kernel<true, 2>),
+                            hipFuncAttributeMaxDynamicSharedMemorySize, 2 * most) != hipSuccess)
       return EAGLE_ERR_HIP;
     configured = true;
   }
   const dim3 grid((N + 127) / 128, slabs);
   hipStream_t st = static_cast<hipStream_t>(stream);
-  if (ragged)
-    hipLaunchKernelGGL(qmm_slab_w4g64_kernel<true>, grid, dim3(256), lds, st, static_cast<const half_t*>(x), wq,
-                       static_cast<const half_t*>(scales), static_cast<const half_t*>(biases), partial, M, N,
-                       K, steps_per_slab);
-  else
-    hipLaunchKernelGGL(qmm_slab_w4g64_kernel<false>, grid, dim3(256), lds, st, static_cast<const half_t*>(x), wq,
-                       static_cast<const half_t*>(scales), static_cast<const half_t*>(biases), partial, M, N,
-                       K, steps_per_slab);
+#define EAGLE_SLAB_LAUNCH(RAG, MRV)                                                                      \
+  hipLaunchKernelGGL((qmm_slab_w4g64_kernel<RAG, MRV>), grid, dim3(256), lds, st,                        \
+                     static_cast<const half_t*>(x), wq, static_cast<const half_t*>(scales),              \
+                     static_cast<const half_t*>(biases), partial, M, N, K, steps_per_slab)
+  if (ragged) {
+    if (mr == 2) EAGLE_SLAB_LAUNCH(true, 2); else EAGLE_SLAB_LAUNCH(true, 1);
+  } else {
+    if (mr == 2) EAGLE_SLAB_LAUNCH(false, 2); else EAGLE_SLAB_LAUNCH(false, 1);
+  }
+#undef EAGLE_SLAB_LAUNCH
   return eagle_launch_status();
 }
 
 EAGLE_EXPORT int eagle_slab_sum_f16(const float* partial, int slabs, const void* bias, void* out, int M,
                                     int N, eagle_stream_t stream) {
   if (!partial || !out) return EAGLE_ERR_NULL;
-  if (slabs < 1 || M < 1 || M > SLAB_ROWS || N < 8 || (N % 8) != 0) return EAGLE_ERR_SHAPE;
+  if (slabs < 1 || M < 1 || M > 2 * SLAB_ROWS || N < 8 || (N % 8) != 0) return EAGLE_ERR_SHAPE;
   if (!eagle_aligned16(partial) || !eagle_aligned16(out) || (bias && !eagle_aligned16(bias))) return EAGLE_ERR_ALIGN;
   const long total = (long)M * (N / 8);
   hipLaunchKernelGGL(slab_sum_kernel, dim3((unsigned)((total + 255) / 256)), dim3(256), 0,

@@ -158,7 +158,7 @@ __global__ void rope_kv_append_slabs_kernel(const float* __restrict__ partial, i
   const int hh = (int)((idx / per_row) % heads);
   const int t = (int)(idx / ((long)per_row * heads));
   const size_t ld = (size_t)heads * hd;
-  const size_t stride = 32 * ld;
+  const size_t stride = (size_t)eagle_slab_rows(T) * ld;
   const float* p = partial + (size_t)t * ld + (size_t)hh * hd + c;
   // the cache length, cos / sin and the bias are requested with the slabs
   const long P = *len_dev;
@@ -237,7 +237,8 @@ __global__ __launch_bounds__(BLOCK) void rmsnorm_kernel(const half_t* __restrict
                                                         half_t* __restrict__ h_out,
                                                         half_t* __restrict__ out, int D,
                                                         const float* __restrict__ partial, int nslab) {
-  // partial != nullptr: x is held as fp32 partial sums of nslab K slabs, [slab][32][D]
+  // partial != nullptr: x is held as fp32 partial sums of nslab K slabs, [slab][32 or 64][D]
+  // (64 when the launch has more than 32 rows)
   constexpr int NV = 256 * RMS_MAXV / BLOCK;     // vectors per thread
   __shared__ float red[BLOCK / 64];
   const int t = blockIdx.x;
@@ -254,7 +255,7 @@ __global__ __launch_bounds__(BLOCK) void rmsnorm_kernel(const half_t* __restrict
       if (res) r8 = *reinterpret_cast<const half8_t*>(res + (long)t * D + c * 8);
       half8_t a;
       if (partial)
-        a = eagle_slab_sum8(partial, nslab, (size_t)32 * D, (size_t)t * D + c * 8, nullptr);
+        a = eagle_slab_sum8(partial, nslab, (size_t)eagle_slab_rows(gridDim.x) * D, (size_t)t * D + c * 8, nullptr);
       else
         a = *reinterpret_cast<const half8_t*>(xr + c * 8);
       if (res) {
@@ -489,7 +490,7 @@ EAGLE_EXPORT int eagle_rope_kv_append_slabs_f16(const float* partial, int slabs,
                                                 int H, int G, int hd, long capacity,
                                                 eagle_stream_t stream) {
   if (!partial || !rope_cs || !q_out || !k_cache || !v_cache || !cache_len_dev) return EAGLE_ERR_NULL;
-  if (slabs < 1 || T < 1 || T > 32 || H < 1 || G < 1 || (H % G) != 0 || hd < 16 || (hd % 16) != 0 ||
+  if (slabs < 1 || T < 1 || T > 64 || H < 1 || G < 1 || (H % G) != 0 || hd < 16 || (hd % 16) != 0 ||
       capacity < T)
     return EAGLE_ERR_SHAPE;
   if (!eagle_aligned16(partial) || !eagle_aligned16(rope_cs) || !eagle_aligned16(q_out) ||
@@ -525,7 +526,7 @@ EAGLE_EXPORT int eagle_rmsnorm_slabs_f16(const float* partial, int slabs, const 
                                          const void* w, float eps, void* h_out, void* out, int T, int D,
                                          eagle_stream_t stream) {
   if (!partial || !w || !out || (residual && !h_out)) return EAGLE_ERR_NULL;
-  if (slabs < 1 || T < 1 || T > 32 || D < 8 || (D % 8) != 0 || D > 256 * 8 * RMS_MAXV) return EAGLE_ERR_SHAPE;
+  if (slabs < 1 || T < 1 || T > 64 || D < 8 || (D % 8) != 0 || D > 256 * 8 * RMS_MAXV) return EAGLE_ERR_SHAPE;
   if (!eagle_aligned16(partial) || !eagle_aligned16(w) || !eagle_aligned16(out) ||
       (residual && (!eagle_aligned16(residual) || !eagle_aligned16(h_out))))
     return EAGLE_ERR_ALIGN;

@@ -406,8 +406,6 @@ def slab_plan(model, T, forced=None, fused=True, rope_launch=True):
     H, G, hd = args.num_attention_heads, args.num_key_value_heads, args.head_dim
     layer = model.model.layers[0]
     shapes = {"qkv": ((H + 2 * G) * hd, D), "o": (D, H * hd), "down": (D, I)}
-    if T > MAXT:      # the slab kernel holds 32 rows
-        return {name: 0 for name in shapes}
     plan = {}
     for name, (n, k) in shapes.items():
         s = ops.slab_steps(T, n, k) if forced is None else int(forced.get(name, 0))
@@ -422,12 +420,12 @@ def slab_plan(model, T, forced=None, fused=True, rope_launch=True):
     return plan
 
 
-def slab_partial_buffer(model, plan):
-    """fp32 buffer large enough for the partial sums of any projection in `plan`."""
+def slab_partial_buffer(model, plan, T=MAXT):
+    """fp32 buffer large enough for the partial sums of any projection in `plan` of a pass of T rows."""
     args = model.args
     D, I = args.hidden_size, args.intermediate_size
     H, G, hd = args.num_attention_heads, args.num_key_value_heads, args.head_dim
-    need = max([1] + [ops.slab_count(k, plan[name]) * 32 * n
+    need = max([1] + [ops.slab_count(k, plan[name]) * ops.slab_rows(T) * n
                       for name, n, k in (("qkv", (H + 2 * G) * hd, D), ("o", D, H * hd), ("down", D, I))
                       if plan[name]])
     return torch.empty(need, dtype=torch.float32, device=model.device)
@@ -486,9 +484,10 @@ class TreeVerifier:
                                       f"(total_tokens <= {TREE_SLOTS - 1})")
         self.V = total_tokens
         self.T = T = total_tokens + 1
-        # above 32 tree tokens: the matmuls in two passes of the 32-row streaming kernel, two mask
-        # words per token and attention in pieces of 32 query rows (one launch pair); the slab,
-        # resident and chained forms hold 32 rows and do not apply
+        # above 32 tree tokens: q|k|v, o and down in the slab form with 64-row partial tiles, the
+        # other matmuls in two passes of the 32-row streaming kernel, two mask words per token and
+        # attention in pieces of 32 query rows (one launch pair); the resident and chained forms
+        # hold 32 rows and do not apply
         self.wide = T > MAXT
         if self.wide and (not fuse or one_launch_attention or chain or resident_gate_up):
             raise ValueError(f"a tree of more than {MAXT} tokens runs with the fused projections and "
@@ -550,7 +549,7 @@ class TreeVerifier:
         self.act = torch.empty((T, I), **f16)
         self.down = torch.empty((T, D), **f16)
         self.logits = torch.empty((T, args.vocab_size), **f16)
-        self.partial = slab_partial_buffer(model, self.slab)
+        self.partial = slab_partial_buffer(model, self.slab, T)
         self.len_dev = cache[0].len_dev
         self.cache_ptrs = torch.tensor([c.keys.data_ptr() for c in cache]
                                        + [c.values.data_ptr() for c in cache],

@@ -145,10 +145,17 @@ def slab_steps(M, N, K):
     return _lib.lib().eagle_qmm_slab_steps(int(M), int(N), int(K))
 
 
+def slab_rows(M):
+    """Rows of a partial tile of the slab form for M rows of x."""
+    if M < 1 or M > 64:
+        raise ValueError("the slab form takes 1..64 rows")
+    return 64 if M > 32 else 32
+
+
 def quantized_matmul_slabs(x, w_q, scales, biases, steps_per_slab, partial=None):
-    """The product for 1..32 rows as fp32 partial sums of K slabs, [slabs, 32, N]: the result
-    is fp16(partial.sum(0)) (+ bias), formed by `slab_sum`, `rms_norm_slabs` or
-    `rope_kv_append_slabs`.  K % 512 == 0."""
+    """The product for 1..64 rows as fp32 partial sums of K slabs, [slabs, R, N] with R = 32 up
+    to 32 rows and 64 above (`slab_rows`): the result is fp16(partial.sum(0)) (+ bias), formed by
+    `slab_sum`, `rms_norm_slabs` or `rope_kv_append_slabs`.  K % 128 == 0."""
     _need_cuda(x, w_q, scales, biases)
     x = _f16(x, "x")
     w_q = as_packed_u32(w_q)
@@ -162,10 +169,11 @@ def quantized_matmul_slabs(x, w_q, scales, biases, steps_per_slab, partial=None)
     slabs = slab_count(K, steps_per_slab)
     if slabs < 1:
         raise ValueError(f"the slab form does not take K = {K} with {steps_per_slab} steps per slab")
+    R = slab_rows(M)
     if partial is None:
-        partial = torch.empty((slabs, 32, N), dtype=torch.float32, device=x.device)
-    elif partial.dtype != torch.float32 or partial.numel() < slabs * 32 * N or not partial.is_contiguous():
-        raise ValueError("partial must be a contiguous fp32 buffer of at least slabs * 32 * N elements")
+        partial = torch.empty((slabs, R, N), dtype=torch.float32, device=x.device)
+    elif partial.dtype != torch.float32 or partial.numel() < slabs * R * N or not partial.is_contiguous():
+        raise ValueError(f"partial must be a contiguous fp32 buffer of at least slabs * {R} * N elements")
     rc = _lib.lib().eagle_qmm_slab_partial_w4g64(_ptr(x), _ptr(w_q), _ptr(scales), _ptr(biases),
                                                  _ptr(partial), partial.numel() * 4, M, N, K, 64, 4,
                                                  int(steps_per_slab), _stream())
@@ -473,8 +481,8 @@ def rope_kv_append(q_lin, k_lin, v_lin, positions, inv_freqs, scaling_factor, q_
 
 
 def rope_kv_append_slabs(partial, slabs, bias, rope_cs, q_out, k_cache, v_cache, cache_len_dev, T, H, G, hd):
-    """`rope_kv_append` (table form) of the fused q|k|v projection held as [slabs, 32, (H+2G) hd]
-    fp32 partial sums; `bias` is the projection's fp16 bias or None."""
+    """`rope_kv_append` (table form) of the fused q|k|v projection held as
+    [slabs, slab_rows(T), (H+2G) hd] fp32 partial sums; `bias` is the projection's fp16 bias or None."""
     rc = _lib.lib().eagle_rope_kv_append_slabs_f16(
         _ptr(partial), int(slabs), _ptr(bias), _ptr(rope_cs), _ptr(q_out), _ptr(k_cache), _ptr(v_cache),
         _ptr(cache_len_dev), T, H, G, hd, k_cache.shape[1], _stream())
@@ -701,7 +709,7 @@ def rms_norm(x, weight, eps, residual=None, out=None, h_out=None):
 
 
 def rms_norm_slabs(partial, slabs, weight, eps, T, residual=None, out=None, h_out=None):
-    """`rms_norm` of x = fp16(sum of the slabs) held as [slabs, 32, D] fp32 partial sums."""
+    """`rms_norm` of x = fp16(sum of the slabs) held as [slabs, slab_rows(T), D] fp32 partial sums."""
     _need_cuda(partial, weight, residual)
     D = weight.shape[-1]
     if out is None:

@@ -1,4 +1,4 @@
-"""Slab form of the 4-bit group-64 matmul for up to 32 rows: fp32 partial sums per K slab,
+"""Slab form of the 4-bit group-64 matmul for up to 64 rows: fp32 partial sums per K slab,
 added by the consumer (plain sum, RMSNorm, rotary embedding + KV append), and the verification
 step built on it."""
 import numpy as np
@@ -29,7 +29,13 @@ def ordered_sum_f16(partial, slabs, M):
                                               (13, 136, 1536, 16, False),
                                               # K a multiple of 128 only: partial last chunk, 4-byte scale fetches
                                               (8, 1152, 896, 8, True), (8, 896, 4864, 8, False), (32, 896, 4864, 32, False),
-                                              (32, 200, 128, 8, True), (5, 128, 640, 8, False), (32, 264, 1920, 16, True)])
+                                              (32, 200, 128, 8, True), (5, 128, 640, 8, False), (32, 264, 1920, 16, True),
+                                              # 33..64 rows: 64-row partial tiles
+                                              (40, 4608, 3584, 8, True), (64, 3584, 3584, 8, False),
+                                              (33, 200, 1536, 8, True), (40, 3584, 18944, 32, False),
+                                              (64, 1000, 4096, 16, True), (47, 136, 1024, 24, False),
+                                              (40, 1152, 896, 8, True), (64, 896, 4864, 32, False),
+                                              (50, 264, 1920, 16, True), (64, 128, 128, 8, False)])
 def test_slab_partials_match_oracle(dev, M, N, K, steps, bias):
     print(f"slab M={M} N={N} K={K} steps={steps}", flush=True)
     rng = np.random.default_rng(M + N + K + steps)
@@ -39,7 +45,7 @@ def test_slab_partials_match_oracle(dev, M, N, K, steps, bias):
     d = layer_to_dev(layer, dev)
     slabs = ops.slab_count(K, steps)
     assert slabs == -(-(K // 64) // steps)
-    partial = torch.full((slabs, 32, N), float("nan"), dtype=torch.float32, device=dev)
+    partial = torch.full((slabs, ops.slab_rows(M), N), float("nan"), dtype=torch.float32, device=dev)
     ops.quantized_matmul_slabs(to_dev(x, dev), d["weight"], d["scales"], d["biases"], steps, partial=partial)
     assert torch.isfinite(partial[:, :M]).all()
     assert torch.isnan(partial[:, M:]).all(), "rows past M must stay untouched"
@@ -80,20 +86,23 @@ def test_slab_form_rejects_bad_arguments(dev):
     with pytest.raises(ValueError):
         ops.quantized_matmul_slabs(x[:, :832].contiguous(), w[:, :104].contiguous(), s[:, :13].contiguous(),
                                    s[:, :13].contiguous(), 8)          # K not a multiple of 128
-    x = torch.zeros((33, 1024), dtype=torch.float16, device=dev)
+    x = torch.zeros((65, 1024), dtype=torch.float16, device=dev)
     w = torch.zeros((64, 128), dtype=torch.int32, device=dev)
     s = torch.zeros((64, 16), dtype=torch.float16, device=dev)
     with pytest.raises(ValueError):
-        ops.quantized_matmul_slabs(x, w, s, s, 8)                      # more than 32 rows
+        ops.quantized_matmul_slabs(x, w, s, s, 8)                      # more than 64 rows
     with pytest.raises(ValueError):
         ops.quantized_matmul_slabs(x[:8], w, s, s, 8, partial=torch.zeros(100, device=dev))
+    with pytest.raises(ValueError):                                    # 33 rows need 64-row tiles
+        ops.quantized_matmul_slabs(x[:33], w, s, s, 8, partial=torch.zeros(2 * 32 * 64, device=dev))
 
 
 @pytest.mark.parametrize("T,D,slabs,residual", [(32, 3584, 7, True), (5, 512, 1, True), (32, 1024, 10, False),
-                                                (17, 4096, 8, True)])
+                                                (17, 4096, 8, True), (40, 3584, 7, True), (64, 1024, 10, False),
+                                                (33, 4096, 3, True)])
 def test_rms_norm_of_slabs_equals_norm_of_their_sum(dev, T, D, slabs, residual):
     g = torch.Generator(device="cpu").manual_seed(T + D + slabs)
-    partial = torch.randn((slabs, 32, D), generator=g).to(dev)
+    partial = torch.randn((slabs, ops.slab_rows(T), D), generator=g).to(dev)
     weight = (1 + 0.1 * torch.randn(D, generator=g)).half().to(dev)
     res = torch.randn((T, D), generator=g).half().to(dev) if residual else None
     x = ops.slab_sum(partial, slabs, T, D)
@@ -109,11 +118,12 @@ def test_rms_norm_of_slabs_equals_norm_of_their_sum(dev, T, D, slabs, residual):
 
 
 @pytest.mark.parametrize("T,H,G,hd,slabs,bias", [(32, 28, 4, 128, 7, True), (9, 4, 2, 64, 2, False),
-                                                 (32, 8, 8, 128, 8, False)])
+                                                 (32, 8, 8, 128, 8, False), (40, 28, 4, 128, 7, True),
+                                                 (64, 4, 2, 64, 2, False), (33, 8, 8, 128, 3, True)])
 def test_rope_append_of_slabs_equals_rope_append_of_their_sum(dev, T, H, G, hd, slabs, bias):
     g = torch.Generator(device="cpu").manual_seed(T + H + hd)
     N = (H + 2 * G) * hd
-    partial = torch.randn((slabs, 32, N), generator=g).to(dev)
+    partial = torch.randn((slabs, ops.slab_rows(T), N), generator=g).to(dev)
     b = torch.randn(N, generator=g).half().to(dev) if bias else None
     P, cap = 50, 128
     len_dev = torch.tensor([P], dtype=torch.int32, device=dev)

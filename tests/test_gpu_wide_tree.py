@@ -88,7 +88,7 @@ def test_fused_step_of_a_wide_tree(dev, name, T):
                                      s2["model"], s2["cache"])[0]
     ver = run_verifier(s, dev, graph=False)
     assert ver.wide and tuple(ver.mask_bits.shape) == (T, 2)
-    assert ver.slab == {"qkv": 0, "o": 0, "down": 0}
+    assert ver.slab == eagle.slab_plan(s["model"], T)       # the library's choice, as for 32 tokens
     ver.step()
     torch.cuda.synchronize()
     assert rel_err(ver.logits.cpu().numpy(), ref_logits.cpu().numpy()) <= TOL

@@ -184,22 +184,28 @@ def test_slab_form_entry_points_reject_bad_arguments():
     assert L.eagle_qmm_slab_steps(32, 4608, 3584) == 8 and L.eagle_qmm_slab_steps(32, 3584, 18944) == 32
     assert L.eagle_qmm_slab_steps(8, 4096, 4096) == 8 and L.eagle_qmm_slab_steps(32, 4096, 14336) == 32
     assert L.eagle_qmm_slab_steps(32, 37888, 3584) == 0 and L.eagle_qmm_slab_steps(32, 152064, 3584) == 0
-    assert L.eagle_qmm_slab_steps(32, 1152, 896) == 0 and L.eagle_qmm_slab_steps(33, 4608, 3584) == 0
+    assert L.eagle_qmm_slab_steps(32, 1152, 896) == 0 and L.eagle_qmm_slab_steps(65, 4608, 3584) == 0
+    # 33..64 rows (a tree above 32 tokens): the same choice, partial tiles of 64 rows
+    assert L.eagle_qmm_slab_steps(40, 4608, 3584) == 8 and L.eagle_qmm_slab_steps(64, 3584, 18944) == 32
+    assert L.eagle_qmm_slab_partial_bytes_rows(32, 4608, 3584, 8) == 7 * 32 * 4608 * 4
+    assert L.eagle_qmm_slab_partial_bytes_rows(33, 4608, 3584, 8) == 7 * 64 * 4608 * 4
+    assert L.eagle_qmm_slab_partial_bytes_rows(65, 4608, 3584, 8) == 0
     call = lambda **kw: L.eagle_qmm_slab_partial_w4g64(
         kw.get("x", p), p, p, p, kw.get("partial", p), kw.get("bytes", big), kw.get("M", 32), kw.get("N", 128),
         kw.get("K", 1024), kw.get("gs", 64), kw.get("bits", 4), kw.get("steps", 8), None)
     assert call(x=None) == 1 and call(partial=None) == 1
-    assert call(M=33) == 2 and call(N=100) == 2 and call(K=832) == 2 and call(steps=12) == 2
+    assert call(M=65) == 2 and call(N=100) == 2 and call(K=832) == 2 and call(steps=12) == 2
+    assert call(M=33, bytes=2 * 32 * 128 * 4) == 5
     assert call(x=p + 2) == 3
     assert call(gs=32) == 4
     assert call(bytes=1024) == 5
     assert L.eagle_slab_sum_f16(p, 0, None, p, 8, 128, None) == 2
-    assert L.eagle_slab_sum_f16(p, 2, None, p, 33, 128, None) == 2
+    assert L.eagle_slab_sum_f16(p, 2, None, p, 65, 128, None) == 2
     assert L.eagle_slab_sum_f16(p, 2, p + 2, p, 8, 128, None) == 3
-    assert L.eagle_rmsnorm_slabs_f16(p, 2, None, p, 1e-6, None, p, 33, 128, None) == 2
+    assert L.eagle_rmsnorm_slabs_f16(p, 2, None, p, 1e-6, None, p, 65, 128, None) == 2
     assert L.eagle_rmsnorm_slabs_f16(p, 0, None, p, 1e-6, None, p, 8, 128, None) == 2
     assert L.eagle_rmsnorm_slabs_f16(p, 2, p, p, 1e-6, None, p, 8, 128, None) == 1     # residual needs h_out
-    assert L.eagle_rope_kv_append_slabs_f16(p, 2, None, p, p, p, p, p, 33, 4, 2, 64, 100, None) == 2
+    assert L.eagle_rope_kv_append_slabs_f16(p, 2, None, p, p, p, p, p, 65, 4, 2, 64, 100, None) == 2
     assert L.eagle_rope_kv_append_slabs_f16(p, 2, None, p, p, p, p, p, 8, 4, 3, 64, 100, None) == 2
     assert L.eagle_rope_kv_append_slabs_f16(p, 2, p + 2, p, p, p, p, p, 8, 4, 2, 64, 100, None) == 3
     assert L.eagle_rope_kv_append_slabs_f16(None, 2, None, p, p, p, p, p, 8, 4, 2, 64, 100, None) == 1
