@@ -34,7 +34,8 @@ enum eagle_status {
   EAGLE_ERR_ARCH = 7         /* current device is not gfx950 */
 };
 
-#define EAGLE_MAX_TREE 32    /* tree tokens per fused verify step (root + 31 nodes): matmul rows, one mask word */
+#define EAGLE_MAX_TREE 32    /* tree tokens per matmul launch and mask word (root + 31 nodes); larger trees take
+                                two mask words and the entry points that say so */
 #define EAGLE_MAX_TREE_SLOTS 64 /* tree tokens the tree-layout kernels take (root + 63 nodes; the reference's
                                    default is 39 nodes, mlx_eagle.py:390,510) */
 #define EAGLE_MAX_CHUNK 1024 /* rows of one causal pass over a prompt chunk */

@@ -12,8 +12,8 @@ import torch
 from . import _lib, ops
 from .layer import emit_layer
 
-MAXT = 32            # tree tokens of the fused verification step (matmul rows, one mask word)
-TREE_SLOTS = 64      # tree tokens the tree-layout kernels and the module path take
+MAXT = 32            # tree tokens per matmul launch and per mask word; larger trees: two of each
+TREE_SLOTS = 64      # tree tokens the tree-layout kernels, the module path and the fused step take
 
 
 def _ptr(t):
@@ -244,10 +244,9 @@ def accept_candidate(cache, accept_indices, accept_length, offset):
 
 
 def _check_tree_size(verify_num_tokens):
-    """The tree kernels lay a tree out in 64 slots (root + 63 nodes): the reference's default of
-    39 nodes (mlx_eagle.py:390,510) runs on the module path (matmuls of more than 32 rows as
-    tiled GEMMs, attention over two mask words per query in pieces of 32 queries); the fused
-    `TreeVerifier` / `SpeculativeDecoder` step takes 32 tree tokens."""
+    """The tree kernels lay a tree out in 64 slots (root + 63 nodes), which covers the reference's
+    default of 39 nodes (mlx_eagle.py:390,510): above 32 tokens the matmuls run as two passes of
+    32 rows and attention over two mask words per query in pieces of 32 queries."""
     if verify_num_tokens + 1 > TREE_SLOTS:
         raise NotImplementedError(
             f"verify_num_tokens={verify_num_tokens}: this build verifies at most {TREE_SLOTS - 1} draft nodes "
