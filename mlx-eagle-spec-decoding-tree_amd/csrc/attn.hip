@@ -33,9 +33,17 @@ namespace {
 constexpr int KT = 32;   // keys per tile
 
 // splits that get work when `ntiles` key tiles are dealt to a grid of `nsplit` splits
-__host__ __device__ inline int active_splits(int ntiles, int nsplit) {
+// `lanes` = KV groups x pieces of query rows, the (group, piece) pairs that share the GPU: with
+// many of them (a prompt chunk) the keys are split less, so that the launch has about
+// SPLIT_TARGET_WGS workgroups in all and each covers more tiles per partial result it writes
+// (8B shape, 512-row chunk, us per launch pair with 2 / 4 / 8 / 16 tiles at least: 33 / 29 / 33 / 44
+// on an empty cache, 94 / 78 / 70 / 66 behind 1536 rows).
+constexpr int SPLIT_TARGET_WGS = 512;
+__host__ __device__ inline int active_splits(int ntiles, int nsplit, int lanes = 1) {
   int tpw = (ntiles + nsplit - 1) / nsplit;
-  if (tpw < 2) tpw = 2;
+  int min_tiles = (lanes * ntiles + SPLIT_TARGET_WGS - 1) / SPLIT_TARGET_WGS;
+  if (min_tiles < 2) min_tiles = 2;
+  if (tpw < min_tiles) tpw = min_tiles;
   return (ntiles + tpw - 1) / tpw;
 }
 
@@ -107,7 +115,7 @@ __global__ __launch_bounds__(512) void tree_attn_split_kernel(
   // least (with one, writing and merging the partials costs more than reading the keys).
   // The tile count of the busiest workgroup sets the time, so the tiles are spread evenly
   // over exactly as many workgroups as that takes; the rest of the grid leaves at once.
-  const int nactive = active_splits(ntiles, nsplit);
+  const int nactive = active_splits(ntiles, nsplit, gridDim.x * gridDim.z);
   if (split >= nactive) return;
   half8_t qreg[KSTEPS];
 #pragma unroll
@@ -331,7 +339,7 @@ __global__ void tree_attn_merge_kernel(const half_t* __restrict__ part_o,
                                        const float* __restrict__ part_ml,
                                        half_t* __restrict__ out, int T, int H, int nsplit,
                                        const int32_t* __restrict__ len_dev, long cap,
-                                       int Tk, int q_rows, int len_stride) {
+                                       int Tk, int q_rows, int len_stride, int groups) {
   const int piece = blockIdx.z;                     // as in the split kernel
   if (T > q_rows - piece * 32) T = q_rows - piece * 32;
   part_o += (long)piece * H * nsplit * 32 * HD;
@@ -369,7 +377,7 @@ __global__ void tree_attn_merge_kernel(const half_t* __restrict__ part_o,
   int P = len_dev[piece * len_stride];
   if (P > cap - Tk) P = (int)(cap - Tk);    // as in the split kernel
   if (P < 0) P = 0;
-  const int nact = active_splits((P + Tk + KT - 1) / KT, nsplit);   // as in the split kernel
+  const int nact = active_splits((P + Tk + KT - 1) / KT, nsplit, groups * gridDim.z);   // as in the split kernel
 #pragma unroll
   for (int k = 0; k < TPW; ++k) {
     const float m = lane < nact ? ml[k][0] : -INFINITY;
@@ -437,7 +445,7 @@ int launch_attention(const half_t* q, half_t* kc, half_t* vc, const uint32_t* bi
                      q_rows, len_stride);
   hipLaunchKernelGGL(tree_attn_merge_kernel<HD>, dim3(H, (T + MERGE_TOK - 1) / MERGE_TOK, pieces),
                      dim3(MERGE_TOK * HD / 4), 0, st, part_o, part_ml, (half_t*)out, T, H, nsplit,
-                     len, cap, Tk, q_rows, len_stride);
+                     len, cap, Tk, q_rows, len_stride, G);
   return eagle_launch_status();
 }
 
