@@ -282,7 +282,8 @@ int eagle_rope_kv_append_f16(const void* q_lin, const void* k_lin, const void* v
  *   tree_mask_bits [T] uint32: bit j of word i set iff tree token j is visible
  *   to tree token i; prefix rows are visible to every token.
  *   out [T,H*hd] fp16 = softmax(scale*q.k + mask) v, laid out for o_proj.
- * hd must be 64 or 128.  Replaces scaled_dot_product_attention with the additive
+ * hd must be 64 or 128, scale positive (this and the other attention entry points return
+ * EAGLE_ERR_SHAPE otherwise).  Replaces scaled_dot_product_attention with the additive
  * tree mask (mlx_llama.py:185-195, mask from mlx_eagle.py:337-338).
  * ------------------------------------------------------------------------- */
 /* max_len bounds prefix + tree rows (P + T) for every launch that uses the workspace. */

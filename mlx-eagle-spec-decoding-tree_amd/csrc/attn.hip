@@ -31,6 +31,16 @@
 namespace {
 
 constexpr int KT = 32;   // keys per tile
+constexpr float M_FLOOR = -3.0e38f;   // running maximum of a row that has seen no key yet
+
+// ds_read_b64_tr_b16: 16 lanes x 4 halves, transposed (lane i of a group of 16 receives element
+// i % 4 of the lanes 4 j + i / 4, j = 0..3 of the group); the address is 8-byte aligned
+typedef __fp16 fp16x4_t __attribute__((__vector_size__(4 * sizeof(__fp16))));
+__device__ inline half4_t lds_read_tr16(const unsigned char* p) {
+  const fp16x4_t v = __builtin_amdgcn_ds_read_tr16_b64_v4f16(
+      (__attribute__((address_space(3))) fp16x4_t*)(p));
+  return __builtin_bit_cast(half4_t, v);
+}
 
 // splits that get work when `ntiles` key tiles are dealt to a grid of `nsplit` splits
 // `lanes` = KV groups x pieces of query rows, the (group, piece) pairs that share the GPU: with
@@ -67,7 +77,14 @@ __device__ inline void rotate_pair(half8_t& lo, half8_t& hi, const float* cs) {
 // taken from k_lin / v_lin instead of the cache, and the workgroup that owns a tile with tree
 // rows appends them to the cache (every tile has exactly one owner per KV group, and no
 // workgroup reads a cache row at or beyond P, so the append races with nothing).
-template <int HD, bool ROPE, bool WIDE = false>
+// NVU: 16-byte vectors of a K (or V) tile per thread, a power of two with NVU * blockDim.x >= the
+// vectors of a tile.  DEPTH: tiles requested ahead, each in registers of its own (a tile's way
+// from the L2 into LDS takes longer than its arithmetic: with one tile ahead the loop runs at one
+// load latency per tile).
+template <int V>
+struct Stage { static constexpr int value = V; };
+
+template <int HD, bool ROPE, bool WIDE, int NVU, int DEPTH>
 __global__ __launch_bounds__(512) void tree_attn_split_kernel(
     const half_t* __restrict__ q, half_t* kc, half_t* vc,
     const uint32_t* __restrict__ mask_bits, const int32_t* __restrict__ len_dev,
@@ -132,7 +149,10 @@ __global__ __launch_bounds__(512) void tree_attn_split_kernel(
   const uint32_t mybits = ql < T ? (mask_bits ? mask_bits[WIDE ? 2 * qrow : ql] : (2u << ql) - 1u) : 0u;
   const uint32_t mybits_hi = (WIDE && ql < T && mask_bits) ? mask_bits[2 * qrow + 1] : 0u;
 
-  float m_run = -INFINITY, l_run = 0.f;
+  float m_run = M_FLOOR, l_run = 0.f;
+  // this lane's address for the transposing loads of V (see the O^T step below)
+  const unsigned char* vt_base =
+      ldsV + (4 * hb + ((lane & 15) >> 2)) * STR + (16 * ((lane >> 4) & 1) + 4 * (lane & 3)) * 2;
   float16_t o_acc[DB];
 #pragma unroll
   for (int db = 0; db < DB; ++db)
@@ -144,17 +164,16 @@ __global__ __launch_bounds__(512) void tree_attn_split_kernel(
   const half_t* klin = ROPE ? k_lin + (long)g * HD : nullptr;
   const half_t* vlin = ROPE ? v_lin + (long)g * HD : nullptr;
 
-  // This workgroup's tiles are split, split + nsplit, ...: all workgroups share the live part
-  // of the cache however short it is.  The next tile is fetched into registers while the
-  // current one is being used.
+  // This workgroup's tiles are split, split + nactive, ...: all workgroups share the live part
+  // of the cache however short it is.  The next DEPTH tiles are in flight into registers while
+  // the current one is being used.
   constexpr int NVEC = KT * VEC_ROW;                 // 16-byte vectors per K (or V) tile
-  constexpr int NV = NVEC / 64;                      // per thread, for as little as one wave
-  half8_t kreg[NV], vreg[NV];
-  auto fetch = [&](int tile) {
+  half8_t kreg[DEPTH][NVU], vreg[DEPTH][NVU];
+  auto fetch = [&](auto S, int tile) {
+    constexpr int st = decltype(S)::value;
     const int kb = tile * KT;
 #pragma unroll
-    for (int it = 0; it < NV; ++it) {
-      if (it * nthr >= NVEC) break;
+    for (int it = 0; it < NVU; ++it) {
       int v = tid + it * nthr;
       if (v > NVEC - 1) v = NVEC - 1;
       const int row = v / VEC_ROW;
@@ -167,25 +186,36 @@ __global__ __launch_bounds__(512) void tree_attn_split_kernel(
         kp = klin + (long)(kidx - P) * ld;
         vp = vlin + (long)(kidx - P) * ld;
       }
-      kreg[it] = *reinterpret_cast<const half8_t*>(kp + c * 8);
-      vreg[it] = *reinterpret_cast<const half8_t*>(vp + c * 8);
+      kreg[st][it] = *reinterpret_cast<const half8_t*>(kp + c * 8);
+      vreg[st][it] = *reinterpret_cast<const half8_t*>(vp + c * 8);
     }
   };
-  auto stash = [&]() {
+  auto stash = [&](auto S) {
+    constexpr int st = decltype(S)::value;
 #pragma unroll
-    for (int it = 0; it < NV; ++it) {
-      if (it * nthr >= NVEC) break;
+    for (int it = 0; it < NVU; ++it) {
       const int v = tid + it * nthr;
       if (v < NVEC) {
         const int row = v / VEC_ROW;
         const int c = v % VEC_ROW;
-        *reinterpret_cast<half8_t*>(ldsK + row * STR + c * 16) = kreg[it];
-        *reinterpret_cast<half8_t*>(ldsV + row * STR + c * 16) = vreg[it];
+        *reinterpret_cast<half8_t*>(ldsK + row * STR + c * 16) = kreg[st][it];
+        *reinterpret_cast<half8_t*>(ldsV + row * STR + c * 16) = vreg[st][it];
       }
     }
   };
 
-  fetch(split);
+  // Every fetch is issued whether or not its tile exists (the index is clamped to the last
+  // tile, whose rows are in the cache): with a fetch under a condition the compiler no longer
+  // knows how many loads are outstanding where a stage is waited for, and waits for all of them.
+  auto tile_at = [&](int t) { return t < ntiles ? t : ntiles - 1; };
+  // (and the stages are requested in the order in which they are waited for, here as in the loop)
+  __builtin_amdgcn_sched_barrier(0);
+  fetch(Stage<0>{}, split);
+  __builtin_amdgcn_sched_barrier(0);
+  if constexpr (DEPTH > 1) fetch(Stage<1>{}, tile_at(split + nactive));
+  __builtin_amdgcn_sched_barrier(0);
+  if constexpr (DEPTH > 2) fetch(Stage<2>{}, tile_at(split + 2 * nactive));
+  __builtin_amdgcn_sched_barrier(0);
   if (ROPE) {
     for (int v = tid; v < T * HALF / 2; v += nthr)
       *reinterpret_cast<float4_t*>(cs_lds + 4 * v) = *reinterpret_cast<const float4_t*>(rope_cs + 4 * v);
@@ -196,22 +226,24 @@ __global__ __launch_bounds__(512) void tree_attn_split_kernel(
         rotate_pair(qreg[kk], qreg[kk + KSTEPS / 2], cs_lds + (ql * HALF + kk * 16 + hb * 8) * 2);
     }
   }
-  for (int tile = split; tile < ntiles; tile += nactive) {
+  // one tile: its registers (stage S) into LDS, the tile DEPTH ahead requested into the same
+  // registers, then the arithmetic on LDS
+  auto do_tile = [&](auto S, int tile) {
+    constexpr int st = decltype(S)::value;
     const int kb = tile * KT;
     __syncthreads();   // every wave is done with the previous tile
     if (ROPE && kb + KT > P) {
       // tree rows: append the values as they are
 #pragma unroll
-      for (int it = 0; it < NV; ++it) {
-        if (it * nthr >= NVEC) break;
+      for (int it = 0; it < NVU; ++it) {
         const int v = tid + it * nthr;
         const int kidx = kb + v / VEC_ROW;
         if (v < NVEC && kidx >= P && kidx < Ltot)
-          *reinterpret_cast<half8_t*>(vc + ((long)g * cap + kidx) * HD + (v % VEC_ROW) * 8) = vreg[it];
+          *reinterpret_cast<half8_t*>(vc + ((long)g * cap + kidx) * HD + (v % VEC_ROW) * 8) = vreg[st][it];
       }
     }
-    stash();
-    if (tile + nactive < ntiles) fetch(tile + nactive);
+    stash(S);
+    fetch(S, tile_at(tile + DEPTH * nactive));
     __syncthreads();
     if (ROPE && kb + KT > P) {
       // rotate the tree keys in LDS (one thread per pair of 16-byte pieces) and append them
@@ -243,14 +275,16 @@ __global__ __launch_bounds__(512) void tree_attn_split_kernel(
       sacc = __builtin_amdgcn_mfma_f32_32x32x16_f16(a, qreg[kk], sacc, 0, 0, 0);
     }
 
-    // accumulator register i of this lane is key 8*(i/4) + 4*hb + i%4 of the tile
+    // accumulator register i of this lane is key 8*(i/4) + 4*hb + i%4 of the tile.  The scores
+    // stay unscaled: the scale (> 0) goes into the exponent's fused multiply-add, and the running
+    // maximum starts at a finite floor instead of -inf, so that no case needs a select.
     float sv[16];
-    float bm = -INFINITY;
+    float bm = M_FLOOR;
     if (kb + KT <= P) {
       // a tile of prefix rows: visible to every token, no mask arithmetic
 #pragma unroll
       for (int i = 0; i < 16; ++i) {
-        sv[i] = sacc[i] * scale_log2e;
+        sv[i] = sacc[i];
         bm = fmaxf(bm, sv[i]);
       }
     } else {
@@ -259,27 +293,22 @@ __global__ __launch_bounds__(512) void tree_attn_split_kernel(
         const int key = kb + 8 * (i >> 2) + 4 * hb + (i & 3);
         const int rel = key - P;
         const uint32_t word = (WIDE && rel >= 32) ? mybits_hi : mybits;
-        const bool vis = (key < P) || (key < Ltot && ((word >> (rel & 31)) & 1u));
-        sv[i] = vis ? sacc[i] * scale_log2e : -INFINITY;
+        // (bitwise, not short-circuit: straight-line selects instead of a branch per key)
+        const bool vis = (rel < 0) | ((key < Ltot) & (((word >> (rel & 31)) & 1u) != 0u));
+        sv[i] = vis ? sacc[i] : -INFINITY;
         bm = fmaxf(bm, sv[i]);
       }
     }
     bm = fmaxf(bm, __shfl_xor(bm, 32, 64));
-    const float m_new = fmaxf(m_run, bm);
-    float alpha = 1.f;
+    const float m_new = fmaxf(m_run, bm * scale_log2e);
+    // arguments are <= 0: the bare hardware exp2 (results below 2^-126 flush to zero, -inf gives 0)
+    const float alpha = __builtin_amdgcn_exp2f(m_run - m_new);
     float psum = 0.f;
     float p[16];
-    if (m_new == -INFINITY) {
 #pragma unroll
-      for (int i = 0; i < 16; ++i) p[i] = 0.f;
-    } else {
-      // arguments are <= 0: the bare hardware exp2 (results below 2^-126 flush to zero)
-      alpha = __builtin_amdgcn_exp2f(m_run - m_new);
-#pragma unroll
-      for (int i = 0; i < 16; ++i) {
-        p[i] = __builtin_amdgcn_exp2f(sv[i] - m_new);
-        psum += p[i];
-      }
+    for (int i = 0; i < 16; ++i) {
+      p[i] = __builtin_amdgcn_exp2f(fmaf(sv[i], scale_log2e, -m_new));
+      psum += p[i];
     }
     psum += __shfl_xor(psum, 32, 64);
     l_run = l_run * alpha + psum;
@@ -292,7 +321,10 @@ __global__ __launch_bounds__(512) void tree_attn_split_kernel(
     }
 
     // O^T[d][token] += sum_key V[key][d] P[token][key]; step u covers accumulator
-    // registers 8u..8u+7, i.e. keys 8*(2u + j/4) + 4*hb + j%4, j = 0..7.
+    // registers 8u..8u+7, i.e. keys 8*(2u + j/4) + 4*hb + j%4, j = 0..7.  The V^T operand comes
+    // from the row-major tile through the transposing LDS load: within 16 lanes, lane i receives
+    // element i % 4 of the four lanes 4 jj + i / 4, so lane s of a group asks for key row s / 4
+    // at the four d columns 4 (s % 4) .. + 3 of the group's 16 and gets four keys of its own d.
 #pragma unroll
     for (int u = 0; u < 2; ++u) {
       half8_t bp;
@@ -300,14 +332,26 @@ __global__ __launch_bounds__(512) void tree_attn_split_kernel(
       for (int j = 0; j < 8; ++j) bp[j] = (half_t)p[8 * u + j];
 #pragma unroll
       for (int db = 0; db < DB; ++db) {
-        half8_t a;
-#pragma unroll
-        for (int j = 0; j < 8; ++j) {
-          const int key = 8 * (2 * u + (j >> 2)) + 4 * hb + (j & 3);
-          a[j] = *reinterpret_cast<const half_t*>(ldsV + key * STR + (db * 32 + ql) * 2);
-        }
+        const half4_t lo = lds_read_tr16(vt_base + (16 * u) * STR + db * 64);
+        const half4_t hi = lds_read_tr16(vt_base + (16 * u + 8) * STR + db * 64);
+        const half8_t a = half8_t{lo[0], lo[1], lo[2], lo[3], hi[0], hi[1], hi[2], hi[3]};
         o_acc[db] = __builtin_amdgcn_mfma_f32_32x32x16_f16(a, bp, o_acc[db], 0, 0, 0);
       }
+    }
+  };
+  // whole rounds of DEPTH tiles (no condition between the stages of a round, so that the loads
+  // outstanding at every wait are known), then the last DEPTH - 1 tiles at most
+  int t0 = split;
+  for (; t0 + (DEPTH - 1) * nactive < ntiles; t0 += DEPTH * nactive) {
+    do_tile(Stage<0>{}, t0);
+    if constexpr (DEPTH > 1) do_tile(Stage<1>{}, t0 + nactive);
+    if constexpr (DEPTH > 2) do_tile(Stage<2>{}, t0 + 2 * nactive);
+  }
+  if constexpr (DEPTH > 1) {
+    if (t0 < ntiles) {
+      do_tile(Stage<0>{}, t0);
+      if constexpr (DEPTH > 2)
+        if (t0 + nactive < ntiles) do_tile(Stage<1>{}, t0 + nactive);
     }
   }
 
@@ -369,15 +413,27 @@ __global__ void tree_attn_merge_kernel(const half_t* __restrict__ part_o,
   const int t = blockIdx.y * MERGE_TOK + tl;
   const int t_c = t < T ? t : T - 1;
   const half_t* src = part_o + ((long)head * nsplit * 32 + t_c) * HD + dq * 4;
+  // One or two pieces of query rows (the tree step: most splits of the grid are active): every
+  // split's partial output is requested before the length is known.  More pieces (a prompt
+  // chunk: a few active splits out of a grid sized for the longest cache): only the active
+  // ones, after it (8B shape, 16 pieces behind 1536 cache rows: 20 -> 9 us).
+  const bool eager = gridDim.z <= 2;
   half4_t pre[PRE];
+  if (eager) {
 #pragma unroll
-  for (int k = 0; k < PRE; ++k)
-    if (k < nsplit) pre[k] = *reinterpret_cast<const half4_t*>(src + (long)k * 32 * HD);
+    for (int k = 0; k < PRE; ++k)
+      if (k < nsplit) pre[k] = *reinterpret_cast<const half4_t*>(src + (long)k * 32 * HD);
+  }
 
   int P = len_dev[piece * len_stride];
   if (P > cap - Tk) P = (int)(cap - Tk);    // as in the split kernel
   if (P < 0) P = 0;
   const int nact = active_splits((P + Tk + KT - 1) / KT, nsplit, groups * gridDim.z);   // as in the split kernel
+  if (!eager) {
+#pragma unroll
+    for (int k = 0; k < PRE; ++k)
+      if (k < nact) pre[k] = *reinterpret_cast<const half4_t*>(src + (long)k * 32 * HD);
+  }
 #pragma unroll
   for (int k = 0; k < TPW; ++k) {
     const float m = lane < nact ? ml[k][0] : -INFINITY;
@@ -440,9 +496,17 @@ int launch_attention(const half_t* q, half_t* kc, half_t* vc, const uint32_t* bi
   const float sl2 = scale * 1.4426950408889634f;
   const int rep = H / G;
   const size_t lds = 2 * KT * (HD * 2 + 16) + (ROPE ? (size_t)EAGLE_MAX_TREE * HD * 4 : 0);
-  hipLaunchKernelGGL((tree_attn_split_kernel<HD, ROPE, WIDE>), dim3(G, nsplit, pieces), dim3(rep * 64), lds,
-                     st, q, kc, vc, bits, len, part_o, part_ml, T, H, G, cap, 0, sl2, k_lin, v_lin, ld, cs, Tk,
-                     q_rows, len_stride);
+  // vectors of a tile per thread (a power of two) and the tiles in flight that its registers allow
+  const int need = (KT * (HD / 8) + rep * 64 - 1) / (rep * 64);
+#define EAGLE_ATTN_SPLIT(NVU, DEPTH)                                                                     \
+  hipLaunchKernelGGL((tree_attn_split_kernel<HD, ROPE, WIDE, NVU, ROPE ? 1 : DEPTH>), dim3(G, nsplit, pieces), \
+                     dim3(rep * 64), lds, st, q, kc, vc, bits, len, part_o, part_ml, T, H, G, cap, 0, sl2,      \
+                     k_lin, v_lin, ld, cs, Tk, q_rows, len_stride)
+  if (need <= 1) EAGLE_ATTN_SPLIT(1, 3);
+  else if (need <= 2) EAGLE_ATTN_SPLIT(2, 3);
+  else if (need <= 4) EAGLE_ATTN_SPLIT(4, 2);
+  else EAGLE_ATTN_SPLIT(8, 1);
+#undef EAGLE_ATTN_SPLIT
   hipLaunchKernelGGL(tree_attn_merge_kernel<HD>, dim3(H, (T + MERGE_TOK - 1) / MERGE_TOK, pieces),
                      dim3(MERGE_TOK * HD / 4), 0, st, part_o, part_ml, (half_t*)out, T, H, nsplit,
                      len, cap, Tk, q_rows, len_stride, G);
@@ -478,7 +542,7 @@ EAGLE_EXPORT int eagle_tree_attention_f16(const void* q, const void* k_cache, co
                                           eagle_stream_t stream) {
   if (!q || !k_cache || !v_cache || !tree_mask_bits || !cache_len_dev || !out) return EAGLE_ERR_NULL;
   if (T < 1 || T > EAGLE_MAX_TREE || H < 1 || G < 1 || (H % G) != 0 || (H / G) > 8 ||
-      (hd != 64 && hd != 128) || max_len < T || max_len > capacity)
+      (hd != 64 && hd != 128) || max_len < T || max_len > capacity || !(scale > 0.f))
     return EAGLE_ERR_SHAPE;
   if (!eagle_aligned16(q) || !eagle_aligned16(k_cache) || !eagle_aligned16(v_cache) ||
       !eagle_aligned16(out))
@@ -505,7 +569,7 @@ EAGLE_EXPORT int eagle_draft_attention_f16(const void* q, const void* k_cache, c
                                            size_t workspace_bytes, eagle_stream_t stream) {
   if (!q || !k_cache || !v_cache || !mask_words || !cache_len_dev || !out) return EAGLE_ERR_NULL;
   if (T < 1 || T > EAGLE_MAX_TREE || Tk < 1 || Tk > 2 * EAGLE_MAX_TREE || H < 1 || G < 1 ||
-      (H % G) != 0 || (H / G) > 8 || (hd != 64 && hd != 128) || max_len < Tk || max_len > capacity)
+      (H % G) != 0 || (H / G) > 8 || (hd != 64 && hd != 128) || max_len < Tk || max_len > capacity || !(scale > 0.f))
     return EAGLE_ERR_SHAPE;
   if (!eagle_aligned16(q) || !eagle_aligned16(k_cache) || !eagle_aligned16(v_cache) ||
       !eagle_aligned16(out))
@@ -537,7 +601,7 @@ EAGLE_EXPORT int eagle_tree_attention_wide_f16(const void* q, const void* k_cach
                                                size_t workspace_bytes, eagle_stream_t stream) {
   if (!q || !k_cache || !v_cache || !mask_words || !cache_len_dev || !out) return EAGLE_ERR_NULL;
   if (T < 1 || T > EAGLE_MAX_TREE_SLOTS || Tk < 1 || Tk > EAGLE_MAX_TREE_SLOTS || H < 1 || G < 1 ||
-      (H % G) != 0 || (H / G) > 8 || (hd != 64 && hd != 128) || max_len < Tk || max_len > capacity)
+      (H % G) != 0 || (H / G) > 8 || (hd != 64 && hd != 128) || max_len < Tk || max_len > capacity || !(scale > 0.f))
     return EAGLE_ERR_SHAPE;
   if (!eagle_aligned16(q) || !eagle_aligned16(k_cache) || !eagle_aligned16(v_cache) ||
       !eagle_aligned16(out))
@@ -572,7 +636,7 @@ EAGLE_EXPORT int eagle_causal_attention_f16(const void* q, const void* k_cache, 
                                             eagle_stream_t stream) {
   if (!q || !k_cache || !v_cache || !piece_len_dev || !out) return EAGLE_ERR_NULL;
   if (R < 32 || (R % 32) != 0 || R > EAGLE_MAX_CHUNK || H < 1 || G < 1 || (H % G) != 0 ||
-      (H / G) > 8 || (hd != 64 && hd != 128) || max_len < 32 || max_len > capacity)
+      (H / G) > 8 || (hd != 64 && hd != 128) || max_len < 32 || max_len > capacity || !(scale > 0.f))
     return EAGLE_ERR_SHAPE;
   if (!eagle_aligned16(q) || !eagle_aligned16(k_cache) || !eagle_aligned16(v_cache) ||
       !eagle_aligned16(out))
@@ -622,7 +686,7 @@ EAGLE_EXPORT int eagle_tree_attention_rope_f16(const void* q_lin, const void* k_
     return EAGLE_ERR_NULL;
   if (T < 1 || T > EAGLE_MAX_TREE || H < 1 || G < 1 || (H % G) != 0 || (H / G) > 8 ||
       (hd != 64 && hd != 128) || max_len < T || max_len > capacity || row_stride < hd ||
-      (row_stride % 8) != 0)
+      (row_stride % 8) != 0 || !(scale > 0.f))
     return EAGLE_ERR_SHAPE;
   if (!eagle_aligned16(q_lin) || !eagle_aligned16(k_lin) || !eagle_aligned16(v_lin) ||
       !eagle_aligned16(rope_cs) || !eagle_aligned16(k_cache) || !eagle_aligned16(v_cache) ||
