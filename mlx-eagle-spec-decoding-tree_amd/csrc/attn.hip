@@ -118,7 +118,8 @@ __global__ __launch_bounds__(512) void tree_attn_split_kernel(
   // piece may hold fewer).  The pieces of a causal pass have a cache length each (len_stride 1),
   // those of a tree of more than 32 tokens share one length and the masked rows (len_stride 0,
   // mask words of query row 32 * piece + ql); a single piece otherwise.
-  const int piece = blockIdx.z;
+  // (the last piece of a causal pass sees the most keys: dispatched first)
+  const int piece = gridDim.z - 1 - blockIdx.z;
   const int qrow = piece * 32 + (lane & 31);
   if (!ROPE && T > q_rows - piece * 32) T = q_rows - piece * 32;
   int P = len_dev[piece * len_stride];
@@ -490,7 +491,12 @@ int launch_attention(const half_t* q, half_t* kc, half_t* vc, const uint32_t* bi
                      int Tk = 0, int pieces = 1, int q_rows = 0, int len_stride = 1) {
   if (!WIDE) Tk = T;
   if (q_rows == 0) q_rows = pieces * T;
-  const int nsplit = splits_for(max_len, G);
+  // The grid holds as many splits as the longest length makes active: a workgroup without
+  // work still takes a slot for the 2 us in which it learns that from the cache length, and
+  // thousands of them ahead of the last pieces' workgroups (a chunk of 16 pieces in a grid of 36
+  // splits for 4 active ones) held those back by 18 of 44 us.
+  int nsplit = splits_for(max_len, G);
+  nsplit = active_splits((max_len + KT - 1) / KT, nsplit, G * pieces);
   float* part_ml = static_cast<float*>(workspace);
   half_t* part_o = reinterpret_cast<half_t*>(part_ml + (size_t)pieces * H * nsplit * 32 * 2);
   const float sl2 = scale * 1.4426950408889634f;
