@@ -433,8 +433,27 @@ def main():
     if parity is not None:
         line["parity"] = parity
     if not opt.headline_only:
-        # the other two workloads, driver-timed in the same run (their own keys; the headline
-        # keys above are untouched)
+        # the other workloads, driver-timed in the same run (their own keys; the headline keys
+        # above are untouched)
+        if NODES <= 32:
+            # the same step on a tree of the reference's default size (39 draft nodes, mlx_eagle.py:390,510)
+            wt = 40
+            wparents = synth.random_tree(rng, wt)
+            wdepth, _, wbits = synth.tree_arrays(wparents)
+            wver = eagle.TreeVerifier(model, cache, total_tokens=wt - 1, max_len=cap)
+            wver.set_tree(torch.from_numpy(rng.integers(0, args.vocab_size, wt).astype(np.int32)).to(dev),
+                          torch.from_numpy(wdepth.astype(np.int32)).to(dev), torch.from_numpy(wparents).to(dev),
+                          torch.from_numpy(wbits.view(np.int32)).to(dev))
+
+            def wide_step():
+                wver.len_dev.copy_(len0)
+                wver.forward()
+
+            wt_ms, wgraph = graph_time_ms(torch, wide_step, reps=20)
+            line["wide_tree"] = {"metric": "tree_verify_step_ms at the reference's default tree size",
+                                 "tree_tokens": wt, "value": round(float(np.median(wt_ms)), 4), "unit": "ms",
+                                 "steps": 20}
+            del wver, wgraph
         del ver, graph, model, cache, weights
         torch.cuda.empty_cache()
         extra = argparse.Namespace(**vars(opt))
