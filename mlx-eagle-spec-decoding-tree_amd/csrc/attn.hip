@@ -44,17 +44,26 @@ __device__ inline half4_t lds_read_tr16(const unsigned char* p) {
 
 // splits that get work when `ntiles` key tiles are dealt to a grid of `nsplit` splits
 // `lanes` = KV groups x pieces of query rows, the (group, piece) pairs that share the GPU: with
-// many of them (a prompt chunk) the keys are split less, so that the launch has about
-// SPLIT_TARGET_WGS workgroups in all and each covers more tiles per partial result it writes
-// (8B shape, 512-row chunk, us per launch pair with 2 / 4 / 8 / 16 tiles at least: 33 / 29 / 33 / 44
-// on an empty cache, 94 / 78 / 70 / 66 behind 1536 rows).
-constexpr int SPLIT_TARGET_WGS = 512;
-__host__ __device__ inline int active_splits(int ntiles, int nsplit, int lanes = 1) {
+// many of them (a prompt chunk) the keys are split less, so that the launch has about as many
+// workgroups as the GPU holds at once (`slots`) and each covers more tiles per partial result
+// it writes (8B shape, 512-row chunk, us per launch pair with 2 / 4 / 8 / 16 tiles at least: 33 /
+// 29 / 33 / 44 on an empty cache, 94 / 78 / 70 / 66 behind 1536 rows).
+__host__ __device__ inline int active_splits(int ntiles, int nsplit, int lanes, int slots) {
   int tpw = (ntiles + nsplit - 1) / nsplit;
-  int min_tiles = (lanes * ntiles + SPLIT_TARGET_WGS - 1) / SPLIT_TARGET_WGS;
+  int min_tiles = (lanes * ntiles + slots - 1) / slots;
   if (min_tiles < 2) min_tiles = 2;
   if (tpw < min_tiles) tpw = min_tiles;
   return (ntiles + tpw - 1) / tpw;
+}
+
+// Workgroups of `rep` waves that the 256 compute units hold at once: the split kernel's registers
+// allow two waves per SIMD at head dimension 128 and three at 64.  One workgroup more than that
+// costs a second round (a tree of 40 tokens at seven heads per group: 264 workgroups, 20.6 us;
+// 176 workgroups, one round).
+__host__ __device__ inline int split_slots(int rep, int hd) {
+  const int waves_per_cu = hd > 64 ? 8 : 12;
+  const int per_cu = waves_per_cu / rep;
+  return 256 * (per_cu < 1 ? 1 : per_cu);
 }
 
 // (lo, hi) = elements i0..i0+7 and i0+half..i0+half+7 of a head vector; cs = 8 (cos, sin) pairs
@@ -133,7 +142,7 @@ __global__ __launch_bounds__(512) void tree_attn_split_kernel(
   // least (with one, writing and merging the partials costs more than reading the keys).
   // The tile count of the busiest workgroup sets the time, so the tiles are spread evenly
   // over exactly as many workgroups as that takes; the rest of the grid leaves at once.
-  const int nactive = active_splits(ntiles, nsplit, gridDim.x * gridDim.z);
+  const int nactive = active_splits(ntiles, nsplit, gridDim.x * gridDim.z, split_slots(rep, HD));
   if (split >= nactive) return;
   half8_t qreg[KSTEPS];
 #pragma unroll
@@ -429,7 +438,8 @@ __global__ void tree_attn_merge_kernel(const half_t* __restrict__ part_o,
   int P = len_dev[piece * len_stride];
   if (P > cap - Tk) P = (int)(cap - Tk);    // as in the split kernel
   if (P < 0) P = 0;
-  const int nact = active_splits((P + Tk + KT - 1) / KT, nsplit, groups * gridDim.z);   // as in the split kernel
+  const int nact = active_splits((P + Tk + KT - 1) / KT, nsplit, groups * gridDim.z,
+                                 split_slots(H / groups, HD));   // as in the split kernel
   if (!eager) {
 #pragma unroll
     for (int k = 0; k < PRE; ++k)
@@ -496,7 +506,7 @@ int launch_attention(const half_t* q, half_t* kc, half_t* vc, const uint32_t* bi
   // thousands of them ahead of the last pieces' workgroups (a chunk of 16 pieces in a grid of 36
   // splits for 4 active ones) held those back by 18 of 44 us.
   int nsplit = splits_for(max_len, G);
-  nsplit = active_splits((max_len + KT - 1) / KT, nsplit, G * pieces);
+  nsplit = active_splits((max_len + KT - 1) / KT, nsplit, G * pieces, split_slots(H / G, HD));
   float* part_ml = static_cast<float*>(workspace);
   half_t* part_o = reinterpret_cast<half_t*>(part_ml + (size_t)pieces * H * nsplit * 32 * 2);
   const float sl2 = scale * 1.4426950408889634f;
