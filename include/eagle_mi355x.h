@@ -38,7 +38,7 @@ enum eagle_status {
                                 two mask words and the entry points that say so */
 #define EAGLE_MAX_TREE_SLOTS 64 /* tree tokens the tree-layout kernels take (root + 63 nodes; the reference's
                                    default is 39 nodes, mlx_eagle.py:390,510) */
-#define EAGLE_MAX_CHUNK 1024 /* rows of one causal pass over a prompt chunk */
+#define EAGLE_MAX_CHUNK 2048 /* rows of one causal pass over a prompt chunk */
 #define EAGLE_MAX_M 32       /* rows of x accepted by the quantised matmul */
 
 const char* eagle_status_string(int status);

@@ -340,7 +340,8 @@ def test_device_loop_refuses_to_overrun_the_caches(dev):
         spec.SpeculativeDecoder(target, draft, capacity=128, k=8, depth=3, verify_num_tokens=64)
 
 
-@pytest.mark.parametrize("n,chunk,graphs", [(75, 512, True), (200, 64, False), (32, 512, True)])
+@pytest.mark.parametrize("n,chunk,graphs", [(75, 512, True), (200, 64, False), (32, 512, True),
+                                            (1100, 2048, True), (1300, 1024, False)])
 def test_chunked_prompt_pass_matches_oracle(dev, n, chunk, graphs):
     """spec.CausalPrefill: linear layers over the whole chunk (tiled GEMM form above 32 rows),
     attention per 32-row piece; cache rows and the last token's logits against the oracle."""
@@ -350,9 +351,10 @@ def test_chunked_prompt_pass_matches_oracle(dev, n, chunk, graphs):
     rng = np.random.default_rng(n)
     ids = rng.integers(0, args.vocab_size, n).astype(np.int32)
     inv, sc = synth.inv_freqs(args)
-    side = draft_oracle.Side(args, w, inv, sc, 320)
+    cap = max(320, n + 120)
+    side = draft_oracle.Side(args, w, inv, sc, cap)
     want = side.causal(ids)
-    cache = make_prompt_cache(model, capacity=320)
+    cache = make_prompt_cache(model, capacity=cap)
     pre = spec.CausalPrefill(model, cache, head=True, chunk=chunk, graphs=graphs)
     got = pre(to_dev(ids, dev)).cpu().numpy()
     assert cache[0].offset == n and int(cache[0].len_dev.item()) == n

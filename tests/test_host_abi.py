@@ -140,9 +140,11 @@ def test_draft_side_entry_points_reject_bad_arguments():
     assert L.eagle_draft_attention_f16(p, p, p, p, p, p, 8, 65, 14, 2, 64, 4096, 2048, 0.1, p, big, None) == 2
     assert L.eagle_draft_attention_f16(p, p, p, p, p, p, 8, 24, 14, 2, 64, 4096, 8192, 0.1, p, big, None) == 2
     assert L.eagle_draft_attention_f16(p, p, p, p, p, p, 8, 24, 14, 2, 64, 4096, 2048, 0.1, None, 0, None) == 5
-    # causal chunk attention: rows a multiple of 32, at most 1024
+    # causal chunk attention: rows a multiple of 32, at most 2048; a positive scale
     assert L.eagle_causal_attention_f16(p, p, p, p, p, 48, 14, 2, 64, 4096, 2048, 0.1, p, big, None) == 2
-    assert L.eagle_causal_attention_f16(p, p, p, p, p, 2048, 14, 2, 64, 4096, 2048, 0.1, p, big, None) == 2
+    assert L.eagle_causal_attention_f16(p, p, p, p, p, 2080, 14, 2, 64, 4096, 2048, 0.1, p, big, None) == 2
+    assert L.eagle_causal_attention_f16(p, p, p, p, p, 64, 14, 2, 64, 4096, 2048, 0.0, p, big, None) == 2
+    assert L.eagle_draft_attention_f16(p, p, p, p, p, p, 8, 24, 14, 2, 64, 4096, 2048, -0.1, p, big, None) == 2
     assert L.eagle_causal_attention_f16(p, p, p, p, p, 512, 14, 2, 64, 4096, 2048, 0.1, p, 1024, None) == 5
     assert (L.eagle_causal_attention_workspace_bytes(512, 14, 64, 2048)
             == 16 * L.eagle_tree_attention_workspace_bytes(14, 64, 2048))
