@@ -566,9 +566,32 @@ def attention_bench(opt):
         kv = 2 * G * (P + T) * hd * 2
         rows.append({"prefix": P, **{k: round(v, 2) for k, v in t.items()}, "kv_bytes": kv,
                      "attention_frac_of_hbm_peak": round(kv / t["attention_us"] / 1e3 / HBM_PEAK_GBS, 4)})
+    # causal attention of a prompt chunk (mlx_llama.py:185-192 with the causal mask of :275-276):
+    # all 32-row pieces of the chunk in one launch pair, behind P0 cache rows
+    causal = []
+    for name, (Hc, Gc, hdc) in (("8B target", (32, 8, 128)), ("7B target", (28, 4, 128)), ("0.5B drafter", (14, 2, 64))):
+        for R, P0 in ((512, 0), (512, 1536), (2048, 0)):
+            cap = P0 + R + 256
+            q = torch.randn(Hc, R, hdc, device=dev).half()
+            kc = torch.randn(Gc, cap, hdc, device=dev).half()
+            vc = torch.randn(Gc, cap, hdc, device=dev).half()
+            out = torch.empty(R, Hc * hdc, device=dev, dtype=torch.float16)
+            piece_len = torch.tensor([P0 + 32 * j for j in range(R // 32)], dtype=torch.int32, device=dev)
+            ops.causal_attention(q, kc, vc, piece_len, hdc ** -0.5, max_len=cap, out=out)
+
+            def chunk():
+                for _ in range(8):
+                    ops.causal_attention(q, kc, vc, piece_len, hdc ** -0.5, max_len=cap, out=out)
+
+            us = float(np.median(graph_time_ms(torch, chunk, reps=7)[0])) * 1e3 / 8
+            keys = sum(P0 + 32 * j + 32 for j in range(R // 32))
+            flops = 4.0 * Hc * 32 * keys * hdc          # S and O products over the keys each piece sees
+            causal.append({"shape": name, "rows": R, "cache_rows": P0, "us": round(us, 2),
+                           "tflops": round(flops / us / 1e6, 1)})
+            del q, kc, vc, out
     return {"metric": "tree-position rope + tree-masked attention, us per layer", "unit": "us", "dtype": "f16",
             "data": "synthetic", "config": {"workload": "32 tree tokens, 28 q / 4 kv heads, head_dim 128, theta 1e6"},
-            "rows": rows}
+            "rows": rows, "causal_chunk": causal}
 
 
 def cpu_qmm_bench(opt):
