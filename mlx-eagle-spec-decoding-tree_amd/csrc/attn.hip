@@ -1,4 +1,4 @@
-// Tree-masked grouped-query attention of T <= 32 query tokens against a KV cache (gfx950).
+// Tree-masked grouped-query attention of 32 query tokens per piece against a KV cache (gfx950).
 //
 //   out[t, h*hd + d] = sum_j softmax_j( scale * q[h,t,:] . k[g,j,:] + mask[t,j] ) v[g,j,d]
 //
@@ -12,10 +12,16 @@
 // wave computes S^T = K Q^T with v_mfma_f32_32x32x16_f16 (rows = keys, columns = the 32
 // tree tokens), runs the online softmax on its accumulator (a lane owns one tree token,
 // its partner lane+32 the other half of the keys), and feeds exp(S^T) straight back as
-// the B operand of O^T += V^T P^T; only V needs a transposed (16-bit) read from LDS.
-// Partial (m, l, O) per split go to a workspace and a second kernel merges them.  The key
-// tiles of the live length are dealt evenly to as many splits as give each at most
-// max(2, tiles / grid splits) tiles; the busiest workgroup sets the time.
+// the B operand of O^T += V^T P^T; only V needs a transposed read from LDS
+// (ds_read_b64_tr_b16).  Partial (m, l, O) per split go to a workspace and a second kernel
+// merges them.  The key tiles of the live length are dealt evenly to as many splits as give
+// each at least two tiles and the launch at most as many workgroups as the GPU holds at once;
+// the busiest workgroup sets the time.
+//
+// More than 32 query rows go in pieces of 32 on blockIdx.z, one launch pair for all pieces: the
+// pieces of a causal prompt chunk (mlx_llama.py:275-276; each with its own cache length, the
+// mask generated in the kernel) or of a tree of up to 64 tokens (one length, two mask words per
+// query).
 //
 // The draft-side form (mlx_eagle.py:143-178,207) has fewer query rows than masked key rows: T
 // queries see the P prefix rows and, through masks of one or two 32-bit words per query, the
