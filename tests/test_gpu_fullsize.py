@@ -112,6 +112,28 @@ def test_one_layer_at_7b_width(dev):
         assert rel_err(ver.logits.cpu().numpy(), want) <= TOL
 
 
+def test_one_layer_at_7b_width_with_the_default_tree(dev):
+    """The same layer on a tree of 40 tokens (the reference's default of 39 draft nodes,
+    mlx_eagle.py:390,510): 64-row partial tiles in the slab form, gate|up and the vocabulary
+    projection as two passes of 32 rows, attention in two pieces of query rows."""
+    P, T = 2048, 40
+    s = setup_step(dev, synth.qwen25_7b(), 1, 6, P, T)
+    mask = np.concatenate([np.zeros((T, P), np.float16), tree_oracle.additive_mask(s["anc"])], axis=1)
+    want_h = {}
+    want = model_oracle.tree_forward(s["args"], s["weights"], s["inv"], s["sc"], s["tokens"], s["depth"] + P,
+                                     mask, s["ocache"], P, tap=lambda i, h: want_h.__setitem__(i + 1, h.copy()))
+    ok, ov = s["ocache"][0]
+    for plan in (None, {}):
+        print(f"7B-width layer, 40 tree tokens, slab plan {plan}", flush=True)
+        ver, hid = run_verifier(dev, s, plan, taps={1})
+        assert ver.wide and (plan is None) == bool(ver.slab["qkv"] and ver.slab["o"] and ver.slab["down"])
+        assert rel_err(hid[1], want_h[1]) <= TOL
+        c = s["cache"][0]
+        assert rel_err(c.keys[0, :, P:P + T].cpu().numpy(), ok[:, P:P + T]) <= TOL
+        assert rel_err(c.values[0, :, P:P + T].cpu().numpy(), ov[:, P:P + T]) <= TOL
+        assert rel_err(ver.logits.cpu().numpy(), want) <= TOL
+
+
 # Bound for the residual stream and the logits after all 28 layers.  Every operator meets
 # TOL on its own output (the tests above and those of the operators); through 28 layers the
 # rounding differences of 197 matmuls add up.  The test below prints how the error grows and
