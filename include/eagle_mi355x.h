@@ -242,6 +242,14 @@ int eagle_qmm_slab_partial_w4g64(const void* x, const uint32_t* wq, const void* 
                                  const void* biases, float* partial, size_t partial_bytes,
                                  int M, int N, int K, int group_size, int bits,
                                  int steps_per_slab, eagle_stream_t stream);
+/* gate|up + SwiGLU (mlx_llama.py:214-215) for 1..64 rows on the slab kernel with one slab over all
+ * of K: operands as eagle_qmm_swiglu_w4g64_f16 (gate and up rows interleaved in 16-row tiles, bias
+ * [N] interleaved likewise or NULL), out [M, N/2] fp16 = silu(g) * u with the same roundings.
+ * For 33..64 rows (a tree above 32 tokens) one launch in place of two of the 32-row kernel. */
+int eagle_qmm_slab_swiglu_supported(int M, int N, int K);
+int eagle_qmm_slab_swiglu_w4g64_f16(const void* x, const uint32_t* wq, const void* scales,
+                                    const void* biases, const void* bias, void* out, int M, int N, int K,
+                                    int group_size, int bits, eagle_stream_t stream);
 /* out [M,N] fp16 = fp16(sum of the slabs) (+ bias [N] fp16, 16-byte aligned, may be NULL). */
 int eagle_slab_sum_f16(const float* partial, int slabs, const void* bias, void* out, int M, int N,
                        eagle_stream_t stream);

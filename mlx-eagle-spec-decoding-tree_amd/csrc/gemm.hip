@@ -465,13 +465,23 @@ constexpr int SLAB_XBUF = SLAB_ROWS * SLAB_XR;
 // MR: 32-row tiles of x (1: up to 32 rows, 2: 33..64 rows of a tree above 32 tokens).  With two,
 // every expanded weight operand feeds two matrix instructions, the x chunk in LDS has 64 rows
 // (66 KB per buffer) and the partial tile is [64][N].
-template <bool RAGGED, int MR = 1>
-__global__ __launch_bounds__(256) void qmm_slab_w4g64_kernel(
+// SWI: one slab over all of K (gridDim.y == 1), the weight rows gate and up interleaved in 16-row
+// tiles (a wave's 32 rows are one gate tile and its up tile), and the result silu(g) * u as fp16
+// [M, N / 2] in `swi_out` (bias [N], interleaved like the rows, or null) instead of partial sums.
+// NWV: waves (32-row weight tiles) per workgroup, 4 unless SWI: there the host picks the count
+// that fits the launch into one workgroup per compute unit where it can (37888 rows: 296
+// workgroups of four waves would leave 40 compute units with two of them and everyone waiting
+// for those; 237 of five waves run side by side).  Waves beyond the fourth only multiply.
+template <bool RAGGED, int MR = 1, bool SWI = false, int NWV = 4>
+__global__ __launch_bounds__(64 * NWV) void qmm_slab_w4g64_kernel(
     const half_t* __restrict__ x, const uint32_t* __restrict__ w, const half_t* __restrict__ s,
-    const half_t* __restrict__ b, float* __restrict__ partial, int M, int N, int K, int spz) {
+    const half_t* __restrict__ b, float* __restrict__ partial, int M, int N, int K, int spz, int xbufs,
+    const half_t* __restrict__ swi_bias = nullptr, half_t* __restrict__ swi_out = nullptr) {
+  static_assert(SWI || NWV == 4, "the partial-sum epilogue is laid out for four waves");
   extern __shared__ __attribute__((aligned(16))) half_t xlds[];   // one or two x chunks
   constexpr int XBUF = MR * SLAB_XBUF;
   const int tid = threadIdx.x;
+  const bool mover = NWV == 4 || tid < 256;  // the threads that carry x into LDS
   const int wave = tid >> 6, lane = tid & 63;
   const int ql = lane & 31, hb = lane >> 5;
   const int z = blockIdx.y;
@@ -492,7 +502,7 @@ __global__ __launch_bounds__(256) void qmm_slab_w4g64_kernel(
     const int row = xr + 32 * r;
     xp[r] = x + (long)(row < M ? row : M - 1) * K + g0 * 64 + xc * 8;
   }
-  int nrow = blockIdx.x * 128 + wave * 32 + ql;
+  int nrow = blockIdx.x * (32 * NWV) + wave * 32 + ql;
   if (nrow > N - 1) nrow = N - 1;
   const uint32_t* wp = w + (long)nrow * KW + g0 * 8 + hb * 4;
   const half_t* sp = s + (long)nrow * G + g0;
@@ -502,6 +512,7 @@ __global__ __launch_bounds__(256) void qmm_slab_w4g64_kernel(
   uint4_t wreg[SLAB_RING];
   half8_t s8, b8, s8n, b8n;
   auto fetch_x = [&](int c) {
+    if (!mover) return;
 #pragma unroll
     for (int r = 0; r < MR; ++r)
 #pragma unroll
@@ -527,6 +538,7 @@ __global__ __launch_bounds__(256) void qmm_slab_w4g64_kernel(
     }
   };
   auto stash_x = [&](int buf) {
+    if (!mover) return;
 #pragma unroll
     for (int r = 0; r < MR; ++r)
 #pragma unroll
@@ -578,20 +590,62 @@ __global__ __launch_bounds__(256) void qmm_slab_w4g64_kernel(
       b8 = b8n;
     }
   };
+  // xbufs == 2: the chunks alternate between two LDS buffers.  xbufs == 1 (a slab of one chunk,
+  // or a workgroup that leaves LDS room for a second one on its compute unit): one buffer, and
+  // a barrier before it is overwritten.
+  const int bmask = xbufs - 1;
   for (int c = 0; c + 1 < chunks; ++c) {
-    chunk(c, c & 1, StepIndex<1>{});
+    chunk(c, c & bmask, StepIndex<1>{});
     // x of chunk c + 1 (requested before this chunk's weight reloads, so that waiting for it
     // leaves those in flight) into the buffer that chunk c - 1 used: every wave left that one
     // before the barrier that ended chunk c - 1
-    stash_x((c + 1) & 1);
+    if (xbufs == 1) __syncthreads();
+    stash_x((c + 1) & bmask);
     if (c + 2 < chunks) fetch_x(c + 2);
     __syncthreads();
   }
-  chunk(chunks - 1, (chunks - 1) & 1, StepIndex<0>{});
+  chunk(chunks - 1, (chunks - 1) & bmask, StepIndex<0>{});
 
   // accumulator register i of a lane: weight row 8*(i/4) + 4*hb + i%4 of the wave's tile, x
   // row ql (+ 32 for the second tile).  Through LDS, so that the lanes of a wave store whole
   // 512-byte row segments.
+  if (SWI) {
+    // registers 0..7 of a lane are gate rows 8 (i / 4) + 4 hb + i % 4 of the wave's tile pair,
+    // registers 8..15 the up rows 16 further on: 16 output columns per wave, 64 per workgroup
+    constexpr int HS = 16 * NWV + 8;         // halves per row of the output tile in LDS
+    half_t* ht = xlds;
+    __syncthreads();                         // every wave is done with the x chunks
+    const int ng = blockIdx.x * (32 * NWV) + wave * 32;
+#pragma unroll
+    for (int r = 0; r < MR; ++r)
+#pragma unroll
+      for (int i4 = 0; i4 < 2; ++i4) {
+        const int n = ng + 8 * i4 + 4 * hb;  // gate row; the up row is n + 16
+        half4_t o;
+#pragma unroll
+        for (int e = 0; e < 4; ++e) {
+          half_t g = (half_t)acc[r][4 * i4 + e], u = (half_t)acc[r][8 + 4 * i4 + e];
+          if (swi_bias && n + 16 + e < N) {
+            g = g + swi_bias[n + e];
+            u = u + swi_bias[n + 16 + e];
+          }
+          const float gf = (float)g;
+          const half_t a = (half_t)(gf / (1.0f + expf(-gf)));
+          o[e] = (half_t)((float)a * (float)u);
+        }
+        *reinterpret_cast<half4_t*>(&ht[(ql + 32 * r) * HS + wave * 16 + 8 * i4 + 4 * hb]) = o;
+      }
+    __syncthreads();
+    const int NO = N >> 1;
+    constexpr int U = 2 * NWV;               // 16-byte pieces of a row of the tile
+    for (int idx = tid; idx < MR * 32 * U; idx += 64 * NWV) {
+      const int m = idx / U, c8 = (idx % U) * 8;
+      const int no = blockIdx.x * (16 * NWV) + c8;
+      if (m < M && no < NO)
+        *reinterpret_cast<half8_t*>(swi_out + (size_t)m * NO + no) = *reinterpret_cast<const half8_t*>(&ht[m * HS + c8]);
+    }
+    return;
+  }
   constexpr int OS = 128 + 4;                // floats per row of the tile in LDS
   float* ot = reinterpret_cast<float*>(xlds);
   __syncthreads();                           // every wave is done with the x chunks
@@ -692,13 +746,87 @@ EAGLE_EXPORT int eagle_qmm_slab_partial_w4g64(const void* x, const uint32_t* wq,
 #define EAGLE_SLAB_LAUNCH(RAG, MRV)                                                                      \
   hipLaunchKernelGGL((qmm_slab_w4g64_kernel<RAG, MRV>), grid, dim3(256), lds, st,                        \
                      static_cast<const half_t*>(x), wq, static_cast<const half_t*>(scales),              \
-                     static_cast<const half_t*>(biases), partial, M, N, K, steps_per_slab)
+                     static_cast<const half_t*>(biases), partial, M, N, K, steps_per_slab, bufs)
   if (ragged) {
     if (mr == 2) EAGLE_SLAB_LAUNCH(true, 2); else EAGLE_SLAB_LAUNCH(true, 1);
   } else {
     if (mr == 2) EAGLE_SLAB_LAUNCH(false, 2); else EAGLE_SLAB_LAUNCH(false, 1);
   }
 #undef EAGLE_SLAB_LAUNCH
+  return eagle_launch_status();
+}
+
+EAGLE_EXPORT int eagle_qmm_slab_swiglu_supported(int M, int N, int K) {
+  return M >= 1 && M <= 2 * SLAB_ROWS && N >= 32 && (N % 32) == 0 && K >= 128 && (K % 128) == 0 && K <= 65536;
+}
+
+EAGLE_EXPORT int eagle_qmm_slab_swiglu_w4g64_f16(const void* x, const uint32_t* wq, const void* scales,
+                                                 const void* biases, const void* bias, void* out, int M,
+                                                 int N, int K, int group_size, int bits,
+                                                 eagle_stream_t stream) {
+  if (!x || !wq || !scales || !biases || !out) return EAGLE_ERR_NULL;
+  if (group_size != 64 || bits != 4) return EAGLE_ERR_UNSUPPORTED;
+  if (!eagle_qmm_slab_swiglu_supported(M, N, K)) return EAGLE_ERR_SHAPE;
+  const bool ragged = (K % 512) != 0;
+  const uintptr_t sb_mask = ragged ? 3u : 15u;
+  if (!eagle_aligned16(x) || !eagle_aligned16(wq) || !eagle_aligned16(out) ||
+      (reinterpret_cast<uintptr_t>(scales) & sb_mask) || (reinterpret_cast<uintptr_t>(biases) & sb_mask) ||
+      (bias && (reinterpret_cast<uintptr_t>(bias) & 1u)))
+    return EAGLE_ERR_ALIGN;
+  const int mr = M > SLAB_ROWS ? 2 : 1;
+  const int steps = K / 64;                      // one slab over all of K
+  // waves per workgroup: the fewest that give every compute unit at most one workgroup
+  int nwv = 4;
+  while (nwv < 8 && (N + 32 * nwv - 1) / (32 * nwv) > NUM_CU) nwv += (nwv == 6 ? 2 : 1);
+  const int blocks = (N + 32 * nwv - 1) / (32 * nwv);
+  // two x buffers, except that with 64 rows they would fill the LDS of a compute unit: when the
+  // launch puts two workgroups on some compute units anyway, one buffer each, so that the two
+  // fill each other's waits
+  const int bufs = steps > SLAB_RING && !(mr == 2 && blocks > NUM_CU) ? 2 : 1;
+  const size_t lds = (size_t)bufs * mr * SLAB_XBUF * sizeof(half_t);
+  static bool configured = false;
+  if (!configured) {
+    const int most = 2 * SLAB_XBUF * (int)sizeof(half_t);
+    bool ok = true;
+#define EAGLE_SLAB_SWI_ATTR(NW)                                                                                  \
+  ok = ok &&                                                                                                     \
+       hipFuncSetAttribute(reinterpret_cast<const void*>(&qmm_slab_w4g64_kernel<false, 1, true, NW>),            \
+                           hipFuncAttributeMaxDynamicSharedMemorySize, most) == hipSuccess &&                    \
+       hipFuncSetAttribute(reinterpret_cast<const void*>(&qmm_slab_w4g64_kernel<true, 1, true, NW>),             \
+                           hipFuncAttributeMaxDynamicSharedMemorySize, most) == hipSuccess &&                    \
+       hipFuncSetAttribute(reinterpret_cast<const void*>(&qmm_slab_w4g64_kernel<false, 2, true, NW>),            \
+                           hipFuncAttributeMaxDynamicSharedMemorySize, 2 * most) == hipSuccess &&                \
+       hipFuncSetAttribute(reinterpret_cast<const void*>(&qmm_slab_w4g64_kernel<true, 2, true, NW>),             \
+                           hipFuncAttributeMaxDynamicSharedMemorySize, 2 * most) == hipSuccess
+    EAGLE_SLAB_SWI_ATTR(4);
+    EAGLE_SLAB_SWI_ATTR(5);
+    EAGLE_SLAB_SWI_ATTR(6);
+    EAGLE_SLAB_SWI_ATTR(8);
+#undef EAGLE_SLAB_SWI_ATTR
+    if (!ok) return EAGLE_ERR_HIP;
+    configured = true;
+  }
+  const dim3 grid(blocks, 1);
+  hipStream_t st = static_cast<hipStream_t>(stream);
+#define EAGLE_SLAB_SWI_LAUNCH(RAG, MRV, NW)                                                              \
+  hipLaunchKernelGGL((qmm_slab_w4g64_kernel<RAG, MRV, true, NW>), grid, dim3(64 * NW), lds, st,          \
+                     static_cast<const half_t*>(x), wq, static_cast<const half_t*>(scales),              \
+                     static_cast<const half_t*>(biases), (float*)nullptr, M, N, K, steps, bufs,          \
+                     static_cast<const half_t*>(bias), static_cast<half_t*>(out))
+#define EAGLE_SLAB_SWI_NW(NW)                                                                            \
+  if (ragged) {                                                                                          \
+    if (mr == 2) EAGLE_SLAB_SWI_LAUNCH(true, 2, NW); else EAGLE_SLAB_SWI_LAUNCH(true, 1, NW);            \
+  } else {                                                                                               \
+    if (mr == 2) EAGLE_SLAB_SWI_LAUNCH(false, 2, NW); else EAGLE_SLAB_SWI_LAUNCH(false, 1, NW);          \
+  }
+  switch (nwv) {
+    case 4: EAGLE_SLAB_SWI_NW(4) break;
+    case 5: EAGLE_SLAB_SWI_NW(5) break;
+    case 6: EAGLE_SLAB_SWI_NW(6) break;
+    default: EAGLE_SLAB_SWI_NW(8) break;
+  }
+#undef EAGLE_SLAB_SWI_NW
+#undef EAGLE_SLAB_SWI_LAUNCH
   return eagle_launch_status();
 }
 

@@ -216,12 +216,37 @@ def swiglu_supported(M, I, K):
     return I % 16 == 0 and M >= 1 and K % 64 == 0
 
 
+def quantized_matmul_swiglu_slab(x, w_q, scales, biases, bias=None, out=None):
+    """`quantized_matmul_swiglu` for 1..64 rows on the slab kernel with one slab over all of K
+    (each expanded weight feeds the matrix instructions of both 32-row tiles above 32 rows)."""
+    _need_cuda(x, w_q, scales, biases, bias)
+    x = _f16(x, "x")
+    w_q = as_packed_u32(w_q)
+    scales, biases = _f16(scales, "scales"), _f16(biases, "biases")
+    *lead, K = x.shape
+    M = reduce(lambda a, b: a * b, lead, 1)
+    N = w_q.shape[0]
+    if w_q.shape[1] * 8 != K or tuple(scales.shape) != (N, K // 64) or tuple(biases.shape) != (N, K // 64):
+        raise ValueError(f"shape mismatch: x {tuple(x.shape)}, w {tuple(w_q.shape)}, "
+                         f"scales {tuple(scales.shape)}, biases {tuple(biases.shape)}")
+    if bias is not None:
+        bias = _f16(bias, "bias")
+        if tuple(bias.shape) != (N,):
+            raise ValueError("bias must have shape [N]")
+    if out is None:
+        out = torch.empty((*lead, N // 2), dtype=torch.float16, device=x.device)
+    rc = _lib.lib().eagle_qmm_slab_swiglu_w4g64_f16(_ptr(x), _ptr(w_q), _ptr(scales), _ptr(biases), _ptr(bias),
+                                                    _ptr(out), M, N, K, 64, 4, _stream())
+    _lib.check(rc, "quantized_matmul_swiglu_slab")
+    return out
+
+
 def quantized_matmul_swiglu(x, w_q, scales, biases, bias=None, out=None, gemm=None):
     """silu(x @ Wg.T) * (x @ Wu.T) (mlx_llama.py:214-215) in one launch: w_q / scales / biases
     / bias hold the gate and up projections interleaved by `interleave_gate_up`.  The result
     equals `silu_mul(quantized_matmul(x, gate...), quantized_matmul(x, up...))` bit for bit.
-    33..64 rows run as two passes of the 32-row kernel, more rows as the tiled GEMM form with the
-    same epilogue (`gemm=True`: that form whatever the row count)."""
+    33..64 rows run on the slab kernel with 64-row tiles (`quantized_matmul_swiglu_slab`), more rows
+    as the tiled GEMM form with the same epilogue (`gemm=True`: that form whatever the row count)."""
     _need_cuda(x, w_q, scales, biases, bias)
     x = _f16(x, "x")
     w_q = as_packed_u32(w_q)
@@ -240,6 +265,13 @@ def quantized_matmul_swiglu(x, w_q, scales, biases, bias=None, out=None, gemm=No
         out = torch.empty((*lead, N // 2), dtype=torch.float16, device=x.device)
     L = _lib.lib()
     if ROW_PASS < M <= 2 * ROW_PASS and not gemm:
+        # one launch of the slab kernel with 64-row tiles (35 us against 48..56 us for two passes
+        # of the 32-row kernel at the 7B shape)
+        if L.eagle_qmm_slab_swiglu_supported(M, N, K):
+            rc = L.eagle_qmm_slab_swiglu_w4g64_f16(_ptr(x), _ptr(w_q), _ptr(scales), _ptr(biases), _ptr(bias),
+                                                   _ptr(out), M, N, K, 64, 4, _stream())
+            _lib.check(rc, "quantized_matmul_swiglu")
+            return out
         x2, out2 = x.reshape(M, K), out.view(M, N // 2)
         for r0 in range(0, M, ROW_PASS):
             quantized_matmul_swiglu(x2[r0:r0 + ROW_PASS], w_q, scales, biases, bias=bias,

@@ -8,7 +8,7 @@ import torch
 from mlx_eagle_spec_decoding_tree_amd import eagle, ops, synth
 from oracle import model_oracle, oracle, tree_oracle
 from test_gpu_model import build, margins, run_verifier
-from util import TOL, layer_to_dev, rel_err, to_dev
+from util import TOL, close_fp16, layer_to_dev, rel_err, to_dev
 
 pytestmark = pytest.mark.gpu
 
@@ -59,6 +59,59 @@ def test_slab_partials_match_oracle(dev, M, N, K, steps, bias):
     # and agrees with the streaming kernel to the rounding of the expanded weights
     stream = ops.quantized_matmul(to_dev(x, dev), d["weight"], d["scales"], d["biases"], bias=d.get("bias"))
     assert rel_err(got.cpu().numpy(), stream.cpu().numpy()) <= TOL
+
+
+@pytest.mark.parametrize("M,I,K,bias", [(40, 18944, 3584, True), (64, 14336, 4096, False), (33, 16, 128, True),
+                                        (32, 18944, 3584, True), (8, 4864, 896, True), (64, 272, 1920, False),
+                                        (47, 2432, 896, True), (1, 64, 512, False), (64, 4112, 1024, True)])
+def test_slab_form_with_swiglu(dev, M, I, K, bias):
+    """gate|up + SwiGLU on the slab kernel (one slab over all of K, 64-row tiles above 32 rows,
+    four to eight waves per workgroup by the row count of the weights): every projection is
+    within TOL of its own RMS, so silu(g) * u is within the propagated bound of the oracle's
+    qmm -> silu_mul (as for the GEMM form); against the streaming kernel's SwiGLU form too."""
+    print(f"slab swiglu M={M} I={I} K={K}", flush=True)
+    rng = np.random.default_rng(M + I + K)
+    g = synth.make_qlinear(rng, I, K, bias=bias, gain=1.0)
+    u = synth.make_qlinear(rng, I, K, bias=bias, gain=1.0)
+    x = synth.make_x(rng, M, K)
+    og = oracle.qmm(x, g["weight"], g["scales"], g["biases"], g.get("bias"))
+    ou = oracle.qmm(x, u["weight"], u["scales"], u["biases"], u.get("bias"))
+    want = oracle.silu_mul(og, ou)
+    gd, ud = layer_to_dev(g, dev), layer_to_dev(u, dev)
+    keys = ["weight", "scales", "biases"] + (["bias"] if bias else [])
+    inter = {k: ops.interleave_gate_up(gd[k], ud[k]) for k in keys}
+    xd = to_dev(x, dev)
+    out = torch.full((M + 1, I), float("nan"), dtype=torch.float16, device=dev)
+    ops.quantized_matmul_swiglu_slab(xd, inter["weight"], inter["scales"], inter["biases"], bias=inter.get("bias"),
+                                     out=out[:M])
+    got = out.cpu().numpy()
+    assert np.isnan(got[M].astype(np.float32)).all()                # nothing written past the rows
+    g64, u64 = og.astype(np.float64), ou.astype(np.float64)
+    rms_g, rms_u = np.sqrt(np.mean(g64 * g64)), np.sqrt(np.mean(u64 * u64))
+    w64, got64 = want.astype(np.float64), got[:M].astype(np.float64)
+    assert np.isfinite(got64).all()
+    ulp = 2.0 ** (np.floor(np.log2(np.maximum(np.abs(w64), 2.0 ** -14))) - 10)
+    bound = TOL * (1.1 * np.abs(u64) * rms_g + np.abs(g64 / (1 + np.exp(-g64))) * rms_u) + 2 * ulp
+    assert np.all(np.abs(got64 - w64) <= bound)
+    assert np.sqrt(np.mean((got64 - w64) ** 2)) <= 0.25 * TOL * np.sqrt(np.mean(w64 * w64))
+    # the dispatcher sends 33..64 rows here
+    auto = ops.quantized_matmul_swiglu(xd, inter["weight"], inter["scales"], inter["biases"], bias=inter.get("bias"))
+    if M > 32:
+        assert torch.equal(auto, out[:M])
+    else:
+        close_fp16(auto.cpu().numpy(), got[:M], "streaming form")
+
+
+def test_slab_swiglu_refusals(dev):
+    from mlx_eagle_spec_decoding_tree_amd import _lib
+    L = _lib.lib()
+    assert L.eagle_qmm_slab_swiglu_supported(64, 37888, 3584) == 1 and L.eagle_qmm_slab_swiglu_supported(65, 64, 128) == 0
+    assert L.eagle_qmm_slab_swiglu_supported(8, 48, 128) == 0 and L.eagle_qmm_slab_swiglu_supported(8, 64, 192) == 0
+    x = torch.zeros((8, 192), dtype=torch.float16, device=dev)
+    w = torch.zeros((64, 24), dtype=torch.int32, device=dev)
+    s = torch.zeros((64, 3), dtype=torch.float16, device=dev)
+    with pytest.raises(ValueError):
+        ops.quantized_matmul_swiglu_slab(x, w, s, s)
 
 
 def test_slab_form_integer_exact(dev):
