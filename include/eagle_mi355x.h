@@ -247,6 +247,8 @@ int eagle_qmm_slab_partial_w4g64(const void* x, const uint32_t* wq, const void* 
  * [N] interleaved likewise or NULL), out [M, N/2] fp16 = silu(g) * u with the same roundings.
  * For 33..64 rows (a tree above 32 tokens) one launch in place of two of the 32-row kernel. */
 int eagle_qmm_slab_swiglu_supported(int M, int N, int K);
+/* 1 where this form measured faster than eagle_qmm_swiglu_w4g64_f16 (always above 32 rows). */
+int eagle_qmm_slab_swiglu_preferred(int M, int N, int K);
 int eagle_qmm_slab_swiglu_w4g64_f16(const void* x, const uint32_t* wq, const void* scales,
                                     const void* biases, const void* bias, void* out, int M, int N, int K,
                                     int group_size, int bits, eagle_stream_t stream);

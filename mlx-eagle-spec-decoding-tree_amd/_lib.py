@@ -48,6 +48,7 @@ SIGNATURES = {
     "eagle_qmm_slab_partial_bytes_rows": (c_size_t, [c_int] * 4),
     "eagle_qmm_slab_partial_w4g64": (c_int, [c_void_p] * 5 + [c_size_t] + [c_int] * 6 + [c_void_p]),
     "eagle_qmm_slab_swiglu_supported": (c_int, [c_int] * 3),
+    "eagle_qmm_slab_swiglu_preferred": (c_int, [c_int] * 3),
     "eagle_qmm_slab_swiglu_w4g64_f16": (c_int, [c_void_p] * 6 + [c_int] * 5 + [c_void_p]),
     "eagle_slab_sum_f16": (c_int, [c_void_p, c_int, c_void_p, c_void_p, c_int, c_int, c_void_p]),
     "eagle_rmsnorm_slabs_f16": (c_int, [c_void_p, c_int, c_void_p, c_void_p, c_float, c_void_p, c_void_p,

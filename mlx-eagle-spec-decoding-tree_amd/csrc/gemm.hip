@@ -472,7 +472,10 @@ constexpr int SLAB_XBUF = SLAB_ROWS * SLAB_XR;
 // that fits the launch into one workgroup per compute unit where it can (37888 rows: 296
 // workgroups of four waves would leave 40 compute units with two of them and everyone waiting
 // for those; 237 of five waves run side by side).  Waves beyond the fourth only multiply.
-template <bool RAGGED, int MR = 1, bool SWI = false, int NWV = 4>
+// WR: register sets of eight weight loads per lane (1: the loads of the next chunk are in flight
+// while a chunk is used; 2: those of the next two, for slabs of many chunks, where the time per
+// step is the load latency divided by the loads in flight).
+template <bool RAGGED, int MR = 1, bool SWI = false, int NWV = 4, int WR = 1>
 __global__ __launch_bounds__(64 * NWV) void qmm_slab_w4g64_kernel(
     const half_t* __restrict__ x, const uint32_t* __restrict__ w, const half_t* __restrict__ s,
     const half_t* __restrict__ b, float* __restrict__ partial, int M, int N, int K, int spz, int xbufs,
@@ -509,8 +512,12 @@ __global__ __launch_bounds__(64 * NWV) void qmm_slab_w4g64_kernel(
   const half_t* bp = b + (long)nrow * G + g0;
 
   half8_t xreg[MR][SLAB_RING];
-  uint4_t wreg[SLAB_RING];
+  uint4_t wreg[WR][SLAB_RING];
   half8_t s8, b8, s8n, b8n;
+  // the packed words of one step of this lane's row (steps past the slab repeat its last one)
+  auto wload = [&](int step) {
+    return *reinterpret_cast<const uint4_t*>(wp + (step < steps ? step : steps - 1) * 8);
+  };
   auto fetch_x = [&](int c) {
     if (!mover) return;
 #pragma unroll
@@ -549,7 +556,12 @@ __global__ __launch_bounds__(64 * NWV) void qmm_slab_w4g64_kernel(
   fetch_x(0);
   fetch_sb(0, s8, b8);
 #pragma unroll
-  for (int i = 0; i < SLAB_RING; ++i) wreg[i] = *reinterpret_cast<const uint4_t*>(wp + step_of(i) * 8);
+  for (int i = 0; i < SLAB_RING; ++i) wreg[0][i] = wload(i);
+  if constexpr (WR == 2) {
+    __builtin_amdgcn_sched_barrier(0);
+#pragma unroll
+    for (int i = 0; i < SLAB_RING; ++i) wreg[1][i] = wload(SLAB_RING + i);
+  }
   __builtin_amdgcn_sched_barrier(0);
   stash_x(0);
   if (chunks > 1) fetch_x(1);
@@ -564,8 +576,9 @@ __global__ __launch_bounds__(64 * NWV) void qmm_slab_w4g64_kernel(
 
   // one chunk of eight steps on the x chunk in buffer `buf`; RELOAD: the weight registers are
   // loaded again for the next chunk
-  auto chunk = [&](int c, int buf, auto RELOAD) {
+  auto chunk = [&](int c, int buf, auto RELOAD, auto PAR) {
     constexpr bool reload = decltype(RELOAD)::value != 0;
+    constexpr int par = WR == 2 ? decltype(PAR)::value : 0;   // the register set of this chunk
     if (reload) fetch_sb(c + 1, s8n, b8n);
 #pragma unroll
     for (int e = 0; e < 8; ++e) {
@@ -574,8 +587,9 @@ __global__ __launch_bounds__(64 * NWV) void qmm_slab_w4g64_kernel(
       const half_t bc = (half_t)((float)bi + 8.f * (float)sc);
       half8_t af[4];
 #pragma unroll
-      for (int j = 0; j < 4; ++j) af[j] = dequant_word_centred(wreg[e][j], half2_t{sc, sc}, half2_t{bc, bc});
-      if (reload) wreg[e] = *reinterpret_cast<const uint4_t*>(wp + step_of((c + 1) * 8 + e) * 8);
+      for (int j = 0; j < 4; ++j) af[j] = dequant_word_centred(wreg[par][e][j], half2_t{sc, sc}, half2_t{bc, bc});
+      if constexpr (WR == 2) wreg[par][e] = wload((c + 2) * 8 + e);
+      else if (reload) wreg[0][e] = wload((c + 1) * 8 + e);
 #pragma unroll
       for (int j = 0; j < 4; ++j)
 #pragma unroll
@@ -584,6 +598,9 @@ __global__ __launch_bounds__(64 * NWV) void qmm_slab_w4g64_kernel(
               *reinterpret_cast<const half8_t*>(xrow + buf * XBUF + r * SLAB_XBUF + e * 64 + j * 8);
           acc[r] = __builtin_amdgcn_mfma_f32_32x32x16_f16(af[j], bf, acc[r], 0, 0, 0);
         }
+      // (with two chunk bodies per loop iteration the scheduler otherwise hoists the x operand
+      // reads of many steps to the top and runs out of registers)
+      if constexpr (WR == 2) __builtin_amdgcn_sched_barrier(0);
     }
     if (reload) {
       s8 = s8n;
@@ -594,17 +611,41 @@ __global__ __launch_bounds__(64 * NWV) void qmm_slab_w4g64_kernel(
   // or a workgroup that leaves LDS room for a second one on its compute unit): one buffer, and
   // a barrier before it is overwritten.
   const int bmask = xbufs - 1;
-  for (int c = 0; c + 1 < chunks; ++c) {
-    chunk(c, c & bmask, StepIndex<1>{});
-    // x of chunk c + 1 (requested before this chunk's weight reloads, so that waiting for it
-    // leaves those in flight) into the buffer that chunk c - 1 used: every wave left that one
-    // before the barrier that ended chunk c - 1
+  // x of chunk c + 1 (requested before chunk c's weight reloads, so that waiting for it leaves
+  // those in flight) into the buffer that chunk c - 1 used: every wave left that one before the
+  // barrier that ended chunk c - 1
+  auto next_x = [&](int c) {
+    if constexpr (WR == 2) __builtin_amdgcn_sched_barrier(0);
     if (xbufs == 1) __syncthreads();
     stash_x((c + 1) & bmask);
+    if constexpr (WR == 2) __builtin_amdgcn_sched_barrier(0);
     if (c + 2 < chunks) fetch_x(c + 2);
     __syncthreads();
+    if constexpr (WR == 2) __builtin_amdgcn_sched_barrier(0);
+  };
+  if constexpr (WR == 2) {
+    // chunks in pairs (even ones on register set 0, odd ones on set 1), then the last one or two
+    int c = 0;
+    for (; c + 2 < chunks; c += 2) {
+      chunk(c, c & bmask, StepIndex<1>{}, StepIndex<0>{});
+      next_x(c);
+      chunk(c + 1, (c + 1) & bmask, StepIndex<1>{}, StepIndex<1>{});
+      next_x(c + 1);
+    }
+    if (c + 1 < chunks) {
+      chunk(c, c & bmask, StepIndex<1>{}, StepIndex<0>{});
+      next_x(c);
+      chunk(c + 1, (c + 1) & bmask, StepIndex<0>{}, StepIndex<1>{});
+    } else {
+      chunk(c, c & bmask, StepIndex<0>{}, StepIndex<0>{});
+    }
+  } else {
+    for (int c = 0; c + 1 < chunks; ++c) {
+      chunk(c, c & bmask, StepIndex<1>{}, StepIndex<0>{});
+      next_x(c);
+    }
+    chunk(chunks - 1, (chunks - 1) & bmask, StepIndex<0>{}, StepIndex<0>{});
   }
-  chunk(chunks - 1, (chunks - 1) & bmask, StepIndex<0>{});
 
   // accumulator register i of a lane: weight row 8*(i/4) + 4*hb + i%4 of the wave's tile, x
   // row ql (+ 32 for the second tile).  Through LDS, so that the lanes of a wave store whole
@@ -760,6 +801,21 @@ EAGLE_EXPORT int eagle_qmm_slab_swiglu_supported(int M, int N, int K) {
   return M >= 1 && M <= 2 * SLAB_ROWS && N >= 32 && (N % 32) == 0 && K >= 128 && (K % 128) == 0 && K <= 65536;
 }
 
+EAGLE_EXPORT int eagle_qmm_slab_swiglu_preferred(int M, int N, int K) {
+  // Measured against the streaming kernel's SwiGLU form (gate|up of the 7B and 8B shapes, us):
+  //   rows          8     16     24     32     40     64
+  //   7B slab    29.6   28.7   28.6   28.8   34.6   35.9      (237 workgroups of five waves)
+  //   7B stream  23.5   22.7   27.6   28.7   48.5   56.1      (40, 64: two launches)
+  //   8B slab    23.5   24.1   24.8   24.3   30.7   31.3      (224 workgroups of four waves)
+  //   8B stream  20.8   21.2   26.1   27.0   45.5   52.8
+  // so: always above 32 rows; from 24 rows where workgroups of four waves fill at least half of
+  // the compute units and at most all of them.
+  if (!eagle_qmm_slab_swiglu_supported(M, N, K)) return 0;
+  if (M > SLAB_ROWS) return 1;
+  const long blocks = (N + 127) / 128;
+  return M >= 24 && blocks > NUM_CU / 2 && blocks <= NUM_CU && K >= 2048;
+}
+
 EAGLE_EXPORT int eagle_qmm_slab_swiglu_w4g64_f16(const void* x, const uint32_t* wq, const void* scales,
                                                  const void* biases, const void* bias, void* out, int M,
                                                  int N, int K, int group_size, int bits,
@@ -790,13 +846,13 @@ EAGLE_EXPORT int eagle_qmm_slab_swiglu_w4g64_f16(const void* x, const uint32_t* 
     bool ok = true;
 #define EAGLE_SLAB_SWI_ATTR(NW)                                                                                  \
   ok = ok &&                                                                                                     \
-       hipFuncSetAttribute(reinterpret_cast<const void*>(&qmm_slab_w4g64_kernel<false, 1, true, NW>),            \
+       hipFuncSetAttribute(reinterpret_cast<const void*>(&qmm_slab_w4g64_kernel<false, 1, true, NW, 2>),            \
                            hipFuncAttributeMaxDynamicSharedMemorySize, most) == hipSuccess &&                    \
-       hipFuncSetAttribute(reinterpret_cast<const void*>(&qmm_slab_w4g64_kernel<true, 1, true, NW>),             \
+       hipFuncSetAttribute(reinterpret_cast<const void*>(&qmm_slab_w4g64_kernel<true, 1, true, NW, 2>),             \
                            hipFuncAttributeMaxDynamicSharedMemorySize, most) == hipSuccess &&                    \
-       hipFuncSetAttribute(reinterpret_cast<const void*>(&qmm_slab_w4g64_kernel<false, 2, true, NW>),            \
+       hipFuncSetAttribute(reinterpret_cast<const void*>(&qmm_slab_w4g64_kernel<false, 2, true, NW, 1>),            \
                            hipFuncAttributeMaxDynamicSharedMemorySize, 2 * most) == hipSuccess &&                \
-       hipFuncSetAttribute(reinterpret_cast<const void*>(&qmm_slab_w4g64_kernel<true, 2, true, NW>),             \
+       hipFuncSetAttribute(reinterpret_cast<const void*>(&qmm_slab_w4g64_kernel<true, 2, true, NW, 1>),             \
                            hipFuncAttributeMaxDynamicSharedMemorySize, 2 * most) == hipSuccess
     EAGLE_SLAB_SWI_ATTR(4);
     EAGLE_SLAB_SWI_ATTR(5);
@@ -809,7 +865,7 @@ EAGLE_EXPORT int eagle_qmm_slab_swiglu_w4g64_f16(const void* x, const uint32_t* 
   const dim3 grid(blocks, 1);
   hipStream_t st = static_cast<hipStream_t>(stream);
 #define EAGLE_SLAB_SWI_LAUNCH(RAG, MRV, NW)                                                              \
-  hipLaunchKernelGGL((qmm_slab_w4g64_kernel<RAG, MRV, true, NW>), grid, dim3(64 * NW), lds, st,          \
+  hipLaunchKernelGGL((qmm_slab_w4g64_kernel<RAG, MRV, true, NW, (MRV == 1 ? 2 : 1)>), grid, dim3(64 * NW), lds, st, \
                      static_cast<const half_t*>(x), wq, static_cast<const half_t*>(scales),              \
                      static_cast<const half_t*>(biases), (float*)nullptr, M, N, K, steps, bufs,          \
                      static_cast<const half_t*>(bias), static_cast<half_t*>(out))

@@ -264,14 +264,15 @@ def quantized_matmul_swiglu(x, w_q, scales, biases, bias=None, out=None, gemm=No
     if out is None:
         out = torch.empty((*lead, N // 2), dtype=torch.float16, device=x.device)
     L = _lib.lib()
+    if not gemm and L.eagle_qmm_slab_swiglu_preferred(M, N, K):
+        # the slab kernel with one slab over all of K: above 32 rows one launch with 64-row tiles
+        # (35 us against 48..56 us for two passes of the 32-row kernel at the 7B shape), and from
+        # 24 rows where its workgroups fill the GPU in one round (the 8B shape: 24 against 27 us)
+        rc = L.eagle_qmm_slab_swiglu_w4g64_f16(_ptr(x), _ptr(w_q), _ptr(scales), _ptr(biases), _ptr(bias),
+                                               _ptr(out), M, N, K, 64, 4, _stream())
+        _lib.check(rc, "quantized_matmul_swiglu")
+        return out
     if ROW_PASS < M <= 2 * ROW_PASS and not gemm:
-        # one launch of the slab kernel with 64-row tiles (35 us against 48..56 us for two passes
-        # of the 32-row kernel at the 7B shape)
-        if L.eagle_qmm_slab_swiglu_supported(M, N, K):
-            rc = L.eagle_qmm_slab_swiglu_w4g64_f16(_ptr(x), _ptr(w_q), _ptr(scales), _ptr(biases), _ptr(bias),
-                                                   _ptr(out), M, N, K, 64, 4, _stream())
-            _lib.check(rc, "quantized_matmul_swiglu")
-            return out
         x2, out2 = x.reshape(M, K), out.view(M, N // 2)
         for r0 in range(0, M, ROW_PASS):
             quantized_matmul_swiglu(x2[r0:r0 + ROW_PASS], w_q, scales, biases, bias=bias,
