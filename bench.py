@@ -330,8 +330,7 @@ def main():
     achieved = alg / (qmm_ms * 1e-3) / 1e9
     traffic, traffic_source = read_traffic_record()
     stream_kernel = "qmm_w4g64_kernel"          # (above 32 tree tokens: two launches of it per product)
-    kernels = (stream_kernel if ver.wide else stream_kernel + " + qmm_slab_w4g64_kernel") \
-        + (" + norm_mlp_in_kernel" if ver.chain else "")
+    kernels = stream_kernel + " + qmm_slab_w4g64_kernel" + (" + norm_mlp_in_kernel" if ver.chain else "")
     roofline = {"bound": "hbm", "kernel": kernels, "achieved": round(achieved, 1),
                 "peak": HBM_PEAK_GBS, "unit": "GB/s", "frac": round(achieved / HBM_PEAK_GBS, 4),
                 "traffic": traffic, "traffic_source": traffic_source, "launches_per_step": n_launch,
@@ -341,7 +340,11 @@ def main():
 
     # the same for each kernel on its own launches
     per_kernel = {}
-    for kname, sub in ((stream_kernel, [l for l in launches if l[6] is True or not l[6]]),
+    # (above 32 tree tokens gate|up + SwiGLU runs on the slab kernel too: one slab over all of K)
+    swi_name = "qmm_slab_w4g64_kernel (SwiGLU form)" if ver.wide else stream_kernel
+    groups = ([(swi_name, [l for l in launches if l[6] is True]), (stream_kernel, [l for l in launches if not l[6]])]
+              if ver.wide else [(stream_kernel, [l for l in launches if l[6] is True or not l[6]])])
+    for kname, sub in (*groups,
                        ("qmm_slab_w4g64_kernel", [l for l in launches if l[6] and l[6] is not True and l[6] != "chain"]),
                        ("norm_mlp_in_kernel", [l for l in launches if l[6] == "chain"])):
         if not sub:
