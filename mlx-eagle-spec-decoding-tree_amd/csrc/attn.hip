@@ -8,7 +8,8 @@
 // Call site replaced: mlx_llama.py:185-195.
 //
 // Split-KV: grid (kv head g, key split s); one wave per query head of the group, so a
-// K/V tile is read from memory once per group and shared through LDS.  Per 32-key tile a
+// K/V tile is read from memory once per group and shared through LDS.  Per block of 32 keys
+// (a tile holds one or two) a
 // wave computes S^T = K Q^T with v_mfma_f32_32x32x16_f16 (rows = keys, columns = the 32
 // tree tokens), runs the online softmax on its accumulator (a lane owns one tree token,
 // its partner lane+32 the other half of the keys), and feeds exp(S^T) straight back as
@@ -54,10 +55,10 @@ __device__ inline half4_t lds_read_tr16(const unsigned char* p) {
 // workgroups as the GPU holds at once (`slots`) and each covers more tiles per partial result
 // it writes (8B shape, 512-row chunk, us per launch pair with 2 / 4 / 8 / 16 tiles at least: 33 /
 // 29 / 33 / 44 on an empty cache, 94 / 78 / 70 / 66 behind 1536 rows).
-__host__ __device__ inline int active_splits(int ntiles, int nsplit, int lanes, int slots) {
+__host__ __device__ inline int active_splits(int ntiles, int nsplit, int lanes, int slots, int floor_tiles) {
   int tpw = (ntiles + nsplit - 1) / nsplit;
   int min_tiles = (lanes * ntiles + slots - 1) / slots;
-  if (min_tiles < 2) min_tiles = 2;
+  if (min_tiles < floor_tiles) min_tiles = floor_tiles;
   if (tpw < min_tiles) tpw = min_tiles;
   return (ntiles + tpw - 1) / tpw;
 }
@@ -99,7 +100,10 @@ __device__ inline void rotate_pair(half8_t& lo, half8_t& hi, const float* cs) {
 template <int V>
 struct Stage { static constexpr int value = V; };
 
-template <int HD, bool ROPE, bool WIDE, int NVU, int DEPTH>
+// SUB: 32-key blocks per tile (1 or 2).  With two, the S products, the exponentials and the O
+// products of 64 keys each form one phase of a tile instead of two: the phases of a tile depend on
+// each other inside a wave, so a tile of 64 keys takes little longer than one of 32.
+template <int HD, bool ROPE, bool WIDE, int NVU, int DEPTH, int SUB>
 __global__ __launch_bounds__(512) void tree_attn_split_kernel(
     const half_t* __restrict__ q, half_t* kc, half_t* vc,
     const uint32_t* __restrict__ mask_bits, const int32_t* __restrict__ len_dev,
@@ -113,9 +117,10 @@ __global__ __launch_bounds__(512) void tree_attn_split_kernel(
   constexpr int VEC_ROW = HD / 8;       // 16-byte vectors per K/V row
   extern __shared__ __attribute__((aligned(16))) unsigned char lds[];
   constexpr int HALF = HD / 2;
+  constexpr int KTT = KT * SUB;         // keys per tile
   unsigned char* ldsK = lds;
-  unsigned char* ldsV = lds + KT * STR;
-  float* cs_lds = reinterpret_cast<float*>(lds + 2 * KT * STR);   // ROPE: [T][HALF][2]
+  unsigned char* ldsV = lds + KTT * STR;
+  float* cs_lds = reinterpret_cast<float*>(lds + 2 * KTT * STR);   // ROPE: [T][HALF][2]
 
   const int g = blockIdx.x;
   const int split = blockIdx.y;
@@ -143,12 +148,12 @@ __global__ __launch_bounds__(512) void tree_attn_split_kernel(
   if (P > cap - Tk) P = (int)(cap - Tk);
   if (P < 0) P = 0;
   const int Ltot = P + Tk;                // Tk = T unless WIDE
-  const int ntiles = (Ltot + KT - 1) / KT;
+  const int ntiles = (Ltot + KTT - 1) / KTT;
   // Splits in use for this length: every workgroup gets at most `tpw` key tiles, two at
   // least (with one, writing and merging the partials costs more than reading the keys).
   // The tile count of the busiest workgroup sets the time, so the tiles are spread evenly
   // over exactly as many workgroups as that takes; the rest of the grid leaves at once.
-  const int nactive = active_splits(ntiles, nsplit, gridDim.x * gridDim.z, split_slots(rep, HD));
+  const int nactive = active_splits(ntiles, nsplit, gridDim.x * gridDim.z, split_slots(rep, HD), 3 - SUB);
   if (split >= nactive) return;
   half8_t qreg[KSTEPS];
 #pragma unroll
@@ -183,11 +188,11 @@ __global__ __launch_bounds__(512) void tree_attn_split_kernel(
   // This workgroup's tiles are split, split + nactive, ...: all workgroups share the live part
   // of the cache however short it is.  The next DEPTH tiles are in flight into registers while
   // the current one is being used.
-  constexpr int NVEC = KT * VEC_ROW;                 // 16-byte vectors per K (or V) tile
+  constexpr int NVEC = KTT * VEC_ROW;                // 16-byte vectors per K (or V) tile
   half8_t kreg[DEPTH][NVU], vreg[DEPTH][NVU];
   auto fetch = [&](auto S, int tile) {
     constexpr int st = decltype(S)::value;
-    const int kb = tile * KT;
+    const int kb = tile * KTT;
 #pragma unroll
     for (int it = 0; it < NVU; ++it) {
       int v = tid + it * nthr;
@@ -246,9 +251,9 @@ __global__ __launch_bounds__(512) void tree_attn_split_kernel(
   // registers, then the arithmetic on LDS
   auto do_tile = [&](auto S, int tile) {
     constexpr int st = decltype(S)::value;
-    const int kb = tile * KT;
+    const int kb = tile * KTT;
     __syncthreads();   // every wave is done with the previous tile
-    if (ROPE && kb + KT > P) {
+    if (ROPE && kb + KTT > P) {
       // tree rows: append the values as they are
 #pragma unroll
       for (int it = 0; it < NVU; ++it) {
@@ -261,9 +266,9 @@ __global__ __launch_bounds__(512) void tree_attn_split_kernel(
     stash(S);
     fetch(S, tile_at(tile + DEPTH * nactive));
     __syncthreads();
-    if (ROPE && kb + KT > P) {
+    if (ROPE && kb + KTT > P) {
       // rotate the tree keys in LDS (one thread per pair of 16-byte pieces) and append them
-      for (int v = tid; v < KT * (VEC_ROW / 2); v += nthr) {
+      for (int v = tid; v < KTT * (VEC_ROW / 2); v += nthr) {
         const int row = v / (VEC_ROW / 2);
         const int c = v % (VEC_ROW / 2);
         const int kidx = kb + row;
@@ -281,51 +286,58 @@ __global__ __launch_bounds__(512) void tree_attn_split_kernel(
       __syncthreads();
     }
 
-    // S^T[key][token] = sum_d K[key][d] Q[token][d]
-    float16_t sacc;
+    // S^T[key][token] = sum_d K[key][d] Q[token][d], one accumulator per block of 32 keys
+    float16_t sacc[SUB];
 #pragma unroll
-    for (int i = 0; i < 16; ++i) sacc[i] = 0.f;
+    for (int h = 0; h < SUB; ++h)
 #pragma unroll
-    for (int kk = 0; kk < KSTEPS; ++kk) {
-      const half8_t a = *reinterpret_cast<const half8_t*>(ldsK + ql * STR + kk * 32 + hb * 16);
-      sacc = __builtin_amdgcn_mfma_f32_32x32x16_f16(a, qreg[kk], sacc, 0, 0, 0);
-    }
+      for (int i = 0; i < 16; ++i) sacc[h][i] = 0.f;
+#pragma unroll
+    for (int kk = 0; kk < KSTEPS; ++kk)
+#pragma unroll
+      for (int h = 0; h < SUB; ++h) {
+        const half8_t a = *reinterpret_cast<const half8_t*>(ldsK + (32 * h + ql) * STR + kk * 32 + hb * 16);
+        sacc[h] = __builtin_amdgcn_mfma_f32_32x32x16_f16(a, qreg[kk], sacc[h], 0, 0, 0);
+      }
 
-    // accumulator register i of this lane is key 8*(i/4) + 4*hb + i%4 of the tile.  The scores
+    // accumulator register i of this lane is key 8*(i/4) + 4*hb + i%4 of its block.  The scores
     // stay unscaled: the scale (> 0) goes into the exponent's fused multiply-add, and the running
     // maximum starts at a finite floor instead of -inf, so that no case needs a select.
-    float sv[16];
     float bm = M_FLOOR;
-    if (kb + KT <= P) {
+    if (kb + KTT <= P) {
       // a tile of prefix rows: visible to every token, no mask arithmetic
 #pragma unroll
-      for (int i = 0; i < 16; ++i) {
-        sv[i] = sacc[i];
-        bm = fmaxf(bm, sv[i]);
-      }
+      for (int h = 0; h < SUB; ++h)
+#pragma unroll
+        for (int i = 0; i < 16; ++i) bm = fmaxf(bm, sacc[h][i]);
     } else {
 #pragma unroll
-      for (int i = 0; i < 16; ++i) {
-        const int key = kb + 8 * (i >> 2) + 4 * hb + (i & 3);
-        const int rel = key - P;
-        const uint32_t word = (WIDE && rel >= 32) ? mybits_hi : mybits;
-        // (bitwise, not short-circuit: straight-line selects instead of a branch per key)
-        const bool vis = (rel < 0) | ((key < Ltot) & (((word >> (rel & 31)) & 1u) != 0u));
-        sv[i] = vis ? sacc[i] : -INFINITY;
-        bm = fmaxf(bm, sv[i]);
-      }
+      for (int h = 0; h < SUB; ++h)
+#pragma unroll
+        for (int i = 0; i < 16; ++i) {
+          const int key = kb + 32 * h + 8 * (i >> 2) + 4 * hb + (i & 3);
+          const int rel = key - P;
+          const uint32_t word = (WIDE && rel >= 32) ? mybits_hi : mybits;
+          // (bitwise, not short-circuit: straight-line selects instead of a branch per key)
+          const bool vis = (rel < 0) | ((key < Ltot) & (((word >> (rel & 31)) & 1u) != 0u));
+          sacc[h][i] = vis ? sacc[h][i] : -INFINITY;
+          bm = fmaxf(bm, sacc[h][i]);
+        }
     }
     bm = fmaxf(bm, __shfl_xor(bm, 32, 64));
     const float m_new = fmaxf(m_run, bm * scale_log2e);
     // arguments are <= 0: the bare hardware exp2 (results below 2^-126 flush to zero, -inf gives 0)
     const float alpha = __builtin_amdgcn_exp2f(m_run - m_new);
     float psum = 0.f;
-    float p[16];
+    half8_t bp[SUB][2];     // exp(S^T) as the B operand of the O products: step u = registers 8u..8u+7
 #pragma unroll
-    for (int i = 0; i < 16; ++i) {
-      p[i] = __builtin_amdgcn_exp2f(fmaf(sv[i], scale_log2e, -m_new));
-      psum += p[i];
-    }
+    for (int h = 0; h < SUB; ++h)
+#pragma unroll
+      for (int i = 0; i < 16; ++i) {
+        const float pv = __builtin_amdgcn_exp2f(fmaf(sacc[h][i], scale_log2e, -m_new));
+        psum += pv;
+        bp[h][i >> 3][i & 7] = (half_t)pv;
+      }
     psum += __shfl_xor(psum, 32, 64);
     l_run = l_run * alpha + psum;
     m_run = m_new;
@@ -336,24 +348,22 @@ __global__ __launch_bounds__(512) void tree_attn_split_kernel(
         for (int i = 0; i < 16; ++i) o_acc[db][i] *= alpha;
     }
 
-    // O^T[d][token] += sum_key V[key][d] P[token][key]; step u covers accumulator
-    // registers 8u..8u+7, i.e. keys 8*(2u + j/4) + 4*hb + j%4, j = 0..7.  The V^T operand comes
-    // from the row-major tile through the transposing LDS load: within 16 lanes, lane i receives
-    // element i % 4 of the four lanes 4 jj + i / 4, so lane s of a group asks for key row s / 4
-    // at the four d columns 4 (s % 4) .. + 3 of the group's 16 and gets four keys of its own d.
+    // O^T[d][token] += sum_key V[key][d] P[token][key]; step u of block h covers accumulator
+    // registers 8u..8u+7, i.e. keys 32h + 8*(2u + j/4) + 4*hb + j%4, j = 0..7.  The V^T operand
+    // comes from the row-major tile through the transposing LDS load: within 16 lanes, lane i
+    // receives element i % 4 of the four lanes 4 jj + i / 4, so lane s of a group asks for key row
+    // s / 4 at the four d columns 4 (s % 4) .. + 3 of the group's 16 and gets four keys of its own d.
 #pragma unroll
-    for (int u = 0; u < 2; ++u) {
-      half8_t bp;
+    for (int h = 0; h < SUB; ++h)
 #pragma unroll
-      for (int j = 0; j < 8; ++j) bp[j] = (half_t)p[8 * u + j];
+      for (int u = 0; u < 2; ++u)
 #pragma unroll
-      for (int db = 0; db < DB; ++db) {
-        const half4_t lo = lds_read_tr16(vt_base + (16 * u) * STR + db * 64);
-        const half4_t hi = lds_read_tr16(vt_base + (16 * u + 8) * STR + db * 64);
-        const half8_t a = half8_t{lo[0], lo[1], lo[2], lo[3], hi[0], hi[1], hi[2], hi[3]};
-        o_acc[db] = __builtin_amdgcn_mfma_f32_32x32x16_f16(a, bp, o_acc[db], 0, 0, 0);
-      }
-    }
+        for (int db = 0; db < DB; ++db) {
+          const half4_t lo = lds_read_tr16(vt_base + (32 * h + 16 * u) * STR + db * 64);
+          const half4_t hi = lds_read_tr16(vt_base + (32 * h + 16 * u + 8) * STR + db * 64);
+          const half8_t a = half8_t{lo[0], lo[1], lo[2], lo[3], hi[0], hi[1], hi[2], hi[3]};
+          o_acc[db] = __builtin_amdgcn_mfma_f32_32x32x16_f16(a, bp[h][u], o_acc[db], 0, 0, 0);
+        }
   };
   // whole rounds of DEPTH tiles (no condition between the stages of a round, so that the loads
   // outstanding at every wait are known), then the last DEPTH - 1 tiles at most
@@ -399,7 +409,7 @@ __global__ void tree_attn_merge_kernel(const half_t* __restrict__ part_o,
                                        const float* __restrict__ part_ml,
                                        half_t* __restrict__ out, int T, int H, int nsplit,
                                        const int32_t* __restrict__ len_dev, long cap,
-                                       int Tk, int q_rows, int len_stride, int groups) {
+                                       int Tk, int q_rows, int len_stride, int groups, int sub) {
   const int piece = blockIdx.z;                     // as in the split kernel
   if (T > q_rows - piece * 32) T = q_rows - piece * 32;
   part_o += (long)piece * H * nsplit * 32 * HD;
@@ -444,8 +454,8 @@ __global__ void tree_attn_merge_kernel(const half_t* __restrict__ part_o,
   int P = len_dev[piece * len_stride];
   if (P > cap - Tk) P = (int)(cap - Tk);    // as in the split kernel
   if (P < 0) P = 0;
-  const int nact = active_splits((P + Tk + KT - 1) / KT, nsplit, groups * gridDim.z,
-                                 split_slots(H / groups, HD));   // as in the split kernel
+  const int nact = active_splits((P + Tk + KT * sub - 1) / (KT * sub), nsplit, groups * gridDim.z,
+                                 split_slots(H / groups, HD), 3 - sub);   // as in the split kernel
   if (!eager) {
 #pragma unroll
     for (int k = 0; k < PRE; ++k)
@@ -511,27 +521,39 @@ int launch_attention(const half_t* q, half_t* kc, half_t* vc, const uint32_t* bi
   // work still takes a slot for the 2 us in which it learns that from the cache length, and
   // thousands of them ahead of the last pieces' workgroups (a chunk of 16 pieces in a grid of 36
   // splits for 4 active ones) held those back by 18 of 44 us.
+  const int rep = H / G;
+  // 64 keys per tile where a tile's 16-byte vectors are at most four per thread (three or more
+  // waves per workgroup at head dimension 128, two or more at 64), 32 keys otherwise and in the
+  // form that rotates and appends
+  const int need64 = (2 * KT * (HD / 8) + rep * 64 - 1) / (rep * 64);
+  const int sub = (!ROPE && need64 <= 4) ? 2 : 1;
+  const int ktt = KT * sub;
   int nsplit = splits_for(max_len, G);
-  nsplit = active_splits((max_len + KT - 1) / KT, nsplit, G * pieces, split_slots(H / G, HD));
+  nsplit = active_splits((max_len + ktt - 1) / ktt, nsplit, G * pieces, split_slots(rep, HD), 3 - sub);
   float* part_ml = static_cast<float*>(workspace);
   half_t* part_o = reinterpret_cast<half_t*>(part_ml + (size_t)pieces * H * nsplit * 32 * 2);
   const float sl2 = scale * 1.4426950408889634f;
-  const int rep = H / G;
-  const size_t lds = 2 * KT * (HD * 2 + 16) + (ROPE ? (size_t)EAGLE_MAX_TREE * HD * 4 : 0);
+  const size_t lds = 2 * ktt * (HD * 2 + 16) + (ROPE ? (size_t)EAGLE_MAX_TREE * HD * 4 : 0);
   // vectors of a tile per thread (a power of two) and the tiles in flight that its registers allow
-  const int need = (KT * (HD / 8) + rep * 64 - 1) / (rep * 64);
-#define EAGLE_ATTN_SPLIT(NVU, DEPTH)                                                                     \
-  hipLaunchKernelGGL((tree_attn_split_kernel<HD, ROPE, WIDE, NVU, ROPE ? 1 : DEPTH>), dim3(G, nsplit, pieces), \
-                     dim3(rep * 64), lds, st, q, kc, vc, bits, len, part_o, part_ml, T, H, G, cap, 0, sl2,      \
-                     k_lin, v_lin, ld, cs, Tk, q_rows, len_stride)
-  if (need <= 1) EAGLE_ATTN_SPLIT(1, 3);
-  else if (need <= 2) EAGLE_ATTN_SPLIT(2, 3);
-  else if (need <= 4) EAGLE_ATTN_SPLIT(4, 2);
-  else EAGLE_ATTN_SPLIT(8, 1);
+  const int need = (ktt * (HD / 8) + rep * 64 - 1) / (rep * 64);
+#define EAGLE_ATTN_SPLIT(NVU, DEPTH, SUB)                                                                \
+  hipLaunchKernelGGL((tree_attn_split_kernel<HD, ROPE, WIDE, NVU, ROPE ? 1 : DEPTH, ROPE ? 1 : SUB>),    \
+                     dim3(G, nsplit, pieces), dim3(rep * 64), lds, st, q, kc, vc, bits, len, part_o, part_ml, T, \
+                     H, G, cap, 0, sl2, k_lin, v_lin, ld, cs, Tk, q_rows, len_stride)
+  if (sub == 2) {
+    if (need <= 1) EAGLE_ATTN_SPLIT(1, 3, 2);
+    else if (need <= 2) EAGLE_ATTN_SPLIT(2, 2, 2);
+    else EAGLE_ATTN_SPLIT(4, 1, 2);
+  } else {
+    if (need <= 1) EAGLE_ATTN_SPLIT(1, 3, 1);
+    else if (need <= 2) EAGLE_ATTN_SPLIT(2, 3, 1);
+    else if (need <= 4) EAGLE_ATTN_SPLIT(4, 2, 1);
+    else EAGLE_ATTN_SPLIT(8, 1, 1);
+  }
 #undef EAGLE_ATTN_SPLIT
   hipLaunchKernelGGL(tree_attn_merge_kernel<HD>, dim3(H, (T + MERGE_TOK - 1) / MERGE_TOK, pieces),
                      dim3(MERGE_TOK * HD / 4), 0, st, part_o, part_ml, (half_t*)out, T, H, nsplit,
-                     len, cap, Tk, q_rows, len_stride, G);
+                     len, cap, Tk, q_rows, len_stride, G, sub);
   return eagle_launch_status();
 }
 
