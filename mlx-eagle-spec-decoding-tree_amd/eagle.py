@@ -473,9 +473,10 @@ class TreeVerifier:
         resident_gate_up: gate|up + SwiGLU through the kernel that keeps x in registers and brings
         the weights in by whole cache lines through LDS (`ops.quantized_matmul_resident`) instead of
         the streaming kernel.  Off unless asked for; takes K a multiple of 512 up to 3584 and scales
-        below 0.2499 in magnitude.  Inside the 7B step it is 1.4 us per layer faster (2.661 against
-        2.699 ms per step, A/B on one box); the measurement and profile records of `bench.py` are
-        those of the default form."""
+        below 0.2499 in magnitude.  Inside the 7B step it measured 1.4 us per layer faster when
+        built (2.661 against 2.699 ms per step, A/B on one box) and 0.6 us slower after the later
+        changes to the other kernels (2.632 against 2.616 ms); the measurement and profile records
+        of `bench.py` are those of the default form."""
         args = model.args
         self.model, self.cache, self.args = model, cache, args
         if total_tokens + 1 > TREE_SLOTS:
