@@ -108,7 +108,7 @@ __global__ __launch_bounds__(512) void tree_attn_split_kernel(
     const half_t* __restrict__ q, half_t* kc, half_t* vc,
     const uint32_t* __restrict__ mask_bits, const int32_t* __restrict__ len_dev,
     half_t* __restrict__ part_o, float* __restrict__ part_ml, int T, int H, int G, long cap,
-    int tiles_per_split, float scale_log2e, const half_t* __restrict__ k_lin,
+    float scale_log2e, const half_t* __restrict__ k_lin,
     const half_t* __restrict__ v_lin, long ld, const float* __restrict__ rope_cs, int Tk, int q_rows,
     int len_stride) {
   constexpr int KSTEPS = HD / 16;       // MFMA steps over the head dimension for S
@@ -539,7 +539,7 @@ int launch_attention(const half_t* q, half_t* kc, half_t* vc, const uint32_t* bi
 #define EAGLE_ATTN_SPLIT(NVU, DEPTH, SUB)                                                                \
   hipLaunchKernelGGL((tree_attn_split_kernel<HD, ROPE, WIDE, NVU, ROPE ? 1 : DEPTH, ROPE ? 1 : SUB>),    \
                      dim3(G, nsplit, pieces), dim3(rep * 64), lds, st, q, kc, vc, bits, len, part_o, part_ml, T, \
-                     H, G, cap, 0, sl2, k_lin, v_lin, ld, cs, Tk, q_rows, len_stride)
+                     H, G, cap, sl2, k_lin, v_lin, ld, cs, Tk, q_rows, len_stride)
   if (sub == 2) {
     if (need <= 1) EAGLE_ATTN_SPLIT(1, 3, 2);
     else if (need <= 2) EAGLE_ATTN_SPLIT(2, 2, 2);
