@@ -59,7 +59,7 @@ def write_traffic_record(fetch_csv, write_csv):
                 if r["Counter_Name"] != name:
                     continue
                 kn = r["Kernel_Name"]
-                if "qmm_w4g64" in kn or "qmm_slab_w4g64" in kn or "qmm_res_w4g64" in kn:
+                if "qmm_w4g64" in kn or "qmm_slab_w4g64" in kn:
                     q.append(float(r["Counter_Value"]))
                 if "copyBuffer" in kn or "elementwise" in kn:
                     cp.append(float(r["Counter_Value"]))
@@ -170,9 +170,6 @@ def main():
     ap.add_argument("--no-draft-folded", action="store_true",
                     help="--loop: the drafter's passes with one launch per operator instead of the small-row "
                          "products with norm / residual / SwiGLU folded in")
-    ap.add_argument("--chain", action="store_true",
-                    help="residual add + norm + gate|up + SwiGLU as one launch of a resident grid with a "
-                         "grid-wide barrier inside (off by default: slower than the two launches it replaces)")
     ap.add_argument("--sweep", action="store_true", help="also print the per-shape QMM table to stderr")
     ap.add_argument("--calibrate-copy", action="store_true",
                     help="before anything else run one 1 GiB device copy (a kernel of known traffic: "
@@ -268,8 +265,7 @@ def main():
     slab_plan = None
     if opt.slabs is not None:
         slab_plan = {kv.split("=")[0]: int(kv.split("=")[1]) for kv in opt.slabs.split(",") if kv}
-    ver = eagle.TreeVerifier(model, cache, total_tokens=NODES - 1, max_len=cap, slab_plan=slab_plan,
-                             chain=opt.chain)
+    ver = eagle.TreeVerifier(model, cache, total_tokens=NODES - 1, max_len=cap, slab_plan=slab_plan)
     ver.set_tree(torch.from_numpy(tokens).to(dev), torch.from_numpy(depth.astype(np.int32)).to(dev),
                  torch.from_numpy(parents).to(dev),
                  torch.from_numpy(bits.view(np.int32)).to(dev))
@@ -304,22 +300,15 @@ def main():
     ver.act.normal_()
 
     def qmm_only(subset=None):
-        for wq, sc, bi, bias, x, out, form in (launches if subset is None else subset):
-            if form == "chain":
-                (gw, gs, gb, gbias), nw, nslab = wq, sc, bi
-                ops.norm_mlp_in(x, nslab, ver.h, nw, args.rms_norm_eps, gw, gs, gb, gbias, out,
-                                ver.chain_scratch, ver.chain_err)
-            elif form is True:
-                ops.quantized_matmul_swiglu(x, wq, sc, bi, bias=bias, out=out)
+        for wq, sc, bi, bias, x, out, form, tiled in (launches if subset is None else subset):
+            if form is True:
+                ops.quantized_matmul_swiglu(x, wq, sc, bi, bias=bias, out=out, tiled=tiled)
             elif form:
-                ops.quantized_matmul_slabs(x, wq, sc, bi, form, partial=ver.partial)
+                ops.quantized_matmul_slabs(x, wq, sc, bi, form, partial=ver.partial, tiled=tiled)
             else:
                 ops.quantized_matmul(x, wq, sc, bi, bias=bias, out=out)
 
     def alg_bytes(l):
-        if l[6] == "chain":               # the product inside the chained launch
-            gw = l[0][0]
-            return qmm_bytes(NODES, gw.shape[0], gw.shape[1] * 8, l[5].shape[-1])
         return qmm_bytes(NODES, l[0].shape[0], l[0].shape[1] * 8, l[5].shape[-1])
 
     qt, _ = graph_time_ms(torch, qmm_only, reps=10)
@@ -330,7 +319,7 @@ def main():
     achieved = alg / (qmm_ms * 1e-3) / 1e9
     traffic, traffic_source = read_traffic_record()
     stream_kernel = "qmm_w4g64_kernel"          # (above 32 tree tokens: two launches of it per product)
-    kernels = stream_kernel + " + qmm_slab_w4g64_kernel" + (" + norm_mlp_in_kernel" if ver.chain else "")
+    kernels = stream_kernel + " + qmm_slab_w4g64_kernel"
     roofline = {"bound": "hbm", "kernel": kernels, "achieved": round(achieved, 1),
                 "peak": HBM_PEAK_GBS, "unit": "GB/s", "frac": round(achieved / HBM_PEAK_GBS, 4),
                 "traffic": traffic, "traffic_source": traffic_source, "launches_per_step": n_launch,
@@ -341,12 +330,12 @@ def main():
     # the same for each kernel on its own launches
     per_kernel = {}
     # (above 32 tree tokens gate|up + SwiGLU runs on the slab kernel too: one slab over all of K)
-    swi_name = "qmm_slab_w4g64_kernel (SwiGLU form)" if ver.wide else stream_kernel
+    swi_on_slab = ver.wide or any(l[6] is True and l[7] is not None for l in launches)
+    swi_name = "qmm_slab_w4g64_kernel (SwiGLU form)" if swi_on_slab else stream_kernel
     groups = ([(swi_name, [l for l in launches if l[6] is True]), (stream_kernel, [l for l in launches if not l[6]])]
-              if ver.wide else [(stream_kernel, [l for l in launches if l[6] is True or not l[6]])])
+              if swi_on_slab else [(stream_kernel, [l for l in launches if l[6] is True or not l[6]])])
     for kname, sub in (*groups,
-                       ("qmm_slab_w4g64_kernel", [l for l in launches if l[6] and l[6] is not True and l[6] != "chain"]),
-                       ("norm_mlp_in_kernel", [l for l in launches if l[6] == "chain"])):
+                       ("qmm_slab_w4g64_kernel", [l for l in launches if l[6] and l[6] is not True])):
         if not sub:
             continue
         st, _ = graph_time_ms(torch, lambda: qmm_only(sub), reps=10)
@@ -357,9 +346,6 @@ def main():
                              "achieved": round(sub_alg / (sub_ms * 1e-3) / 1e9, 1),
                              "frac": round(sub_alg / (sub_ms * 1e-3) / 1e9 / HBM_PEAK_GBS, 4)}
     roofline["per_kernel"] = per_kernel
-    if ver.chain and bool(ver.chain_err.item()):
-        print("bench.py: a grid barrier of the chained launch gave up", file=sys.stderr)
-        sys.exit(1)
 
     if opt.sweep:
         sweep(torch, ops, dev, args)

@@ -68,36 +68,6 @@ int eagle_qmm_w4g64_f16(const void* x, const uint32_t* wq, const void* scales,
                         const void* biases, const void* bias, void* out,
                         int M, int N, int K, int group_size, int bits,
                         void* workspace, size_t workspace_bytes, eagle_stream_t stream);
-/* Residual add, RMSNorm, gate|up and SwiGLU of a decoder layer in ONE launch of a resident grid
- * (256 workgroups, one per compute unit): first h += fp16(sum of the K slabs of the product that
- * precedes the norm) and the sums of squares of the new h, spread over the whole grid; then,
- * across a grid-wide barrier, act = silu(g) * u with (g | u) = RMSNorm(h) . Wgu^T, the norm folded
- * into the load of x (mlx_llama.py:240-243, 214-215, 225-228).  The weights of the product are
- * requested at the start of the launch and stay in flight across the barrier, which a kernel
- * boundary cannot do.  Replaces eagle_rmsnorm_slabs_f16 (residual form) followed by
- * eagle_qmm_swiglu_w4g64_f16.
- *   partial [slabs][32][D] fp32 from eagle_qmm_slab_partial_w4g64 (the o projection, no bias);
- *   h [M, D] fp16, updated in place; norm_w [D] fp16; gu_* the gate and up projections [2 I, D]
- *   interleaved in 16-row tiles as for eagle_qmm_swiglu_w4g64_f16, gu_bias [2 I] interleaved or
- *   NULL; act [M, I] fp16.
- * Constraints (eagle_norm_mlp_in_supported): D % 512 == 0, D <= 3584, I % 16 == 0, every scale
- * below 0.2499 (as eagle_qmm_res_w4g64_f16), a device with at least 256 compute units; all
- * pointers 16-byte aligned.
- * `scratch` (eagle_norm_mlp_in_scratch_bytes) holds the sums of squares and the barrier counters;
- * it must be ZERO before the first launch and belongs to this entry point from then on (the
- * counters only grow; launches sharing it must be stream ordered and on one device).
- * The wait at the barrier is bounded: after `spin_limit_ticks` (100 MHz ticks) a workgroup stores 1
- * to *err_dev and the launch ends without the product; the caller then has to zero `scratch` and
- * *err_dev before the next launch.  The grid needs every compute unit of the device to itself
- * for the duration of the launch. */
-size_t eagle_norm_mlp_in_scratch_bytes(void);
-int eagle_norm_mlp_in_supported(int M, int D, int I);
-int eagle_norm_mlp_in_f16(const float* partial, int slabs, void* h, const void* norm_w, float eps,
-                          const uint32_t* gu_wq, const void* gu_scales, const void* gu_biases,
-                          const void* gu_bias, void* act, int M, int D, int I,
-                          void* scratch, size_t scratch_bytes, int* err_dev,
-                          long long spin_limit_ticks, eagle_stream_t stream);
-
 /* The product for a pass of at most 16 rows through a small model (the drafter's passes of the
  * tree loop), with the operators around it folded in, so that a decoder layer needs four of
  * these launches and no norm / add launch (mlx_llama.py:195-196, 214-215, 225-249):
@@ -203,21 +173,6 @@ int eagle_qmm_gemm_swiglu_w4g64_f16(const void* x, const uint32_t* wq, const voi
                                     const void* biases, const void* bias, void* out, int M, int N,
                                     int K, int group_size, int bits, eagle_stream_t stream);
 
-/* The same product (and its SwiGLU form when `swiglu` != 0, weights interleaved as for
- * eagle_qmm_swiglu_w4g64_f16, out [M, N/2]) for 1..32 rows with x resident in registers: one
- * workgroup per compute unit, the K range split in units of 512 over its waves, whole K per
- * workgroup, so no workspace and no counters.  K % 512 == 0 and K <= 3584
- * (eagle_qmm_res_supported returns 1), N % 8 == 0 (N % 32 == 0 with swiglu); x, wq, scales and
- * biases 16-byte aligned, out 8-byte aligned.  Every scale must be below 0.2499 (weights are
- * expanded through fp16 subnormals, scale * 2^18 has to be finite in fp16); larger scales give
- * inf / NaN, never a finite wrong value.
- * Replaces the same call sites as eagle_qmm_w4g64_f16 (qmm_kernel.py:84-164,
- * mlx_model_fwd_bench.py:65-73) and, with swiglu, mlx_llama.py:214-215. */
-int eagle_qmm_res_supported(int M, int N, int K);
-int eagle_qmm_res_w4g64_f16(const void* x, const uint32_t* wq, const void* scales,
-                            const void* biases, const void* bias, void* out, int M, int N, int K,
-                            int group_size, int bits, int swiglu, eagle_stream_t stream);
-
 /* The same product for 1..64 rows in the slab form, with the result left as fp32 partial sums:
  * every workgroup owns 128 weight rows and one K slab of `steps_per_slab` quantisation groups
  * (a multiple of 8), moves x through LDS eight groups at a time and expands the weights to fp16
@@ -252,6 +207,34 @@ int eagle_qmm_slab_swiglu_preferred(int M, int N, int K);
 int eagle_qmm_slab_swiglu_w4g64_f16(const void* x, const uint32_t* wq, const void* scales,
                                     const void* biases, const void* bias, void* out, int M, int N, int K,
                                     int group_size, int bits, eagle_stream_t stream);
+/* The weights of a projection in the layout the 32-row slab kernels stream fastest.  The
+ * reference keeps every matrix row-major ([N, K/8] words, qmm_kernel.py:101-104, and re-orders
+ * them offline only in its swizzle experiment, swizzle.py:41-75); read that way a wave's load
+ * touches 32 cache lines for 1 KB.  eagle_qmm_tile_w4g64 re-lays a matrix out once (not in
+ * place) as
+ *   wt  [N/32 tiles][K/64 groups][64 lanes][4 words]: lane l of a wave holds words 4 (l / 32) ..
+ *       4 (l / 32) + 3 of the group for row 32 tile + l % 32, so a tile's group is one contiguous
+ *       1 KB block in the order the lanes use it;
+ *   sbt [N/32 tiles][K/512 chunks][64 lanes][8 halves]: lanes 0..31 the scales of their row for
+ *       the chunk's eight groups, lanes 32..63 the biases (eagle_qmm_tiled_sb_bytes bytes).
+ * N % 32 == 0, K % 512 == 0, all pointers 16-byte aligned.
+ * eagle_qmm_slab_partial_tiled_w4g64 / eagle_qmm_slab_swiglu_tiled_w4g64_f16 are
+ * eagle_qmm_slab_partial_w4g64 / eagle_qmm_slab_swiglu_w4g64_f16 for 1..32 rows on that copy
+ * (same results, same partial-sum layout, same consumers).  small_scales != 0 promises that
+ * every |scale| is below 0.0624: the nibbles are then expanded through fp16 subnormals (scale *
+ * 2^20 must be a finite fp16; larger scales give inf / NaN, never a finite wrong value).
+ * Replace the same call sites (qmm_kernel.py:84-164, mlx_model_fwd_bench.py:65-73; with the
+ * SwiGLU epilogue mlx_llama.py:214-215). */
+int eagle_qmm_tiled_supported(int M, int N, int K);
+size_t eagle_qmm_tiled_sb_bytes(int N, int K);
+int eagle_qmm_tile_w4g64(const uint32_t* wq, const void* scales, const void* biases, uint32_t* wt,
+                         void* sbt, int N, int K, int group_size, int bits, eagle_stream_t stream);
+int eagle_qmm_slab_partial_tiled_w4g64(const void* x, const uint32_t* wt, const void* sbt,
+                                       float* partial, size_t partial_bytes, int M, int N, int K,
+                                       int steps_per_slab, int small_scales, eagle_stream_t stream);
+int eagle_qmm_slab_swiglu_tiled_w4g64_f16(const void* x, const uint32_t* wt, const void* sbt,
+                                          const void* bias, void* out, int M, int N, int K,
+                                          int small_scales, eagle_stream_t stream);
 /* out [M,N] fp16 = fp16(sum of the slabs) (+ bias [N] fp16, 16-byte aligned, may be NULL). */
 int eagle_slab_sum_f16(const float* partial, int slabs, const void* bias, void* out, int M, int N,
                        eagle_stream_t stream);
@@ -342,7 +325,7 @@ int eagle_rope_kv_append_slabs_f16(const float* partial, int slabs, const void* 
                                    const int32_t* cache_len_dev, int T, int H, int G, int hd,
                                    long capacity, eagle_stream_t stream);
 
-/* cos/sin table for eagle_rope_kv_append_table_f16 and eagle_tree_attention_rope_f16: out[t][i] = (cos, sin)(positions[t] *
+/* cos/sin table for eagle_rope_kv_append_table_f16: out[t][i] = (cos, sin)(positions[t] *
  * scaling_factor * inv_freqs[i]), fp32 [T, half_dim, 2]; the same angles as
  * eagle_rope_arrayed_f16 (mlx_arrayed_rope_kernel.py:60-123).  The table depends on the tree
  * positions only, so one call serves every layer of a step. */
@@ -350,24 +333,6 @@ int eagle_rope_table_f32(const int32_t* positions, const float* inv_freqs, float
                          int T, int half_dim, float* out, eagle_stream_t stream);
 /* Both table forms take up to EAGLE_MAX_CHUNK rows (a prompt chunk); the other tree entry
  * points take at most EAGLE_MAX_TREE. */
-
-/* The attention block of one layer without a separate rope launch (mlx_llama.py:166-195: rope of q and k with
- * per-token positions, cache update, masked SDPA).  q_lin / k_lin / v_lin are the token-major
- * projection outputs ([T, H*hd], [T, G*hd], [T, G*hd]) with a common row stride in elements
- * (columns of one fused q|k|v matrix, or row_stride = the width of each when separate and
- * equal).  Rotated keys and the values of the T tree tokens are written to cache rows
- * P .. P+T-1 (P = *cache_len_dev) and attended to together with the prefix under
- * tree_mask_bits, exactly as eagle_rope_kv_append_f16 followed by eagle_tree_attention_f16
- * (one launch less: tree rows are read from the projections, rotated on the way, and stored
- * to the cache by the workgroup that owns their key tile).  out [T, H*hd].  Calls sharing a
- * workspace must be stream ordered. */
-size_t eagle_tree_attention_rope_workspace_bytes(int H, int hd, int max_len);
-int eagle_tree_attention_rope_f16(const void* q_lin, const void* k_lin, const void* v_lin,
-                                  long row_stride, const float* rope_cs, void* k_cache,
-                                  void* v_cache, const uint32_t* tree_mask_bits,
-                                  const int32_t* cache_len_dev, void* out, int T, int H, int G,
-                                  int hd, long capacity, int max_len, float scale, void* workspace,
-                                  size_t workspace_bytes, eagle_stream_t stream);
 
 /* Attention of the draft-side expansion (mlx_eagle.py:143-178,207 through mlx_llama.py:185-192):
  * T <= 32 query tokens against the P = *cache_len_dev prefix rows (visible to every query) and

@@ -23,10 +23,6 @@ SIGNATURES = {
     "eagle_qmm_w4g64_f16": (c_int, [c_void_p] * 6 + [c_int] * 5 + [c_void_p, c_size_t, c_void_p]),
     "eagle_qmm_noalloc_scratch_bytes": (c_size_t, []),
     "eagle_qmm_w4g64_f16_noalloc": (c_int, [c_void_p] * 6 + [c_int] * 5 + [c_void_p]),
-    "eagle_norm_mlp_in_scratch_bytes": (c_size_t, []),
-    "eagle_norm_mlp_in_supported": (c_int, [c_int] * 3),
-    "eagle_norm_mlp_in_f16": (c_int, [c_void_p, c_int, c_void_p, c_void_p, c_float] + [c_void_p] * 5
-                              + [c_int] * 3 + [c_void_p, c_size_t, c_void_p, c_longlong, c_void_p]),
     "eagle_qmm_small_supported": (c_int, [c_int] * 5),
     "eagle_qmm_small_w4g64_f16": (c_int, [c_void_p, c_void_p, c_float] + [c_void_p] * 6 + [c_int] * 6 + [c_void_p]),
     "eagle_qkv_rope_small_supported": (c_int, [c_int] * 5),
@@ -40,13 +36,16 @@ SIGNATURES = {
     "eagle_qmm_w4g64_f16_tuned": (c_int, [c_void_p] * 6 + [c_int] * 8 + [c_void_p, c_size_t, c_void_p]),
     "eagle_qmm_gemm_w4g64_f16": (c_int, [c_void_p] * 6 + [c_int] * 5 + [c_void_p]),
     "eagle_qmm_gemm_swiglu_w4g64_f16": (c_int, [c_void_p] * 6 + [c_int] * 5 + [c_void_p]),
-    "eagle_qmm_res_supported": (c_int, [c_int] * 3),
-    "eagle_qmm_res_w4g64_f16": (c_int, [c_void_p] * 6 + [c_int] * 6 + [c_void_p]),
     "eagle_qmm_slab_count": (c_int, [c_int] * 2),
     "eagle_qmm_slab_steps": (c_int, [c_int] * 3),
     "eagle_qmm_slab_partial_bytes": (c_size_t, [c_int] * 3),
     "eagle_qmm_slab_partial_bytes_rows": (c_size_t, [c_int] * 4),
     "eagle_qmm_slab_partial_w4g64": (c_int, [c_void_p] * 5 + [c_size_t] + [c_int] * 6 + [c_void_p]),
+    "eagle_qmm_tiled_supported": (c_int, [c_int] * 3),
+    "eagle_qmm_tiled_sb_bytes": (c_size_t, [c_int] * 2),
+    "eagle_qmm_tile_w4g64": (c_int, [c_void_p] * 5 + [c_int] * 4 + [c_void_p]),
+    "eagle_qmm_slab_partial_tiled_w4g64": (c_int, [c_void_p] * 4 + [c_size_t] + [c_int] * 5 + [c_void_p]),
+    "eagle_qmm_slab_swiglu_tiled_w4g64_f16": (c_int, [c_void_p] * 5 + [c_int] * 4 + [c_void_p]),
     "eagle_qmm_slab_swiglu_supported": (c_int, [c_int] * 3),
     "eagle_qmm_slab_swiglu_preferred": (c_int, [c_int] * 3),
     "eagle_qmm_slab_swiglu_w4g64_f16": (c_int, [c_void_p] * 6 + [c_int] * 5 + [c_void_p]),
@@ -79,9 +78,6 @@ SIGNATURES = {
     "eagle_causal_attention_f16": (c_int, [c_void_p] * 5 + [c_int] * 4 + [c_long, c_int, c_float,
                                                                          c_void_p, c_size_t, c_void_p]),
     "eagle_rope_table_f32": (c_int, [c_void_p, c_void_p, c_float, c_int, c_int, c_void_p, c_void_p]),
-    "eagle_tree_attention_rope_workspace_bytes": (c_size_t, [c_int, c_int, c_int]),
-    "eagle_tree_attention_rope_f16": (c_int, [c_void_p] * 3 + [c_long] + [c_void_p] * 6 + [c_int] * 4
-                                      + [c_long, c_int, c_float, c_void_p, c_size_t, c_void_p]),
     "eagle_rmsnorm_f16": (c_int, [c_void_p] * 3 + [c_float] + [c_void_p] * 2 + [c_int] * 2 + [c_void_p]),
     "eagle_silu_mul_f16": (c_int, [c_void_p] * 3 + [c_int] * 2 + [c_void_p]),
     "eagle_add_f16": (c_int, [c_void_p] * 3 + [c_long, c_void_p]),

@@ -92,6 +92,26 @@ __device__ inline half8_t dequant_word_centred(uint32_t w, half2_t s2, half2_t b
   return o;
 }
 
+// Through fp16 subnormals: a masked nibble pair left at mantissa bits 4..7 is (q_i, q_j) * 2^-20
+// exactly, and one packed fma with (s * 2^20, b) gives fp16(s*q + b) with a single rounding and
+// no offset: three shifts, four masks and four fmas per packed word.  |s| * 2^20 has to stay
+// inside fp16: |s| < 0.0624 (beyond it the product is inf / NaN).
+__device__ inline half8_t dequant_word_sub(uint32_t w, half2_t s20, half2_t b2) {
+  union { uint32_t u; half2_t h; } c[4];
+  c[0].u = (w << 4) & 0x00f000f0u;
+  c[1].u = w & 0x00f000f0u;
+  c[2].u = (w >> 4) & 0x00f000f0u;
+  c[3].u = (w >> 8) & 0x00f000f0u;
+  half8_t o;
+#pragma unroll
+  for (int i = 0; i < 4; ++i) {
+    const half2_t v = __builtin_elementwise_fma(c[i].h, s20, b2);
+    o[2 * i] = v[0];
+    o[2 * i + 1] = v[1];
+  }
+  return o;
+}
+
 // MT = 32-row x tiles per wave: 2 (128-row blocks) or 4 (256-row blocks: twice the matrix work
 // per expanded weight and per byte read from LDS).
 template <int E>
@@ -454,6 +474,12 @@ int launch_gemm(const half_t* x, const uint32_t* w, const half_t* s, const half_
 // slab_sum_kernel below).  A last-arriver reduction inside this kernel (partial store, wait,
 // counter, loads of all slabs, store) is a chain of device-scope round trips that took longer
 // than the product itself: 14.1 us against 5.7 us for 32 x 4608 x 3584.
+#ifdef EAGLE_TRACE
+__device__ unsigned long long* g_trace = nullptr;
+#define EAGLE_TR(tr, ev) do { if ((tr) && (threadIdx.x & 63) == 0) (tr)[ev] = wall_clock64(); } while (0)
+#else
+#define EAGLE_TR(tr, ev) do { } while (0)
+#endif
 constexpr int SLAB_RING = 8;
 constexpr int SLAB_ROWS = 32;               // rows of x per accumulator tile
 constexpr int SLAB_XR = SLAB_RING * 64 + 8; // LDS row stride of an x chunk in halves
@@ -475,12 +501,19 @@ constexpr int SLAB_XBUF = SLAB_ROWS * SLAB_XR;
 // WR: register sets of eight weight loads per lane (1: the loads of the next chunk are in flight
 // while a chunk is used; 2: those of the next two, for slabs of many chunks, where the time per
 // step is the load latency divided by the loads in flight).
-template <bool RAGGED, int MR = 1, bool SWI = false, int NWV = 4, int WR = 1>
+// TL: the weights come in the tiled layout (eagle_qmm_tile_w4g64): w is [N/32 tiles][K/64 steps]
+// [64 lanes][4 words], one contiguous 1 KB block per wave and step in the order the lanes hold it,
+// and s is [N/32 tiles][K/512 chunks][64 lanes][8 halves] with the scales of the chunk's eight
+// groups in lanes 0..31 (one row each) and the biases in lanes 32..63; b is not read.  A load
+// instruction then touches eight whole cache lines instead of pieces of 32 or 64.
+// SUBN: expansion through fp16 subnormals (dequant_word_sub), for |scale| < 0.0624.
+template <bool RAGGED, int MR = 1, bool SWI = false, int NWV = 4, int WR = 1, bool TL = false, bool SUBN = false>
 __global__ __launch_bounds__(64 * NWV) void qmm_slab_w4g64_kernel(
     const half_t* __restrict__ x, const uint32_t* __restrict__ w, const half_t* __restrict__ s,
     const half_t* __restrict__ b, float* __restrict__ partial, int M, int N, int K, int spz, int xbufs,
     const half_t* __restrict__ swi_bias = nullptr, half_t* __restrict__ swi_out = nullptr) {
   static_assert(SWI || NWV == 4, "the partial-sum epilogue is laid out for four waves");
+  static_assert(!TL || !RAGGED, "the tiled layout holds whole chunks");
   extern __shared__ __attribute__((aligned(16))) half_t xlds[];   // one or two x chunks
   constexpr int XBUF = MR * SLAB_XBUF;
   const int tid = threadIdx.x;
@@ -507,16 +540,18 @@ __global__ __launch_bounds__(64 * NWV) void qmm_slab_w4g64_kernel(
   }
   int nrow = blockIdx.x * (32 * NWV) + wave * 32 + ql;
   if (nrow > N - 1) nrow = N - 1;
-  const uint32_t* wp = w + (long)nrow * KW + g0 * 8 + hb * 4;
-  const half_t* sp = s + (long)nrow * G + g0;
-  const half_t* bp = b + (long)nrow * G + g0;
+  int tile = blockIdx.x * NWV + wave;        // TL: the wave's 32-row tile (rows past N are never stored)
+  if (tile > (N >> 5) - 1) tile = (N >> 5) - 1;
+  const uint32_t* wp = TL ? w + ((long)tile * G + g0) * 256 + lane * 4 : w + (long)nrow * KW + g0 * 8 + hb * 4;
+  const half_t* sp = TL ? s + ((long)tile * (G >> 3) + (g0 >> 3)) * 512 + lane * 8 : s + (long)nrow * G + g0;
+  const half_t* bp = TL ? nullptr : b + (long)nrow * G + g0;
 
   half8_t xreg[MR][SLAB_RING];
   uint4_t wreg[WR][SLAB_RING];
   half8_t s8, b8, s8n, b8n;
   // the packed words of one step of this lane's row (steps past the slab repeat its last one)
   auto wload = [&](int step) {
-    return *reinterpret_cast<const uint4_t*>(wp + (step < steps ? step : steps - 1) * 8);
+    return *reinterpret_cast<const uint4_t*>(wp + (step < steps ? step : steps - 1) * (TL ? 256 : 8));
   };
   auto fetch_x = [&](int c) {
     if (!mover) return;
@@ -528,7 +563,10 @@ __global__ __launch_bounds__(64 * NWV) void qmm_slab_w4g64_kernel(
   };
   // scales and biases of chunk c: one 16-byte fetch, or four 4-byte fetches kept inside the slab
   auto fetch_sb = [&](int c, half8_t& s_out, half8_t& b_out) {
-    if (!RAGGED) {
+    if constexpr (TL) {
+      // one 16-byte load per lane: scales in the lower half of the wave, biases in the upper
+      s_out = *reinterpret_cast<const half8_t*>(sp + c * 512);
+    } else if (!RAGGED) {
       s_out = *reinterpret_cast<const half8_t*>(sp + c * 8);
       b_out = *reinterpret_cast<const half8_t*>(bp + c * 8);
     } else {
@@ -553,6 +591,12 @@ __global__ __launch_bounds__(64 * NWV) void qmm_slab_w4g64_kernel(
         *reinterpret_cast<half8_t*>(&xlds[buf * XBUF + (xr + 32 * r) * SLAB_XR + i * 64 + xc * 8]) =
             permute8(xreg[r][i]);
   };
+#ifdef EAGLE_TRACE
+  unsigned long long* tr = g_trace ? g_trace + ((size_t)(blockIdx.y * gridDim.x + blockIdx.x) * 16 + wave) * 24 : nullptr;
+#else
+  unsigned long long* tr = nullptr;
+#endif
+  EAGLE_TR(tr, 0);
   fetch_x(0);
   fetch_sb(0, s8, b8);
 #pragma unroll
@@ -563,9 +607,11 @@ __global__ __launch_bounds__(64 * NWV) void qmm_slab_w4g64_kernel(
     for (int i = 0; i < SLAB_RING; ++i) wreg[1][i] = wload(SLAB_RING + i);
   }
   __builtin_amdgcn_sched_barrier(0);
+  EAGLE_TR(tr, 1);
   stash_x(0);
   if (chunks > 1) fetch_x(1);
   __syncthreads();
+  EAGLE_TR(tr, 2);
 
   float16_t acc[MR];
 #pragma unroll
@@ -579,15 +625,31 @@ __global__ __launch_bounds__(64 * NWV) void qmm_slab_w4g64_kernel(
   auto chunk = [&](int c, int buf, auto RELOAD, auto PAR) {
     constexpr bool reload = decltype(RELOAD)::value != 0;
     constexpr int par = WR == 2 ? decltype(PAR)::value : 0;   // the register set of this chunk
+    if constexpr (TL) {
+      // s8 holds what this lane loaded (scales in lanes 0..31, biases in 32..63): exchange the
+      // halves of the wave so that every lane has both
+      union { half8_t h; uint32_t u[4]; } own, oth;
+      own.h = s8;
+#pragma unroll
+      for (int i = 0; i < 4; ++i) oth.u[i] = __shfl_xor(own.u[i], 32, 64);
+      s8 = hb ? oth.h : own.h;
+      b8 = hb ? own.h : oth.h;
+    }
     if (reload) fetch_sb(c + 1, s8n, b8n);
 #pragma unroll
     for (int e = 0; e < 8; ++e) {
       if (RAGGED && !reload && e >= rem) break;            // the last chunk may be partial
       const half_t sc = s8[e], bi = b8[e];
-      const half_t bc = (half_t)((float)bi + 8.f * (float)sc);
       half8_t af[4];
+      if constexpr (SUBN) {
+        const half_t s20 = (half_t)((float)sc * 1048576.f);
 #pragma unroll
-      for (int j = 0; j < 4; ++j) af[j] = dequant_word_centred(wreg[par][e][j], half2_t{sc, sc}, half2_t{bc, bc});
+        for (int j = 0; j < 4; ++j) af[j] = dequant_word_sub(wreg[par][e][j], half2_t{s20, s20}, half2_t{bi, bi});
+      } else {
+        const half_t bc = (half_t)((float)bi + 8.f * (float)sc);
+#pragma unroll
+        for (int j = 0; j < 4; ++j) af[j] = dequant_word_centred(wreg[par][e][j], half2_t{sc, sc}, half2_t{bc, bc});
+      }
       if constexpr (WR == 2) wreg[par][e] = wload((c + 2) * 8 + e);
       else if (reload) wreg[0][e] = wload((c + 1) * 8 + e);
 #pragma unroll
@@ -628,9 +690,13 @@ __global__ __launch_bounds__(64 * NWV) void qmm_slab_w4g64_kernel(
     int c = 0;
     for (; c + 2 < chunks; c += 2) {
       chunk(c, c & bmask, StepIndex<1>{}, StepIndex<0>{});
+      EAGLE_TR(tr, 3 + 2 * c);
       next_x(c);
+      EAGLE_TR(tr, 4 + 2 * c);
       chunk(c + 1, (c + 1) & bmask, StepIndex<1>{}, StepIndex<1>{});
+      EAGLE_TR(tr, 5 + 2 * c);
       next_x(c + 1);
+      EAGLE_TR(tr, 6 + 2 * c);
     }
     if (c + 1 < chunks) {
       chunk(c, c & bmask, StepIndex<1>{}, StepIndex<0>{});
@@ -642,10 +708,13 @@ __global__ __launch_bounds__(64 * NWV) void qmm_slab_w4g64_kernel(
   } else {
     for (int c = 0; c + 1 < chunks; ++c) {
       chunk(c, c & bmask, StepIndex<1>{}, StepIndex<0>{});
+      EAGLE_TR(tr, 3 + 2 * c);
       next_x(c);
+      EAGLE_TR(tr, 4 + 2 * c);
     }
     chunk(chunks - 1, (chunks - 1) & bmask, StepIndex<0>{}, StepIndex<0>{});
   }
+  EAGLE_TR(tr, 22);
 
   // accumulator register i of a lane: weight row 8*(i/4) + 4*hb + i%4 of the wave's tile, x
   // row ql (+ 32 for the second tile).  Through LDS, so that the lanes of a wave store whole
@@ -708,6 +777,299 @@ __global__ __launch_bounds__(64 * NWV) void qmm_slab_w4g64_kernel(
   }
 }
 
+// ------------------------------------------------------------------------------------------
+// The same two products (partial sums of a K slab; gate|up with the SwiGLU epilogue) with every
+// weight request of a wave in flight at once
+// ------------------------------------------------------------------------------------------
+// What bounds the kernel above at 32 rows is the number of bytes a compute unit has in flight:
+// four or five waves with eight or sixteen 16-byte loads per lane are 32 - 80 KB, and at the
+// 3 - 5 us a request takes under load that is 2.3 - 4 TB/s over the whole GPU.  Here a workgroup
+// owns TILES 32-row weight tiles and one K slab of whole chunks, and
+//   * two streaming waves share a weight tile: each takes four of a chunk's eight steps (a
+//     whole 128-byte line of every weight row of the tile per chunk) and keeps the loads of
+//     four chunks in flight, 16 KB per wave, issued before anything else; for a slab of up to
+//     four chunks that is every weight byte of the workgroup at the start of the kernel.
+//     The chunk loop is unrolled over a compile-time chunk count, all loads unconditional;
+//   * two more waves only carry x: a whole chunk per step of their loop (global -> registers ->
+//     LDS in operand order), so that the streaming waves' in-order load counters never wait
+//     for an x load that was issued behind their prefetched weights;
+//   * one LDS-only barrier per chunk; at the end the second wave of a tile hands its
+//     accumulators to the first through LDS, which runs the epilogue of the kernel above.
+// SUBN: expansion through fp16 subnormals (dequant_word_sub), for |scale| < 0.0624.
+#ifndef EAGLE_BURST_CA
+#define EAGLE_BURST_CA 2
+#endif
+constexpr int BURST_CA = EAGLE_BURST_CA;     // chunks of weight loads in flight per wave
+constexpr int BURST_MOVERS = 4;              // waves that only carry x
+constexpr int BURST_XB = 3;                  // x chunks in LDS
+constexpr int BURST_SPW = 4;                 // steps of a chunk per streaming wave
+
+template <bool SUBN, int NCH>
+__device__ inline void burst_stream(const uint32_t* __restrict__ wp, const half_t* __restrict__ sp,
+                                    const half_t* __restrict__ bp, const half_t* xrow, float16_t& acc,
+                                    unsigned long long* tr) {
+  uint4_t wreg[BURST_CA][BURST_SPW];
+  half4_t s4[BURST_CA], b4[BURST_CA];
+  constexpr int PRE = NCH < BURST_CA ? NCH : BURST_CA;
+  // scales and biases first, then the weights chunk by chunk: loads retire in issue order, and
+  // the first chunk must not wait behind the requests of the later ones
+#pragma unroll
+  for (int c = 0; c < PRE; ++c) {
+    s4[c] = *reinterpret_cast<const half4_t*>(sp + c * 8);
+    b4[c] = *reinterpret_cast<const half4_t*>(bp + c * 8);
+  }
+  __builtin_amdgcn_sched_barrier(0);
+#pragma unroll
+  for (int c = 0; c < PRE; ++c) {
+#pragma unroll
+    for (int e = 0; e < BURST_SPW; ++e) wreg[c][e] = *reinterpret_cast<const uint4_t*>(wp + (c * 8 + e) * 8);
+    __builtin_amdgcn_sched_barrier(0);
+  }
+  EAGLE_TR(tr, 1);
+  __syncthreads();                           // x chunk 0 is in LDS
+  EAGLE_TR(tr, 2);
+#pragma unroll
+  for (int c = 0; c < NCH; ++c) {
+    constexpr int XBUF = SLAB_XBUF;
+    const int slot = c % BURST_CA;
+    const half4_t sc4 = s4[slot], bi4 = b4[slot];
+    if (c + BURST_CA < NCH) {
+      s4[slot] = *reinterpret_cast<const half4_t*>(sp + (c + BURST_CA) * 8);
+      b4[slot] = *reinterpret_cast<const half4_t*>(bp + (c + BURST_CA) * 8);
+      __builtin_amdgcn_sched_barrier(0);
+    }
+#pragma unroll
+    for (int e = 0; e < BURST_SPW; ++e) {
+      const half_t sc = sc4[e], bi = bi4[e];
+      half8_t af[4];
+      if constexpr (SUBN) {
+        const half_t s20 = (half_t)((float)sc * 1048576.f);
+#pragma unroll
+        for (int j = 0; j < 4; ++j) af[j] = dequant_word_sub(wreg[slot][e][j], half2_t{s20, s20}, half2_t{bi, bi});
+      } else {
+        const half_t bc = (half_t)((float)bi + 8.f * (float)sc);
+#pragma unroll
+        for (int j = 0; j < 4; ++j) af[j] = dequant_word_centred(wreg[slot][e][j], half2_t{sc, sc}, half2_t{bc, bc});
+      }
+      if (c + BURST_CA < NCH)
+        wreg[slot][e] = *reinterpret_cast<const uint4_t*>(wp + ((c + BURST_CA) * 8 + e) * 8);
+#pragma unroll
+      for (int j = 0; j < 4; ++j) {
+        const half8_t bf = *reinterpret_cast<const half8_t*>(xrow + (c % BURST_XB) * XBUF + e * 64 + j * 8);
+        acc = __builtin_amdgcn_mfma_f32_32x32x16_f16(af[j], bf, acc, 0, 0, 0);
+      }
+      if (c + BURST_CA < NCH) __builtin_amdgcn_sched_barrier(0);   // keeps the reloads in step order
+    }
+    EAGLE_TR(tr, 3 + 2 * c);
+    __syncthreads();                         // every wave is done with chunk c; chunk c + 1 is in LDS
+    EAGLE_TR(tr, 4 + 2 * c);
+  }
+}
+
+template <int TILES, bool SWI, bool SUBN, int NCH, int NLAST>
+__global__ __launch_bounds__(64 * (2 * TILES + BURST_MOVERS)) void qmm_burst_w4g64_kernel(
+    const half_t* __restrict__ x, const uint32_t* __restrict__ w, const half_t* __restrict__ s,
+    const half_t* __restrict__ b, float* __restrict__ partial, int M, int N, int K, int spz,
+    const half_t* __restrict__ swi_bias, half_t* __restrict__ swi_out) {
+  extern __shared__ __attribute__((aligned(16))) half_t xlds[];   // three x chunks
+  constexpr int NSW = 2 * TILES;             // streaming waves
+  constexpr int NT = 64 * (NSW + BURST_MOVERS);
+  constexpr int XBUF = SLAB_XBUF;
+  const int tid = threadIdx.x;
+  const int wv = tid >> 6, lane = tid & 63;
+  const int ql = lane & 31, hb = lane >> 5;
+  const int z = blockIdx.y;
+  const int G = K >> 6, KW = K >> 3;
+  const int g0 = z * spz;
+  const int steps = G - g0 < spz ? G - g0 : spz;   // a multiple of eight
+  const int chunks = steps >> 3;                    // NCH, or NLAST for the last slab
+  const int t = wv % TILES, kp = wv / TILES;        // tile and half of the chunk of a streaming wave
+  float16_t acc;
+#pragma unroll
+  for (int i = 0; i < 16; ++i) acc[i] = 0.f;
+#ifdef EAGLE_TRACE
+  unsigned long long* tr = g_trace ? g_trace + ((size_t)(blockIdx.y * gridDim.x + blockIdx.x) * 16 + wv) * 24 : nullptr;
+#else
+  unsigned long long* tr = nullptr;
+#endif
+  EAGLE_TR(tr, 0);
+
+  if (wv >= NSW) {
+    // piece 256 i + mt of a chunk: row (256 i + mt) / 64, 16-byte column (256 i + mt) % 64.
+    // Two chunks are in flight in registers and up to three sit in LDS: chunk c + 2 is written
+    // during chunk c (into the buffer chunk c - 1 used) and was requested two chunks earlier.
+    const int mt = tid - 64 * NSW;
+    const int r0 = mt >> 6, c8 = mt & 63;
+    half8_t xr[2][8];
+    const half_t* xp[8];
+#pragma unroll
+    for (int i = 0; i < 8; ++i) {
+      const int row = 4 * i + r0;
+      xp[i] = x + (long)(row < M ? row : M - 1) * K + g0 * 64 + c8 * 8;
+    }
+    const int last = chunks - 1;
+    auto fetch = [&](int c, auto SET) {
+      constexpr int set = decltype(SET)::value;
+      const int cc = c < last ? c : last;
+#pragma unroll
+      for (int i = 0; i < 8; ++i) xr[set][i] = *reinterpret_cast<const half8_t*>(xp[i] + cc * 512);
+    };
+    auto stash = [&](int c, auto SET) {
+      constexpr int set = decltype(SET)::value;
+      const int buf = c % BURST_XB;
+#pragma unroll
+      for (int i = 0; i < 8; ++i)
+        *reinterpret_cast<half8_t*>(&xlds[buf * XBUF + (4 * i + r0) * SLAB_XR + c8 * 8]) = permute8(xr[set][i]);
+    };
+    fetch(0, StepIndex<0>{});
+    fetch(1, StepIndex<1>{});
+    stash(0, StepIndex<0>{});
+    fetch(2, StepIndex<0>{});
+    EAGLE_TR(tr, 1);
+    __syncthreads();
+    EAGLE_TR(tr, 2);
+    // during chunk c: chunk c + 1 goes into LDS (requested two chunks ago), chunk c + 3 is requested
+    for (int c = 0; c < chunks; c += 2) {
+      stash(c + 1, StepIndex<1>{});
+      EAGLE_TR(tr, 3 + 3 * c);
+      fetch(c + 3, StepIndex<1>{});
+      EAGLE_TR(tr, 4 + 3 * c);
+      __syncthreads();
+      EAGLE_TR(tr, 5 + 3 * c);
+      if (c + 1 < chunks) {
+        stash(c + 2, StepIndex<0>{});
+        EAGLE_TR(tr, 6 + 3 * c);
+        fetch(c + 4, StepIndex<0>{});
+        EAGLE_TR(tr, 7 + 3 * c);
+        __syncthreads();
+        EAGLE_TR(tr, 8 + 3 * c);
+      }
+    }
+  } else {
+    int nrow = blockIdx.x * (32 * TILES) + t * 32 + ql;
+    if (nrow > N - 1) nrow = N - 1;
+    const uint32_t* wp = w + (long)nrow * KW + (g0 + kp * BURST_SPW) * 8 + hb * 4;
+    const half_t* sp = s + (long)nrow * G + g0 + kp * BURST_SPW;
+    const half_t* bp = b + (long)nrow * G + g0 + kp * BURST_SPW;
+    const half_t* xrow = xlds + ql * SLAB_XR + hb * 32 + kp * BURST_SPW * 64;
+    if (NCH == NLAST || chunks == NCH) burst_stream<SUBN, NCH>(wp, sp, bp, xrow, acc, tr);
+    else burst_stream<SUBN, NLAST>(wp, sp, bp, xrow, acc, tr);
+  }
+
+  // the second wave of a tile hands its accumulators over (register i of lane l at [tile][i][l]),
+  // behind the output tile
+  constexpr int OUT_BYTES = SWI ? 32 * (16 * TILES + 8) * 2 : 32 * (32 * TILES + 4) * 4;
+  float* ex = reinterpret_cast<float*>(reinterpret_cast<char*>(xlds) + ((OUT_BYTES + 255) / 256) * 256) + t * (16 * 64) + lane;
+  if (wv < NSW && kp == 1) {
+#pragma unroll
+    for (int i = 0; i < 16; ++i) ex[i * 64] = acc[i];
+  }
+  __syncthreads();
+  const bool owner = wv < NSW && kp == 0;
+  if (owner) {
+#pragma unroll
+    for (int i = 0; i < 16; ++i) acc[i] += ex[i * 64];
+  }
+  if constexpr (SWI) {
+    constexpr int HS = 16 * TILES + 8;       // halves per row of the output tile in LDS
+    half_t* ht = xlds;
+    if (owner) {
+      const int ng = blockIdx.x * (32 * TILES) + t * 32;
+#pragma unroll
+      for (int i4 = 0; i4 < 2; ++i4) {
+        const int n = ng + 8 * i4 + 4 * hb;  // gate row; the up row is n + 16
+        half4_t o;
+#pragma unroll
+        for (int e = 0; e < 4; ++e) {
+          half_t g = (half_t)acc[4 * i4 + e], u = (half_t)acc[8 + 4 * i4 + e];
+          if (swi_bias && n + 16 + e < N) {
+            g = g + swi_bias[n + e];
+            u = u + swi_bias[n + 16 + e];
+          }
+          const float gf = (float)g;
+          const half_t a = (half_t)(gf / (1.0f + expf(-gf)));
+          o[e] = (half_t)((float)a * (float)u);
+        }
+        *reinterpret_cast<half4_t*>(&ht[ql * HS + t * 16 + 8 * i4 + 4 * hb]) = o;
+      }
+    }
+    __syncthreads();
+    const int NO = N >> 1;
+    constexpr int U = 2 * TILES;             // 16-byte pieces of a row of the tile
+    for (int idx = tid; idx < 32 * U; idx += NT) {
+      const int m = idx / U, c8 = (idx % U) * 8;
+      const int no = blockIdx.x * (16 * TILES) + c8;
+      if (m < M && no < NO)
+        *reinterpret_cast<half8_t*>(swi_out + (size_t)m * NO + no) = *reinterpret_cast<const half8_t*>(&ht[m * HS + c8]);
+    }
+  } else {
+    constexpr int OS = 32 * TILES + 4;       // floats per row of the tile in LDS
+    float* ot = reinterpret_cast<float*>(xlds);
+    if (owner) {
+#pragma unroll
+      for (int i4 = 0; i4 < 4; ++i4)
+        *reinterpret_cast<float4_t*>(&ot[ql * OS + t * 32 + 8 * i4 + 4 * hb]) =
+            float4_t{acc[4 * i4], acc[4 * i4 + 1], acc[4 * i4 + 2], acc[4 * i4 + 3]};
+    }
+    __syncthreads();
+    float* dst = partial + (size_t)z * SLAB_ROWS * N;
+    constexpr int U = 8 * TILES;             // 16-byte pieces of a row of the tile
+    for (int idx = tid; idx < 32 * U; idx += NT) {
+      const int m = idx / U, c4 = (idx % U) * 4;
+      const int n = blockIdx.x * (32 * TILES) + c4;
+      if (m < M && n < N)
+        *reinterpret_cast<float4_t*>(dst + (size_t)m * N + n) = *reinterpret_cast<const float4_t*>(&ot[m * OS + c4]);
+    }
+  }
+  EAGLE_TR(tr, 23);
+}
+
+template <int TILES, bool SWI, bool SUBN, int NCH, int NLAST>
+int launch_burst(const half_t* x, const uint32_t* w, const half_t* s, const half_t* b, float* partial, int M,
+                 int N, int K, int spz, int slabs, const half_t* bias, half_t* out, hipStream_t st) {
+  const size_t lds = BURST_XB * (size_t)SLAB_XBUF * sizeof(half_t);
+  static bool configured = false;
+  if (!configured) {
+    if (hipFuncSetAttribute(reinterpret_cast<const void*>(&qmm_burst_w4g64_kernel<TILES, SWI, SUBN, NCH, NLAST>),
+                            hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds) != hipSuccess)
+      return EAGLE_ERR_HIP;
+    configured = true;
+  }
+  const dim3 grid((N + 32 * TILES - 1) / (32 * TILES), slabs);
+  hipLaunchKernelGGL((qmm_burst_w4g64_kernel<TILES, SWI, SUBN, NCH, NLAST>), grid,
+                     dim3(64 * (2 * TILES + BURST_MOVERS)), lds, st, x, w, s, b, partial, M, N, K, spz, bias, out);
+  return eagle_launch_status();
+}
+
+// The tiled layout of a weight matrix (see TL above) from the row-major one: thread = one 16-byte
+// piece of the output.
+__global__ void tile_weights_kernel(const uint32_t* __restrict__ w, const half_t* __restrict__ s,
+                                    const half_t* __restrict__ b, uint32_t* __restrict__ wt,
+                                    half_t* __restrict__ sbt, int N, int K) {
+  const int G = K >> 6, KW = K >> 3;
+  const long nw = (long)(N >> 5) * G * 64;             // pieces of wt
+  const long nsb = (long)(N >> 5) * (G >> 3) * 64;     // pieces of sbt
+  const long idx = (long)blockIdx.x * blockDim.x + threadIdx.x;
+  if (idx < nw) {
+    const int lane = (int)(idx & 63);
+    const long ts = idx >> 6;
+    const int step = (int)(ts % G);
+    const long tile = ts / G;
+    const long row = tile * 32 + (lane & 31);
+    *reinterpret_cast<uint4_t*>(wt + idx * 4) =
+        *reinterpret_cast<const uint4_t*>(w + row * KW + step * 8 + (lane >> 5) * 4);
+  } else if (idx < nw + nsb) {
+    const long i = idx - nw;
+    const int lane = (int)(i & 63);
+    const long tc = i >> 6;
+    const int chunk = (int)(tc % (G >> 3));
+    const long tile = tc / (G >> 3);
+    const long row = tile * 32 + (lane & 31);
+    const half_t* src = (lane >> 5) ? b : s;
+    *reinterpret_cast<half8_t*>(sbt + i * 8) = *reinterpret_cast<const half8_t*>(src + row * G + chunk * 8);
+  }
+}
+
 // out[m][n] = fp16(sum over the slabs, in slab order) (+ bias): the plain reader of partial sums
 __global__ void slab_sum_kernel(const float* __restrict__ partial, int nslab, const half_t* __restrict__ bias,
                                 half_t* __restrict__ out, int M, int N) {
@@ -720,6 +1082,12 @@ __global__ void slab_sum_kernel(const float* __restrict__ partial, int nslab, co
 }
 
 }  // namespace
+
+#ifdef EAGLE_TRACE
+EAGLE_EXPORT int eagle_debug_trace(void* p) {
+  return (int)hipMemcpyToSymbol(HIP_SYMBOL(g_trace), &p, sizeof(p));
+}
+#endif
 
 EAGLE_EXPORT int eagle_qmm_slab_count(int K, int steps_per_slab) {
   if (K < 128 || (K % 128) != 0 || steps_per_slab < 8 || (steps_per_slab % 8) != 0 || steps_per_slab > 4096)
@@ -782,8 +1150,32 @@ EAGLE_EXPORT int eagle_qmm_slab_partial_w4g64(const void* x, const uint32_t* wq,
       return EAGLE_ERR_HIP;
     configured = true;
   }
-  const dim3 grid((N + 127) / 128, slabs);
   hipStream_t st = static_cast<hipStream_t>(stream);
+#ifdef EAGLE_BURST
+  if (mr == 1 && !ragged && N % 128 == 0) {
+    const int G = K / 64;
+    const int nch = steps_per_slab / 8, nlast = (G - (slabs - 1) * steps_per_slab) / 8;
+#ifdef EAGLE_SLAB_SUBN
+    constexpr bool subn = true;
+#else
+    constexpr bool subn = false;
+#endif
+#define EAGLE_BURST_CASE(A, B)                                                                              \
+  if (nch == A && nlast == B)                                                                               \
+    return launch_burst<4, false, subn, A, B>(static_cast<const half_t*>(x), wq,                             \
+                                              static_cast<const half_t*>(scales),                            \
+                                              static_cast<const half_t*>(biases), partial, M, N, K,          \
+                                              steps_per_slab, slabs, nullptr, nullptr, st);
+    EAGLE_BURST_CASE(5, 2)
+    EAGLE_BURST_CASE(4, 1)
+    EAGLE_BURST_CASE(4, 4)
+#ifdef EAGLE_BURST_ONE
+    EAGLE_BURST_CASE(1, 1)
+#endif
+#undef EAGLE_BURST_CASE
+  }
+#endif
+  const dim3 grid((N + 127) / 128, slabs);
 #define EAGLE_SLAB_LAUNCH(RAG, MRV)                                                                      \
   hipLaunchKernelGGL((qmm_slab_w4g64_kernel<RAG, MRV>), grid, dim3(256), lds, st,                        \
                      static_cast<const half_t*>(x), wq, static_cast<const half_t*>(scales),              \
@@ -812,6 +1204,9 @@ EAGLE_EXPORT int eagle_qmm_slab_swiglu_preferred(int M, int N, int K) {
   // the compute units and at most all of them.
   if (!eagle_qmm_slab_swiglu_supported(M, N, K)) return 0;
   if (M > SLAB_ROWS) return 1;
+#ifdef EAGLE_SWI_SLAB_ALWAYS
+  if (M >= 24) return 1;
+#endif
   const long blocks = (N + 127) / 128;
   return M >= 24 && blocks > NUM_CU / 2 && blocks <= NUM_CU && K >= 2048;
 }
@@ -831,6 +1226,23 @@ EAGLE_EXPORT int eagle_qmm_slab_swiglu_w4g64_f16(const void* x, const uint32_t* 
     return EAGLE_ERR_ALIGN;
   const int mr = M > SLAB_ROWS ? 2 : 1;
   const int steps = K / 64;                      // one slab over all of K
+#ifdef EAGLE_BURST
+  if (mr == 1 && !ragged && (steps == 56 || steps == 64)) {
+#ifdef EAGLE_SLAB_SUBN
+    constexpr bool subn = true;
+#else
+    constexpr bool subn = false;
+#endif
+    hipStream_t bst = static_cast<hipStream_t>(stream);
+    if (steps == 56)
+      return launch_burst<5, true, subn, 7, 7>(static_cast<const half_t*>(x), wq, static_cast<const half_t*>(scales),
+                                               static_cast<const half_t*>(biases), nullptr, M, N, K, steps, 1,
+                                               static_cast<const half_t*>(bias), static_cast<half_t*>(out), bst);
+    return launch_burst<4, true, subn, 8, 8>(static_cast<const half_t*>(x), wq, static_cast<const half_t*>(scales),
+                                             static_cast<const half_t*>(biases), nullptr, M, N, K, steps, 1,
+                                             static_cast<const half_t*>(bias), static_cast<half_t*>(out), bst);
+  }
+#endif
   // waves per workgroup: the fewest that give every compute unit at most one workgroup
   int nwv = 4;
   while (nwv < 8 && (N + 32 * nwv - 1) / (32 * nwv) > NUM_CU) nwv += (nwv == 6 ? 2 : 1);
@@ -895,6 +1307,119 @@ EAGLE_EXPORT int eagle_slab_sum_f16(const float* partial, int slabs, const void*
   hipLaunchKernelGGL(slab_sum_kernel, dim3((unsigned)((total + 255) / 256)), dim3(256), 0,
                      static_cast<hipStream_t>(stream), partial, slabs, static_cast<const half_t*>(bias),
                      static_cast<half_t*>(out), M, N);
+  return eagle_launch_status();
+}
+
+EAGLE_EXPORT int eagle_qmm_tiled_supported(int M, int N, int K) {
+  return M >= 1 && M <= SLAB_ROWS && N >= 32 && (N % 32) == 0 && K >= 512 && (K % 512) == 0 && K <= 65536;
+}
+
+EAGLE_EXPORT size_t eagle_qmm_tiled_sb_bytes(int N, int K) {
+  if (N < 32 || (N % 32) != 0 || K < 512 || (K % 512) != 0) return 0;
+  return (size_t)N * (K / 64) * 2 * sizeof(half_t);
+}
+
+EAGLE_EXPORT int eagle_qmm_tile_w4g64(const uint32_t* wq, const void* scales, const void* biases, uint32_t* wt,
+                                      void* sbt, int N, int K, int group_size, int bits, eagle_stream_t stream) {
+  if (!wq || !scales || !biases || !wt || !sbt) return EAGLE_ERR_NULL;
+  if (group_size != 64 || bits != 4) return EAGLE_ERR_UNSUPPORTED;
+  if (N < 32 || (N % 32) != 0 || K < 512 || (K % 512) != 0) return EAGLE_ERR_SHAPE;
+  if (!eagle_aligned16(wq) || !eagle_aligned16(scales) || !eagle_aligned16(biases) || !eagle_aligned16(wt) ||
+      !eagle_aligned16(sbt))
+    return EAGLE_ERR_ALIGN;
+  if (wt == wq || sbt == scales || sbt == biases) return EAGLE_ERR_SHAPE;    // not in place
+  const long G = K / 64;
+  const long total = (long)(N / 32) * G * 64 + (long)(N / 32) * (G / 8) * 64;
+  hipLaunchKernelGGL(tile_weights_kernel, dim3((unsigned)((total + 255) / 256)), dim3(256), 0,
+                     static_cast<hipStream_t>(stream), wq, static_cast<const half_t*>(scales),
+                     static_cast<const half_t*>(biases), wt, static_cast<half_t*>(sbt), N, K);
+  return eagle_launch_status();
+}
+
+EAGLE_EXPORT int eagle_qmm_slab_partial_tiled_w4g64(const void* x, const uint32_t* wt, const void* sbt,
+                                                    float* partial, size_t partial_bytes, int M, int N, int K,
+                                                    int steps_per_slab, int small_scales, eagle_stream_t stream) {
+  if (!x || !wt || !sbt || !partial) return EAGLE_ERR_NULL;
+  if (!eagle_qmm_tiled_supported(M, N, K)) return EAGLE_ERR_SHAPE;
+  const int slabs = eagle_qmm_slab_count(K, steps_per_slab);
+  if (slabs < 1 || slabs > 65535) return EAGLE_ERR_SHAPE;
+  if (!eagle_aligned16(x) || !eagle_aligned16(wt) || !eagle_aligned16(sbt) || !eagle_aligned16(partial))
+    return EAGLE_ERR_ALIGN;
+  if (partial_bytes < eagle_qmm_slab_partial_bytes_rows(M, N, K, steps_per_slab)) return EAGLE_ERR_WORKSPACE;
+  const int bufs = steps_per_slab > SLAB_RING ? 2 : 1;
+  const size_t lds = (size_t)bufs * SLAB_XBUF * sizeof(half_t);
+  static bool configured = false;
+  if (!configured) {
+    const int most = 2 * SLAB_XBUF * (int)sizeof(half_t);
+    if (hipFuncSetAttribute(reinterpret_cast<const void*>(&qmm_slab_w4g64_kernel<false, 1, false, 4, 1, true, false>),
+                            hipFuncAttributeMaxDynamicSharedMemorySize, most) != hipSuccess ||
+        hipFuncSetAttribute(reinterpret_cast<const void*>(&qmm_slab_w4g64_kernel<false, 1, false, 4, 1, true, true>),
+                            hipFuncAttributeMaxDynamicSharedMemorySize, most) != hipSuccess)
+      return EAGLE_ERR_HIP;
+    configured = true;
+  }
+  const dim3 grid((N + 127) / 128, slabs);
+  hipStream_t st = static_cast<hipStream_t>(stream);
+  const half_t* xh = static_cast<const half_t*>(x);
+  const half_t* sb = static_cast<const half_t*>(sbt);
+  if (small_scales)
+    hipLaunchKernelGGL((qmm_slab_w4g64_kernel<false, 1, false, 4, 1, true, true>), grid, dim3(256), lds, st, xh, wt,
+                       sb, (const half_t*)nullptr, partial, M, N, K, steps_per_slab, bufs);
+  else
+    hipLaunchKernelGGL((qmm_slab_w4g64_kernel<false, 1, false, 4, 1, true, false>), grid, dim3(256), lds, st, xh, wt,
+                       sb, (const half_t*)nullptr, partial, M, N, K, steps_per_slab, bufs);
+  return eagle_launch_status();
+}
+
+EAGLE_EXPORT int eagle_qmm_slab_swiglu_tiled_w4g64_f16(const void* x, const uint32_t* wt, const void* sbt,
+                                                       const void* bias, void* out, int M, int N, int K,
+                                                       int small_scales, eagle_stream_t stream) {
+  if (!x || !wt || !sbt || !out) return EAGLE_ERR_NULL;
+  if (!eagle_qmm_tiled_supported(M, N, K)) return EAGLE_ERR_SHAPE;
+  if (!eagle_aligned16(x) || !eagle_aligned16(wt) || !eagle_aligned16(sbt) || !eagle_aligned16(out) ||
+      (bias && (reinterpret_cast<uintptr_t>(bias) & 1u)))
+    return EAGLE_ERR_ALIGN;
+  const int steps = K / 64;                      // one slab over all of K
+  int nwv = 4;
+  while (nwv < 8 && (N + 32 * nwv - 1) / (32 * nwv) > NUM_CU) nwv += (nwv == 6 ? 2 : 1);
+  const int blocks = (N + 32 * nwv - 1) / (32 * nwv);
+  const int bufs = steps > SLAB_RING ? 2 : 1;
+  const size_t lds = (size_t)bufs * SLAB_XBUF * sizeof(half_t);
+  static bool configured = false;
+  if (!configured) {
+    const int most = 2 * SLAB_XBUF * (int)sizeof(half_t);
+    bool ok = true;
+#define EAGLE_TL_SWI_ATTR(NW)                                                                                    \
+  ok = ok &&                                                                                                     \
+       hipFuncSetAttribute(reinterpret_cast<const void*>(&qmm_slab_w4g64_kernel<false, 1, true, NW, 2, true, false>), \
+                           hipFuncAttributeMaxDynamicSharedMemorySize, most) == hipSuccess &&                    \
+       hipFuncSetAttribute(reinterpret_cast<const void*>(&qmm_slab_w4g64_kernel<false, 1, true, NW, 2, true, true>),  \
+                           hipFuncAttributeMaxDynamicSharedMemorySize, most) == hipSuccess
+    EAGLE_TL_SWI_ATTR(4);
+    EAGLE_TL_SWI_ATTR(5);
+    EAGLE_TL_SWI_ATTR(6);
+    EAGLE_TL_SWI_ATTR(8);
+#undef EAGLE_TL_SWI_ATTR
+    if (!ok) return EAGLE_ERR_HIP;
+    configured = true;
+  }
+  const dim3 grid(blocks, 1);
+  hipStream_t st = static_cast<hipStream_t>(stream);
+#define EAGLE_TL_SWI_LAUNCH(NW, SUB)                                                                     \
+  hipLaunchKernelGGL((qmm_slab_w4g64_kernel<false, 1, true, NW, 2, true, SUB>), grid, dim3(64 * NW), lds, st, \
+                     static_cast<const half_t*>(x), wt, static_cast<const half_t*>(sbt),                 \
+                     (const half_t*)nullptr, (float*)nullptr, M, N, K, steps, bufs,                      \
+                     static_cast<const half_t*>(bias), static_cast<half_t*>(out))
+#define EAGLE_TL_SWI_NW(NW)                                                                              \
+  if (small_scales) EAGLE_TL_SWI_LAUNCH(NW, true); else EAGLE_TL_SWI_LAUNCH(NW, false);
+  switch (nwv) {
+    case 4: EAGLE_TL_SWI_NW(4) break;
+    case 5: EAGLE_TL_SWI_NW(5) break;
+    case 6: EAGLE_TL_SWI_NW(6) break;
+    default: EAGLE_TL_SWI_NW(8) break;
+  }
+#undef EAGLE_TL_SWI_NW
+#undef EAGLE_TL_SWI_LAUNCH
   return eagle_launch_status();
 }
 

@@ -394,7 +394,35 @@ def fuse_projections(model, swiglu):
     return qkv_w, gu_w
 
 
-def slab_plan(model, T, forced=None, fused=True, rope_launch=True):
+def tiled_projections(model, qkv_w, gu_w, plan, swiglu):
+    """`ops.TiledWeights` copies of the projections a pass of up to 32 rows runs through the slab
+    kernels: q|k|v, o and down where `plan` sends them there, and the interleaved gate|up when
+    the SwiGLU form is on.  {"qkv": [...], "o": [...], "down": [...], "gu": [...]} with one entry
+    per layer (None where the shape is not taken); one set per model, shared by its pass objects."""
+    done = getattr(model, "_tiled_projections", None)
+    if done is None:
+        done = model._tiled_projections = {}
+    key = (bool(plan["qkv"]), bool(plan["o"]), bool(plan["down"]), bool(swiglu))
+    if key in done:
+        return done[key]
+
+    def tile(w, sc, bi):
+        n, k = w.shape[0], w.shape[1] * 8
+        return ops.tile_weights(w, sc, bi) if ops.tiled_supported(32, n, k) else None
+
+    out = {"qkv": [], "o": [], "down": [], "gu": []}
+    for i, layer in enumerate(model.model.layers):
+        at, mlp = layer.self_attn, layer.mlp
+        out["qkv"].append(tile(*qkv_w[i][:3]) if plan["qkv"] else None)
+        out["o"].append(tile(at.o_proj.weight, at.o_proj.scales, at.o_proj.biases) if plan["o"] else None)
+        out["down"].append(tile(mlp.down_proj.weight, mlp.down_proj.scales, mlp.down_proj.biases)
+                           if plan["down"] else None)
+        out["gu"].append(tile(*gu_w[i][:3]) if swiglu else None)
+    done[key] = out
+    return out
+
+
+def slab_plan(model, T, forced=None, fused=True):
     """K steps per slab for the q|k|v, o and down projections of a pass of T rows (0: streaming
     kernel): the library's choice per shape, or `forced` ({"qkv": s, "o": s, "down": s}).  The
     slab form leaves the product as partial sums for its consumer to add, so it needs the fused
@@ -409,8 +437,6 @@ def slab_plan(model, T, forced=None, fused=True, rope_launch=True):
     for name, (n, k) in shapes.items():
         s = ops.slab_steps(T, n, k) if forced is None else int(forced.get(name, 0))
         ok = fused and s > 0 and ops.slab_count(k, s) > 0
-        if name == "qkv":
-            ok = ok and rope_launch
         if name == "o":
             ok = ok and layer.self_attn.o_proj.bias is None
         if name == "down":
@@ -461,22 +487,13 @@ class TreeVerifier:
     Same kernels and operator order as Model.__call__ + the host functions above."""
 
     def __init__(self, model, cache, total_tokens=31, max_len=None, compact=True, fuse=True,
-                 swiglu=True, one_launch_attention=False, slab_plan=None, chain=None, resident_gate_up=None):
+                 swiglu=True, slab_plan=None, tiled=None):
         """slab_plan: {"qkv": s, "o": s, "down": s}, K steps per slab for the projections that go
         through the slab form of the matmul (their consumer adds the slabs), 0 for the
         streaming kernel; None: the library's choice for this shape.
-        chain: the residual add after the o projection, the norm and gate|up + SwiGLU of a layer as
-        ONE launch of a resident grid with a grid-wide barrier inside (`ops.norm_mlp_in`; needs the
-        o projection in the slab form).  Off unless asked for: measured inside the 7B step it takes
-        43.7 us against 5.3 + 30.6 us for the two launches it replaces (step 2.99 against 2.70 ms).
-        `chain_error()` reports a barrier that gave up.
-        resident_gate_up: gate|up + SwiGLU through the kernel that keeps x in registers and brings
-        the weights in by whole cache lines through LDS (`ops.quantized_matmul_resident`) instead of
-        the streaming kernel.  Off unless asked for; takes K a multiple of 512 up to 3584 and scales
-        below 0.2499 in magnitude.  Inside the 7B step it measured 1.4 us per layer faster when
-        built (2.661 against 2.699 ms per step, A/B on one box) and 0.6 us slower after the later
-        changes to the other kernels (2.632 against 2.616 ms); the measurement and profile records
-        of `bench.py` are those of the default form."""
+        tiled: the slab products (and gate|up + SwiGLU) read a copy of their weights in the tiled
+        layout (`ops.tile_weights`; doubles the memory of those matrices).  None: on for the fused
+        step of up to 32 tree tokens."""
         args = model.args
         self.model, self.cache, self.args = model, cache, args
         if total_tokens + 1 > TREE_SLOTS:
@@ -486,12 +503,10 @@ class TreeVerifier:
         self.T = T = total_tokens + 1
         # above 32 tree tokens: q|k|v, o and down in the slab form with 64-row partial tiles, the
         # other matmuls in two passes of the 32-row streaming kernel, two mask words per token and
-        # attention in pieces of 32 query rows (one launch pair); the resident and chained forms
-        # hold 32 rows and do not apply
+        # attention in pieces of 32 query rows (one launch pair)
         self.wide = T > MAXT
-        if self.wide and (not fuse or one_launch_attention or chain or resident_gate_up):
-            raise ValueError(f"a tree of more than {MAXT} tokens runs with the fused projections and "
-                             "none of the 32-row options")
+        if self.wide and not fuse:
+            raise ValueError(f"a tree of more than {MAXT} tokens runs with the fused projections only")
         dev = model.device
         self.dev = dev
         D, I = args.hidden_size, args.intermediate_size
@@ -502,24 +517,14 @@ class TreeVerifier:
         self.fuse = fuse
         # gate|up with the SwiGLU epilogue when the matmul covers the shape in one K slab
         self.swiglu = bool(fuse and swiglu and ops.swiglu_supported(T, I, D))
-        # rope and KV append inside the attention launch instead of a launch of their own (as
-        # fast inside a captured graph, one launch less per layer outside one)
-        self.one_launch_attention = bool(fuse and one_launch_attention)
         if fuse:
             self._fuse_projections()
         self.slab = self._slab_plan(slab_plan)
-        can_res = bool(self.swiglu and ops.resident_supported(T, 2 * I, D)
-                       and all(float(g[1].abs().max()) < ops.SMALL_SCALE_LIMIT for g in self.gu_w))
-        if resident_gate_up and not can_res:
-            raise ValueError("the resident form of gate|up does not take this model")
-        self.resident_gate_up = bool(resident_gate_up)
-        can_chain = bool(self.swiglu and self.slab["o"] and ops.norm_mlp_in_supported(T, D, I)
-                         and torch.cuda.get_device_properties(dev).multi_processor_count >= 256)
-        if chain and not can_chain:
-            raise ValueError("the chained launch does not take this model shape")
-        self.chain = bool(chain)
-        if self.chain:
-            self.chain_scratch, self.chain_err = ops.norm_mlp_in_scratch(dev)
+        if tiled and (self.wide or not fuse):
+            raise ValueError("the tiled weight layout serves the fused step of up to 32 tree tokens")
+        self.tiled = None
+        if (tiled or tiled is None) and fuse and not self.wide:
+            self.tiled = tiled_projections(model, self.qkv_w, self.gu_w, self.slab, self.swiglu)
         i32 = dict(dtype=torch.int32, device=dev)
         f16 = dict(dtype=torch.float16, device=dev)
         self.tokens = torch.zeros(T, **i32)
@@ -570,54 +575,46 @@ class TreeVerifier:
                    for rows in ((T,) if not self.wide else (MAXT, T - MAXT)))
         ops.workspace("qmm", need, dev)
         ops.workspace("attn", L.eagle_tree_attention_wide_workspace_bytes(T, H, hd, self.max_len), dev)
-        ops.workspace("attn_rope", L.eagle_tree_attention_rope_workspace_bytes(H, hd, self.max_len), dev)
         ops.workspace("argmax", L.eagle_argmax_workspace_bytes(T, args.vocab_size), dev)
 
     def _fuse_projections(self):
         self.qkv_w, self.gu_w = fuse_projections(self.model, self.swiglu)
 
     def _slab_plan(self, forced):
-        return slab_plan(self.model, self.T, forced, fused=self.fuse,
-                         rope_launch=not self.one_launch_attention)
+        return slab_plan(self.model, self.T, forced, fused=self.fuse)
 
     def qmm_launches(self):
-        """(weight, scales, biases, bias, x, out, form) of every quantised matmul of one step,
-        in order; `form` is True for the launches that go through `quantized_matmul_swiglu`,
+        """(weight, scales, biases, bias, x, out, form, tiled) of every quantised matmul of one
+        step, in order; `form` is True for the launches that go through `quantized_matmul_swiglu`,
         the K steps per slab for those that go through `quantized_matmul_slabs` (into
-        `self.partial`), False for `quantized_matmul`; "chain" entries are (gate|up tuple, norm
-        weight, slabs, None, partial, out, "chain") for `norm_mlp_in`."""
+        `self.partial`), False for `quantized_matmul`; `tiled` the `ops.TiledWeights` copy those
+        two forms read, or None."""
         m = self.model
         out = []
         for i, layer in enumerate(m.model.layers):
             at, mlp = layer.self_attn, layer.mlp
             if self.fuse:
-                out.append((*self.qkv_w[i], self.hn, self.qkv, self.slab["qkv"] or False))
+                out.append((*self.qkv_w[i], self.hn, self.qkv, self.slab["qkv"] or False, self._tiled("qkv", i)))
             else:
                 for lin, o in ((at.q_proj, self.q), (at.k_proj, self.k), (at.v_proj, self.v)):
-                    out.append((lin.weight, lin.scales, lin.biases, lin.bias, self.hn, o, False))
-            if self.chain:
-                # the o projection as slabs; gate|up + SwiGLU inside the chained launch that adds them
-                out.append((at.o_proj.weight, at.o_proj.scales, at.o_proj.biases, at.o_proj.bias,
-                            self.attn, self.o, self.slab["o"]))
-                out.append((self.gu_w[i], layer.post_attention_layernorm.weight,
-                            ops.slab_count(at.o_proj.weight.shape[1] * 8, self.slab["o"]), None, self.partial,
-                            self.act, "chain"))
-                out.append((mlp.down_proj.weight, mlp.down_proj.scales, mlp.down_proj.biases,
-                            mlp.down_proj.bias, self.act, self.down, self.slab["down"] or False))
-                continue
+                    out.append((lin.weight, lin.scales, lin.biases, lin.bias, self.hn, o, False, None))
             out.append((at.o_proj.weight, at.o_proj.scales, at.o_proj.biases, at.o_proj.bias,
-                        self.attn, self.o, self.slab["o"] or False))
+                        self.attn, self.o, self.slab["o"] or False, self._tiled("o", i)))
             if self.fuse:
                 out.append((*self.gu_w[i], self.hn, self.act if self.swiglu else self.gate_up,
-                            self.swiglu))
+                            self.swiglu, self._tiled("gu", i)))
             else:
                 for lin, o in ((mlp.gate_proj, self.gate), (mlp.up_proj, self.up)):
-                    out.append((lin.weight, lin.scales, lin.biases, lin.bias, self.hn, o, False))
+                    out.append((lin.weight, lin.scales, lin.biases, lin.bias, self.hn, o, False, None))
             out.append((mlp.down_proj.weight, mlp.down_proj.scales, mlp.down_proj.biases,
-                        mlp.down_proj.bias, self.act, self.down, self.slab["down"] or False))
+                        mlp.down_proj.bias, self.act, self.down, self.slab["down"] or False,
+                        self._tiled("down", i)))
         head = m.model.embed_tokens if self.args.tie_word_embeddings else m.lm_head
-        out.append((head.weight, head.scales, head.biases, None, self.hn, self.logits, False))
+        out.append((head.weight, head.scales, head.biases, None, self.hn, self.logits, False, None))
         return out
+
+    def _tiled(self, name, i):
+        return self.tiled[name][i] if self.tiled else None
 
     def set_tree(self, tokens, tree_position_ids, mask_index, mask_bits):
         self.tokens.copy_(tokens.reshape(-1))
@@ -651,15 +648,9 @@ class TreeVerifier:
             ops.tree_attention(self.q_rot, c.keys[0], c.values[0], self.mask_bits, self.len_dev, at.scale,
                                max_len=self.max_len, out=self.attn)
 
-        def attend_with_rope(at, c, q_lin, k_lin, v_lin):
-            ops.tree_attention_rope(q_lin, k_lin, v_lin, self.rope_cs, c.keys[0], c.values[0], self.mask_bits,
-                                    self.len_dev, at.scale, H, G, hd, row_stride=(H + 2 * G) * hd,
-                                    max_len=self.max_len, out=self.attn)
-
         for i, layer in enumerate(layers):
             if self.fuse:
-                emit_layer(self, i, self.len_dev, attend, positions=self.positions,
-                           attend_with_rope=attend_with_rope if self.one_launch_attention else None)
+                emit_layer(self, i, self.len_dev, attend, positions=self.positions)
             else:
                 self._layer_one_launch_per_projection(i, layer)
             if tap is not None:
@@ -735,17 +726,6 @@ class TreeVerifier:
             self.graph.replay()
         else:
             self.forward()
-
-    def chain_error(self):
-        """True if a grid barrier of the chained launch gave up since the last call (one
-        device-to-host copy); the scratch is zeroed again so that later steps can run."""
-        if not self.chain:
-            return False
-        bad = bool(self.chain_err.item())
-        if bad:
-            self.chain_scratch.zero_()
-            self.chain_err.zero_()
-        return bad
 
     def sync_host_offsets(self):
         """Bring the host-side cache offsets in line with the device length (one D2H copy)."""

@@ -152,12 +152,15 @@ def slab_rows(M):
     return 64 if M > 32 else 32
 
 
-def quantized_matmul_slabs(x, w_q, scales, biases, steps_per_slab, partial=None):
+def quantized_matmul_slabs(x, w_q, scales, biases, steps_per_slab, partial=None, tiled=None):
     """The product for 1..64 rows as fp32 partial sums of K slabs, [slabs, R, N] with R = 32 up
     to 32 rows and 64 above (`slab_rows`): the result is fp16(partial.sum(0)) (+ bias), formed by
-    `slab_sum`, `rms_norm_slabs` or `rope_kv_append_slabs`.  K % 128 == 0."""
+    `slab_sum`, `rms_norm_slabs` or `rope_kv_append_slabs`.  K % 128 == 0.
+    tiled: the same matrix as `TiledWeights`; up to 32 rows then read that copy."""
     _need_cuda(x, w_q, scales, biases)
     x = _f16(x, "x")
+    if tiled is not None and x.numel() // x.shape[-1] <= 32:
+        return _matmul_slabs_tiled(x, tiled, steps_per_slab, partial)
     w_q = as_packed_u32(w_q)
     scales, biases = _f16(scales, "scales"), _f16(biases, "biases")
     *lead, K = x.shape
@@ -178,6 +181,26 @@ def quantized_matmul_slabs(x, w_q, scales, biases, steps_per_slab, partial=None)
                                                  _ptr(partial), partial.numel() * 4, M, N, K, 64, 4,
                                                  int(steps_per_slab), _stream())
     _lib.check(rc, "quantized_matmul_slabs")
+    return partial
+
+
+def _matmul_slabs_tiled(x, tiled, steps_per_slab, partial):
+    *lead, K = x.shape
+    M = reduce(lambda a, b: a * b, lead, 1)
+    N = tiled.N
+    if K != tiled.K:
+        raise ValueError(f"shape mismatch: x {tuple(x.shape)}, tiled weights [{N}, {tiled.K}]")
+    slabs = slab_count(K, steps_per_slab)
+    if slabs < 1:
+        raise ValueError(f"the slab form does not take K = {K} with {steps_per_slab} steps per slab")
+    if partial is None:
+        partial = torch.empty((slabs, 32, N), dtype=torch.float32, device=x.device)
+    elif partial.dtype != torch.float32 or partial.numel() < slabs * 32 * N or not partial.is_contiguous():
+        raise ValueError("partial must be a contiguous fp32 buffer of at least slabs * 32 * N elements")
+    rc = _lib.lib().eagle_qmm_slab_partial_tiled_w4g64(_ptr(x), _ptr(tiled.wt), _ptr(tiled.sbt), _ptr(partial),
+                                                       partial.numel() * 4, M, N, K, int(steps_per_slab),
+                                                       int(tiled.small), _stream())
+    _lib.check(rc, "quantized_matmul_slabs (tiled)")
     return partial
 
 
@@ -241,14 +264,33 @@ def quantized_matmul_swiglu_slab(x, w_q, scales, biases, bias=None, out=None):
     return out
 
 
-def quantized_matmul_swiglu(x, w_q, scales, biases, bias=None, out=None, gemm=None):
+def quantized_matmul_swiglu(x, w_q, scales, biases, bias=None, out=None, gemm=None, tiled=None):
     """silu(x @ Wg.T) * (x @ Wu.T) (mlx_llama.py:214-215) in one launch: w_q / scales / biases
-    / bias hold the gate and up projections interleaved by `interleave_gate_up`.  The result
-    equals `silu_mul(quantized_matmul(x, gate...), quantized_matmul(x, up...))` bit for bit.
-    33..64 rows run on the slab kernel with 64-row tiles (`quantized_matmul_swiglu_slab`), more rows
-    as the tiled GEMM form with the same epilogue (`gemm=True`: that form whatever the row count)."""
+    / bias hold the gate and up projections interleaved by `interleave_gate_up`.  With more than
+    one row on the streaming kernel the result equals `silu_mul(quantized_matmul(x, gate...),
+    quantized_matmul(x, up...))` bit for bit; the other forms agree with it to the tolerance of
+    the product.  33..64 rows run on the slab kernel with 64-row tiles
+    (`quantized_matmul_swiglu_slab`), more rows as the tiled GEMM form with the same epilogue
+    (`gemm=True`: that form whatever the row count).
+    tiled: the interleaved matrix as `TiledWeights`; up to 32 rows then run the slab kernel on
+    that copy."""
     _need_cuda(x, w_q, scales, biases, bias)
     x = _f16(x, "x")
+    if tiled is not None and not gemm and x.numel() // x.shape[-1] <= 32:
+        *lead, K = x.shape
+        M = reduce(lambda a, b: a * b, lead, 1)
+        if K != tiled.K:
+            raise ValueError(f"shape mismatch: x {tuple(x.shape)}, tiled weights [{tiled.N}, {tiled.K}]")
+        if bias is not None:
+            bias = _f16(bias, "bias")
+            if tuple(bias.shape) != (tiled.N,):
+                raise ValueError("bias must have shape [N]")
+        if out is None:
+            out = torch.empty((*lead, tiled.N // 2), dtype=torch.float16, device=x.device)
+        rc = _lib.lib().eagle_qmm_slab_swiglu_tiled_w4g64_f16(_ptr(x), _ptr(tiled.wt), _ptr(tiled.sbt), _ptr(bias),
+                                                              _ptr(out), M, tiled.N, K, int(tiled.small), _stream())
+        _lib.check(rc, "quantized_matmul_swiglu (tiled)")
+        return out
     w_q = as_packed_u32(w_q)
     scales, biases = _f16(scales, "scales"), _f16(biases, "biases")
     *lead, K = x.shape
@@ -291,39 +333,45 @@ def quantized_matmul_swiglu(x, w_q, scales, biases, bias=None, out=None, gemm=No
     return out
 
 
-CHAIN_SPIN_TICKS = 5_000_000     # 50 ms at 100 MHz: the bounded wait of the in-kernel grid barrier
+# |scale| below this: the kernels may expand nibbles through fp16 subnormals (scale * 2^20 is a
+# finite fp16), three vector instructions fewer per packed word
+TILED_SMALL_SCALE = 0.0624
 
 
-def norm_mlp_in_supported(M, D, I):
-    return bool(_lib.lib().eagle_norm_mlp_in_supported(M, D, I))
+class TiledWeights:
+    """A 4-bit group-64 weight matrix [N, K] in the layout the 32-row slab kernels stream
+    fastest (`tile_weights`): `wt` [N/32, K/64, 64, 4] int32, one contiguous 1 KB block per
+    32-row tile and quantisation group in the order the lanes of a wave hold it, and `sbt`
+    [N/32, K/512, 64, 8] fp16 with the scales of a tile's rows for eight groups in lanes 0..31
+    and the biases in lanes 32..63.  `small` says that every |scale| is below TILED_SMALL_SCALE."""
+
+    def __init__(self, wt, sbt, N, K, small):
+        self.wt, self.sbt, self.N, self.K, self.small = wt, sbt, int(N), int(K), bool(small)
 
 
-def norm_mlp_in_scratch(device):
-    """Zeroed scratch (sums of squares + barrier counters) and error word for `norm_mlp_in`;
-    one pair per pass object, kept for its lifetime."""
-    n = _lib.lib().eagle_norm_mlp_in_scratch_bytes()
-    return (torch.zeros(n, dtype=torch.uint8, device=device), torch.zeros(1, dtype=torch.int32, device=device))
+def tiled_supported(M, N, K):
+    """True when the tiled forms (`quantized_matmul_slabs` / `quantized_matmul_swiglu` with
+    `tiled=`) take this product: up to 32 rows, N a multiple of 32, K a multiple of 512."""
+    return bool(_lib.lib().eagle_qmm_tiled_supported(int(M), int(N), int(K)))
 
 
-def norm_mlp_in(partial, slabs, h, norm_weight, eps, gu_w, gu_scales, gu_biases, gu_bias, act, scratch, err,
-                spin_ticks=CHAIN_SPIN_TICKS):
-    """h += fp16(sum of the slabs); act = silu(g) * u with (g | u) = rms_norm(h) @ Wgu.T, in one
-    launch of a resident grid with a grid-wide barrier between the two parts
-    (mlx_llama.py:240-243, 214-215).  `partial` [slabs, 32, D] from `quantized_matmul_slabs`,
-    gate|up interleaved by `interleave_gate_up`.  `scratch`, `err` from `norm_mlp_in_scratch`;
-    err[0] != 0 afterwards means the barrier gave up."""
-    _need_cuda(partial, h, gu_w, act)
-    M, D = h.shape
-    I = act.shape[-1]
-    rc = _lib.lib().eagle_norm_mlp_in_f16(
-        _ptr(partial), int(slabs), _ptr(h), _ptr(norm_weight), float(eps), _ptr(as_packed_u32(gu_w)),
-        _ptr(gu_scales), _ptr(gu_biases), _ptr(gu_bias), _ptr(act), M, D, I, _ptr(scratch), scratch.numel(),
-        _ptr(err), int(spin_ticks), _stream())
-    _lib.check(rc, "norm_mlp_in")
-    return act
-
-
-SMALL_SCALE_LIMIT = 0.2499       # |scale| * 2^18 has to stay a finite fp16
+def tile_weights(w_q, scales, biases):
+    """Re-lay a weight matrix in the MLX layout (`w_q` [N, K/8] uint32, `scales`, `biases`
+    [N, K/64] fp16) out as `TiledWeights` (one device launch; the inputs are left as they are)."""
+    _need_cuda(w_q, scales, biases)
+    w_q = as_packed_u32(w_q)
+    scales, biases = _f16(scales, "scales"), _f16(biases, "biases")
+    N, K = w_q.shape[0], w_q.shape[1] * 8
+    L = _lib.lib()
+    nsb = L.eagle_qmm_tiled_sb_bytes(N, K)
+    if not nsb or tuple(scales.shape) != (N, K // 64) or tuple(biases.shape) != (N, K // 64):
+        raise ValueError(f"the tiled layout takes N % 32 == 0 and K % 512 == 0, got [{N}, {K}]")
+    wt = torch.empty((N // 32, K // 64, 64, 4), dtype=torch.int32, device=w_q.device)
+    sbt = torch.empty((N // 32, K // 512, 64, 8), dtype=torch.float16, device=w_q.device)
+    rc = L.eagle_qmm_tile_w4g64(_ptr(w_q), _ptr(scales), _ptr(biases), _ptr(wt), _ptr(sbt), N, K, 64, 4, _stream())
+    _lib.check(rc, "tile_weights")
+    small = bool(scales.abs().max().item() < TILED_SMALL_SCALE)
+    return TiledWeights(wt, sbt, N, K, small)
 
 
 def small_supported(T, N, K, norm=False, swiglu=False):
@@ -418,37 +466,6 @@ def quantized_matvec(x, w_q, scales, biases, bias=None, out=None):
     rc = _lib.lib().eagle_qmv_w4g64_f16(_ptr(x), _ptr(w_q), _ptr(scales), _ptr(biases), _ptr(bias),
                                         _ptr(out), N, K, 64, 4, _stream())
     _lib.check(rc, "quantized_matvec")
-    return out
-
-
-def resident_supported(M, N, K):
-    """True when `quantized_matmul_resident` takes this shape (K a multiple of 512, <= 3584)."""
-    return bool(_lib.lib().eagle_qmm_res_supported(M, N, K))
-
-
-def quantized_matmul_resident(x, w_q, scales, biases, bias=None, out=None, swiglu=False):
-    """The same product as `quantized_matmul` (or `quantized_matmul_swiglu` with swiglu=True)
-    through the kernel that keeps x in registers and splits K over the waves of one workgroup
-    per compute unit (mlx_model_fwd_bench.py:65-73; mlx_llama.py:214-215)."""
-    _need_cuda(x, w_q, scales, biases, bias)
-    x = _f16(x, "x")
-    w_q = as_packed_u32(w_q)
-    scales, biases = _f16(scales, "scales"), _f16(biases, "biases")
-    *lead, K = x.shape
-    M = reduce(lambda a, b: a * b, lead, 1)
-    N = w_q.shape[0]
-    if w_q.shape[1] * 8 != K or tuple(scales.shape) != (N, K // 64) or tuple(biases.shape) != (N, K // 64):
-        raise ValueError(f"shape mismatch: x {tuple(x.shape)}, w {tuple(w_q.shape)}, "
-                         f"scales {tuple(scales.shape)}, biases {tuple(biases.shape)}")
-    if bias is not None:
-        bias = _f16(bias, "bias")
-        if tuple(bias.shape) != (N,):
-            raise ValueError("bias must have shape [N]")
-    if out is None:
-        out = torch.empty((*lead, N // 2 if swiglu else N), dtype=torch.float16, device=x.device)
-    rc = _lib.lib().eagle_qmm_res_w4g64_f16(_ptr(x), _ptr(w_q), _ptr(scales), _ptr(biases), _ptr(bias),
-                                            _ptr(out), M, N, K, 64, 4, int(bool(swiglu)), _stream())
-    _lib.check(rc, "quantized_matmul_resident")
     return out
 
 
@@ -568,7 +585,7 @@ def tree_attention(q, k_cache, v_cache, tree_mask_bits, cache_len_dev, scale, ma
 
 def rope_table(positions, inv_freqs, scaling_factor=1.0, out=None):
     """fp32 [T, hd/2, 2] table of (cos, sin)(positions[t] * scaling_factor * inv_freqs[i]) for
-    `tree_attention_rope`; the angles are those of `arrayed_rope`."""
+    the rope launches; the angles are those of `arrayed_rope`."""
     _need_cuda(positions, inv_freqs)
     T, half = positions.numel(), inv_freqs.numel()
     if out is None:
@@ -576,33 +593,6 @@ def rope_table(positions, inv_freqs, scaling_factor=1.0, out=None):
     rc = _lib.lib().eagle_rope_table_f32(_ptr(positions), _ptr(inv_freqs), float(scaling_factor),
                                          T, half, _ptr(out), _stream())
     _lib.check(rc, "rope_table")
-    return out
-
-
-def tree_attention_rope(q_lin, k_lin, v_lin, rope_cs, k_cache, v_cache, tree_mask_bits,
-                        cache_len_dev, scale, H, G, hd, row_stride=0, max_len=None, out=None):
-    """`rope_kv_append` + `tree_attention` without the rope launch: q_lin [T,H*hd], k_lin / v_lin [T,G*hd]
-    (row_stride > 0: column blocks of one [T,row_stride] matrix), rope_cs from `rope_table`.
-    Appends the rotated keys and the values to cache rows P..P+T-1 and returns [T, H*hd]."""
-    _need_cuda(q_lin, k_lin, v_lin, rope_cs, k_cache, v_cache, tree_mask_bits, cache_len_dev)
-    T = q_lin.shape[0]
-    cap = k_cache.shape[1]
-    if row_stride == 0:
-        if H != G:
-            raise ValueError("separate q and k/v matrices of different widths need row_stride")
-        row_stride = H * hd
-    if max_len is None:
-        max_len = cap
-    if out is None:
-        out = torch.empty((T, H * hd), dtype=torch.float16, device=q_lin.device)
-    L = _lib.lib()
-    need = L.eagle_tree_attention_rope_workspace_bytes(H, hd, max_len)
-    ws = workspace("attn_rope", need, q_lin.device)
-    rc = L.eagle_tree_attention_rope_f16(
-        _ptr(q_lin), _ptr(k_lin), _ptr(v_lin), int(row_stride), _ptr(rope_cs), _ptr(k_cache),
-        _ptr(v_cache), _ptr(tree_mask_bits), _ptr(cache_len_dev), _ptr(out), T, H, G, hd, cap,
-        max_len, float(scale), _ptr(ws), ws.numel(), _stream())
-    _lib.check(rc, "tree_attention_rope")
     return out
 
 

@@ -1,6 +1,6 @@
 """Parity at the sizes the benchmark configurations name, through the C ABI:
-the projection shapes of a Qwen2.5-7B-shaped model at M in {1, 8, 16, 24, 32} (streaming, slab and
-resident forms of the matmul), one decoder layer of that width over a 2048-token prefix, and the
+the projection shapes of a Qwen2.5-7B-shaped model at M in {1, 8, 16, 24, 32} (streaming and slab
+forms of the matmul), one decoder layer of that width over a 2048-token prefix, and the
 whole 28-layer verification step with the error followed through the layers for both forms of
 the matmul and both weight-rounding modes of the oracle."""
 import numpy as np
@@ -40,10 +40,6 @@ def test_cfg2_projection_shapes(dev, name, N, K):
             got = ops.slab_sum(part, ops.slab_count(K, s), M, N)
             torch.cuda.synchronize()
             assert rel_err(got.cpu().numpy(), want) <= TOL, f"slab form {name} M={M}"
-        if ops.resident_supported(M, N, K):
-            got = ops.quantized_matmul_resident(xd, d["weight"], d["scales"], d["biases"])
-            torch.cuda.synchronize()
-            assert rel_err(got.cpu().numpy(), want) <= TOL, f"resident form {name} M={M}"
 
 
 def setup_step(dev, args, layers, seed, P, T):

@@ -125,37 +125,6 @@ def test_fused_step_equals_module_path_and_oracle(dev, name):
 
 
 @pytest.mark.parametrize("name", list(CONFIGS))
-def test_one_launch_attention_step(dev, name):
-    """The step with rope + append inside the attention launch, and with a rope launch of its
-    own: logits within tolerance of each other and of the oracle; a captured graph replays to
-    the same bits."""
-    P, T = 200, 32
-    s = build(dev, name, P, T, seed=7)
-    base = run_verifier(s, dev, graph=False, one_launch_attention=False)
-    base.step()
-    s2 = build(dev, name, P, T, seed=7)
-    one = run_verifier(s2, dev, graph=False, one_launch_attention=True)
-    one.step()
-    torch.cuda.synchronize()
-    assert rel_err(one.logits.cpu().numpy(), base.logits.cpu().numpy()) <= TOL
-    want = model_oracle.verify_step(s["args"], s["weights"], s["inv"], s["sc"], s["tokens"], s["depth"],
-                                    s["parents"], s["anc"], s["ocache"], P)
-    assert rel_err(one.logits.cpu().numpy(), want["logits"]) <= TOL
-    s3 = build(dev, name, P, T, seed=7)
-    g = run_verifier(s3, dev, graph=True, one_launch_attention=True)
-    for rep in range(3):
-        s3["cache"][0].offset = P
-        s3["cache"][0].sync_len()
-        torch.cuda.synchronize()
-        g.step()
-        torch.cuda.synchronize()
-        assert torch.equal(g.logits, one.logits), f"replay {rep}"
-        assert torch.equal(g.result, one.result), f"replay {rep}"
-    for c, c2 in zip(s2["cache"], s3["cache"]):
-        assert torch.equal(c.keys, c2.keys) and torch.equal(c.values, c2.values)
-
-
-@pytest.mark.parametrize("name", list(CONFIGS))
 def test_graph_replays_match_eager(dev, name):
     """Replay the captured step several times with eager work and synchronisation in
     between; every replay must reproduce the eager result."""

@@ -155,96 +155,6 @@ def test_sdpa_signature(dev):
     assert rel_err(got[0].cpu().numpy(), want) <= TOL
 
 
-@pytest.mark.parametrize("H,G,hd,P,T", [(28, 4, 128, 1024, 32), (28, 4, 128, 2048, 32), (28, 4, 128, 2050, 32),
-                                        (14, 2, 64, 515, 32), (32, 8, 128, 100, 8), (4, 2, 64, 0, 16),
-                                        (8, 8, 128, 31, 24), (4, 4, 64, 7, 1)])
-def test_tree_attention_rope_one_launch(dev, H, G, hd, P, T):
-    """rope(q, k) + cache append inside the attention launch: against the oracle's
-    rope -> append -> attention, and against the device path with a separate rope launch."""
-    print(f"attn+rope H={H} G={G} hd={hd} P={P} T={T}", flush=True)
-    rng = np.random.default_rng(H + P + T + 1)
-    cap = P + T + 13
-    _, k, v, depth, anc = make_attention_case(rng, H, G, hd, P, T, cap)
-    k[:, P:] = np.nan                                   # rows the launch must write or never read
-    v[:, P:] = np.nan
-    W = (H + 2 * G) * hd
-    qkv = synth.make_x(rng, T, W)
-    pos = (P + depth).astype(np.int32)
-    inv = ops.default_inv_freqs(hd, 1000000.0, device=None).numpy()
-    sc = 1.0
-    # oracle: rotate, append, attend
-    ql = qkv[:, :H * hd].reshape(T, H, hd).transpose(1, 0, 2)[None]
-    kl = qkv[:, H * hd:(H + G) * hd].reshape(T, G, hd).transpose(1, 0, 2)[None]
-    vl = qkv[:, (H + G) * hd:].reshape(T, G, hd).transpose(1, 0, 2)
-    q_rot = oracle.rope_arrayed(ql, pos[None], inv, sc)[0]
-    k_rot = oracle.rope_arrayed(kl, pos[None], inv, sc)[0]
-    k_ref, v_ref = k.copy(), v.copy()
-    k_ref[:, P:P + T] = k_rot
-    v_ref[:, P:P + T] = vl
-    mask = np.concatenate([np.zeros((T, P), np.float16), tree_oracle.additive_mask(anc)], axis=1)
-    scale = hd ** -0.5
-    want = oracle.tree_attention(q_rot, k_ref, v_ref, mask, scale, S=P + T)
-    want_t = np.ascontiguousarray(want.transpose(1, 0, 2)).reshape(T, H * hd)
-
-    bits = to_dev(tree_oracle.mask_bits(anc).view(np.int32), dev)
-    len_dev = torch.tensor([P], dtype=torch.int32, device=dev)
-    qkv_d, pos_d, inv_d = to_dev(qkv, dev), to_dev(pos, dev), to_dev(inv, dev)
-    cs = ops.rope_table(pos_d, inv_d, sc)
-    for max_len in (P + T, cap):
-        kd, vd = to_dev(k, dev), to_dev(v, dev)
-        got = ops.tree_attention_rope(qkv_d, qkv_d[:, H * hd:], qkv_d[:, (H + G) * hd:], cs, kd, vd, bits,
-                                      len_dev, scale, H, G, hd, row_stride=W, max_len=max_len)
-        torch.cuda.synchronize()
-        got = got.cpu().numpy()
-        assert np.isfinite(got.astype(np.float32)).all()
-        assert rel_err(got, want_t) <= TOL
-        kg, vg = kd.cpu().numpy(), vd.cpu().numpy()
-        assert np.array_equal(vg[:, P:P + T], vl), "appended values are copies"
-        assert rel_err(kg[:, P:P + T], k_rot) <= TOL
-        assert np.isnan(kg[:, P + T:].astype(np.float32)).all(), "rows past P+T untouched"
-        assert np.array_equal(kg[:, :P], k[:, :P]) and np.array_equal(vg[:, :P], v[:, :P])
-    # the two-launch path appends the same rows and agrees on the output
-    kd2, vd2 = to_dev(k, dev), to_dev(v, dev)
-    q_out = torch.empty((H, T, hd), dtype=torch.float16, device=dev)
-    ops.rope_kv_append(qkv_d, qkv_d[:, H * hd:], qkv_d[:, (H + G) * hd:], pos_d, inv_d, sc, q_out, kd2, vd2,
-                       len_dev, H, G, hd, row_stride=W)
-    two = ops.tree_attention(q_out, kd2, vd2, bits, len_dev, scale, max_len=cap)
-    torch.cuda.synchronize()
-    assert torch.equal(vd2[:, P:P + T], vd[:, P:P + T])
-    assert rel_err(kd[:, P:P + T].cpu().numpy(), kd2[:, P:P + T].cpu().numpy()) <= 1e-3
-    assert rel_err(got, two.cpu().numpy()) <= TOL
-
-
-def test_tree_attention_rope_repeated_calls_share_workspace(dev):
-    """Calls with different lengths share one workspace."""
-    rng = np.random.default_rng(5)
-    H, G, hd, T = 8, 2, 64, 32
-    cap = 700
-    W = (H + 2 * G) * hd
-    inv = ops.default_inv_freqs(hd, 10000.0, device=None).numpy()
-    for P in (600, 40, 333):
-        _, k, v, depth, anc = make_attention_case(rng, H, G, hd, P, T, cap)
-        qkv = synth.make_x(rng, T, W)
-        pos = (P + depth).astype(np.int32)
-        ql = qkv[:, :H * hd].reshape(T, H, hd).transpose(1, 0, 2)[None]
-        kl = qkv[:, H * hd:(H + G) * hd].reshape(T, G, hd).transpose(1, 0, 2)[None]
-        vl = qkv[:, (H + G) * hd:].reshape(T, G, hd).transpose(1, 0, 2)
-        k[:, P:P + T] = oracle.rope_arrayed(kl, pos[None], inv, 1.0)[0]
-        v[:, P:P + T] = vl
-        mask = np.concatenate([np.zeros((T, P), np.float16), tree_oracle.additive_mask(anc)], axis=1)
-        want = oracle.tree_attention(oracle.rope_arrayed(ql, pos[None], inv, 1.0)[0], k, v, mask, hd ** -0.5,
-                                     S=P + T)
-        want_t = np.ascontiguousarray(want.transpose(1, 0, 2)).reshape(T, H * hd)
-        qkv_d = to_dev(qkv, dev)
-        cs = ops.rope_table(to_dev(pos, dev), to_dev(inv, dev), 1.0)
-        got = ops.tree_attention_rope(qkv_d, qkv_d[:, H * hd:], qkv_d[:, (H + G) * hd:], cs, to_dev(k, dev),
-                                      to_dev(v, dev), to_dev(tree_oracle.mask_bits(anc).view(np.int32), dev),
-                                      torch.tensor([P], dtype=torch.int32, device=dev), hd ** -0.5, H, G, hd,
-                                      row_stride=W, max_len=cap)
-        torch.cuda.synchronize()
-        assert rel_err(got.cpu().numpy(), want_t) <= TOL
-
-
 @pytest.mark.parametrize("H,G,hd,T", [(28, 4, 128, 32), (14, 2, 64, 17), (4, 4, 64, 1)])
 def test_rope_kv_append_from_table(dev, H, G, hd, T):
     """Angles from the per-step cos/sin table instead of sincos in the launch: the values are
