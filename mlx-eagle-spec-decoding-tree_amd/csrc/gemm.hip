@@ -805,24 +805,22 @@ constexpr int BURST_XB = 3;                  // x chunks in LDS
 constexpr int BURST_SPW = 4;                 // steps of a chunk per streaming wave
 
 template <bool SUBN, int NCH>
-__device__ inline void burst_stream(const uint32_t* __restrict__ wp, const half_t* __restrict__ sp,
-                                    const half_t* __restrict__ bp, const half_t* xrow, float16_t& acc,
-                                    unsigned long long* tr) {
+__device__ inline void burst_stream(const uint32_t* __restrict__ wp, const half_t* __restrict__ sp, int kp, int hb,
+                                    const half_t* xrow, float16_t& acc, unsigned long long* tr) {
+  // wp: the wave's first block of the tiled weights (+ lane), 256 words per step; sp: the
+  // tile's first block of scales | biases (+ lane), 512 halves per chunk
   uint4_t wreg[BURST_CA][BURST_SPW];
-  half4_t s4[BURST_CA], b4[BURST_CA];
+  half8_t sb[BURST_CA];
   constexpr int PRE = NCH < BURST_CA ? NCH : BURST_CA;
   // scales and biases first, then the weights chunk by chunk: loads retire in issue order, and
   // the first chunk must not wait behind the requests of the later ones
 #pragma unroll
-  for (int c = 0; c < PRE; ++c) {
-    s4[c] = *reinterpret_cast<const half4_t*>(sp + c * 8);
-    b4[c] = *reinterpret_cast<const half4_t*>(bp + c * 8);
-  }
+  for (int c = 0; c < PRE; ++c) sb[c] = *reinterpret_cast<const half8_t*>(sp + c * 512);
   __builtin_amdgcn_sched_barrier(0);
 #pragma unroll
   for (int c = 0; c < PRE; ++c) {
 #pragma unroll
-    for (int e = 0; e < BURST_SPW; ++e) wreg[c][e] = *reinterpret_cast<const uint4_t*>(wp + (c * 8 + e) * 8);
+    for (int e = 0; e < BURST_SPW; ++e) wreg[c][e] = *reinterpret_cast<const uint4_t*>(wp + (c * 8 + e) * 256);
     __builtin_amdgcn_sched_barrier(0);
   }
   EAGLE_TR(tr, 1);
@@ -832,15 +830,24 @@ __device__ inline void burst_stream(const uint32_t* __restrict__ wp, const half_
   for (int c = 0; c < NCH; ++c) {
     constexpr int XBUF = SLAB_XBUF;
     const int slot = c % BURST_CA;
-    const half4_t sc4 = s4[slot], bi4 = b4[slot];
+    // this lane loaded eight scales (lanes 0..31) or biases (32..63); the wave's four steps are
+    // words 2 kp, 2 kp + 1; exchange the halves of the wave so that every lane has both
+    union { half8_t h; uint32_t u[4]; } own;
+    own.h = sb[slot];
+    const uint32_t m0 = kp ? own.u[2] : own.u[0], m1 = kp ? own.u[3] : own.u[1];
+    const uint32_t o0 = __shfl_xor(m0, 32, 64), o1 = __shfl_xor(m1, 32, 64);
+    union { uint32_t u[2]; half4_t h; } sc4, bi4;
+    sc4.u[0] = hb ? o0 : m0;
+    sc4.u[1] = hb ? o1 : m1;
+    bi4.u[0] = hb ? m0 : o0;
+    bi4.u[1] = hb ? m1 : o1;
     if (c + BURST_CA < NCH) {
-      s4[slot] = *reinterpret_cast<const half4_t*>(sp + (c + BURST_CA) * 8);
-      b4[slot] = *reinterpret_cast<const half4_t*>(bp + (c + BURST_CA) * 8);
+      sb[slot] = *reinterpret_cast<const half8_t*>(sp + (c + BURST_CA) * 512);
       __builtin_amdgcn_sched_barrier(0);
     }
 #pragma unroll
     for (int e = 0; e < BURST_SPW; ++e) {
-      const half_t sc = sc4[e], bi = bi4[e];
+      const half_t sc = sc4.h[e], bi = bi4.h[e];
       half8_t af[4];
       if constexpr (SUBN) {
         const half_t s20 = (half_t)((float)sc * 1048576.f);
@@ -852,7 +859,7 @@ __device__ inline void burst_stream(const uint32_t* __restrict__ wp, const half_
         for (int j = 0; j < 4; ++j) af[j] = dequant_word_centred(wreg[slot][e][j], half2_t{sc, sc}, half2_t{bc, bc});
       }
       if (c + BURST_CA < NCH)
-        wreg[slot][e] = *reinterpret_cast<const uint4_t*>(wp + ((c + BURST_CA) * 8 + e) * 8);
+        wreg[slot][e] = *reinterpret_cast<const uint4_t*>(wp + ((c + BURST_CA) * 8 + e) * 256);
 #pragma unroll
       for (int j = 0; j < 4; ++j) {
         const half8_t bf = *reinterpret_cast<const half8_t*>(xrow + (c % BURST_XB) * XBUF + e * 64 + j * 8);
@@ -879,7 +886,7 @@ __global__ __launch_bounds__(64 * (2 * TILES + BURST_MOVERS)) void qmm_burst_w4g
   const int wv = tid >> 6, lane = tid & 63;
   const int ql = lane & 31, hb = lane >> 5;
   const int z = blockIdx.y;
-  const int G = K >> 6, KW = K >> 3;
+  const int G = K >> 6;
   const int g0 = z * spz;
   const int steps = G - g0 < spz ? G - g0 : spz;   // a multiple of eight
   const int chunks = steps >> 3;                    // NCH, or NLAST for the last slab
@@ -946,14 +953,13 @@ __global__ __launch_bounds__(64 * (2 * TILES + BURST_MOVERS)) void qmm_burst_w4g
       }
     }
   } else {
-    int nrow = blockIdx.x * (32 * TILES) + t * 32 + ql;
-    if (nrow > N - 1) nrow = N - 1;
-    const uint32_t* wp = w + (long)nrow * KW + (g0 + kp * BURST_SPW) * 8 + hb * 4;
-    const half_t* sp = s + (long)nrow * G + g0 + kp * BURST_SPW;
-    const half_t* bp = b + (long)nrow * G + g0 + kp * BURST_SPW;
+    int tile = blockIdx.x * TILES + t;         // rows past N are never stored
+    if (tile > (N >> 5) - 1) tile = (N >> 5) - 1;
+    const uint32_t* wp = w + ((long)tile * G + g0 + kp * BURST_SPW) * 256 + lane * 4;
+    const half_t* sp = s + ((long)tile * (G >> 3) + (g0 >> 3)) * 512 + lane * 8;
     const half_t* xrow = xlds + ql * SLAB_XR + hb * 32 + kp * BURST_SPW * 64;
-    if (NCH == NLAST || chunks == NCH) burst_stream<SUBN, NCH>(wp, sp, bp, xrow, acc, tr);
-    else burst_stream<SUBN, NLAST>(wp, sp, bp, xrow, acc, tr);
+    if (NCH == NLAST || chunks == NCH) burst_stream<SUBN, NCH>(wp, sp, kp, hb, xrow, acc, tr);
+    else burst_stream<SUBN, NLAST>(wp, sp, kp, hb, xrow, acc, tr);
   }
 
   // the second wave of a tile hands its accumulators over (register i of lane l at [tile][i][l]),
@@ -1151,30 +1157,6 @@ EAGLE_EXPORT int eagle_qmm_slab_partial_w4g64(const void* x, const uint32_t* wq,
     configured = true;
   }
   hipStream_t st = static_cast<hipStream_t>(stream);
-#ifdef EAGLE_BURST
-  if (mr == 1 && !ragged && N % 128 == 0) {
-    const int G = K / 64;
-    const int nch = steps_per_slab / 8, nlast = (G - (slabs - 1) * steps_per_slab) / 8;
-#ifdef EAGLE_SLAB_SUBN
-    constexpr bool subn = true;
-#else
-    constexpr bool subn = false;
-#endif
-#define EAGLE_BURST_CASE(A, B)                                                                              \
-  if (nch == A && nlast == B)                                                                               \
-    return launch_burst<4, false, subn, A, B>(static_cast<const half_t*>(x), wq,                             \
-                                              static_cast<const half_t*>(scales),                            \
-                                              static_cast<const half_t*>(biases), partial, M, N, K,          \
-                                              steps_per_slab, slabs, nullptr, nullptr, st);
-    EAGLE_BURST_CASE(5, 2)
-    EAGLE_BURST_CASE(4, 1)
-    EAGLE_BURST_CASE(4, 4)
-#ifdef EAGLE_BURST_ONE
-    EAGLE_BURST_CASE(1, 1)
-#endif
-#undef EAGLE_BURST_CASE
-  }
-#endif
   const dim3 grid((N + 127) / 128, slabs);
 #define EAGLE_SLAB_LAUNCH(RAG, MRV)                                                                      \
   hipLaunchKernelGGL((qmm_slab_w4g64_kernel<RAG, MRV>), grid, dim3(256), lds, st,                        \
@@ -1204,9 +1186,6 @@ EAGLE_EXPORT int eagle_qmm_slab_swiglu_preferred(int M, int N, int K) {
   // the compute units and at most all of them.
   if (!eagle_qmm_slab_swiglu_supported(M, N, K)) return 0;
   if (M > SLAB_ROWS) return 1;
-#ifdef EAGLE_SWI_SLAB_ALWAYS
-  if (M >= 24) return 1;
-#endif
   const long blocks = (N + 127) / 128;
   return M >= 24 && blocks > NUM_CU / 2 && blocks <= NUM_CU && K >= 2048;
 }
@@ -1226,23 +1205,6 @@ EAGLE_EXPORT int eagle_qmm_slab_swiglu_w4g64_f16(const void* x, const uint32_t* 
     return EAGLE_ERR_ALIGN;
   const int mr = M > SLAB_ROWS ? 2 : 1;
   const int steps = K / 64;                      // one slab over all of K
-#ifdef EAGLE_BURST
-  if (mr == 1 && !ragged && (steps == 56 || steps == 64)) {
-#ifdef EAGLE_SLAB_SUBN
-    constexpr bool subn = true;
-#else
-    constexpr bool subn = false;
-#endif
-    hipStream_t bst = static_cast<hipStream_t>(stream);
-    if (steps == 56)
-      return launch_burst<5, true, subn, 7, 7>(static_cast<const half_t*>(x), wq, static_cast<const half_t*>(scales),
-                                               static_cast<const half_t*>(biases), nullptr, M, N, K, steps, 1,
-                                               static_cast<const half_t*>(bias), static_cast<half_t*>(out), bst);
-    return launch_burst<4, true, subn, 8, 8>(static_cast<const half_t*>(x), wq, static_cast<const half_t*>(scales),
-                                             static_cast<const half_t*>(biases), nullptr, M, N, K, steps, 1,
-                                             static_cast<const half_t*>(bias), static_cast<half_t*>(out), bst);
-  }
-#endif
   // waves per workgroup: the fewest that give every compute unit at most one workgroup
   int nwv = 4;
   while (nwv < 8 && (N + 32 * nwv - 1) / (32 * nwv) > NUM_CU) nwv += (nwv == 6 ? 2 : 1);
@@ -1380,6 +1342,19 @@ EAGLE_EXPORT int eagle_qmm_slab_swiglu_tiled_w4g64_f16(const void* x, const uint
       (bias && (reinterpret_cast<uintptr_t>(bias) & 1u)))
     return EAGLE_ERR_ALIGN;
   const int steps = K / 64;                      // one slab over all of K
+  // the two K sizes of the benchmark targets go to the kernel with two waves per weight tile
+  if (steps == 56 || steps == 64) {
+    hipStream_t bst = static_cast<hipStream_t>(stream);
+    const half_t* xh = static_cast<const half_t*>(x);
+    const half_t* sb = static_cast<const half_t*>(sbt);
+    const half_t* bh = static_cast<const half_t*>(bias);
+    half_t* oh = static_cast<half_t*>(out);
+    if (steps == 56)
+      return small_scales ? launch_burst<5, true, true, 7, 7>(xh, wt, sb, nullptr, nullptr, M, N, K, steps, 1, bh, oh, bst)
+                          : launch_burst<5, true, false, 7, 7>(xh, wt, sb, nullptr, nullptr, M, N, K, steps, 1, bh, oh, bst);
+    return small_scales ? launch_burst<4, true, true, 8, 8>(xh, wt, sb, nullptr, nullptr, M, N, K, steps, 1, bh, oh, bst)
+                        : launch_burst<4, true, false, 8, 8>(xh, wt, sb, nullptr, nullptr, M, N, K, steps, 1, bh, oh, bst);
+  }
   int nwv = 4;
   while (nwv < 8 && (N + 32 * nwv - 1) / (32 * nwv) > NUM_CU) nwv += (nwv == 6 ? 2 : 1);
   const int blocks = (N + 32 * nwv - 1) / (32 * nwv);

@@ -374,6 +374,9 @@ def tile_weights(w_q, scales, biases):
     return TiledWeights(wt, sbt, N, K, small)
 
 
+SMALL_SCALE_LIMIT = 0.2499       # |scale| * 2^18 has to stay a finite fp16 (the small-row kernels)
+
+
 def small_supported(T, N, K, norm=False, swiglu=False):
     """True when `quantized_matmul_small` takes this shape."""
     return bool(_lib.lib().eagle_qmm_small_supported(T, N, K, int(bool(norm)), int(bool(swiglu))))

@@ -121,8 +121,11 @@ def test_swiglu(dev, M, I, K, bias):
                                     out=out[:M], tiled=t)
         got = out.cpu().numpy()
         assert np.isnan(got[M].astype(np.float32)).all()
-        if not small:
+        if not small and K not in (3584, 4096):
+            # (those two K sizes run two waves per weight tile, which add their halves of K at the end)
             assert torch.equal(out[:M], plain)
+        else:
+            close_fp16(got[:M], plain.cpu().numpy(), "against the row-major form")
         g64, u64 = og.astype(np.float64), ou.astype(np.float64)
         rms_g, rms_u = np.sqrt(np.mean(g64 * g64)), np.sqrt(np.mean(u64 * u64))
         w64, got64 = want.astype(np.float64), got[:M].astype(np.float64)
