@@ -373,7 +373,9 @@ def main():
         print(f"[bench] CPU baseline: full steps on {cores} host threads ...", file=sys.stderr, flush=True)
         set_omp_threads(cores)
         cpu_step()                                      # warm-up: pages in the 4.3 GB of weights
-        want, cpu_ms = cpu_step()
+        cpu_runs = [cpu_step() for _ in range(3)]
+        want = cpu_runs[0][0]
+        cpu_ms = float(np.median([t for _, t in cpu_runs]))
         # one thread: a step of 1 layer and a step of 3 layers (+ embedding, head, acceptance);
         # the difference prices a layer, the full step is extrapolated from it
         print("[bench] CPU baseline: 1-layer and 3-layer steps on one host thread ...", file=sys.stderr, flush=True)
@@ -385,11 +387,12 @@ def main():
         cpu = {"value": round(cpu_ms, 1), "unit": "ms", "cores": cores, "cores_available": have,
                "cpu_model": cpu_model(), "kind": "port",
                "sample": "1 full step (28 layers + head, 32 nodes, 2048-token prefix), same weights and inputs, "
-                         "OpenMP C restatement, timed once after one warm-up step",
+                         "OpenMP C restatement, median of 3 timed steps after one warm-up step",
+               "runs_ms": [round(t, 1) for _, t in cpu_runs],
                "single_thread": {"value": round(single_est, 1), "unit": "ms", "cores": 1,
-                                 "sample": "extrapolated to 28 layers from a 1-layer step "
-                                           f"({t1:.0f} ms) and a 3-layer step ({t3:.0f} ms), both with embedding, "
-                                           "head and acceptance, one thread"}}
+                                 "measured": {"one_layer_step_ms": round(t1, 1), "three_layer_step_ms": round(t3, 1)},
+                                 "sample": "measured on one thread: a 1-layer step and a 3-layer step (both with "
+                                           "embedding, head and acceptance); `value` extrapolates them to 28 layers"}}
         wl = want["logits"].astype(np.float32)
         gl = gpu_logits.astype(np.float32)
         abs_err = float(np.abs(gl - wl).max())
@@ -452,6 +455,8 @@ def main():
         line["loop"] = {k: lp[k] for k in ("metric", "value", "unit", "steps", "ms_per_step", "tokens_per_step",
                                            "prefill_ms", "parity")}
         line["loop"]["workload"] = lp["config"]["workload"]
+        torch.cuda.empty_cache()
+        line["qmm_sweep"] = qmm_sweep(torch, ops, dev, with_cpu=not opt.no_cpu)
         extra.steps, extra.warmup = 10, 2
         gm = gemm_bench(extra)
         line["prompt_gemm"] = {"metric": gm["metric"], "value": gm["value"], "unit": gm["unit"],
@@ -623,9 +628,10 @@ def cpu_qmm_bench(opt):
 
 
 def small_m_bench(opt):
-    """M = 1 over the projection shapes of the Qwen2.5-7B-shaped model: eagle_qmv_w4g64_f16
-    (v_dot2_f32_f16 + DPP row sums) beside eagle_qmm_w4g64_f16 (16-row MFMA tiles, 15 rows idle),
-    each launch on its own copy of the weights (> 1 GB in rotation)."""
+    """M in {1, 2, 4, 8} over the projection shapes of the Qwen2.5-7B-shaped model:
+    eagle_qmv_rows_w4g64_f16 (v_dot2_f32_f16 + DPP row sums, the expanded nibbles shared by the rows)
+    beside eagle_qmm_w4g64_f16 (16-row MFMA tiles with the other rows idle), each launch on its own
+    copy of the weights (> 1 GB in rotation)."""
     import torch
     from mlx_eagle_spec_decoding_tree_amd import _lib, ops
 
@@ -641,33 +647,39 @@ def small_m_bench(opt):
         ws = [torch.randint(-2 ** 31, 2 ** 31 - 1, (N, K // 8), dtype=torch.int32, device=dev) for _ in range(ncopy)]
         ss = [(torch.rand(N, K // 64, device=dev) * 0.015 + 0.005).half() for _ in range(ncopy)]
         bs = [(-8 * s.float()).half() for s in ss]
-        x = torch.randn(1, K, device=dev).half()
-        o = torch.empty(1, N, device=dev, dtype=torch.float16)
-        wsp = ops.workspace("qmm", L.eagle_qmm_workspace_bytes(1, N, K), dev)
-        iters = 24
+        for M in (1, 2, 4, 8):
+            x = torch.randn(M, K, device=dev).half()
+            o = torch.empty(M, N, device=dev, dtype=torch.float16)
+            wsp = ops.workspace("qmm", L.eagle_qmm_workspace_bytes(M, N, K), dev)
+            iters = 24
 
-        def mfma():
-            for i in range(iters):
-                j = i % ncopy
-                _lib.check(L.eagle_qmm_w4g64_f16(x.data_ptr(), ws[j].data_ptr(), ss[j].data_ptr(), bs[j].data_ptr(),
-                                                 None, o.data_ptr(), 1, N, K, 64, 4, wsp.data_ptr(), wsp.numel(),
-                                                 st()), "qmm")
+            def mfma():
+                for i in range(iters):
+                    j = i % ncopy
+                    _lib.check(L.eagle_qmm_w4g64_f16(x.data_ptr(), ws[j].data_ptr(), ss[j].data_ptr(), bs[j].data_ptr(),
+                                                     None, o.data_ptr(), M, N, K, 64, 4, wsp.data_ptr(), wsp.numel(),
+                                                     st()), "qmm")
 
-        def valu():
-            for i in range(iters):
-                j = i % ncopy
-                _lib.check(L.eagle_qmv_w4g64_f16(x.data_ptr(), ws[j].data_ptr(), ss[j].data_ptr(), bs[j].data_ptr(),
-                                                 None, o.data_ptr(), N, K, 64, 4, st()), "qmv")
+            def valu():
+                for i in range(iters):
+                    j = i % ncopy
+                    _lib.check(L.eagle_qmv_rows_w4g64_f16(x.data_ptr(), ws[j].data_ptr(), ss[j].data_ptr(),
+                                                          bs[j].data_ptr(), None, o.data_ptr(), M, N, K, 64, 4, st()),
+                               "qmv")
 
-        t_m = float(np.median(graph_time_ms(torch, mfma, reps=7)[0])) * 1e3 / iters
-        t_v = float(np.median(graph_time_ms(torch, valu, reps=7)[0])) * 1e3 / iters
-        byts = qmm_bytes(1, N, K)
-        rows.append({"name": name, "N": N, "K": K, "mfma_us": round(t_m, 2), "valu_us": round(t_v, 2),
-                     "mfma_frac": round(byts / t_m / 1e3 / HBM_PEAK_GBS, 4),
-                     "valu_frac": round(byts / t_v / 1e3 / HBM_PEAK_GBS, 4),
-                     "dispatched_to": "valu" if ops.qmv_preferred(N, K) else "mfma"})
+            t_m = float(np.median(graph_time_ms(torch, mfma, reps=7)[0])) * 1e3 / iters
+            rec = {"name": name, "N": N, "K": K, "M": M, "mfma_us": round(t_m, 2)}
+            byts = qmm_bytes(M, N, K)
+            rec["mfma_frac"] = round(byts / t_m / 1e3 / HBM_PEAK_GBS, 4)
+            if L.eagle_qmv_rows_supported(M, N, K):
+                t_v = float(np.median(graph_time_ms(torch, valu, reps=7)[0])) * 1e3 / iters
+                rec["valu_us"] = round(t_v, 2)
+                rec["valu_frac"] = round(byts / t_v / 1e3 / HBM_PEAK_GBS, 4)
+            rec["dispatched_to"] = "valu" if ops.qmv_preferred(N, K, M) else "mfma"
+            rows.append(rec)
+            print(f"[small-m] {rec}", file=sys.stderr, flush=True)
         del ws, ss, bs
-    return {"metric": "one-row quantised product, us per launch (vector ALU beside matrix tiles)", "unit": "us",
+    return {"metric": "quantised product of 1..8 rows, us per launch (vector ALU beside matrix tiles)", "unit": "us",
             "dtype": "f16", "data": "synthetic", "rows": rows}
 
 
@@ -756,6 +768,80 @@ def loop_bench(opt):
                    "stream_equal": agree == len(emitted)},
     }
     return line
+
+
+def qmm_sweep(torch, ops, dev, with_cpu=True):
+    """Per-shape table for the JSON line: the single-matmul configuration (8192 x 2048) and the
+    five projection shapes of the 7B-shaped target at M in {1, 8, 16, 24, 32}.  GPU: us per launch
+    of `quantized_matmul` (graph-timed, weights rotated over more than 1 GB of copies), and of the
+    partial-sum slab form on the tiled weight layout where the verification step uses it (its sum
+    is taken by the kernel that reads it); algorithmic GB/s and fraction of 8 TB/s of the faster
+    one.  CPU: the OpenMP C restatement on all host threads given to the run, median of 20 calls
+    after 10 warm-up calls (the reference's own loop drops 10 of 30, utils.py:59-72)."""
+    from mlx_eagle_spec_decoding_tree_amd import synth
+    shapes = [("cfg1", 8192, 2048), ("q_o", 3584, 3584), ("k_v", 512, 3584), ("gate_up", 18944, 3584),
+              ("down", 3584, 18944), ("lm_head", 152064, 3584)]
+    rows = []
+    cores = None
+    if with_cpu:
+        from oracle import oracle
+        oracle.build()
+        cores = int(os.environ.get("OMP_NUM_THREADS", 0)) or min(16, os.cpu_count() or 1)
+        set_omp_threads(cores)
+    rng = np.random.default_rng(42)
+    for name, N, K in shapes:
+        wbytes = 0.5625 * N * K
+        ncopy = 4 if wbytes > 3e8 else min(40, max(2, int(1.2e9 // wbytes)))
+        ws = [torch.randint(-2 ** 31, 2 ** 31 - 1, (N, K // 8), dtype=torch.int32, device=dev) for _ in range(ncopy)]
+        ss = [(torch.rand(N, K // 64, device=dev) * 0.015 + 0.005).half() for _ in range(ncopy)]
+        bs = [(-8 * s.float()).half() for s in ss]
+        steps = ops.slab_steps(32, N, K)
+        tiled = [ops.tile_weights(ws[i], ss[i], bs[i]) for i in range(ncopy)] if steps and ops.tiled_supported(32, N, K) else None
+        layer = synth.make_qlinear(rng, N, K) if with_cpu else None
+        for M in (1, 8, 16, 24, 32):
+            x = torch.randn(M, K, device=dev).half()
+            o = torch.empty(M, N, device=dev, dtype=torch.float16)
+            iters = 40
+
+            def fn():
+                for i in range(iters):
+                    ops.quantized_matmul(x, ws[i % ncopy], ss[i % ncopy], bs[i % ncopy], out=o)
+
+            ts, g = graph_time_ms(torch, fn, reps=5)
+            us = float(np.median(ts)) * 1e3 / iters
+            rec = {"shape": name, "N": N, "K": K, "M": M, "gpu_us": round(us, 2)}
+            best = us
+            if tiled is not None:
+                part = torch.empty(ops.slab_count(K, steps) * 32 * N, dtype=torch.float32, device=dev)
+
+                def fn_slab():
+                    for i in range(iters):
+                        ops.quantized_matmul_slabs(x, ws[i % ncopy], ss[i % ncopy], bs[i % ncopy], steps, partial=part,
+                                                   tiled=tiled[i % ncopy])
+
+                ts, g = graph_time_ms(torch, fn_slab, reps=5)
+                rec["slab_us"] = round(float(np.median(ts)) * 1e3 / iters, 2)
+                best = min(best, rec["slab_us"])
+            gbs = qmm_bytes(M, N, K) / best / 1e3
+            rec["gbs"] = round(gbs)
+            rec["frac"] = round(gbs / HBM_PEAK_GBS, 3)
+            if with_cpu:
+                xc = synth.make_x(rng, M, K)
+                ts = []
+                for it in range(30):
+                    t0 = time.perf_counter()
+                    oracle.qmm(xc, layer["weight"], layer["scales"], layer["biases"])
+                    if it >= 10:
+                        ts.append((time.perf_counter() - t0) * 1e6)
+                rec["cpu_us"] = round(float(np.median(ts)), 1)
+            rows.append(rec)
+            del g
+        del ws, ss, bs, tiled
+        torch.cuda.empty_cache()
+    return {"gpu": "us per launch, graph-timed, weights rotated over > 1 GB; slab_us = partial-sum slab form on "
+                   "the tiled layout (summed by its reader); gbs / frac: algorithmic bytes over the faster form",
+            "cpu": f"OpenMP C restatement, {cores} threads, median of 20 calls after 10 warm-up calls" if with_cpu else None,
+            "rows": rows}
 
 
 def sweep(torch, ops, dev, args):

@@ -116,6 +116,14 @@ int eagle_qmv_supported(int N, int K);
 int eagle_qmv_w4g64_f16(const void* x, const uint32_t* wq, const void* scales, const void* biases,
                         const void* bias, void* out, int N, int K, int group_size, int bits,
                         eagle_stream_t stream);
+/* The same for 1..8 rows of x (eagle_qmv_rows_supported): the expanded nibbles of a packed word
+ * serve every row, as the reference's batched vector kernel does (kernels/qmv/1b.metal:100-147,
+ * qmv.py:226-241); x [M, K], out [M, N].  Measured against the matrix-tile kernel at M = 2, 4, 8
+ * by `bench.py --small-m`. */
+int eagle_qmv_rows_supported(int M, int N, int K);
+int eagle_qmv_rows_w4g64_f16(const void* x, const uint32_t* wq, const void* scales,
+                             const void* biases, const void* bias, void* out, int M, int N, int K,
+                             int group_size, int bits, eagle_stream_t stream);
 
 /* The same matmul for callers that cannot allocate or bring a workspace (code under HIP graph
  * capture, tight serving loops, harnesses that forbid hipMalloc).  It has no counterpart in the
@@ -219,7 +227,7 @@ int eagle_qmm_slab_swiglu_w4g64_f16(const void* x, const uint32_t* wq, const voi
  *       the chunk's eight groups, lanes 32..63 the biases (eagle_qmm_tiled_sb_bytes bytes).
  * N % 32 == 0, K % 512 == 0, all pointers 16-byte aligned.
  * eagle_qmm_slab_partial_tiled_w4g64 / eagle_qmm_slab_swiglu_tiled_w4g64_f16 are
- * eagle_qmm_slab_partial_w4g64 / eagle_qmm_slab_swiglu_w4g64_f16 for 1..32 rows on that copy
+ * eagle_qmm_slab_partial_w4g64 / eagle_qmm_slab_swiglu_w4g64_f16 for 1..64 rows on that copy
  * (same results, same partial-sum layout, same consumers).  small_scales != 0 promises that
  * every |scale| is below 0.0624: the nibbles are then expanded through fp16 subnormals (scale *
  * 2^20 must be a finite fp16; larger scales give inf / NaN, never a finite wrong value).

@@ -30,6 +30,8 @@ SIGNATURES = {
                                        + [c_long, c_int, c_int, c_void_p]),
     "eagle_qmv_supported": (c_int, [c_int] * 2),
     "eagle_qmv_w4g64_f16": (c_int, [c_void_p] * 6 + [c_int] * 4 + [c_void_p]),
+    "eagle_qmv_rows_supported": (c_int, [c_int] * 3),
+    "eagle_qmv_rows_w4g64_f16": (c_int, [c_void_p] * 6 + [c_int] * 5 + [c_void_p]),
     "eagle_qmm_plan": (c_int, [c_int, c_int, c_int, c_void_p]),
     "eagle_qmm_swiglu_w4g64_f16": (c_int, [c_void_p] * 6 + [c_int] * 5 + [c_void_p, c_size_t, c_void_p]),
     "eagle_qmm_workspace_bytes_tuned": (c_size_t, [c_int] * 3),

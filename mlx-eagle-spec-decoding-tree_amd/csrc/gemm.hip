@@ -1273,7 +1273,7 @@ EAGLE_EXPORT int eagle_slab_sum_f16(const float* partial, int slabs, const void*
 }
 
 EAGLE_EXPORT int eagle_qmm_tiled_supported(int M, int N, int K) {
-  return M >= 1 && M <= SLAB_ROWS && N >= 32 && (N % 32) == 0 && K >= 512 && (K % 512) == 0 && K <= 65536;
+  return M >= 1 && M <= 2 * SLAB_ROWS && N >= 32 && (N % 32) == 0 && K >= 512 && (K % 512) == 0 && K <= 65536;
 }
 
 EAGLE_EXPORT size_t eagle_qmm_tiled_sb_bytes(int N, int K) {
@@ -1308,15 +1308,20 @@ EAGLE_EXPORT int eagle_qmm_slab_partial_tiled_w4g64(const void* x, const uint32_
   if (!eagle_aligned16(x) || !eagle_aligned16(wt) || !eagle_aligned16(sbt) || !eagle_aligned16(partial))
     return EAGLE_ERR_ALIGN;
   if (partial_bytes < eagle_qmm_slab_partial_bytes_rows(M, N, K, steps_per_slab)) return EAGLE_ERR_WORKSPACE;
+  const int mr = M > SLAB_ROWS ? 2 : 1;
   const int bufs = steps_per_slab > SLAB_RING ? 2 : 1;
-  const size_t lds = (size_t)bufs * SLAB_XBUF * sizeof(half_t);
+  const size_t lds = (size_t)bufs * mr * SLAB_XBUF * sizeof(half_t);
   static bool configured = false;
   if (!configured) {
     const int most = 2 * SLAB_XBUF * (int)sizeof(half_t);
     if (hipFuncSetAttribute(reinterpret_cast<const void*>(&qmm_slab_w4g64_kernel<false, 1, false, 4, 1, true, false>),
                             hipFuncAttributeMaxDynamicSharedMemorySize, most) != hipSuccess ||
         hipFuncSetAttribute(reinterpret_cast<const void*>(&qmm_slab_w4g64_kernel<false, 1, false, 4, 1, true, true>),
-                            hipFuncAttributeMaxDynamicSharedMemorySize, most) != hipSuccess)
+                            hipFuncAttributeMaxDynamicSharedMemorySize, most) != hipSuccess ||
+        hipFuncSetAttribute(reinterpret_cast<const void*>(&qmm_slab_w4g64_kernel<false, 2, false, 4, 1, true, false>),
+                            hipFuncAttributeMaxDynamicSharedMemorySize, 2 * most) != hipSuccess ||
+        hipFuncSetAttribute(reinterpret_cast<const void*>(&qmm_slab_w4g64_kernel<false, 2, false, 4, 1, true, true>),
+                            hipFuncAttributeMaxDynamicSharedMemorySize, 2 * most) != hipSuccess)
       return EAGLE_ERR_HIP;
     configured = true;
   }
@@ -1324,12 +1329,15 @@ EAGLE_EXPORT int eagle_qmm_slab_partial_tiled_w4g64(const void* x, const uint32_
   hipStream_t st = static_cast<hipStream_t>(stream);
   const half_t* xh = static_cast<const half_t*>(x);
   const half_t* sb = static_cast<const half_t*>(sbt);
-  if (small_scales)
-    hipLaunchKernelGGL((qmm_slab_w4g64_kernel<false, 1, false, 4, 1, true, true>), grid, dim3(256), lds, st, xh, wt,
-                       sb, (const half_t*)nullptr, partial, M, N, K, steps_per_slab, bufs);
-  else
-    hipLaunchKernelGGL((qmm_slab_w4g64_kernel<false, 1, false, 4, 1, true, false>), grid, dim3(256), lds, st, xh, wt,
-                       sb, (const half_t*)nullptr, partial, M, N, K, steps_per_slab, bufs);
+#define EAGLE_TL_PARTIAL(MRV, SUB)                                                                         \
+  hipLaunchKernelGGL((qmm_slab_w4g64_kernel<false, MRV, false, 4, 1, true, SUB>), grid, dim3(256), lds, st, xh, wt, \
+                     sb, (const half_t*)nullptr, partial, M, N, K, steps_per_slab, bufs)
+  if (mr == 2) {
+    if (small_scales) EAGLE_TL_PARTIAL(2, true); else EAGLE_TL_PARTIAL(2, false);
+  } else {
+    if (small_scales) EAGLE_TL_PARTIAL(1, true); else EAGLE_TL_PARTIAL(1, false);
+  }
+#undef EAGLE_TL_PARTIAL
   return eagle_launch_status();
 }
 
@@ -1343,7 +1351,7 @@ EAGLE_EXPORT int eagle_qmm_slab_swiglu_tiled_w4g64_f16(const void* x, const uint
     return EAGLE_ERR_ALIGN;
   const int steps = K / 64;                      // one slab over all of K
   // the two K sizes of the benchmark targets go to the kernel with two waves per weight tile
-  if (steps == 56 || steps == 64) {
+  if (M <= SLAB_ROWS && (steps == 56 || steps == 64)) {
     hipStream_t bst = static_cast<hipStream_t>(stream);
     const half_t* xh = static_cast<const half_t*>(x);
     const half_t* sb = static_cast<const half_t*>(sbt);
@@ -1355,11 +1363,12 @@ EAGLE_EXPORT int eagle_qmm_slab_swiglu_tiled_w4g64_f16(const void* x, const uint
     return small_scales ? launch_burst<4, true, true, 8, 8>(xh, wt, sb, nullptr, nullptr, M, N, K, steps, 1, bh, oh, bst)
                         : launch_burst<4, true, false, 8, 8>(xh, wt, sb, nullptr, nullptr, M, N, K, steps, 1, bh, oh, bst);
   }
+  const int mr = M > SLAB_ROWS ? 2 : 1;
   int nwv = 4;
   while (nwv < 8 && (N + 32 * nwv - 1) / (32 * nwv) > NUM_CU) nwv += (nwv == 6 ? 2 : 1);
   const int blocks = (N + 32 * nwv - 1) / (32 * nwv);
-  const int bufs = steps > SLAB_RING ? 2 : 1;
-  const size_t lds = (size_t)bufs * SLAB_XBUF * sizeof(half_t);
+  const int bufs = steps > SLAB_RING && !(mr == 2 && blocks > NUM_CU) ? 2 : 1;   // as the row-major form
+  const size_t lds = (size_t)bufs * mr * SLAB_XBUF * sizeof(half_t);
   static bool configured = false;
   if (!configured) {
     const int most = 2 * SLAB_XBUF * (int)sizeof(half_t);
@@ -1369,7 +1378,11 @@ EAGLE_EXPORT int eagle_qmm_slab_swiglu_tiled_w4g64_f16(const void* x, const uint
        hipFuncSetAttribute(reinterpret_cast<const void*>(&qmm_slab_w4g64_kernel<false, 1, true, NW, 2, true, false>), \
                            hipFuncAttributeMaxDynamicSharedMemorySize, most) == hipSuccess &&                    \
        hipFuncSetAttribute(reinterpret_cast<const void*>(&qmm_slab_w4g64_kernel<false, 1, true, NW, 2, true, true>),  \
-                           hipFuncAttributeMaxDynamicSharedMemorySize, most) == hipSuccess
+                           hipFuncAttributeMaxDynamicSharedMemorySize, most) == hipSuccess &&                    \
+       hipFuncSetAttribute(reinterpret_cast<const void*>(&qmm_slab_w4g64_kernel<false, 2, true, NW, 1, true, false>), \
+                           hipFuncAttributeMaxDynamicSharedMemorySize, 2 * most) == hipSuccess &&                \
+       hipFuncSetAttribute(reinterpret_cast<const void*>(&qmm_slab_w4g64_kernel<false, 2, true, NW, 1, true, true>),  \
+                           hipFuncAttributeMaxDynamicSharedMemorySize, 2 * most) == hipSuccess
     EAGLE_TL_SWI_ATTR(4);
     EAGLE_TL_SWI_ATTR(5);
     EAGLE_TL_SWI_ATTR(6);
@@ -1380,13 +1393,17 @@ EAGLE_EXPORT int eagle_qmm_slab_swiglu_tiled_w4g64_f16(const void* x, const uint
   }
   const dim3 grid(blocks, 1);
   hipStream_t st = static_cast<hipStream_t>(stream);
-#define EAGLE_TL_SWI_LAUNCH(NW, SUB)                                                                     \
-  hipLaunchKernelGGL((qmm_slab_w4g64_kernel<false, 1, true, NW, 2, true, SUB>), grid, dim3(64 * NW), lds, st, \
-                     static_cast<const half_t*>(x), wt, static_cast<const half_t*>(sbt),                 \
-                     (const half_t*)nullptr, (float*)nullptr, M, N, K, steps, bufs,                      \
-                     static_cast<const half_t*>(bias), static_cast<half_t*>(out))
+#define EAGLE_TL_SWI_LAUNCH(NW, MRV, SUB)                                                                \
+  hipLaunchKernelGGL((qmm_slab_w4g64_kernel<false, MRV, true, NW, (MRV == 1 ? 2 : 1), true, SUB>), grid,  \
+                     dim3(64 * NW), lds, st, static_cast<const half_t*>(x), wt,                          \
+                     static_cast<const half_t*>(sbt), (const half_t*)nullptr, (float*)nullptr, M, N, K,  \
+                     steps, bufs, static_cast<const half_t*>(bias), static_cast<half_t*>(out))
 #define EAGLE_TL_SWI_NW(NW)                                                                              \
-  if (small_scales) EAGLE_TL_SWI_LAUNCH(NW, true); else EAGLE_TL_SWI_LAUNCH(NW, false);
+  if (mr == 2) {                                                                                         \
+    if (small_scales) EAGLE_TL_SWI_LAUNCH(NW, 2, true); else EAGLE_TL_SWI_LAUNCH(NW, 2, false);          \
+  } else {                                                                                               \
+    if (small_scales) EAGLE_TL_SWI_LAUNCH(NW, 1, true); else EAGLE_TL_SWI_LAUNCH(NW, 1, false);          \
+  }
   switch (nwv) {
     case 4: EAGLE_TL_SWI_NW(4) break;
     case 5: EAGLE_TL_SWI_NW(5) break;

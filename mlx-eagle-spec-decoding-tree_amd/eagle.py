@@ -493,7 +493,7 @@ class TreeVerifier:
         streaming kernel; None: the library's choice for this shape.
         tiled: the slab products (and gate|up + SwiGLU) read a copy of their weights in the tiled
         layout (`ops.tile_weights`; doubles the memory of those matrices).  None: on for the fused
-        step of up to 32 tree tokens."""
+        step."""
         args = model.args
         self.model, self.cache, self.args = model, cache, args
         if total_tokens + 1 > TREE_SLOTS:
@@ -520,10 +520,10 @@ class TreeVerifier:
         if fuse:
             self._fuse_projections()
         self.slab = self._slab_plan(slab_plan)
-        if tiled and (self.wide or not fuse):
-            raise ValueError("the tiled weight layout serves the fused step of up to 32 tree tokens")
+        if tiled and not fuse:
+            raise ValueError("the tiled weight layout serves the fused step")
         self.tiled = None
-        if (tiled or tiled is None) and fuse and not self.wide:
+        if (tiled or tiled is None) and fuse:
             self.tiled = tiled_projections(model, self.qkv_w, self.gu_w, self.slab, self.swiglu)
         i32 = dict(dtype=torch.int32, device=dev)
         f16 = dict(dtype=torch.float16, device=dev)

@@ -107,11 +107,12 @@ def quantized_matmul(x, w_q, scales, biases, transpose=True, group_size=64, bits
                                         _ptr(out), M, N, K, group_size, bits, _stream())
         _lib.check(rc, "quantized_matmul")
         return out
-    if tuned is None and M == 1 and qmv_preferred(N, K) and group_size == 64 and bits == 4:
-        # one row: the vector-ALU kernel (faster than a 16-row matrix tile with 15 rows idle
-        # wherever the matrix has enough rows to fill the GPU with short K)
-        rc = L.eagle_qmv_w4g64_f16(_ptr(x), _ptr(w_q), _ptr(scales), _ptr(biases), _ptr(bias),
-                                   _ptr(out), N, K, group_size, bits, _stream())
+    if tuned is None and M <= QMV_MAX_ROWS and qmv_preferred(N, K, M) and group_size == 64 and bits == 4:
+        # one row (or the few rows `qmv_preferred` takes): the vector-ALU kernel, faster than a 16-row
+        # matrix tile with most rows idle wherever the matrix has enough rows to fill the GPU with
+        # short K
+        rc = L.eagle_qmv_rows_w4g64_f16(_ptr(x), _ptr(w_q), _ptr(scales), _ptr(biases), _ptr(bias),
+                                        _ptr(out), M, N, K, group_size, bits, _stream())
         _lib.check(rc, "quantized_matmul")
         return out
     if tuned is None:
@@ -156,10 +157,10 @@ def quantized_matmul_slabs(x, w_q, scales, biases, steps_per_slab, partial=None,
     """The product for 1..64 rows as fp32 partial sums of K slabs, [slabs, R, N] with R = 32 up
     to 32 rows and 64 above (`slab_rows`): the result is fp16(partial.sum(0)) (+ bias), formed by
     `slab_sum`, `rms_norm_slabs` or `rope_kv_append_slabs`.  K % 128 == 0.
-    tiled: the same matrix as `TiledWeights`; up to 32 rows then read that copy."""
+    tiled: the same matrix as `TiledWeights`; the kernel then reads that copy."""
     _need_cuda(x, w_q, scales, biases)
     x = _f16(x, "x")
-    if tiled is not None and x.numel() // x.shape[-1] <= 32:
+    if tiled is not None and x.numel() // x.shape[-1] <= 64:
         return _matmul_slabs_tiled(x, tiled, steps_per_slab, partial)
     w_q = as_packed_u32(w_q)
     scales, biases = _f16(scales, "scales"), _f16(biases, "biases")
@@ -193,10 +194,11 @@ def _matmul_slabs_tiled(x, tiled, steps_per_slab, partial):
     slabs = slab_count(K, steps_per_slab)
     if slabs < 1:
         raise ValueError(f"the slab form does not take K = {K} with {steps_per_slab} steps per slab")
+    R = slab_rows(M)
     if partial is None:
-        partial = torch.empty((slabs, 32, N), dtype=torch.float32, device=x.device)
-    elif partial.dtype != torch.float32 or partial.numel() < slabs * 32 * N or not partial.is_contiguous():
-        raise ValueError("partial must be a contiguous fp32 buffer of at least slabs * 32 * N elements")
+        partial = torch.empty((slabs, R, N), dtype=torch.float32, device=x.device)
+    elif partial.dtype != torch.float32 or partial.numel() < slabs * R * N or not partial.is_contiguous():
+        raise ValueError(f"partial must be a contiguous fp32 buffer of at least slabs * {R} * N elements")
     rc = _lib.lib().eagle_qmm_slab_partial_tiled_w4g64(_ptr(x), _ptr(tiled.wt), _ptr(tiled.sbt), _ptr(partial),
                                                        partial.numel() * 4, M, N, K, int(steps_per_slab),
                                                        int(tiled.small), _stream())
@@ -272,11 +274,11 @@ def quantized_matmul_swiglu(x, w_q, scales, biases, bias=None, out=None, gemm=No
     the product.  33..64 rows run on the slab kernel with 64-row tiles
     (`quantized_matmul_swiglu_slab`), more rows as the tiled GEMM form with the same epilogue
     (`gemm=True`: that form whatever the row count).
-    tiled: the interleaved matrix as `TiledWeights`; up to 32 rows then run the slab kernel on
+    tiled: the interleaved matrix as `TiledWeights`; up to 64 rows then run the slab kernel on
     that copy."""
     _need_cuda(x, w_q, scales, biases, bias)
     x = _f16(x, "x")
-    if tiled is not None and not gemm and x.numel() // x.shape[-1] <= 32:
+    if tiled is not None and not gemm and x.numel() // x.shape[-1] <= 64:
         *lead, K = x.shape
         M = reduce(lambda a, b: a * b, lead, 1)
         if K != tiled.K:
@@ -351,7 +353,7 @@ class TiledWeights:
 
 def tiled_supported(M, N, K):
     """True when the tiled forms (`quantized_matmul_slabs` / `quantized_matmul_swiglu` with
-    `tiled=`) take this product: up to 32 rows, N a multiple of 32, K a multiple of 512."""
+    `tiled=`) take this product: up to 64 rows, N a multiple of 32, K a multiple of 512."""
     return bool(_lib.lib().eagle_qmm_tiled_supported(int(M), int(N), int(K)))
 
 
@@ -441,24 +443,37 @@ def qkv_rope_small(x, w_q, scales, biases, bias, rope_cs, q_rot, k_cache, v_cach
     return q_rot
 
 
-def qmv_preferred(N, K):
-    """True where the vector-ALU kernel is the faster form for one row of x: measured on the
-    projection shapes of the 7B model (M = 1: 5.7 against 8.5 us for 3584 x 3584, 12.5 against
-    16.2 us for 18944 x 3584); a long K over few rows (3584 x 18944: 28.8 against 18.6 us) and the
-    vocabulary projection (66.8 against 62.8 us) stay on the matrix kernel."""
-    return bool(_lib.lib().eagle_qmv_supported(N, K)) and K <= 4096 and N <= 65536
+# rows of x up to which `quantized_matmul` considers the vector-ALU kernel (`bench.py --small-m`
+# has the measurements behind QMV_MAX_ROWS and `qmv_preferred`)
+QMV_MAX_ROWS = 2
+
+
+def qmv_preferred(N, K, M=1):
+    """True where the vector-ALU kernel is the faster form for M rows of x.  Measured on the
+    projection shapes of the 7B model, vector ALU against matrix tiles, us per launch:
+      M = 1: 5.8 / 8.5 (3584 x 3584), 4.4 / 6.7 (512 x 3584), 12.6 / 16.1 (18944 x 3584), 5.3 / 7.1
+             (8192 x 2048); a long K over few rows (3584 x 18944: 28.3 / 18.9) and the vocabulary
+             projection (66.6 / 63.2) stay on the matrix kernel;
+      M = 2: 7.2 / 8.5, 5.8 / 6.9, 16.3 / 15.9, 6.6 / 7.2: the vector ALU up to a few thousand rows;
+      M = 4: 9.4 / 8.6, 8.4 / 7.0, 28.7 / 16.1, 8.9 / 7.3; M = 8: 15.1 / 8.7, 14.3 / 7.1, 44.2 / 16.1,
+             14.2 / 7.4: matrix tiles everywhere (5 + 4 M vector instructions per packed word)."""
+    if M > QMV_MAX_ROWS or not _lib.lib().eagle_qmv_rows_supported(M, N, K) or K > 4096:
+        return False
+    return N <= 65536 if M == 1 else N <= 16384
 
 
 def quantized_matvec(x, w_q, scales, biases, bias=None, out=None):
-    """One row of x times the quantised matrix on the vector ALU (no matrix instructions):
-    the M = 1 case of `quantized_matmul` (mlx_model_fwd_bench.py:65-73)."""
+    """One to eight rows of x times the quantised matrix on the vector ALU (no matrix
+    instructions): the M = 1 case of `quantized_matmul` (mlx_model_fwd_bench.py:65-73) and the
+    reference's batched vector form (qmv.py:226-241)."""
     _need_cuda(x, w_q, scales, biases, bias)
     x = _f16(x, "x")
     w_q = as_packed_u32(w_q)
     scales, biases = _f16(scales, "scales"), _f16(biases, "biases")
     K = x.shape[-1]
     N = w_q.shape[0]
-    if x.numel() != K or w_q.shape[1] * 8 != K or tuple(scales.shape) != (N, K // 64) \
+    M = x.numel() // K
+    if M < 1 or M > 8 or w_q.shape[1] * 8 != K or tuple(scales.shape) != (N, K // 64) \
             or tuple(biases.shape) != (N, K // 64):
         raise ValueError(f"shape mismatch: x {tuple(x.shape)}, w {tuple(w_q.shape)}, "
                          f"scales {tuple(scales.shape)}, biases {tuple(biases.shape)}")
@@ -466,8 +481,8 @@ def quantized_matvec(x, w_q, scales, biases, bias=None, out=None):
         bias = _f16(bias, "bias")
     if out is None:
         out = torch.empty((*x.shape[:-1], N), dtype=torch.float16, device=x.device)
-    rc = _lib.lib().eagle_qmv_w4g64_f16(_ptr(x), _ptr(w_q), _ptr(scales), _ptr(biases), _ptr(bias),
-                                        _ptr(out), N, K, 64, 4, _stream())
+    rc = _lib.lib().eagle_qmv_rows_w4g64_f16(_ptr(x), _ptr(w_q), _ptr(scales), _ptr(biases), _ptr(bias),
+                                             _ptr(out), M, N, K, 64, 4, _stream())
     _lib.check(rc, "quantized_matvec")
     return out
 

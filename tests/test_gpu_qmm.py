@@ -212,3 +212,28 @@ def test_swiglu_form_with_k_slabs(dev):
         torch.cuda.synchronize()
         assert torch.equal(got, two), f"M={M} I={I} K={K}"
         assert rel_err(got.cpu().numpy(), want) <= TOL
+
+
+@pytest.mark.parametrize("N,K", [(3584, 3584), (512, 3584), (8192, 2048), (40, 512), (136, 4096)])
+@pytest.mark.parametrize("M", [1, 2, 3, 4, 5, 8])
+def test_vector_alu_rows(dev, M, N, K):
+    """The vector-ALU kernel for 1..8 rows of x (the expanded nibbles of a packed word shared by
+    the rows) against the oracle, with a bias; rows past M are neither read nor written."""
+    rng = np.random.default_rng(M * 7 + N + K)
+    layer = synth.make_qlinear(rng, N, K, bias=True)
+    x = synth.make_x(rng, M, K)
+    want = oracle.qmm(x, layer["weight"], layer["scales"], layer["biases"], layer["bias"])
+    d = layer_to_dev(layer, dev)
+    out = torch.full((M + 1, N), float("nan"), dtype=torch.float16, device=dev)
+    ops.quantized_matvec(to_dev(x, dev), d["weight"], d["scales"], d["biases"], bias=d["bias"], out=out[:M])
+    got = out.cpu().numpy()
+    assert np.isnan(got[M].astype(np.float32)).all()
+    assert rel_err(got[:M], want) <= TOL
+
+
+def test_vector_alu_rows_refusals(dev):
+    from mlx_eagle_spec_decoding_tree_amd import _lib
+    L = _lib.lib()
+    assert L.eagle_qmv_rows_supported(8, 3584, 3584) == 1 and L.eagle_qmv_rows_supported(9, 3584, 3584) == 0
+    assert L.eagle_qmv_rows_supported(1, 3584, 18944) == 1 and L.eagle_qmv_rows_supported(4, 3584, 18944) == 0   # x beyond LDS
+    assert L.eagle_qmv_rows_supported(2, 64, 896) == 0

@@ -38,7 +38,9 @@ def test_layout(dev, N, K):
 
 @pytest.mark.parametrize("M,N,K,steps", [(32, 4608, 3584, 8), (32, 3584, 3584, 8), (32, 3584, 18944, 32),
                                          (17, 96, 1536, 8), (1, 128, 1024, 16), (24, 4096, 14336, 32),
-                                         (8, 6144, 4096, 8), (32, 160, 512, 8)])
+                                         (8, 6144, 4096, 8), (32, 160, 512, 8),
+                                         # 33..64 rows: 64-row partial tiles
+                                         (40, 4608, 3584, 8), (64, 3584, 18944, 32), (33, 96, 1024, 8)])
 def test_partial_sums(dev, M, N, K, steps):
     print(f"tiled slab M={M} N={N} K={K} steps={steps}", flush=True)
     rng = np.random.default_rng(M + N + K)
@@ -52,7 +54,7 @@ def test_partial_sums(dev, M, N, K, steps):
     plain = ops.quantized_matmul_slabs(xd, d["weight"], d["scales"], d["biases"], steps)
     for small in (False, True):
         t.small = small
-        part = torch.full((slabs, 32, N), float("nan"), dtype=torch.float32, device=dev)
+        part = torch.full((slabs, ops.slab_rows(M), N), float("nan"), dtype=torch.float32, device=dev)
         ops.quantized_matmul_slabs(xd, d["weight"], d["scales"], d["biases"], steps, partial=part, tiled=t)
         assert torch.isfinite(part[:, :M]).all() and torch.isnan(part[:, M:]).all()
         if not small:
@@ -97,7 +99,8 @@ def test_large_scales_take_the_other_expansion(dev):
 
 
 @pytest.mark.parametrize("M,I,K,bias", [(32, 18944, 3584, True), (32, 14336, 4096, False), (8, 4864, 1024, True),
-                                        (1, 64, 512, False), (27, 272, 1536, True)])
+                                        (1, 64, 512, False), (27, 272, 1536, True), (40, 18944, 3584, True),
+                                        (64, 14336, 4096, False), (47, 272, 1536, True)])
 def test_swiglu(dev, M, I, K, bias):
     print(f"tiled swiglu M={M} I={I} K={K}", flush=True)
     rng = np.random.default_rng(M + I + K)
@@ -121,7 +124,7 @@ def test_swiglu(dev, M, I, K, bias):
                                     out=out[:M], tiled=t)
         got = out.cpu().numpy()
         assert np.isnan(got[M].astype(np.float32)).all()
-        if not small and K not in (3584, 4096):
+        if not small and (K not in (3584, 4096) or M > 32):
             # (those two K sizes run two waves per weight tile, which add their halves of K at the end)
             assert torch.equal(out[:M], plain)
         else:
@@ -137,7 +140,7 @@ def test_swiglu(dev, M, I, K, bias):
 
 def test_refusals(dev):
     L = _lib.lib()
-    assert L.eagle_qmm_tiled_supported(32, 4608, 3584) == 1 and L.eagle_qmm_tiled_supported(33, 4608, 3584) == 0
+    assert L.eagle_qmm_tiled_supported(64, 4608, 3584) == 1 and L.eagle_qmm_tiled_supported(65, 4608, 3584) == 0
     assert L.eagle_qmm_tiled_supported(8, 1152, 896) == 0 and L.eagle_qmm_tiled_supported(8, 48, 512) == 0
     assert L.eagle_qmm_tiled_sb_bytes(4608, 3584) == 4608 * 56 * 4 and L.eagle_qmm_tiled_sb_bytes(48, 512) == 0
     rng = np.random.default_rng(1)
