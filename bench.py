@@ -59,7 +59,7 @@ def write_traffic_record(fetch_csv, write_csv):
                 if r["Counter_Name"] != name:
                     continue
                 kn = r["Kernel_Name"]
-                if "qmm_w4g64" in kn or "qmm_slab_w4g64" in kn:
+                if "qmm_w4g64" in kn or "qmm_slab_w4g64" in kn or "qmm_burst_w4g64" in kn:
                     q.append(float(r["Counter_Value"]))
                 if "copyBuffer" in kn or "elementwise" in kn:
                     cp.append(float(r["Counter_Value"]))
@@ -319,7 +319,8 @@ def main():
     achieved = alg / (qmm_ms * 1e-3) / 1e9
     traffic, traffic_source = read_traffic_record()
     stream_kernel = "qmm_w4g64_kernel"          # (above 32 tree tokens: two launches of it per product)
-    kernels = stream_kernel + " + qmm_slab_w4g64_kernel"
+    burst = (not ver.wide) and any(l[6] is True and l[7] is not None for l in launches)
+    kernels = stream_kernel + " + qmm_slab_w4g64_kernel" + (" + qmm_burst_w4g64_kernel" if burst else "")
     roofline = {"bound": "hbm", "kernel": kernels, "achieved": round(achieved, 1),
                 "peak": HBM_PEAK_GBS, "unit": "GB/s", "frac": round(achieved / HBM_PEAK_GBS, 4),
                 "traffic": traffic, "traffic_source": traffic_source, "launches_per_step": n_launch,
@@ -331,7 +332,8 @@ def main():
     per_kernel = {}
     # (above 32 tree tokens gate|up + SwiGLU runs on the slab kernel too: one slab over all of K)
     swi_on_slab = ver.wide or any(l[6] is True and l[7] is not None for l in launches)
-    swi_name = "qmm_slab_w4g64_kernel (SwiGLU form)" if swi_on_slab else stream_kernel
+    swi_name = ("qmm_burst_w4g64_kernel (gate|up + SwiGLU)" if burst else
+                "qmm_slab_w4g64_kernel (SwiGLU form)" if swi_on_slab else stream_kernel)
     groups = ([(swi_name, [l for l in launches if l[6] is True]), (stream_kernel, [l for l in launches if not l[6]])]
               if swi_on_slab else [(stream_kernel, [l for l in launches if l[6] is True or not l[6]])])
     for kname, sub in (*groups,

@@ -9,8 +9,7 @@ import os
 from ctypes import c_char_p, c_float, c_int, c_int32, c_long, c_longlong, c_size_t, c_void_p
 
 HERE = os.path.dirname(os.path.abspath(__file__))
-# EAGLE_MI355X_LIB selects another build of the same library (kernel experiments)
-LIB_PATH = os.environ.get("EAGLE_MI355X_LIB") or os.path.join(HERE, "libeagle_mi355x.so")
+LIB_PATH = os.path.join(HERE, "libeagle_mi355x.so")
 
 _lib = None
 

@@ -27,10 +27,6 @@
 // The draft-side form (mlx_eagle.py:143-178,207) has fewer query rows than masked key rows: T
 // queries see the P prefix rows and, through masks of one or two 32-bit words per query, the
 // Tk <= 64 rows P .. P+Tk-1 written by the earlier expansion levels and this one.
-//
-// A second form of the split kernel takes the un-rotated projection outputs instead
-// (mlx_llama.py:166-183): it rotates q and the tree keys itself and appends the tree rows to
-// the cache, which saves the separate rope / append launch.
 #include "common.h"
 
 #include <math.h>
@@ -73,26 +69,7 @@ __host__ __device__ inline int split_slots(int rep, int hd) {
   return 256 * (per_cu < 1 ? 1 : per_cu);
 }
 
-// (lo, hi) = elements i0..i0+7 and i0+half..i0+half+7 of a head vector; cs = 8 (cos, sin) pairs
-__device__ inline void rotate_pair(half8_t& lo, half8_t& hi, const float* cs) {
-  float4_t c[4];
-#pragma unroll
-  for (int k = 0; k < 4; ++k) c[k] = *reinterpret_cast<const float4_t*>(cs + 4 * k);
-#pragma unroll
-  for (int j = 0; j < 8; ++j) {
-    const float co = c[j >> 1][(j & 1) * 2], sn = c[j >> 1][(j & 1) * 2 + 1];
-    const float x1 = (float)lo[j], x2 = (float)hi[j];
-    lo[j] = (half_t)__builtin_fmaf(x1, co, -(x2 * sn));
-    hi[j] = (half_t)__builtin_fmaf(x1, sn, x2 * co);
-  }
-}
-
-// ROPE = false: q [H,T,hd] is rotated already and the cache holds the tree rows.
-// ROPE = true: q, k_lin, v_lin are the token-major projection outputs (row stride ld); q and
-// the tree keys are rotated here with the cos/sin table rope_cs [T][hd/2][2], tree rows are
-// taken from k_lin / v_lin instead of the cache, and the workgroup that owns a tile with tree
-// rows appends them to the cache (every tile has exactly one owner per KV group, and no
-// workgroup reads a cache row at or beyond P, so the append races with nothing).
+// q [H,T,hd] is rotated already and the cache holds the tree rows.
 // NVU: 16-byte vectors of a K (or V) tile per thread, a power of two with NVU * blockDim.x >= the
 // vectors of a tile.  DEPTH: tiles requested ahead, each in registers of its own (a tile's way
 // from the L2 into LDS takes longer than its arithmetic: with one tile ahead the loop runs at one
@@ -103,24 +80,20 @@ struct Stage { static constexpr int value = V; };
 // SUB: 32-key blocks per tile (1 or 2).  With two, the S products, the exponentials and the O
 // products of 64 keys each form one phase of a tile instead of two: the phases of a tile depend on
 // each other inside a wave, so a tile of 64 keys takes little longer than one of 32.
-template <int HD, bool ROPE, bool WIDE, int NVU, int DEPTH, int SUB>
+template <int HD, bool WIDE, int NVU, int DEPTH, int SUB>
 __global__ __launch_bounds__(512) void tree_attn_split_kernel(
     const half_t* __restrict__ q, half_t* kc, half_t* vc,
     const uint32_t* __restrict__ mask_bits, const int32_t* __restrict__ len_dev,
     half_t* __restrict__ part_o, float* __restrict__ part_ml, int T, int H, int G, long cap,
-    float scale_log2e, const half_t* __restrict__ k_lin,
-    const half_t* __restrict__ v_lin, long ld, const float* __restrict__ rope_cs, int Tk, int q_rows,
-    int len_stride) {
+    float scale_log2e, int Tk, int q_rows, int len_stride) {
   constexpr int KSTEPS = HD / 16;       // MFMA steps over the head dimension for S
   constexpr int DB = HD / 32;           // 32-wide blocks of the head dimension for O
   constexpr int STR = HD * 2 + 16;      // LDS row stride in bytes (pad: conflict-free reads)
   constexpr int VEC_ROW = HD / 8;       // 16-byte vectors per K/V row
   extern __shared__ __attribute__((aligned(16))) unsigned char lds[];
-  constexpr int HALF = HD / 2;
   constexpr int KTT = KT * SUB;         // keys per tile
   unsigned char* ldsK = lds;
   unsigned char* ldsV = lds + KTT * STR;
-  float* cs_lds = reinterpret_cast<float*>(lds + 2 * KTT * STR);   // ROPE: [T][HALF][2]
 
   const int g = blockIdx.x;
   const int split = blockIdx.y;
@@ -141,7 +114,7 @@ __global__ __launch_bounds__(512) void tree_attn_split_kernel(
   // (the last piece of a causal pass sees the most keys: dispatched first)
   const int piece = gridDim.z - 1 - blockIdx.z;
   const int qrow = piece * 32 + (lane & 31);
-  if (!ROPE && T > q_rows - piece * 32) T = q_rows - piece * 32;
+  if (T > q_rows - piece * 32) T = q_rows - piece * 32;
   int P = len_dev[piece * len_stride];
   // never index past the cache, whatever the counter says (a graph replayed beyond the
   // capacity would otherwise read beyond the last head's buffer)
@@ -160,8 +133,7 @@ __global__ __launch_bounds__(512) void tree_attn_split_kernel(
   for (int kk = 0; kk < KSTEPS; ++kk) {
     qreg[kk] = half8_t{0, 0, 0, 0, 0, 0, 0, 0};
     if (ql < T) {
-      const half_t* qp = ROPE ? q + (long)ql * ld + (long)head * HD
-                              : q + ((long)head * q_rows + qrow) * HD;
+      const half_t* qp = q + ((long)head * q_rows + qrow) * HD;
       qreg[kk] = *reinterpret_cast<const half8_t*>(qp + kk * 16 + hb * 8);
     }
   }
@@ -182,8 +154,6 @@ __global__ __launch_bounds__(512) void tree_attn_split_kernel(
 
   const half_t* kbase_ptr = kc + (long)g * cap * HD;
   const half_t* vbase_ptr = vc + (long)g * cap * HD;
-  const half_t* klin = ROPE ? k_lin + (long)g * HD : nullptr;
-  const half_t* vlin = ROPE ? v_lin + (long)g * HD : nullptr;
 
   // This workgroup's tiles are split, split + nactive, ...: all workgroups share the live part
   // of the cache however short it is.  The next DEPTH tiles are in flight into registers while
@@ -203,10 +173,6 @@ __global__ __launch_bounds__(512) void tree_attn_split_kernel(
       if (kidx > Ltot - 1) kidx = Ltot - 1;          // rows past the end are masked out below
       const half_t* kp = kbase_ptr + (long)kidx * HD;
       const half_t* vp = vbase_ptr + (long)kidx * HD;
-      if (ROPE && kidx >= P) {
-        kp = klin + (long)(kidx - P) * ld;
-        vp = vlin + (long)(kidx - P) * ld;
-      }
       kreg[st][it] = *reinterpret_cast<const half8_t*>(kp + c * 8);
       vreg[st][it] = *reinterpret_cast<const half8_t*>(vp + c * 8);
     }
@@ -237,54 +203,15 @@ __global__ __launch_bounds__(512) void tree_attn_split_kernel(
   __builtin_amdgcn_sched_barrier(0);
   if constexpr (DEPTH > 2) fetch(Stage<2>{}, tile_at(split + 2 * nactive));
   __builtin_amdgcn_sched_barrier(0);
-  if (ROPE) {
-    for (int v = tid; v < T * HALF / 2; v += nthr)
-      *reinterpret_cast<float4_t*>(cs_lds + 4 * v) = *reinterpret_cast<const float4_t*>(rope_cs + 4 * v);
-    __syncthreads();
-    if (ql < T) {
-#pragma unroll
-      for (int kk = 0; kk < KSTEPS / 2; ++kk)
-        rotate_pair(qreg[kk], qreg[kk + KSTEPS / 2], cs_lds + (ql * HALF + kk * 16 + hb * 8) * 2);
-    }
-  }
   // one tile: its registers (stage S) into LDS, the tile DEPTH ahead requested into the same
   // registers, then the arithmetic on LDS
   auto do_tile = [&](auto S, int tile) {
     constexpr int st = decltype(S)::value;
     const int kb = tile * KTT;
     __syncthreads();   // every wave is done with the previous tile
-    if (ROPE && kb + KTT > P) {
-      // tree rows: append the values as they are
-#pragma unroll
-      for (int it = 0; it < NVU; ++it) {
-        const int v = tid + it * nthr;
-        const int kidx = kb + v / VEC_ROW;
-        if (v < NVEC && kidx >= P && kidx < Ltot)
-          *reinterpret_cast<half8_t*>(vc + ((long)g * cap + kidx) * HD + (v % VEC_ROW) * 8) = vreg[st][it];
-      }
-    }
     stash(S);
     fetch(S, tile_at(tile + DEPTH * nactive));
     __syncthreads();
-    if (ROPE && kb + KTT > P) {
-      // rotate the tree keys in LDS (one thread per pair of 16-byte pieces) and append them
-      for (int v = tid; v < KTT * (VEC_ROW / 2); v += nthr) {
-        const int row = v / (VEC_ROW / 2);
-        const int c = v % (VEC_ROW / 2);
-        const int kidx = kb + row;
-        if (kidx >= P && kidx < Ltot) {
-          half8_t lo = *reinterpret_cast<const half8_t*>(ldsK + row * STR + c * 16);
-          half8_t hi = *reinterpret_cast<const half8_t*>(ldsK + row * STR + (c + VEC_ROW / 2) * 16);
-          rotate_pair(lo, hi, cs_lds + ((kidx - P) * HALF + c * 8) * 2);
-          *reinterpret_cast<half8_t*>(ldsK + row * STR + c * 16) = lo;
-          *reinterpret_cast<half8_t*>(ldsK + row * STR + (c + VEC_ROW / 2) * 16) = hi;
-          half_t* dst = kc + ((long)g * cap + kidx) * HD;
-          *reinterpret_cast<half8_t*>(dst + c * 8) = lo;
-          *reinterpret_cast<half8_t*>(dst + HALF + c * 8) = hi;
-        }
-      }
-      __syncthreads();
-    }
 
     // S^T[key][token] = sum_d K[key][d] Q[token][d], one accumulator per block of 32 keys
     float16_t sacc[SUB];
@@ -510,10 +437,10 @@ int splits_for(int max_len, int G) {
   return n;
 }
 
-template <int HD, bool ROPE, bool WIDE = false>
+template <int HD, bool WIDE = false>
 int launch_attention(const half_t* q, half_t* kc, half_t* vc, const uint32_t* bits, const int32_t* len,
                      void* out, int T, int H, int G, long cap, int max_len, float scale, void* workspace,
-                     const half_t* k_lin, const half_t* v_lin, long ld, const float* cs, hipStream_t st,
+                     hipStream_t st,
                      int Tk = 0, int pieces = 1, int q_rows = 0, int len_stride = 1) {
   if (!WIDE) Tk = T;
   if (q_rows == 0) q_rows = pieces * T;
@@ -523,23 +450,22 @@ int launch_attention(const half_t* q, half_t* kc, half_t* vc, const uint32_t* bi
   // splits for 4 active ones) held those back by 18 of 44 us.
   const int rep = H / G;
   // 64 keys per tile where a tile's 16-byte vectors are at most four per thread (three or more
-  // waves per workgroup at head dimension 128, two or more at 64), 32 keys otherwise and in the
-  // form that rotates and appends
+  // waves per workgroup at head dimension 128, two or more at 64), 32 keys otherwise
   const int need64 = (2 * KT * (HD / 8) + rep * 64 - 1) / (rep * 64);
-  const int sub = (!ROPE && need64 <= 4) ? 2 : 1;
+  const int sub = need64 <= 4 ? 2 : 1;
   const int ktt = KT * sub;
   int nsplit = splits_for(max_len, G);
   nsplit = active_splits((max_len + ktt - 1) / ktt, nsplit, G * pieces, split_slots(rep, HD), 3 - sub);
   float* part_ml = static_cast<float*>(workspace);
   half_t* part_o = reinterpret_cast<half_t*>(part_ml + (size_t)pieces * H * nsplit * 32 * 2);
   const float sl2 = scale * 1.4426950408889634f;
-  const size_t lds = 2 * ktt * (HD * 2 + 16) + (ROPE ? (size_t)EAGLE_MAX_TREE * HD * 4 : 0);
+  const size_t lds = 2 * ktt * (HD * 2 + 16);
   // vectors of a tile per thread (a power of two) and the tiles in flight that its registers allow
   const int need = (ktt * (HD / 8) + rep * 64 - 1) / (rep * 64);
 #define EAGLE_ATTN_SPLIT(NVU, DEPTH, SUB)                                                                \
-  hipLaunchKernelGGL((tree_attn_split_kernel<HD, ROPE, WIDE, NVU, ROPE ? 1 : DEPTH, ROPE ? 1 : SUB>),    \
+  hipLaunchKernelGGL((tree_attn_split_kernel<HD, WIDE, NVU, DEPTH, SUB>),                                \
                      dim3(G, nsplit, pieces), dim3(rep * 64), lds, st, q, kc, vc, bits, len, part_o, part_ml, T, \
-                     H, G, cap, sl2, k_lin, v_lin, ld, cs, Tk, q_rows, len_stride)
+                     H, G, cap, sl2, Tk, q_rows, len_stride)
   if (sub == 2) {
     if (need <= 1) EAGLE_ATTN_SPLIT(1, 3, 2);
     else if (need <= 2) EAGLE_ATTN_SPLIT(2, 2, 2);
@@ -599,11 +525,10 @@ EAGLE_EXPORT int eagle_tree_attention_f16(const void* q, const void* k_cache, co
   half_t* kc = const_cast<half_t*>(static_cast<const half_t*>(k_cache));
   half_t* vc = const_cast<half_t*>(static_cast<const half_t*>(v_cache));
   if (hd == 128)
-    return launch_attention<128, false>((const half_t*)q, kc, vc, tree_mask_bits, cache_len_dev, out, T, H,
-                                        G, capacity, max_len, scale, workspace, nullptr, nullptr, 0,
-                                        nullptr, st);
-  return launch_attention<64, false>((const half_t*)q, kc, vc, tree_mask_bits, cache_len_dev, out, T, H, G,
-                                     capacity, max_len, scale, workspace, nullptr, nullptr, 0, nullptr, st);
+    return launch_attention<128>((const half_t*)q, kc, vc, tree_mask_bits, cache_len_dev, out, T, H,
+                                        G, capacity, max_len, scale, workspace, st);
+  return launch_attention<64>((const half_t*)q, kc, vc, tree_mask_bits, cache_len_dev, out, T, H, G,
+                                     capacity, max_len, scale, workspace, st);
 }
 
 EAGLE_EXPORT int eagle_draft_attention_f16(const void* q, const void* k_cache, const void* v_cache,
@@ -625,12 +550,10 @@ EAGLE_EXPORT int eagle_draft_attention_f16(const void* q, const void* k_cache, c
   half_t* kc = const_cast<half_t*>(static_cast<const half_t*>(k_cache));
   half_t* vc = const_cast<half_t*>(static_cast<const half_t*>(v_cache));
   if (hd == 128)
-    return launch_attention<128, false, true>((const half_t*)q, kc, vc, mask_words, cache_len_dev, out, T,
-                                              H, G, capacity, max_len, scale, workspace, nullptr, nullptr,
-                                              0, nullptr, st, Tk);
-  return launch_attention<64, false, true>((const half_t*)q, kc, vc, mask_words, cache_len_dev, out, T, H,
-                                           G, capacity, max_len, scale, workspace, nullptr, nullptr, 0,
-                                           nullptr, st, Tk);
+    return launch_attention<128, true>((const half_t*)q, kc, vc, mask_words, cache_len_dev, out, T,
+                                              H, G, capacity, max_len, scale, workspace, st, Tk);
+  return launch_attention<64, true>((const half_t*)q, kc, vc, mask_words, cache_len_dev, out, T, H,
+                                           G, capacity, max_len, scale, workspace, st, Tk);
 }
 
 EAGLE_EXPORT size_t eagle_tree_attention_wide_workspace_bytes(int T, int H, int hd, int max_len) {
@@ -660,12 +583,10 @@ EAGLE_EXPORT int eagle_tree_attention_wide_f16(const void* q, const void* k_cach
   const int pieces = (T + 31) / 32;
   const int rows = T < 32 ? T : 32;
   if (hd == 128)
-    return launch_attention<128, false, true>((const half_t*)q, kc, vc, mask_words, cache_len_dev, out, rows,
-                                              H, G, capacity, max_len, scale, workspace, nullptr, nullptr,
-                                              0, nullptr, st, Tk, pieces, T, 0);
-  return launch_attention<64, false, true>((const half_t*)q, kc, vc, mask_words, cache_len_dev, out, rows, H,
-                                           G, capacity, max_len, scale, workspace, nullptr, nullptr, 0,
-                                           nullptr, st, Tk, pieces, T, 0);
+    return launch_attention<128, true>((const half_t*)q, kc, vc, mask_words, cache_len_dev, out, rows,
+                                              H, G, capacity, max_len, scale, workspace, st, Tk, pieces, T, 0);
+  return launch_attention<64, true>((const half_t*)q, kc, vc, mask_words, cache_len_dev, out, rows, H,
+                                           G, capacity, max_len, scale, workspace, st, Tk, pieces, T, 0);
 }
 
 EAGLE_EXPORT size_t eagle_causal_attention_workspace_bytes(int R, int H, int hd, int max_len) {
@@ -693,12 +614,10 @@ EAGLE_EXPORT int eagle_causal_attention_f16(const void* q, const void* k_cache, 
   half_t* vc = const_cast<half_t*>(static_cast<const half_t*>(v_cache));
   // the two-word form of the kernel: it keeps the cache length inside the buffer
   if (hd == 128)
-    return launch_attention<128, false, true>((const half_t*)q, kc, vc, nullptr, piece_len_dev, out, 32, H,
-                                              G, capacity, max_len, scale, workspace, nullptr, nullptr, 0,
-                                              nullptr, st, 32, R / 32);
-  return launch_attention<64, false, true>((const half_t*)q, kc, vc, nullptr, piece_len_dev, out, 32, H, G,
-                                           capacity, max_len, scale, workspace, nullptr, nullptr, 0, nullptr,
-                                           st, 32, R / 32);
+    return launch_attention<128, true>((const half_t*)q, kc, vc, nullptr, piece_len_dev, out, 32, H,
+                                              G, capacity, max_len, scale, workspace, st, 32, R / 32);
+  return launch_attention<64, true>((const half_t*)q, kc, vc, nullptr, piece_len_dev, out, 32, H, G,
+                                           capacity, max_len, scale, workspace, st, 32, R / 32);
 }
 
 EAGLE_EXPORT int eagle_rope_table_f32(const int32_t* positions, const float* inv_freqs,
@@ -712,41 +631,4 @@ EAGLE_EXPORT int eagle_rope_table_f32(const int32_t* positions, const float* inv
                      static_cast<hipStream_t>(stream), positions, inv_freqs, scaling_factor, out, T,
                      half_dim);
   return eagle_launch_status();
-}
-
-EAGLE_EXPORT size_t eagle_tree_attention_rope_workspace_bytes(int H, int hd, int max_len) {
-  return eagle_tree_attention_workspace_bytes(H, hd, max_len);
-}
-
-EAGLE_EXPORT int eagle_tree_attention_rope_f16(const void* q_lin, const void* k_lin, const void* v_lin,
-                                               long row_stride, const float* rope_cs, void* k_cache,
-                                               void* v_cache, const uint32_t* tree_mask_bits,
-                                               const int32_t* cache_len_dev, void* out, int T, int H,
-                                               int G, int hd, long capacity, int max_len, float scale,
-                                               void* workspace, size_t workspace_bytes,
-                                               eagle_stream_t stream) {
-  if (!q_lin || !k_lin || !v_lin || !rope_cs || !k_cache || !v_cache || !tree_mask_bits ||
-      !cache_len_dev || !out)
-    return EAGLE_ERR_NULL;
-  if (T < 1 || T > EAGLE_MAX_TREE || H < 1 || G < 1 || (H % G) != 0 || (H / G) > 8 ||
-      (hd != 64 && hd != 128) || max_len < T || max_len > capacity || row_stride < hd ||
-      (row_stride % 8) != 0 || !(scale > 0.f))
-    return EAGLE_ERR_SHAPE;
-  if (!eagle_aligned16(q_lin) || !eagle_aligned16(k_lin) || !eagle_aligned16(v_lin) ||
-      !eagle_aligned16(rope_cs) || !eagle_aligned16(k_cache) || !eagle_aligned16(v_cache) ||
-      !eagle_aligned16(out))
-    return EAGLE_ERR_ALIGN;
-  if (!workspace || !eagle_aligned16(workspace) ||
-      workspace_bytes < eagle_tree_attention_rope_workspace_bytes(H, hd, max_len))
-    return EAGLE_ERR_WORKSPACE;
-  hipStream_t st = static_cast<hipStream_t>(stream);
-  if (hd == 128)
-    return launch_attention<128, true>((const half_t*)q_lin, (half_t*)k_cache, (half_t*)v_cache,
-                                       tree_mask_bits, cache_len_dev, out, T, H, G, capacity, max_len, scale,
-                                       workspace, (const half_t*)k_lin, (const half_t*)v_lin, row_stride,
-                                       rope_cs, st);
-  return launch_attention<64, true>((const half_t*)q_lin, (half_t*)k_cache, (half_t*)v_cache,
-                                    tree_mask_bits, cache_len_dev, out, T, H, G, capacity, max_len, scale,
-                                    workspace, (const half_t*)k_lin, (const half_t*)v_lin, row_stride,
-                                    rope_cs, st);
 }

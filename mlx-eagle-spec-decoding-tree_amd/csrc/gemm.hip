@@ -474,12 +474,6 @@ int launch_gemm(const half_t* x, const uint32_t* w, const half_t* s, const half_
 // slab_sum_kernel below).  A last-arriver reduction inside this kernel (partial store, wait,
 // counter, loads of all slabs, store) is a chain of device-scope round trips that took longer
 // than the product itself: 14.1 us against 5.7 us for 32 x 4608 x 3584.
-#ifdef EAGLE_TRACE
-__device__ unsigned long long* g_trace = nullptr;
-#define EAGLE_TR(tr, ev) do { if ((tr) && (threadIdx.x & 63) == 0) (tr)[ev] = wall_clock64(); } while (0)
-#else
-#define EAGLE_TR(tr, ev) do { } while (0)
-#endif
 constexpr int SLAB_RING = 8;
 constexpr int SLAB_ROWS = 32;               // rows of x per accumulator tile
 constexpr int SLAB_XR = SLAB_RING * 64 + 8; // LDS row stride of an x chunk in halves
@@ -591,12 +585,6 @@ __global__ __launch_bounds__(64 * NWV) void qmm_slab_w4g64_kernel(
         *reinterpret_cast<half8_t*>(&xlds[buf * XBUF + (xr + 32 * r) * SLAB_XR + i * 64 + xc * 8]) =
             permute8(xreg[r][i]);
   };
-#ifdef EAGLE_TRACE
-  unsigned long long* tr = g_trace ? g_trace + ((size_t)(blockIdx.y * gridDim.x + blockIdx.x) * 16 + wave) * 24 : nullptr;
-#else
-  unsigned long long* tr = nullptr;
-#endif
-  EAGLE_TR(tr, 0);
   fetch_x(0);
   fetch_sb(0, s8, b8);
 #pragma unroll
@@ -607,11 +595,9 @@ __global__ __launch_bounds__(64 * NWV) void qmm_slab_w4g64_kernel(
     for (int i = 0; i < SLAB_RING; ++i) wreg[1][i] = wload(SLAB_RING + i);
   }
   __builtin_amdgcn_sched_barrier(0);
-  EAGLE_TR(tr, 1);
   stash_x(0);
   if (chunks > 1) fetch_x(1);
   __syncthreads();
-  EAGLE_TR(tr, 2);
 
   float16_t acc[MR];
 #pragma unroll
@@ -690,13 +676,9 @@ __global__ __launch_bounds__(64 * NWV) void qmm_slab_w4g64_kernel(
     int c = 0;
     for (; c + 2 < chunks; c += 2) {
       chunk(c, c & bmask, StepIndex<1>{}, StepIndex<0>{});
-      EAGLE_TR(tr, 3 + 2 * c);
       next_x(c);
-      EAGLE_TR(tr, 4 + 2 * c);
       chunk(c + 1, (c + 1) & bmask, StepIndex<1>{}, StepIndex<1>{});
-      EAGLE_TR(tr, 5 + 2 * c);
       next_x(c + 1);
-      EAGLE_TR(tr, 6 + 2 * c);
     }
     if (c + 1 < chunks) {
       chunk(c, c & bmask, StepIndex<1>{}, StepIndex<0>{});
@@ -708,13 +690,10 @@ __global__ __launch_bounds__(64 * NWV) void qmm_slab_w4g64_kernel(
   } else {
     for (int c = 0; c + 1 < chunks; ++c) {
       chunk(c, c & bmask, StepIndex<1>{}, StepIndex<0>{});
-      EAGLE_TR(tr, 3 + 2 * c);
       next_x(c);
-      EAGLE_TR(tr, 4 + 2 * c);
     }
     chunk(chunks - 1, (chunks - 1) & bmask, StepIndex<0>{}, StepIndex<0>{});
   }
-  EAGLE_TR(tr, 22);
 
   // accumulator register i of a lane: weight row 8*(i/4) + 4*hb + i%4 of the wave's tile, x
   // row ql (+ 32 for the second tile).  Through LDS, so that the lanes of a wave store whole
@@ -806,7 +785,7 @@ constexpr int BURST_SPW = 4;                 // steps of a chunk per streaming w
 
 template <bool SUBN, int NCH>
 __device__ inline void burst_stream(const uint32_t* __restrict__ wp, const half_t* __restrict__ sp, int kp, int hb,
-                                    const half_t* xrow, float16_t& acc, unsigned long long* tr) {
+                                    const half_t* xrow, float16_t& acc) {
   // wp: the wave's first block of the tiled weights (+ lane), 256 words per step; sp: the
   // tile's first block of scales | biases (+ lane), 512 halves per chunk
   uint4_t wreg[BURST_CA][BURST_SPW];
@@ -823,9 +802,7 @@ __device__ inline void burst_stream(const uint32_t* __restrict__ wp, const half_
     for (int e = 0; e < BURST_SPW; ++e) wreg[c][e] = *reinterpret_cast<const uint4_t*>(wp + (c * 8 + e) * 256);
     __builtin_amdgcn_sched_barrier(0);
   }
-  EAGLE_TR(tr, 1);
   __syncthreads();                           // x chunk 0 is in LDS
-  EAGLE_TR(tr, 2);
 #pragma unroll
   for (int c = 0; c < NCH; ++c) {
     constexpr int XBUF = SLAB_XBUF;
@@ -867,9 +844,7 @@ __device__ inline void burst_stream(const uint32_t* __restrict__ wp, const half_
       }
       if (c + BURST_CA < NCH) __builtin_amdgcn_sched_barrier(0);   // keeps the reloads in step order
     }
-    EAGLE_TR(tr, 3 + 2 * c);
     __syncthreads();                         // every wave is done with chunk c; chunk c + 1 is in LDS
-    EAGLE_TR(tr, 4 + 2 * c);
   }
 }
 
@@ -894,12 +869,6 @@ __global__ __launch_bounds__(64 * (2 * TILES + BURST_MOVERS)) void qmm_burst_w4g
   float16_t acc;
 #pragma unroll
   for (int i = 0; i < 16; ++i) acc[i] = 0.f;
-#ifdef EAGLE_TRACE
-  unsigned long long* tr = g_trace ? g_trace + ((size_t)(blockIdx.y * gridDim.x + blockIdx.x) * 16 + wv) * 24 : nullptr;
-#else
-  unsigned long long* tr = nullptr;
-#endif
-  EAGLE_TR(tr, 0);
 
   if (wv >= NSW) {
     // piece 256 i + mt of a chunk: row (256 i + mt) / 64, 16-byte column (256 i + mt) % 64.
@@ -932,24 +901,16 @@ __global__ __launch_bounds__(64 * (2 * TILES + BURST_MOVERS)) void qmm_burst_w4g
     fetch(1, StepIndex<1>{});
     stash(0, StepIndex<0>{});
     fetch(2, StepIndex<0>{});
-    EAGLE_TR(tr, 1);
     __syncthreads();
-    EAGLE_TR(tr, 2);
     // during chunk c: chunk c + 1 goes into LDS (requested two chunks ago), chunk c + 3 is requested
     for (int c = 0; c < chunks; c += 2) {
       stash(c + 1, StepIndex<1>{});
-      EAGLE_TR(tr, 3 + 3 * c);
       fetch(c + 3, StepIndex<1>{});
-      EAGLE_TR(tr, 4 + 3 * c);
       __syncthreads();
-      EAGLE_TR(tr, 5 + 3 * c);
       if (c + 1 < chunks) {
         stash(c + 2, StepIndex<0>{});
-        EAGLE_TR(tr, 6 + 3 * c);
         fetch(c + 4, StepIndex<0>{});
-        EAGLE_TR(tr, 7 + 3 * c);
         __syncthreads();
-        EAGLE_TR(tr, 8 + 3 * c);
       }
     }
   } else {
@@ -958,8 +919,8 @@ __global__ __launch_bounds__(64 * (2 * TILES + BURST_MOVERS)) void qmm_burst_w4g
     const uint32_t* wp = w + ((long)tile * G + g0 + kp * BURST_SPW) * 256 + lane * 4;
     const half_t* sp = s + ((long)tile * (G >> 3) + (g0 >> 3)) * 512 + lane * 8;
     const half_t* xrow = xlds + ql * SLAB_XR + hb * 32 + kp * BURST_SPW * 64;
-    if (NCH == NLAST || chunks == NCH) burst_stream<SUBN, NCH>(wp, sp, kp, hb, xrow, acc, tr);
-    else burst_stream<SUBN, NLAST>(wp, sp, kp, hb, xrow, acc, tr);
+    if (NCH == NLAST || chunks == NCH) burst_stream<SUBN, NCH>(wp, sp, kp, hb, xrow, acc);
+    else burst_stream<SUBN, NLAST>(wp, sp, kp, hb, xrow, acc);
   }
 
   // the second wave of a tile hands its accumulators over (register i of lane l at [tile][i][l]),
@@ -1027,7 +988,6 @@ __global__ __launch_bounds__(64 * (2 * TILES + BURST_MOVERS)) void qmm_burst_w4g
         *reinterpret_cast<float4_t*>(dst + (size_t)m * N + n) = *reinterpret_cast<const float4_t*>(&ot[m * OS + c4]);
     }
   }
-  EAGLE_TR(tr, 23);
 }
 
 template <int TILES, bool SWI, bool SUBN, int NCH, int NLAST>
@@ -1089,11 +1049,6 @@ __global__ void slab_sum_kernel(const float* __restrict__ partial, int nslab, co
 
 }  // namespace
 
-#ifdef EAGLE_TRACE
-EAGLE_EXPORT int eagle_debug_trace(void* p) {
-  return (int)hipMemcpyToSymbol(HIP_SYMBOL(g_trace), &p, sizeof(p));
-}
-#endif
 
 EAGLE_EXPORT int eagle_qmm_slab_count(int K, int steps_per_slab) {
   if (K < 128 || (K % 128) != 0 || steps_per_slab < 8 || (steps_per_slab % 8) != 0 || steps_per_slab > 4096)
