@@ -41,6 +41,7 @@ TRAFFIC_FILE = os.path.join(ROOT, "profiles", "qmm_traffic.json")
 FULL_DEPTH_BOUND = 6e-2
 PREFIX = 2048
 NODES = 32
+ACCEPT_CHAIN = 3        # draft tokens of the benchmark tree that the target accepts (see tree_verify)
 
 
 def write_traffic_record(fetch_csv, write_csv):
@@ -120,6 +121,15 @@ def qmm_shapes(args):
     per_layer = [("q", H * hd, D), ("k", G * hd, D), ("v", G * hd, D), ("o", D, H * hd),
                  ("gate", I, D), ("up", I, D), ("down", D, I)]
     return per_layer, ("lm_head", V, D)
+
+
+def pass_bytes(args, M, prefix):
+    """Algorithmic bytes of one pass of M rows through a model behind `prefix` cached tokens:
+    every quantised product once (qmm_bytes) and the K / V rows of every layer read once."""
+    per_layer, head = qmm_shapes(args)
+    L, G, hd = args.num_hidden_layers, args.num_key_value_heads, args.head_dim
+    mats = L * sum(qmm_bytes(M, n, k) for _, n, k in per_layer) + qmm_bytes(M, head[1], head[2])
+    return mats + 2.0 * L * G * (prefix + M) * hd * 2
 
 
 def graph_time_ms(torch, fn, reps, warm=2):
@@ -275,6 +285,20 @@ def main():
         ver.len_dev.copy_(len0)               # rewind: every step sees the same 2048-token prefix
         ver.forward()
 
+    # A tree of random tokens is rejected at the root.  The draft tokens along one root-to-leaf
+    # path are therefore set to what the target itself predicts there (one eager step per level:
+    # a node's logits depend on its ancestors' tokens only), so that the timed step accepts a
+    # chain of ACCEPT_CHAIN tokens and compacts their K / V rows, as a step of the loop does.
+    path = [int(np.argmax(depth))]
+    while path[-1] != 0:
+        path.append(int(parents[path[-1] - 1]))
+    path = path[::-1][:ACCEPT_CHAIN + 1]
+    for parent, child in zip(path[:-1], path[1:]):
+        one_step()
+        tokens[child] = int(ver.node_argmax[parent].item())
+        ver.set_tree(torch.from_numpy(tokens).to(dev), torch.from_numpy(depth.astype(np.int32)).to(dev),
+                     torch.from_numpy(parents).to(dev), torch.from_numpy(bits.view(np.int32)).to(dev))
+
     # ---- timed region: W warm-up replays, then exactly K replays ----
     _, graph = graph_time_ms(torch, one_step, reps=1, warm=0)
     for _ in range(opt.warmup):
@@ -409,6 +433,7 @@ def main():
                   "nodes_with_clear_margin": int(clear.sum()),
                   "clear_margin_argmax_equal": int((am_gpu[clear] == want["node_argmax"][clear]).sum()),
                   "nodes": NODES,
+                  "accept_length": int(result[1]), "accept_length_cpu": int(want["accept_length"]),
                   "accept_equal": bool(result[0] == want["best"] and result[1] == want["accept_length"]
                                        and result[3] == want["next_token"])}
         parity["ok"] = bool(parity["finite"] and err <= FULL_DEPTH_BOUND and parity["accept_equal"]
@@ -753,6 +778,18 @@ def loop_bench(opt):
         agree += int(ops.argmax_rows(logits.half()[None].contiguous()).item()) == tok
         logits = target(torch.tensor([[tok]], dtype=torch.int64, device=dev), cache=ref_cache)[0, -1].float()
     rms = float(logits.pow(2).mean().sqrt())
+    # what a step has to move at least: 1 + depth passes of k rows through the drafter and one pass of
+    # the tree's rows through the target, each reading its weights once (K / V rows priced at the
+    # prompt's length: the caches grow by a few rows per step)
+    step_bytes = (1 + depth) * pass_bytes(dargs, k, prompt_len) + pass_bytes(targs, nodes + 1, prompt_len)
+    achieved = step_bytes / (ms / steps * 1e-3) / 1e9
+    roofline = {"bound": "hbm", "kernel": f"whole loop step: {1 + depth} drafter passes of {k} rows + one target "
+                                          f"pass of {nodes + 1} rows (no single kernel dominates)",
+                "achieved": round(achieved, 1), "peak": HBM_PEAK_GBS, "unit": "GB/s",
+                "frac": round(achieved / HBM_PEAK_GBS, 4), "traffic": None,
+                "algorithmic_bytes_per_step": round(step_bytes),
+                "target_pass_bytes": round(pass_bytes(targs, nodes + 1, prompt_len)),
+                "drafter_pass_bytes": round(pass_bytes(dargs, k, prompt_len))}
     line = {
         "metric": "end-to-end tree loop, generated tokens per second (greedy)",
         "value": round(n / ms * 1e3, 2), "unit": "tokens/s", "n_gpus": 1, "steps": steps,
@@ -765,6 +802,7 @@ def loop_bench(opt):
                    "prompt_len": prompt_len, "k": k, "depth": depth, "verify_num_tokens": nodes},
         "tokens": n, "tokens_per_step": round(n / steps, 4), "prefill_ms": round(prefill_ms, 1),
         "gpu_ms_total": round(gpu_ms, 2), "wall_ms_total": round(wall_ms, 2),
+        "roofline": roofline,
         "parity": {"checked_tokens": len(emitted), "equal_to_target_greedy_stream": agree,
                    "max_logit_deficit_over_rms": round(worst / max(rms, 1e-9), 5),
                    "stream_equal": agree == len(emitted)},

@@ -243,7 +243,8 @@ int eagle_qmm_slab_partial_tiled_w4g64(const void* x, const uint32_t* wt, const 
 int eagle_qmm_slab_swiglu_tiled_w4g64_f16(const void* x, const uint32_t* wt, const void* sbt,
                                           const void* bias, void* out, int M, int N, int K,
                                           int small_scales, eagle_stream_t stream);
-/* out [M,N] fp16 = fp16(sum of the slabs) (+ bias [N] fp16, 16-byte aligned, may be NULL). */
+/* out [M,N] fp16 = fp16(sum of the slabs) (+ bias [N] fp16, 16-byte aligned, may be NULL).  M must
+ * be the M of the call that wrote the partial sums (the rows per slab, 32 or 64, follow from it). */
 int eagle_slab_sum_f16(const float* partial, int slabs, const void* bias, void* out, int M, int N,
                        eagle_stream_t stream);
 
@@ -302,8 +303,9 @@ int eagle_tree_attention_f16(const void* q, const void* k_cache, const void* v_c
 int eagle_rmsnorm_f16(const void* x, const void* residual, const void* w, float eps,
                       void* h_out, void* out, int T, int D, eagle_stream_t stream);
 /* The same with x held as fp32 partial sums of K slabs (eagle_qmm_slab_partial_w4g64 with
- * N = D): x = fp16(sum of the slabs).  T <= 64 (partial rows as that entry point lays them out
- * for M = T). */
+ * N = D): x = fp16(sum of the slabs).  T <= 64, and T must be the M of the call that wrote the
+ * partial sums: a slab holds 32 rows for M <= 32 and 64 rows above, and this kernel derives that
+ * stride from T (a smaller T over 64-row slabs would read the wrong rows). */
 int eagle_rmsnorm_slabs_f16(const float* partial, int slabs, const void* residual, const void* w,
                             float eps, void* h_out, void* out, int T, int D, eagle_stream_t stream);
 
@@ -327,7 +329,8 @@ int eagle_rope_kv_append_table_f16(const void* q_lin, const void* k_lin, const v
 /* The same with the fused q|k|v projection held as fp32 partial sums of K slabs
  * (eagle_qmm_slab_partial_w4g64 with N = (H + 2G) hd, rows [q heads | k heads | v heads]):
  * every value is fp16(sum of the slabs) + bias (bias [N] fp16, 16-byte aligned, may be NULL)
- * before the rotation.  T <= 64 (partial rows as that entry point lays them out for M = T). */
+ * before the rotation.  T <= 64, and T must be the M of the call that wrote the partial sums (the
+ * rows per slab, 32 or 64, follow from it). */
 int eagle_rope_kv_append_slabs_f16(const float* partial, int slabs, const void* bias,
                                    const float* rope_cs, void* q_out, void* k_cache, void* v_cache,
                                    const int32_t* cache_len_dev, int T, int H, int G, int hd,

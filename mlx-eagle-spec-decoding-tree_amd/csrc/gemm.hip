@@ -166,12 +166,12 @@ __global__ __launch_bounds__(256 * KGRP, (KGRP == 1 ? 2 : 1)) void qmm_gemm_w4g6
   // wave covers eight whole 128-byte rows of the step (the rate of cache lines touched, not
   // bytes, bounds the loads of this kernel)
   const int xr = tid >> 3, xc = tid & 7;
-  const half_t* xp[PP];
+  uint32_t xo[PP];                          // element offsets (the host checks M * K < 2^31)
 #pragma unroll
   for (int g = 0; g < PP; ++g) {
     int xrow = m0 + xr + 32 * g;
     if (xrow > M - 1) xrow = M - 1;         // rows past the end are never stored
-    xp[g] = x + (long)xrow * K + xc * 8;
+    xo[g] = (uint32_t)xrow * (uint32_t)K + xc * 8;
   }
   int nrow[NTW];
 #pragma unroll
@@ -196,7 +196,7 @@ __global__ __launch_bounds__(256 * KGRP, (KGRP == 1 ? 2 : 1)) void qmm_gemm_w4g6
                                             // step's as soon as this step's matrix instructions have read it
   auto fetch_x = [&](int ks, int set) {
 #pragma unroll
-    for (int g = 0; g < PP; ++g) xreg[set][g] = *reinterpret_cast<const half8_t*>(xp[g] + (long)ks * BK);
+    for (int g = 0; g < PP; ++g) xreg[set][g] = *reinterpret_cast<const half8_t*>(x + (xo[g] + (uint32_t)(ks * BK)));
   };
   auto fetch_w = [&](int ks, int p) {
 #pragma unroll
@@ -1377,6 +1377,7 @@ static int gemm_dispatch(const void* x, const uint32_t* wq, const void* scales, 
   if (group_size != 64 || bits != 4) return EAGLE_ERR_UNSUPPORTED;
   if (M < 1 || N < 8 || (N % 8) != 0 || K < 64 || (K % 64) != 0) return EAGLE_ERR_SHAPE;
   if (swiglu && (N % 32) != 0) return EAGLE_ERR_SHAPE;
+  if ((long)M * K >= (1L << 31)) return EAGLE_ERR_SHAPE;      // the kernel indexes x with 32 bits
   if (!eagle_aligned16(x) || !eagle_aligned16(wq) || !eagle_aligned16(out) ||
       (bias && (reinterpret_cast<uintptr_t>(bias) & 7u)))
     return EAGLE_ERR_ALIGN;
@@ -1416,7 +1417,7 @@ static int gemm_dispatch(const void* x, const uint32_t* wq, const void* scales, 
   if (swiglu) {
     // the wide gate|up matrix: the 128 x 256 block where it pays, else 128 x 128
     switch (sbw) {
-      case 8: return big ? launch_gemm<2, 4, 8, 1, true>(xh, wq, sh, bh, bi, oh, M, N, K, st)
+      case 8: return big ? launch_gemm<2, 4, 4, 1, true>(xh, wq, sh, bh, bi, oh, M, N, K, st)
                          : launch_gemm<1, 4, 8, 1, true>(xh, wq, sh, bh, bi, oh, M, N, K, st);
       case 4: return launch_gemm<1, 4, 4, 1, true>(xh, wq, sh, bh, bi, oh, M, N, K, st);
       case 2: return launch_gemm<1, 4, 2, 1, true>(xh, wq, sh, bh, bi, oh, M, N, K, st);
@@ -1429,6 +1430,9 @@ static int gemm_dispatch(const void* x, const uint32_t* wq, const void* scales, 
     if (!big) return launch_gemm<1, 4, 8, 2>(xh, wq, sh, bh, bi, oh, M, N, K, st);
   }
   if (small) { EAGLE_GEMM_SHAPE(1, 2) }
+  // (the 128 x 256 block takes its scales four groups per fetch at most: with eight it spills
+  // twenty registers and is no faster, 149-153 us against 143-152 us for 512 x 28672 x 4096)
+  if (big && sbw == 8) return launch_gemm<2, 4, 4>(xh, wq, sh, bh, bi, oh, M, N, K, st);
   if (big) { EAGLE_GEMM_SHAPE(2, 4) }
   EAGLE_GEMM_SHAPE(1, 4)
 #undef EAGLE_GEMM_SHAPE

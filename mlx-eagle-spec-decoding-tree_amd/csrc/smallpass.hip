@@ -103,7 +103,7 @@ enum { SMALL_PLAIN = 0, SMALL_SWIGLU = 1, SMALL_ROPE = 2 };
 constexpr int SMALL_MAXC = 3;
 constexpr int SMALL_XROW = 256 + 16;       // bytes per staged x row: 128 columns, padded against bank conflicts
 
-template <int NW, int RP, int MODE>
+template <int NW, int RP, int MODE, bool NORM>
 __global__ __launch_bounds__(NW * 64) void qmm_small_kernel(SmallArgs a) {
   constexpr int NT = MODE == SMALL_PLAIN ? 1 : 2;
   constexpr int MAXC = SMALL_MAXC;
@@ -159,7 +159,7 @@ __global__ __launch_bounds__(NW * 64) void qmm_small_kernel(SmallArgs a) {
     }
   }
   half8_t nw[MAXC][4];
-  if (a.norm_w) {
+  if (NORM && a.norm_w) {
     const half_t* np = a.norm_w + kb + kq * 32;
 #pragma unroll
     for (int c = 0; c < MAXC; ++c)
@@ -213,7 +213,7 @@ __global__ __launch_bounds__(NW * 64) void qmm_small_kernel(SmallArgs a) {
   }
 
   // ---- RMSNorm folded into x ----
-  if (a.norm_w) {
+  if (NORM && a.norm_w) {
     float ss = 0.f;
 #pragma unroll
     for (int c = 0; c < MAXC; ++c) {
@@ -366,19 +366,24 @@ constexpr int SMALL_K16 = 16 * SMALL_MAXC * 128;
 template <int MODE>
 void small_launch(const SmallArgs& a, int grid, hipStream_t st) {
   const bool tall = a.T > 8;
-#define SMALL_GO(NW)                                                                                   \
+#define SMALL_GO(NW, NORM)                                                                                \
   do {                                                                                                 \
     if (tall)                                                                                          \
-      hipLaunchKernelGGL((qmm_small_kernel<NW, 4, MODE>), dim3(grid), dim3(NW * 64), 0, st, a);        \
+      hipLaunchKernelGGL((qmm_small_kernel<NW, 4, MODE, NORM>), dim3(grid), dim3(NW * 64), 0, st, a);  \
     else                                                                                               \
-      hipLaunchKernelGGL((qmm_small_kernel<NW, 2, MODE>), dim3(grid), dim3(NW * 64), 0, st, a);        \
+      hipLaunchKernelGGL((qmm_small_kernel<NW, 2, MODE, NORM>), dim3(grid), dim3(NW * 64), 0, st, a);  \
   } while (0)
+  // Sixteen waves leave a wave 128 registers: the norm weights of its chunks (48 of them) only
+  // have room in a build of their own, so the products without a norm (o, down) get one that
+  // does not hold them.
   if (a.K <= SMALL_K4)
-    SMALL_GO(4);
+    SMALL_GO(4, true);
   else if (a.K <= SMALL_K8)
-    SMALL_GO(8);
+    SMALL_GO(8, true);
+  else if (a.norm_w)
+    SMALL_GO(16, true);
   else
-    SMALL_GO(16);
+    SMALL_GO(16, false);
 #undef SMALL_GO
 }
 

@@ -240,3 +240,24 @@ def test_length_budget_bounds_the_device_length():
     b.reset(168)
     true_len[0] = 168
     b.reserve(read)                          # 168 + 32 == 200 still fits
+
+
+def test_build_fails_on_registers_spilled_to_scratch_memory():
+    """The build reads the compiler's per-kernel resource report: a kernel outside the allowed
+    list with a non-zero scratch size is an error, one on the list is reported, none is fine."""
+    from mlx_eagle_spec_decoding_tree_amd import build
+    remark = ("a.hip:7:1: remark: Function Name: {n} [-Rpass-analysis=kernel-resource-usage]\n"
+              "a.hip:7:1: remark:     VGPRs: 128 [-Rpass-analysis=kernel-resource-usage]\n"
+              "a.hip:7:1: remark:     ScratchSize [bytes/lane]: {b} [-Rpass-analysis=kernel-resource-usage]\n")
+    clean = "_ZN12_GLOBAL__N_121qmm_burst_w4g64_kernelILi5ELb1ELb1ELi7ELi7EEEvPKDF16_"
+    listed = "_ZN12_GLOBAL__N_121qmm_gemm_w4g64_kernelILi2ELi4ELi4ELi1ELb0EEEvPKDF16_PKjS2_S2_S2_PDF16_iii"
+    rep = build.scratch_report(remark.format(n=clean, b=0) + remark.format(n=listed, b=8))
+    assert rep == {clean: 0, listed: 8}
+    allowed = build.check_scratch(rep)
+    assert list(allowed) == [listed] and allowed[listed][0] == 8
+    with pytest.raises(RuntimeError, match="spilled to scratch"):
+        build.check_scratch(build.scratch_report(remark.format(n=clean, b=48)))
+    # the drafter's down projection (sixteen waves, one tile, no norm) is not on the list
+    small = "_ZN12_GLOBAL__N_116qmm_small_kernelILi16ELi2ELi0ELb0EEEvNS_9SmallArgsE"
+    with pytest.raises(RuntimeError):
+        build.check_scratch({small: 4})
