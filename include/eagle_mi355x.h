@@ -10,6 +10,17 @@
  *
  * Each declaration cites the reference interface it replaces
  * (file:line in 0seba/mlx-eagle-spec-decoding-tree).
+ *
+ * Two groups.  DEFAULT: what the library's own verification step, draft loop and prompt pass
+ * call when nothing is chosen by hand: eagle_qmm_w4g64_f16 (+ _workspace_bytes), eagle_qmm_swiglu_*,
+ * eagle_qmm_slab_* (partial sums, SwiGLU, their tiled forms and eagle_qmm_tile_w4g64),
+ * eagle_qmv_w4g64_f16 / eagle_qmv_rows_w4g64_f16 (one and two rows), eagle_qmm_small_* and
+ * eagle_qkv_rope_small_* (a drafter's passes), eagle_qmm_gemm_* (prompt chunks), every rope, norm,
+ * attention, embedding, argmax, tree and loop-state entry point.  ON REQUEST: complete and tested,
+ * but picked by a caller only: eagle_qmm_plan / eagle_qmm_w4g64_f16_tuned (a launch shape chosen by
+ * hand), eagle_slab_sum_f16 (partial sums written out as a plain product),
+ * eagle_qmv_rows_w4g64_f16 at three to eight rows, eagle_qmm_w4g64_f16_noalloc (callers that cannot
+ * allocate).  There are no experimental entry points.
  */
 #ifndef EAGLE_MI355X_H
 #define EAGLE_MI355X_H
@@ -216,8 +227,9 @@ int eagle_qmm_slab_swiglu_w4g64_f16(const void* x, const uint32_t* wq, const voi
                                     const void* biases, const void* bias, void* out, int M, int N, int K,
                                     int group_size, int bits, eagle_stream_t stream);
 /* The weights of a projection in the layout the 32-row slab kernels stream fastest.  The
- * reference keeps every matrix row-major ([N, K/8] words, qmm_kernel.py:101-104, and re-orders
- * them offline only in its swizzle experiment, swizzle.py:41-75); read that way a wave's load
+ * reference keeps every matrix row-major ([N, K/8] words: M = w.shape[0], qmm_kernel.py:99-101)
+ * and re-orders the words offline only under its --swizzle option (swizzle.py:41-55, applied at
+ * qmm_kernel.py:221-225); read row-major, a wave's load
  * touches 32 cache lines for 1 KB.  eagle_qmm_tile_w4g64 re-lays a matrix out once (not in
  * place) as
  *   wt  [N/32 tiles][K/64 groups][64 lanes][4 words]: lane l of a wave holds words 4 (l / 32) ..

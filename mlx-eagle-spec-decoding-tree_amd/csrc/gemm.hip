@@ -757,21 +757,22 @@ __global__ __launch_bounds__(64 * NWV) void qmm_slab_w4g64_kernel(
 }
 
 // ------------------------------------------------------------------------------------------
-// The same two products (partial sums of a K slab; gate|up with the SwiGLU epilogue) with every
-// weight request of a wave in flight at once
+// The same two products (partial sums of a K slab; gate|up with the SwiGLU epilogue) with two
+// waves per weight tile and waves of their own for x
 // ------------------------------------------------------------------------------------------
-// What bounds the kernel above at 32 rows is the number of bytes a compute unit has in flight:
-// four or five waves with eight or sixteen 16-byte loads per lane are 32 - 80 KB, and at the
-// 3 - 5 us a request takes under load that is 2.3 - 4 TB/s over the whole GPU.  Here a workgroup
-// owns TILES 32-row weight tiles and one K slab of whole chunks, and
+// What bounds the kernel above at 32 rows is the rate at which a compute unit takes in bytes
+// (its weight tiles and the x chunks it re-reads from L2 alike) and the time a wave spends per
+// tile and K step when it has a SIMD to itself.  Here a workgroup owns TILES 32-row weight tiles
+// and one K slab of whole chunks (tiled weight layout only), and
 //   * two streaming waves share a weight tile: each takes four of a chunk's eight steps (a
 //     whole 128-byte line of every weight row of the tile per chunk) and keeps the loads of
-//     four chunks in flight, 16 KB per wave, issued before anything else; for a slab of up to
-//     four chunks that is every weight byte of the workgroup at the start of the kernel.
+//     BURST_CA chunks in flight, issued in the order they are needed, scales and biases first:
+//     loads retire in issue order, and every request of a long slab issued at the start puts
+//     the first chunk, which the waves wait for, behind microseconds of later ones.
 //     The chunk loop is unrolled over a compile-time chunk count, all loads unconditional;
-//   * two more waves only carry x: a whole chunk per step of their loop (global -> registers ->
-//     LDS in operand order), so that the streaming waves' in-order load counters never wait
-//     for an x load that was issued behind their prefetched weights;
+//   * BURST_MOVERS more waves only carry x: a whole chunk per step of their loop (global ->
+//     registers -> LDS in operand order, two chunks in flight in registers, BURST_XB buffers in
+//     LDS), so that the streaming waves' in-order load counters never wait for an x load;
 //   * one LDS-only barrier per chunk; at the end the second wave of a tile hands its
 //     accumulators to the first through LDS, which runs the epilogue of the kernel above.
 // SUBN: expansion through fp16 subnormals (dequant_word_sub), for |scale| < 0.0624.
