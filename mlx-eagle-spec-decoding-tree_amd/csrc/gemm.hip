@@ -776,10 +776,7 @@ __global__ __launch_bounds__(64 * NWV) void qmm_slab_w4g64_kernel(
 //   * one LDS-only barrier per chunk; at the end the second wave of a tile hands its
 //     accumulators to the first through LDS, which runs the epilogue of the kernel above.
 // SUBN: expansion through fp16 subnormals (dequant_word_sub), for |scale| < 0.0624.
-#ifndef EAGLE_BURST_CA
-#define EAGLE_BURST_CA 2
-#endif
-constexpr int BURST_CA = EAGLE_BURST_CA;     // chunks of weight loads in flight per wave
+constexpr int BURST_CA = 2;                  // chunks of weight loads in flight per wave
 constexpr int BURST_MOVERS = 4;              // waves that only carry x
 constexpr int BURST_XB = 3;                  // x chunks in LDS
 constexpr int BURST_SPW = 4;                 // steps of a chunk per streaming wave
