@@ -60,7 +60,7 @@ def write_traffic_record(fetch_csv, write_csv):
                 if r["Counter_Name"] != name:
                     continue
                 kn = r["Kernel_Name"]
-                if "qmm_w4g64" in kn or "qmm_slab_w4g64" in kn or "qmm_burst_w4g64" in kn:
+                if any(k in kn for k in ("qmm_w4g64", "qmm_slab_w4g64", "qmm_burst_w4g64", "qmm_rows_tiled")):
                     q.append(float(r["Counter_Value"]))
                 if "copyBuffer" in kn or "elementwise" in kn:
                     cp.append(float(r["Counter_Value"]))
@@ -327,6 +327,8 @@ def main():
         for wq, sc, bi, bias, x, out, form, tiled in (launches if subset is None else subset):
             if form is True:
                 ops.quantized_matmul_swiglu(x, wq, sc, bi, bias=bias, out=out, tiled=tiled)
+            elif form == "rows":
+                ops.quantized_matmul_tiled(x, tiled, bias=bias, out=out)
             elif form:
                 ops.quantized_matmul_slabs(x, wq, sc, bi, form, partial=ver.partial, tiled=tiled)
             else:
@@ -344,7 +346,10 @@ def main():
     traffic, traffic_source = read_traffic_record()
     stream_kernel = "qmm_w4g64_kernel"          # (above 32 tree tokens: two launches of it per product)
     burst = (not ver.wide) and any(l[6] is True and l[7] is not None for l in launches)
-    kernels = stream_kernel + " + qmm_slab_w4g64_kernel" + (" + qmm_burst_w4g64_kernel" if burst else "")
+    rows_form = any(l[6] == "rows" for l in launches)
+    kernels = ((stream_kernel if any(not l[6] for l in launches) else "qmm_rows_tiled_kernel")
+               + " + qmm_slab_w4g64_kernel" + (" + qmm_burst_w4g64_kernel" if burst else "")
+               + (" + qmm_rows_tiled_kernel" if rows_form and any(not l[6] for l in launches) else ""))
     roofline = {"bound": "hbm", "kernel": kernels, "achieved": round(achieved, 1),
                 "peak": HBM_PEAK_GBS, "unit": "GB/s", "frac": round(achieved / HBM_PEAK_GBS, 4),
                 "traffic": traffic, "traffic_source": traffic_source, "launches_per_step": n_launch,
@@ -361,7 +366,8 @@ def main():
     groups = ([(swi_name, [l for l in launches if l[6] is True]), (stream_kernel, [l for l in launches if not l[6]])]
               if swi_on_slab else [(stream_kernel, [l for l in launches if l[6] is True or not l[6]])])
     for kname, sub in (*groups,
-                       ("qmm_slab_w4g64_kernel", [l for l in launches if l[6] and l[6] is not True])):
+                       ("qmm_rows_tiled_kernel (vocabulary projection)", [l for l in launches if l[6] == "rows"]),
+                       ("qmm_slab_w4g64_kernel", [l for l in launches if l[6] and l[6] is not True and l[6] != "rows"])):
         if not sub:
             continue
         st, _ = graph_time_ms(torch, lambda: qmm_only(sub), reps=10)

@@ -255,6 +255,16 @@ int eagle_qmm_slab_partial_tiled_w4g64(const void* x, const uint32_t* wt, const 
 int eagle_qmm_slab_swiglu_tiled_w4g64_f16(const void* x, const uint32_t* wt, const void* sbt,
                                           const void* bias, void* out, int M, int N, int K,
                                           int small_scales, eagle_stream_t stream);
+/* The whole product from the tiled copy, out [M,N] fp16 (+ bias [N] fp16 or NULL, added in fp16
+ * after rounding), for up to 32 rows and a matrix of very many rows: the vocabulary projection
+ * (mlx_llama.py:309-312: `lm_head`, or the tied embedding's `as_linear`).  One workgroup per compute
+ * unit owns 16 or 20 32-row tiles over all of K, so that a compute unit reads x once.  M <= 32,
+ * N % 32 == 0, K % 512 == 0; small_scales as above.  Same value as eagle_qmm_w4g64_f16 to the
+ * rounding of the fp16 weights (tolerance of the tests, not bit-identical). */
+int eagle_qmm_rows_tiled_supported(int M, int N, int K);
+int eagle_qmm_rows_tiled_w4g64_f16(const void* x, const uint32_t* wt, const void* sbt, const void* bias,
+                                   void* out, int M, int N, int K, int small_scales,
+                                   eagle_stream_t stream);
 /* out [M,N] fp16 = fp16(sum of the slabs) (+ bias [N] fp16, 16-byte aligned, may be NULL).  M must
  * be the M of the call that wrote the partial sums (the rows per slab, 32 or 64, follow from it). */
 int eagle_slab_sum_f16(const float* partial, int slabs, const void* bias, void* out, int M, int N,

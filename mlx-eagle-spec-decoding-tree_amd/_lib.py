@@ -47,6 +47,8 @@ SIGNATURES = {
     "eagle_qmm_tile_w4g64": (c_int, [c_void_p] * 5 + [c_int] * 4 + [c_void_p]),
     "eagle_qmm_slab_partial_tiled_w4g64": (c_int, [c_void_p] * 4 + [c_size_t] + [c_int] * 5 + [c_void_p]),
     "eagle_qmm_slab_swiglu_tiled_w4g64_f16": (c_int, [c_void_p] * 5 + [c_int] * 4 + [c_void_p]),
+    "eagle_qmm_rows_tiled_supported": (c_int, [c_int] * 3),
+    "eagle_qmm_rows_tiled_w4g64_f16": (c_int, [c_void_p] * 5 + [c_int] * 4 + [c_void_p]),
     "eagle_qmm_slab_swiglu_supported": (c_int, [c_int] * 3),
     "eagle_qmm_slab_swiglu_preferred": (c_int, [c_int] * 3),
     "eagle_qmm_slab_swiglu_w4g64_f16": (c_int, [c_void_p] * 6 + [c_int] * 5 + [c_void_p]),

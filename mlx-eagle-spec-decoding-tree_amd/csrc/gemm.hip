@@ -1005,6 +1005,202 @@ int launch_burst(const half_t* x, const uint32_t* w, const half_t* s, const half
   return eagle_launch_status();
 }
 
+// ------------------------------------------------------------------------------------------
+// The whole product of up to 32 rows with a matrix of very many rows (a vocabulary projection),
+// fp16 out, from the tiled weight layout
+// ------------------------------------------------------------------------------------------
+// A compute unit takes in bytes at a fixed rate, the x chunks it re-reads from L2 included, so
+// the cheapest division gives every compute unit ONE pass over x: a workgroup per compute unit
+// owns 2 NSW 32-row weight tiles over all of K.  Each of its NSW streaming waves owns two tiles
+// and walks K once: per chunk of eight steps sixteen (step, tile) items, the x operand of a step
+// read from LDS once for both tiles, the packed weights of the next eight items in flight in a
+// register ring (the register of an item is loaded again for the item eight ahead as soon as it
+// has been expanded; all loads unconditional, the chunk loop's body the same every time, so the
+// wait counts are exact).  Two more waves only carry x (as in the kernel above).  At the end the
+// tile [32 x 64 NSW] goes through LDS and is stored as whole rows, bias added in fp16.
+constexpr int ROWS_MOVERS = 2;
+
+template <int NSW, bool SUBN>
+__global__ __launch_bounds__(64 * (NSW + ROWS_MOVERS)) void qmm_rows_tiled_kernel(
+    const half_t* __restrict__ x, const uint32_t* __restrict__ w, const half_t* __restrict__ s,
+    const half_t* __restrict__ bias, half_t* __restrict__ out, int M, int N, int K) {
+  extern __shared__ __attribute__((aligned(16))) half_t xlds[];   // three x chunks, then the output tile
+  constexpr int NT = 64 * (NSW + ROWS_MOVERS);
+  constexpr int XBUF = SLAB_XBUF;
+  // (step, tile) items of packed weights in flight per lane.  Sixteen (a whole chunk) were slower
+  // (74 against 68 us for 32 x 152064 x 3584) and four the same: the depth is not what bounds it.
+  constexpr int ROWS_RING = 8;
+  const int tid = threadIdx.x;
+  const int wv = tid >> 6, lane = tid & 63;
+  const int ql = lane & 31, hb = lane >> 5;
+  const int G = K >> 6;
+  const int chunks = G >> 3;
+  float16_t acc[2];
+#pragma unroll
+  for (int j = 0; j < 2; ++j)
+#pragma unroll
+    for (int i = 0; i < 16; ++i) acc[j][i] = 0.f;
+
+  if (wv >= NSW) {
+    // piece 128 i + mt of a chunk: row (128 i + mt) / 64, 16-byte column (128 i + mt) % 64
+    const int mt = tid - 64 * NSW;
+    const int r0 = mt >> 6, c8 = mt & 63;
+    half8_t xr[2][16];
+    const half_t* xb = x + c8 * 8;
+    uint32_t xo[16];                                 // element offsets of the thread's rows (M * K < 2^31)
+#pragma unroll
+    for (int i = 0; i < 16; ++i) {
+      const int row = 2 * i + r0;
+      xo[i] = (uint32_t)(row < M ? row : M - 1) * (uint32_t)K;
+    }
+    const int last = chunks - 1;
+    auto fetch = [&](int c, auto SET) {
+      constexpr int set = decltype(SET)::value;
+      const int cc = c < last ? c : last;
+#pragma unroll
+      for (int i = 0; i < 16; ++i) xr[set][i] = *reinterpret_cast<const half8_t*>(xb + (xo[i] + (uint32_t)(cc * 512)));
+    };
+    auto stash = [&](int c, auto SET) {
+      constexpr int set = decltype(SET)::value;
+      const int buf = c % BURST_XB;
+#pragma unroll
+      for (int i = 0; i < 16; ++i)
+        *reinterpret_cast<half8_t*>(&xlds[buf * XBUF + (2 * i + r0) * SLAB_XR + c8 * 8]) = permute8(xr[set][i]);
+    };
+    fetch(0, StepIndex<0>{});
+    fetch(1, StepIndex<1>{});
+    stash(0, StepIndex<0>{});
+    fetch(2, StepIndex<0>{});
+    __syncthreads();
+    for (int c = 0; c < chunks; c += 2) {
+      stash(c + 1, StepIndex<1>{});
+      fetch(c + 3, StepIndex<1>{});
+      __syncthreads();
+      if (c + 1 < chunks) {
+        stash(c + 2, StepIndex<0>{});
+        fetch(c + 4, StepIndex<0>{});
+        __syncthreads();
+      }
+    }
+  } else {
+    const int ntiles = N >> 5;
+    const uint32_t* wp[2];
+    const half_t* sp[2];
+#pragma unroll
+    for (int j = 0; j < 2; ++j) {
+      int tile = (blockIdx.x * NSW + wv) * 2 + j;    // rows past N are never stored
+      if (tile > ntiles - 1) tile = ntiles - 1;
+      wp[j] = w + (long)tile * G * 256 + lane * 4;
+      sp[j] = s + (long)tile * (G >> 3) * 512 + lane * 8;
+    }
+    const half_t* xrow = xlds + ql * SLAB_XR + hb * 32;
+    uint4_t wreg[ROWS_RING];                         // item i = 2 e + j (step e of the chunk, tile j) in register i % ROWS_RING
+    half8_t sb[2];
+#pragma unroll
+    for (int j = 0; j < 2; ++j) sb[j] = *reinterpret_cast<const half8_t*>(sp[j]);
+    __builtin_amdgcn_sched_barrier(0);
+#pragma unroll
+    for (int i = 0; i < ROWS_RING; ++i) wreg[i] = *reinterpret_cast<const uint4_t*>(wp[i & 1] + (i >> 1) * 256);
+    __builtin_amdgcn_sched_barrier(0);
+    __syncthreads();                                 // x chunk 0 is in LDS
+    const int last = chunks - 1;
+    for (int c = 0; c < chunks; ++c) {
+      // this lane loaded eight scales (lanes 0..31) or biases (32..63) per tile; exchange the
+      // halves of the wave so that every lane has both, then request the next chunk's
+      const int cn = c < last ? c + 1 : last;
+      union { half8_t h; uint32_t u[4]; } own, oth;
+      half8_t s8[2], b8[2];
+#pragma unroll
+      for (int j = 0; j < 2; ++j) {
+        own.h = sb[j];
+#pragma unroll
+        for (int i = 0; i < 4; ++i) oth.u[i] = __shfl_xor(own.u[i], 32, 64);
+        s8[j] = hb ? oth.h : own.h;
+        b8[j] = hb ? own.h : oth.h;
+        sb[j] = *reinterpret_cast<const half8_t*>(sp[j] + cn * 512);
+      }
+      __builtin_amdgcn_sched_barrier(0);
+      const half_t* xc = xrow + (c % BURST_XB) * XBUF;
+#pragma unroll
+      for (int e = 0; e < 8; ++e) {
+        half8_t bf[4];
+#pragma unroll
+        for (int k = 0; k < 4; ++k) bf[k] = *reinterpret_cast<const half8_t*>(xc + e * 64 + k * 8);
+#pragma unroll
+        for (int j = 0; j < 2; ++j) {
+          const int r = (2 * e + j) % ROWS_RING;
+          const half_t sc = s8[j][e], bi = b8[j][e];
+          half8_t af[4];
+          if constexpr (SUBN) {
+            const half_t s20 = (half_t)((float)sc * 1048576.f);
+#pragma unroll
+            for (int k = 0; k < 4; ++k) af[k] = dequant_word_sub(wreg[r][k], half2_t{s20, s20}, half2_t{bi, bi});
+          } else {
+            const half_t bc = (half_t)((float)bi + 8.f * (float)sc);
+#pragma unroll
+            for (int k = 0; k < 4; ++k) af[k] = dequant_word_centred(wreg[r][k], half2_t{sc, sc}, half2_t{bc, bc});
+          }
+          // the item ROWS_RING ahead: a later step of this chunk, or a step of the next
+          constexpr int AH = ROWS_RING / 2;          // steps ahead
+          wreg[r] = *reinterpret_cast<const uint4_t*>(wp[j] + ((e + AH < 8 ? c * 8 + e + AH : cn * 8 + e + AH - 8)) * 256);
+#pragma unroll
+          for (int k = 0; k < 4; ++k) acc[j] = __builtin_amdgcn_mfma_f32_32x32x16_f16(af[k], bf[k], acc[j], 0, 0, 0);
+        }
+        __builtin_amdgcn_sched_barrier(0);           // keeps the reloads in item order
+      }
+      __syncthreads();                               // every wave is done with chunk c; chunk c + 1 is in LDS
+    }
+  }
+
+  // accumulator register i of a lane: weight row 8 (i / 4) + 4 hb + i % 4 of the tile, x row ql
+  constexpr int HS = 64 * NSW + 8;                   // halves per row of the output tile in LDS
+  half_t* ht = xlds;
+  if (wv < NSW) {
+#pragma unroll
+    for (int j = 0; j < 2; ++j) {
+      const int col = (2 * wv + j) * 32;
+      const int n0 = blockIdx.x * (64 * NSW) + col;
+#pragma unroll
+      for (int i4 = 0; i4 < 4; ++i4) {
+        const int n = n0 + 8 * i4 + 4 * hb;
+        half4_t o;
+#pragma unroll
+        for (int e = 0; e < 4; ++e) {
+          o[e] = (half_t)acc[j][4 * i4 + e];
+          if (bias && n + e < N) o[e] = o[e] + bias[n + e];
+        }
+        *reinterpret_cast<half4_t*>(&ht[ql * HS + col + 8 * i4 + 4 * hb]) = o;
+      }
+    }
+  }
+  __syncthreads();
+  constexpr int U = 8 * NSW;                         // 16-byte pieces of a row of the tile
+  for (int idx = tid; idx < 32 * U; idx += NT) {
+    const int m = idx / U, c8 = (idx % U) * 8;
+    const int n = blockIdx.x * (64 * NSW) + c8;
+    if (m < M && n < N)
+      *reinterpret_cast<half8_t*>(out + (size_t)m * N + n) = *reinterpret_cast<const half8_t*>(&ht[m * HS + c8]);
+  }
+}
+
+template <int NSW, bool SUBN>
+int launch_rows_tiled(const half_t* x, const uint32_t* w, const half_t* s, const half_t* bias, half_t* out, int M,
+                      int N, int K, hipStream_t st) {
+  const size_t lds = BURST_XB * (size_t)SLAB_XBUF * sizeof(half_t);
+  static_assert(BURST_XB * SLAB_XBUF >= 32 * (64 * NSW + 8), "the output tile reuses the x buffers");
+  static bool configured = false;
+  if (!configured) {
+    if (hipFuncSetAttribute(reinterpret_cast<const void*>(&qmm_rows_tiled_kernel<NSW, SUBN>),
+                            hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds) != hipSuccess)
+      return EAGLE_ERR_HIP;
+    configured = true;
+  }
+  const int blocks = ((N >> 5) + 2 * NSW - 1) / (2 * NSW);
+  hipLaunchKernelGGL((qmm_rows_tiled_kernel<NSW, SUBN>), dim3(blocks), dim3(64 * (NSW + ROWS_MOVERS)), lds, st, x, w, s,
+                     bias, out, M, N, K);
+  return eagle_launch_status();
+}
+
 // The tiled layout of a weight matrix (see TL above) from the row-major one: thread = one 16-byte
 // piece of the output.
 __global__ void tile_weights_kernel(const uint32_t* __restrict__ w, const half_t* __restrict__ s,
@@ -1366,6 +1562,35 @@ EAGLE_EXPORT int eagle_qmm_slab_swiglu_tiled_w4g64_f16(const void* x, const uint
 #undef EAGLE_TL_SWI_NW
 #undef EAGLE_TL_SWI_LAUNCH
   return eagle_launch_status();
+}
+
+EAGLE_EXPORT int eagle_qmm_rows_tiled_supported(int M, int N, int K) {
+  return M >= 1 && M <= SLAB_ROWS && N >= 32 && (N % 32) == 0 && K >= 512 && (K % 512) == 0 && K <= 65536;
+}
+
+EAGLE_EXPORT int eagle_qmm_rows_tiled_w4g64_f16(const void* x, const uint32_t* wt, const void* sbt, const void* bias,
+                                                void* out, int M, int N, int K, int small_scales,
+                                                eagle_stream_t stream) {
+  if (!x || !wt || !sbt || !out) return EAGLE_ERR_NULL;
+  if (!eagle_qmm_rows_tiled_supported(M, N, K)) return EAGLE_ERR_SHAPE;
+  if (!eagle_aligned16(x) || !eagle_aligned16(wt) || !eagle_aligned16(sbt) || !eagle_aligned16(out) ||
+      (bias && (reinterpret_cast<uintptr_t>(bias) & 1u)))
+    return EAGLE_ERR_ALIGN;
+  if (x == out) return EAGLE_ERR_UNSUPPORTED;
+  hipStream_t st = static_cast<hipStream_t>(stream);
+  const half_t* xh = static_cast<const half_t*>(x);
+  const half_t* sb = static_cast<const half_t*>(sbt);
+  const half_t* bh = static_cast<const half_t*>(bias);
+  half_t* oh = static_cast<half_t*>(out);
+  // ten streaming waves (twenty tiles per workgroup) unless eight give a launch that still fits
+  // one workgroup per compute unit and fills more of them
+  const int tiles = N >> 5;
+  const bool eight = (tiles + 15) / 16 <= NUM_CU;
+  if (eight)
+    return small_scales ? launch_rows_tiled<8, true>(xh, wt, sb, bh, oh, M, N, K, st)
+                        : launch_rows_tiled<8, false>(xh, wt, sb, bh, oh, M, N, K, st);
+  return small_scales ? launch_rows_tiled<10, true>(xh, wt, sb, bh, oh, M, N, K, st)
+                      : launch_rows_tiled<10, false>(xh, wt, sb, bh, oh, M, N, K, st);
 }
 
 static int gemm_dispatch(const void* x, const uint32_t* wq, const void* scales, const void* biases,

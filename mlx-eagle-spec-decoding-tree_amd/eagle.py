@@ -422,6 +422,19 @@ def tiled_projections(model, qkv_w, gu_w, plan, swiglu):
     return out
 
 
+def tiled_head(model):
+    """`ops.TiledWeights` copy of the vocabulary projection (the tied embedding or `lm_head`,
+    mlx_llama.py:309-312) where the whole-K form on the tiled layout takes it and the matrix has
+    enough rows to give every compute unit a workgroup of that form; None otherwise.  One copy
+    per model."""
+    if not hasattr(model, "_tiled_head"):
+        head = model.model.embed_tokens if model.args.tie_word_embeddings else model.lm_head
+        n, k = head.weight.shape[0], head.weight.shape[1] * 8
+        ok = ops.rows_tiled_supported(32, n, k) and n >= 32 * 16 * 128
+        model._tiled_head = ops.tile_weights(head.weight, head.scales, head.biases) if ok else None
+    return model._tiled_head
+
+
 def slab_plan(model, T, forced=None, fused=True):
     """K steps per slab for the q|k|v, o and down projections of a pass of T rows (0: streaming
     kernel): the library's choice per shape, or `forced` ({"qkv": s, "o": s, "down": s}).  The
@@ -523,8 +536,10 @@ class TreeVerifier:
         if tiled and not fuse:
             raise ValueError("the tiled weight layout serves the fused step")
         self.tiled = None
+        self.head_tiled = None
         if (tiled or tiled is None) and fuse:
             self.tiled = tiled_projections(model, self.qkv_w, self.gu_w, self.slab, self.swiglu)
+            self.head_tiled = tiled_head(model)
         i32 = dict(dtype=torch.int32, device=dev)
         f16 = dict(dtype=torch.float16, device=dev)
         self.tokens = torch.zeros(T, **i32)
@@ -587,8 +602,9 @@ class TreeVerifier:
         """(weight, scales, biases, bias, x, out, form, tiled) of every quantised matmul of one
         step, in order; `form` is True for the launches that go through `quantized_matmul_swiglu`,
         the K steps per slab for those that go through `quantized_matmul_slabs` (into
-        `self.partial`), False for `quantized_matmul`; `tiled` the `ops.TiledWeights` copy those
-        two forms read, or None."""
+        `self.partial`), "rows" for `quantized_matmul_tiled` (the vocabulary projection on the
+        tiled layout), False for `quantized_matmul`; `tiled` the `ops.TiledWeights` copy the first
+        three forms read, or None."""
         m = self.model
         out = []
         for i, layer in enumerate(m.model.layers):
@@ -610,7 +626,8 @@ class TreeVerifier:
                         mlp.down_proj.bias, self.act, self.down, self.slab["down"] or False,
                         self._tiled("down", i)))
         head = m.model.embed_tokens if self.args.tie_word_embeddings else m.lm_head
-        out.append((head.weight, head.scales, head.biases, None, self.hn, self.logits, False, None))
+        out.append((head.weight, head.scales, head.biases, None, self.hn, self.logits,
+                    "rows" if self.head_tiled is not None else False, self.head_tiled))
         return out
 
     def _tiled(self, name, i):
@@ -655,8 +672,11 @@ class TreeVerifier:
                 self._layer_one_launch_per_projection(i, layer)
             if tap is not None:
                 tap(i, self.h)
-        head = m.model.embed_tokens if args.tie_word_embeddings else m.lm_head
-        ops.quantized_matmul(self.hn, head.weight, head.scales, head.biases, out=self.logits)
+        if self.head_tiled is not None:
+            ops.quantized_matmul_tiled(self.hn, self.head_tiled, out=self.logits)
+        else:
+            head = m.model.embed_tokens if args.tie_word_embeddings else m.lm_head
+            ops.quantized_matmul(self.hn, head.weight, head.scales, head.biases, out=self.logits)
         ops.argmax_rows(self.logits, out=self.node_argmax)
         _lib.check(L.eagle_greedy_accept(_ptr(self.node_argmax), _ptr(self.tokens),
                                          _ptr(self.retrieve), _ptr(self.shape), T,

@@ -241,6 +241,40 @@ def swiglu_supported(M, I, K):
     return I % 16 == 0 and M >= 1 and K % 64 == 0
 
 
+def rows_tiled_supported(M, N, K):
+    """Whether `quantized_matmul_tiled` takes the shape (1..32 rows per pass, N % 32 == 0, K % 512 == 0)."""
+    return bool(_lib.lib().eagle_qmm_rows_tiled_supported(int(M), int(N), int(K)))
+
+
+def quantized_matmul_tiled(x, tiled, bias=None, out=None):
+    """`quantized_matmul` of up to 32 rows (64: two passes) from the tiled copy of a matrix with
+    very many rows (the vocabulary projection, mlx_llama.py:309-312): one workgroup per compute
+    unit walks all of K over its share of the weight rows, so every compute unit reads x once.
+    Agrees with `quantized_matmul` to the tolerance of the product (fp16 weights)."""
+    _need_cuda(x, tiled.wt, tiled.sbt, bias)
+    x = _f16(x, "x")
+    *lead, K = x.shape
+    M = reduce(lambda a, b: a * b, lead, 1)
+    if K != tiled.K:
+        raise ValueError(f"shape mismatch: x {tuple(x.shape)}, tiled weights [{tiled.N}, {tiled.K}]")
+    if M < 1 or M > 64:
+        raise ValueError("quantized_matmul_tiled takes 1..64 rows")
+    if bias is not None:
+        bias = _f16(bias, "bias")
+        if tuple(bias.shape) != (tiled.N,):
+            raise ValueError("bias must have shape [N]")
+    if out is None:
+        out = torch.empty((*lead, tiled.N), dtype=torch.float16, device=x.device)
+    x2, o2 = x.reshape(M, K), out.view(M, tiled.N)
+    L = _lib.lib()
+    for r0 in range(0, M, 32):
+        r1 = min(M, r0 + 32)
+        rc = L.eagle_qmm_rows_tiled_w4g64_f16(_ptr(x2[r0:r1]), _ptr(tiled.wt), _ptr(tiled.sbt), _ptr(bias),
+                                              _ptr(o2[r0:r1]), r1 - r0, tiled.N, K, int(tiled.small), _stream())
+        _lib.check(rc, "quantized_matmul_tiled")
+    return out
+
+
 def quantized_matmul_swiglu_slab(x, w_q, scales, biases, bias=None, out=None):
     """`quantized_matmul_swiglu` for 1..64 rows on the slab kernel with one slab over all of K
     (each expanded weight feeds the matrix instructions of both 32-row tiles above 32 rows)."""

@@ -154,3 +154,69 @@ def test_refusals(dev):
     x = torch.zeros((8, 1024), dtype=torch.float16, device=dev)
     with pytest.raises(ValueError):
         ops.quantized_matmul_slabs(x, d["weight"], d["scales"], d["biases"], 8, tiled=t)
+
+
+@pytest.mark.parametrize("M,N,K,bias", [(32, 20 * 32 * 2 + 96, 1024, True), (8, 640, 512, False), (1, 32, 512, True),
+                                        (31, 16 * 32 + 32, 1536, False), (32, 152064, 3584, False),
+                                        (32, 128256, 4096, False), (8, 152064, 3584, True)])
+def test_whole_product_from_the_tiled_layout(dev, M, N, K, bias):
+    """`quantized_matmul_tiled` (the vocabulary projection's form: whole K per workgroup, fp16 out)
+    against the oracle, with both expansions; workgroups with fewer tiles than they own and rows
+    beyond M must leave the rest of `out` alone."""
+    print(f"tiled whole product M={M} N={N} K={K} bias={bias}", flush=True)
+    rng = np.random.default_rng(M + N + K)
+    layer = synth.make_qlinear(rng, N, K, bias=bias)
+    x = synth.make_x(rng, M, K)
+    want = oracle.qmm(x, layer["weight"], layer["scales"], layer["biases"], layer.get("bias"))
+    d = layer_to_dev(layer, dev)
+    t = ops.tile_weights(d["weight"], d["scales"], d["biases"])
+    assert ops.rows_tiled_supported(M, N, K)
+    for small in (True, False):
+        t.small = small
+        out = torch.full((M + 1, N), float("nan"), dtype=torch.float16, device=dev)
+        ops.quantized_matmul_tiled(to_dev(x, dev), t, bias=d.get("bias"), out=out[:M])
+        torch.cuda.synchronize()
+        assert torch.isnan(out[M:]).all()
+        assert rel_err(out[:M].cpu().numpy(), want) <= TOL, f"small={small}"
+
+
+def test_whole_product_one_hot_and_two_passes(dev):
+    """One-hot rows give fp16(s q + b) exactly (nibble order and single rounding of this kernel's
+    expansion); 40 rows run as two passes and agree with the oracle."""
+    rng = np.random.default_rng(21)
+    N, K, M = 672, 1024, 32
+    layer = synth.make_qlinear(rng, N, K)
+    d = layer_to_dev(layer, dev)
+    t = ops.tile_weights(d["weight"], d["scales"], d["biases"])
+    assert t.small
+    cols = rng.choice(K, size=M, replace=False)
+    x = np.zeros((M, K), np.float16)
+    x[np.arange(M), cols] = 1.0
+    got = ops.quantized_matmul_tiled(to_dev(x, dev), t).cpu().numpy()
+    qv = synth.unpack_nibbles(layer["weight"])[:, cols].astype(np.float32)
+    s = layer["scales"].astype(np.float32)[:, cols // 64]
+    b = layer["biases"].astype(np.float32)[:, cols // 64]
+    assert np.array_equal(got, (s * qv + b).astype(np.float16).T)
+    x = synth.make_x(rng, 40, K)
+    got = ops.quantized_matmul_tiled(to_dev(x, dev), t).cpu().numpy()
+    assert rel_err(got, oracle.qmm(x, layer["weight"], layer["scales"], layer["biases"])) <= TOL
+
+
+def test_whole_product_refusals(dev):
+    L = _lib.lib()
+    assert L.eagle_qmm_rows_tiled_supported(32, 152064, 3584) == 1
+    assert L.eagle_qmm_rows_tiled_supported(33, 152064, 3584) == 0
+    assert L.eagle_qmm_rows_tiled_supported(8, 152064, 896) == 0 and L.eagle_qmm_rows_tiled_supported(8, 48, 512) == 0
+    rng = np.random.default_rng(2)
+    layer = synth.make_qlinear(rng, 64, 512)
+    d = layer_to_dev(layer, dev)
+    t = ops.tile_weights(d["weight"], d["scales"], d["biases"])
+    with pytest.raises(ValueError):
+        ops.quantized_matmul_tiled(torch.zeros((8, 1024), dtype=torch.float16, device=dev), t)
+    with pytest.raises(ValueError):
+        ops.quantized_matmul_tiled(torch.zeros((65, 512), dtype=torch.float16, device=dev), t)
+    x = torch.zeros((8, 512), dtype=torch.float16, device=dev)
+    assert L.eagle_qmm_rows_tiled_w4g64_f16(x.data_ptr(), t.wt.data_ptr(), t.sbt.data_ptr(), None, x.data_ptr(),
+                                            8, 64, 512, 1, None) == 4          # in place
+    assert L.eagle_qmm_rows_tiled_w4g64_f16(x.data_ptr(), None, t.sbt.data_ptr(), None, x.data_ptr(),
+                                            8, 64, 512, 1, None) == 1
