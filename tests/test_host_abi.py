@@ -261,3 +261,12 @@ def test_build_fails_on_registers_spilled_to_scratch_memory():
     small = "_ZN12_GLOBAL__N_116qmm_small_kernelILi16ELi2ELi0ELb0EEEvNS_9SmallArgsE"
     with pytest.raises(RuntimeError):
         build.check_scratch({small: 4})
+
+
+def test_gemm_refuses_an_x_beyond_32_bit_indexing():
+    """The many-row matmul indexes x with 32 bits: M * K >= 2^31 is a shape error on the host."""
+    L = _lib.lib()
+    buf = (ctypes.c_char * 4096)()
+    p = (ctypes.addressof(buf) + 15) & ~15
+    assert L.eagle_qmm_gemm_w4g64_f16(p, p, p, p, None, p, 1 << 20, 64, 2048, 64, 4, None) == 2
+    assert L.eagle_qmm_gemm_w4g64_f16(None, p, p, p, None, p, 64, 64, 2048, 64, 4, None) == 1
