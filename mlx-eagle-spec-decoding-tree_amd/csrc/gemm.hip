@@ -870,8 +870,8 @@ __global__ __launch_bounds__(64 * (2 * TILES + BURST_MOVERS)) void qmm_burst_w4g
 
   if (wv >= NSW) {
     // piece 256 i + mt of a chunk: row (256 i + mt) / 64, 16-byte column (256 i + mt) % 64.
-    // Two chunks are in flight in registers and up to three sit in LDS: chunk c + 2 is written
-    // during chunk c (into the buffer chunk c - 1 used) and was requested two chunks earlier.
+    // Two chunks are in flight in registers and up to three sit in LDS: chunk c + 1 is written
+    // during chunk c (into the buffer chunk c - 2 used) and was requested two chunks earlier.
     const int mt = tid - 64 * NSW;
     const int r0 = mt >> 6, c8 = mt & 63;
     half8_t xr[2][8];

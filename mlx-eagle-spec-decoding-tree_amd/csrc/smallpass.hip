@@ -20,8 +20,9 @@
 //     workgroup repeats it, so it is kept short: v_dot2 for the sums, x / rms rounded to fp16 and
 //     then multiplied by the norm weight in packed fp16 (two roundings where the norm launch has
 //     one).
-//   * Expansion of the nibbles through fp16 subnormals as in csrc/resident.hip: fp16(s q + b),
-//     single rounding; scales below 0.2499.
+//   * Expansion of the nibbles through fp16 subnormals (a masked nibble pair at mantissa bits
+//     6..9 is q * 2^-18 exactly; one packed fma with (s * 2^18, b)): fp16(s q + b), single
+//     rounding; scales below 0.2499.
 //
 // Measured on the way (8 rows, the 0.5B drafter's shapes, launches back to back in a graph):
 //   - one wave per tile over the whole K: 2500 instructions on one wave per SIMD, 15 us per launch;
